@@ -1,0 +1,59 @@
+"""Builds libgptrs_hip.so (HIP kernels + C++ host runtime + C ABI) for gfx950 with hipcc.
+
+hipcc cross-compiles without a GPU, so this runs on any machine with ROCm installed.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libgptrs_hip.so")
+
+SOURCES = ["ptir.cpp", "fuse.cpp", "plan.cpp", "api.cpp", "kernels_generic.hip", "kernels_fused.hip",
+           "kernels_linear.hip", "kernels_attn.hip", "kernels_mfma.hip"]
+
+# -packed-fp32-ops is switched off: the compiler must not form v_pk_*_f32 from float code.
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-fast-math", "-ffp-contract=off",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
+        if cand and (os.path.isabs(cand) and os.path.exists(cand) or not os.path.isabs(cand)):
+            return cand
+    raise RuntimeError("hipcc not found")
+
+
+def _compile(src: str, obj: str, force: bool):
+    path = os.path.join(CSRC, src)
+    deps = [path] + [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")]
+    deps.append(os.path.join(HERE, "..", "include", "gptrs_hip.h"))
+    if not force and os.path.exists(obj) and all(os.path.getmtime(obj) >= os.path.getmtime(d) for d in deps):
+        return
+    cmd = [_hipcc()] + FLAGS + (["-x", "hip"] if src.endswith(".cpp") else []) + ["-c", path, "-o", obj]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src}:\n{out}")
+    if out.strip():
+        sys.stderr.write(out + "\n")
+
+
+def build_library(force: bool = False, jobs: int = 8) -> str:
+    objdir = os.path.join(CSRC, "build")
+    os.makedirs(objdir, exist_ok=True)
+    objs = [os.path.join(objdir, s.rsplit(".", 1)[0] + ".o") for s in SOURCES]
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        list(ex.map(lambda so: _compile(so[0], so[1], force), zip(SOURCES, objs)))
+    if force or not os.path.exists(LIB) or any(os.path.getmtime(o) > os.path.getmtime(LIB) for o in objs):
+        cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
+        subprocess.check_call(cmd)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build_library(force="--force" in sys.argv))

@@ -1,0 +1,550 @@
+// Backend implementation and the extern "C" surface declared in include/gptrs_hip.h.
+#include <cstring>
+
+#include "../../include/gptrs_hip.h"
+#include "runtime.hpp"
+
+namespace gptrs {
+
+// ------------------------------------------------------------------------------ device pool
+size_t DevicePool::bucket(size_t n) {
+    if (n <= 4096) return (n + 255) / 256 * 256;
+    size_t p = 4096;
+    while (p * 2 <= n) p *= 2;  // p <= n < 2p
+    const size_t step = p / 8;
+    return (n + step - 1) / step * step;
+}
+void* DevicePool::alloc(size_t bytes, size_t* cap_out) {
+    const size_t cap = bucket(bytes ? bytes : 1);
+    *cap_out = cap;
+    auto it = free_.find(cap);
+    if (it != free_.end() && !it->second.empty()) {
+        void* p = it->second.back();
+        it->second.pop_back();
+        return p;
+    }
+    void* p = nullptr;
+    hipError_t e = hipMalloc(&p, cap);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        trim();
+        e = hipMalloc(&p, cap);
+        if (e != hipSuccess) fail_exec(std::string("device allocation of ") + std::to_string(cap) + " bytes failed: " + hipGetErrorString(e));
+    }
+    bytes_allocated += cap;
+    return p;
+}
+void DevicePool::release(void* p, size_t cap) { free_[cap].push_back(p); }
+void DevicePool::trim() {
+    for (auto& kv : free_) {
+        for (void* p : kv.second) { (void)hipFree(p); bytes_allocated -= kv.first; }
+        kv.second.clear();
+    }
+}
+
+Buffer::~Buffer() {
+    if (ptr && owner) owner->release_block(ptr, cap);
+}
+
+// ------------------------------------------------------------------------------ backend
+Backend::Backend(int dev) : device(dev) {
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0)
+        fail_exec("no HIP device is visible: the hip backend has no CPU fallback");
+    if (dev < 0 || dev >= count) fail_exec("device index out of range");
+    GPTRS_HIP_CHECK(hipSetDevice(dev));
+    GPTRS_HIP_CHECK(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
+    GPTRS_HIP_CHECK(hipMalloc((void**)&d_err_flag_, 256));
+    GPTRS_HIP_CHECK(hipMalloc((void**)&d_counters_, k::kLinearCounters * sizeof(int)));
+    GPTRS_HIP_CHECK(hipMalloc((void**)&d_argmax_val_, 1024 * sizeof(float)));
+    GPTRS_HIP_CHECK(hipMalloc((void**)&d_argmax_idx_, 1024 * sizeof(int32_t)));
+    GPTRS_HIP_CHECK(hipMalloc((void**)&d_token_, 256));
+    GPTRS_HIP_CHECK(hipHostMalloc(&h_pinned_, 256, hipHostMallocDefault));
+    k::fill_zero(stream, d_err_flag_, 256);
+    k::fill_zero(stream, d_counters_, k::kLinearCounters * sizeof(int));
+    GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
+}
+
+Backend::~Backend() {
+    (void)hipSetDevice(device);
+    if (stream) (void)hipStreamSynchronize(stream);
+    for (auto& kv : params_) {
+        if (kv.second->refs.fetch_sub(1) == 1) delete kv.second;
+    }
+    params_.clear();
+    plan_index_.clear();
+    plan_lru_.clear();
+    pool_.trim();
+    (void)hipFree(d_err_flag_);
+    (void)hipFree(d_counters_);
+    (void)hipFree(d_argmax_val_);
+    (void)hipFree(d_argmax_idx_);
+    (void)hipFree(d_token_);
+    if (h_pinned_) (void)hipHostFree(h_pinned_);
+    if (stream) (void)hipStreamDestroy(stream);
+}
+
+BufferP Backend::new_buffer(size_t bytes) {
+    auto b = std::make_shared<Buffer>();
+    b->ptr = pool_.alloc(bytes, &b->cap);
+    b->owner = this;
+    return b;
+}
+
+gptrs_hip_tensor* Backend::materialize(const Spec& spec, const void* host, size_t nbytes) {
+    GPTRS_HIP_CHECK(hipSetDevice(device));
+    const size_t want = spec.bytes();
+    if (host && nbytes != want) fail_exec("literal byte length mismatch");
+    auto* t = new gptrs_hip_tensor();
+    t->spec = spec;
+    try {
+        t->buf = new_buffer(want);
+        if (!want) return t;
+        if (!host) {
+            k::fill_zero(stream, t->buf->ptr, want);
+        } else if (want <= sizeof(k::SmallPayload)) {
+            k::SmallPayload p;
+            memset(&p, 0, sizeof(p));
+            memcpy(p.w, host, want);
+            k::store_small(stream, t->buf->ptr, p, (int)want);
+        } else {
+            // pageable source: the copy is staged by the runtime; wait so the caller may reuse `host`
+            GPTRS_HIP_CHECK(hipMemcpyAsync(t->buf->ptr, host, want, hipMemcpyHostToDevice, stream));
+            GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
+        }
+    } catch (...) {
+        delete t;
+        throw;
+    }
+    return t;
+}
+
+void Backend::check_device_errors() {
+    // called after a stream synchronisation
+    int* flag = (int*)h_pinned_ + 32;
+    GPTRS_HIP_CHECK(hipMemcpyAsync(flag, d_err_flag_, sizeof(int), hipMemcpyDeviceToHost, stream));
+    GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
+    if (*flag) {
+        k::fill_zero(stream, d_err_flag_, 256);
+        fail_exec("take index out of bounds");  // cpu.rs:1632-1634
+    }
+}
+
+void Backend::to_literal(const gptrs_hip_tensor* t, void* dst, size_t cap) {
+    GPTRS_HIP_CHECK(hipSetDevice(device));
+    if (t->consumed) fail_exec("tensor handle was donated to run_program and can no longer be read");
+    const size_t n = t->spec.bytes();
+    if (cap < n) fail_exec("to_literal destination too small");
+    if (n) GPTRS_HIP_CHECK(hipMemcpyAsync(dst, t->data(), n, hipMemcpyDeviceToHost, stream));
+    GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
+    check_device_errors();
+}
+
+void Backend::synchronize() {
+    GPTRS_HIP_CHECK(hipSetDevice(device));
+    GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
+    check_device_errors();
+}
+
+gptrs_hip_tensor* Backend::param_get(const std::array<uint8_t, 16>& id) {
+    auto it = params_.find(id);
+    if (it == params_.end()) return nullptr;
+    it->second->refs.fetch_add(1);
+    return it->second;
+}
+void Backend::param_set(const std::array<uint8_t, 16>& id, gptrs_hip_tensor* t) {
+    t->refs.fetch_add(1);
+    auto it = params_.find(id);
+    if (it != params_.end()) {
+        if (it->second->refs.fetch_sub(1) == 1) delete it->second;
+        it->second = t;
+    } else {
+        params_[id] = t;
+    }
+}
+
+int64_t Backend::sample(const gptrs_hip_tensor* logits, float temperature, bool has_top_k, bool has_u, float u) {
+    GPTRS_HIP_CHECK(hipSetDevice(device));
+    if (logits->consumed) fail_exec("tensor handle was donated to run_program and can no longer be read");
+    const Spec& s = logits->spec;
+    if (!dtype_is_float(s.dtype) || s.rank() < 1 || s.rank() > 2 || s.count() == 0)
+        fail_exec("sample_decode_token expects non-empty f32/bf16 logits of rank 1 or 2");
+    const int64_t vocab = s.dims.back(), rows = s.rank() == 2 ? s.dims[0] : 1;
+    if (has_top_k) return -1;  // Ok(None): host sampler handles top-k
+    if (temperature <= 0.0f) {
+        k::argmax_last_row(stream, (int)s.dtype, logits->data(), rows, vocab, d_token_, d_argmax_val_, d_argmax_idx_, 1024);
+        n_launches += 2;
+    } else {
+        if (!has_u) return -1;
+        k::sample_temperature_last_row(stream, (int)s.dtype, logits->data(), rows, vocab, temperature, u, d_token_);
+        n_launches += 1;
+    }
+    int64_t* host = (int64_t*)h_pinned_;
+    GPTRS_HIP_CHECK(hipMemcpyAsync(host, d_token_, sizeof(int64_t), hipMemcpyDeviceToHost, stream));
+    GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
+    check_device_errors();
+    return *host;
+}
+
+std::shared_ptr<Plan> Backend::get_plan(const char* json, size_t len, uint64_t key, const uint8_t* donate, size_t n_in) {
+    uint64_t k2 = key;
+    if (key) {
+        // donation pattern and fusion switch are part of the compiled form
+        k2 = key * 1099511628211ull + (opt_fusion ? 0x9e3779b97f4a7c15ull : 0);
+        for (size_t i = 0; i < n_in; ++i) k2 = (k2 ^ (donate && donate[i] ? 0xA5 : 0x11)) * 1099511628211ull;
+        if (!k2) k2 = 1;
+        auto it = plan_index_.find(k2);
+        if (it != plan_index_.end()) {
+            plan_lru_.splice(plan_lru_.begin(), plan_lru_, it->second);
+            ++n_cache_hits;
+            return it->second->second;
+        }
+    }
+    std::vector<bool> don(n_in, false);
+    for (size_t i = 0; i < n_in; ++i) don[i] = donate && donate[i];
+    auto plan = std::make_shared<Plan>();
+    plan->fn = parse_program(json, len);
+    if (plan->fn.param_ids.size() != n_in) fail_exec("entry input arity mismatch");
+    {
+        // validate the program as written before any rewrite touches it
+        Plan check;
+        check.fn = plan->fn;
+        build_plan(check, don);
+    }
+    if (opt_fusion) plan->fused_ops = fuse_function(plan->fn);
+    build_plan(*plan, don);
+    if (plan->workspace_bytes) plan->workspace = new_buffer(plan->workspace_bytes);
+    if (!plan->const_host.empty()) {
+        plan->consts = new_buffer(plan->const_host.size());
+        GPTRS_HIP_CHECK(hipMemcpyAsync(plan->consts->ptr, plan->const_host.data(), plan->const_host.size(), hipMemcpyHostToDevice, stream));
+        GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
+    }
+    ++n_compiled;
+    n_fused += plan->fused_ops;
+    if (key) {
+        plan_lru_.emplace_front(k2, plan);
+        plan_index_[k2] = plan_lru_.begin();
+        while (plan_lru_.size() > 64) {  // program LRU of 64, as the reference arena keeps (plan.rs:20-29)
+            plan_index_.erase(plan_lru_.back().first);
+            plan_lru_.pop_back();
+        }
+    }
+    return plan;
+}
+
+void Backend::execute(Plan& plan, gptrs_hip_tensor* const* inputs, const uint8_t* donate, gptrs_hip_tensor** outputs) {
+    const Function& fn = plan.fn;
+    const size_t n_in = fn.param_ids.size();
+    for (size_t i = 0; i < n_in; ++i) {
+        if (!inputs[i]) fail_exec("null input handle");
+        if (inputs[i]->consumed) fail_exec("input " + std::to_string(i) + " was donated to an earlier run_program call");
+        if (inputs[i]->spec != fn.param_specs[i])
+            fail_exec("entry input " + std::to_string(i) + " is " + inputs[i]->spec.str() + " but the program expects " + fn.param_specs[i].str());
+    }
+    // a buffer donated for in-place update must not be reachable through another input or handle
+    std::vector<bool> inplace_ok(n_in, false);
+    for (size_t ob = 0; ob < plan.out_buffer_inplace_input.size(); ++ob) {
+        const int ip = plan.out_buffer_inplace_input[ob];
+        if (ip < 0) continue;
+        bool ok = donate && donate[ip] && inputs[ip]->refs.load() == 1 && inputs[ip]->buf.use_count() == 1;
+        for (size_t j = 0; j < n_in && ok; ++j)
+            if ((int)j != ip && inputs[j]->buf == inputs[ip]->buf) ok = false;
+        inplace_ok[ip] = ok;
+    }
+    // output buffers
+    std::vector<BufferP> out_bufs(plan.out_buffer_bytes.size());
+    for (size_t ob = 0; ob < out_bufs.size(); ++ob) {
+        const int ip = plan.out_buffer_inplace_input[ob];
+        if (ip >= 0 && inplace_ok[ip]) {
+            out_bufs[ob] = inputs[ip]->buf;
+            ++n_inplace;
+        } else {
+            out_bufs[ob] = new_buffer(plan.out_buffer_bytes[ob]);
+        }
+    }
+    ExecCtx cx;
+    cx.be = this;
+    cx.stream = stream;
+    cx.ws = plan.workspace ? (char*)plan.workspace->ptr : nullptr;
+    cx.consts = plan.consts ? (char*)plan.consts->ptr : nullptr;
+    cx.err_flag = d_err_flag_;
+    cx.counters = d_counters_;
+    cx.ptr.assign(plan.values.size(), nullptr);
+    for (size_t v = 0; v < plan.values.size(); ++v) {
+        if (!plan.values[v].defined) continue;
+        int r = plan.values[v].root;
+        while (plan.values[r].root != r) r = plan.values[r].root;
+        const RootStorage& rs = plan.storage[r];
+        switch (rs.kind) {
+            case Storage::Input: cx.ptr[v] = inputs[rs.index]->data(); break;
+            case Storage::Output: cx.ptr[v] = out_bufs[rs.index]->ptr; break;
+            case Storage::Const: cx.ptr[v] = cx.consts + rs.offset; break;
+            case Storage::Temp: cx.ptr[v] = cx.ws ? cx.ws + rs.offset : nullptr; break;
+            case Storage::InPlace: break;
+        }
+    }
+    for (const Step& st : plan.steps) run_step(plan, st, cx);
+    {
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) fail_exec(std::string("kernel launch failed: ") + hipGetErrorString(e));
+    }
+    n_launches += cx.launches;
+    last_launches = cx.launches;
+    // results
+    for (size_t i = 0; i < fn.result_ids.size(); ++i) {
+        auto* t = new gptrs_hip_tensor();
+        t->spec = fn.result_specs[i];
+        if (plan.result_input_alias[i] >= 0) t->buf = inputs[plan.result_input_alias[i]]->buf;
+        else t->buf = out_bufs[plan.out_buffer_of_result[i]];
+        outputs[i] = t;
+    }
+    for (size_t ip = 0; ip < n_in; ++ip)
+        if (inplace_ok[ip]) inputs[ip]->consumed = true;
+}
+
+void Backend::run_program(const char* json, size_t len, uint64_t key, gptrs_hip_tensor* const* inputs,
+                          const uint8_t* donate, size_t n_in, gptrs_hip_tensor** outputs, size_t n_out) {
+    GPTRS_HIP_CHECK(hipSetDevice(device));
+    auto plan = get_plan(json, len, key, donate, n_in);
+    if (plan->fn.result_ids.size() != n_out)
+        fail_exec("program produces " + std::to_string(plan->fn.result_ids.size()) + " results but " + std::to_string(n_out) + " were requested");
+    execute(*plan, inputs, donate, outputs);
+}
+
+}  // namespace gptrs
+
+// ================================================================================ C ABI
+using gptrs::Backend;
+using gptrs::BackendError;
+
+struct gptrs_hip_backend {
+    Backend impl;
+    explicit gptrs_hip_backend(int dev) : impl(dev) {}
+};
+
+static thread_local std::string g_last_error;
+
+template <typename F>
+static int guarded(F&& f) {
+    try {
+        f();
+        return GPTRS_HIP_OK;
+    } catch (const BackendError& e) {
+        g_last_error = e.what();
+        return (int)e.kind;
+    } catch (const std::exception& e) {
+        g_last_error = std::string("backend execution failure: ") + e.what();
+        return GPTRS_HIP_ERR_EXECUTION;
+    }
+}
+
+static gptrs::Spec spec_from_desc(const gptrs_hip_tensor_desc* d) {
+    if (!d) gptrs::fail_exec("null tensor descriptor");
+    gptrs::Spec s;
+    switch (d->dtype) {
+        case GPTRS_HIP_F32: s.dtype = gptrs::DType::F32; break;
+        case GPTRS_HIP_BF16: s.dtype = gptrs::DType::BF16; break;
+        case GPTRS_HIP_SI32: s.dtype = gptrs::DType::SI32; break;
+        case GPTRS_HIP_I1: s.dtype = gptrs::DType::I1; break;
+        case GPTRS_HIP_SI8: s.dtype = gptrs::DType::SI8; break;
+        case GPTRS_HIP_UI8: s.dtype = gptrs::DType::UI8; break;
+        default: gptrs::fail_spec("dtype_not_supported (dtype tag " + std::to_string(d->dtype) + ")");
+    }
+    if (d->rank > 8) gptrs::fail_spec("rank above 8");
+    for (uint32_t i = 0; i < d->rank; ++i) {
+        if (d->dims[i] < 0) gptrs::fail_spec("negative dimension");
+        s.dims.push_back(d->dims[i]);
+    }
+    return s;
+}
+
+extern "C" {
+
+int gptrs_hip_create(int device, gptrs_hip_backend** out) {
+    return guarded([&] {
+        if (!out) gptrs::fail_exec("null output pointer");
+        *out = new gptrs_hip_backend(device);
+    });
+}
+
+void gptrs_hip_destroy(gptrs_hip_backend* b) { delete b; }
+
+const char* gptrs_hip_backend_name(const gptrs_hip_backend*) { return "hip"; }
+
+int gptrs_hip_materialize(gptrs_hip_backend* b, const gptrs_hip_tensor_desc* desc, const void* host_bytes, size_t nbytes,
+                          gptrs_hip_tensor** out) {
+    return guarded([&] {
+        if (!b || !out) gptrs::fail_exec("null argument");
+        const gptrs::Spec s = spec_from_desc(desc);
+        std::lock_guard<std::mutex> g(b->impl.mu);
+        *out = b->impl.materialize(s, host_bytes, nbytes);
+    });
+}
+
+int gptrs_hip_to_literal(gptrs_hip_backend* b, const gptrs_hip_tensor* t, void* host_dst, size_t cap) {
+    return guarded([&] {
+        if (!b || !t || (!host_dst && cap)) gptrs::fail_exec("null argument");
+        std::lock_guard<std::mutex> g(b->impl.mu);
+        b->impl.to_literal(t, host_dst, cap);
+    });
+}
+
+void gptrs_hip_tensor_retain(gptrs_hip_tensor* t) {
+    if (t) t->refs.fetch_add(1);
+}
+
+void gptrs_hip_tensor_release(gptrs_hip_tensor* t) {
+    if (!t) return;
+    if (t->refs.fetch_sub(1) == 1) {
+        // returning the block to the pool touches backend state
+        gptrs::Backend* owner = t->buf ? t->buf->owner : nullptr;
+        if (owner) {
+            std::lock_guard<std::mutex> g(owner->mu);
+            delete t;
+        } else {
+            delete t;
+        }
+    }
+}
+
+int gptrs_hip_tensor_spec(const gptrs_hip_tensor* t, uint32_t* dtype_out, int64_t* dims_out, size_t dims_cap) {
+    if (!t) return -1;
+    if (dtype_out) *dtype_out = (uint32_t)t->spec.dtype;
+    for (size_t i = 0; i < t->spec.dims.size() && i < dims_cap; ++i) dims_out[i] = t->spec.dims[i];
+    return t->spec.rank();
+}
+
+int gptrs_hip_run_program_donate(gptrs_hip_backend* b, const char* program_json, size_t json_len, uint64_t program_key,
+                                 gptrs_hip_tensor* const* inputs, const uint8_t* donate, size_t n_in,
+                                 gptrs_hip_tensor** outputs, size_t n_out) {
+    return guarded([&] {
+        if (!b || !program_json || (n_in && !inputs) || (n_out && !outputs)) gptrs::fail_exec("null argument");
+        std::lock_guard<std::mutex> g(b->impl.mu);
+        b->impl.run_program(program_json, json_len, program_key, inputs, donate, n_in, outputs, n_out);
+    });
+}
+
+int gptrs_hip_run_program(gptrs_hip_backend* b, const char* program_json, size_t json_len, uint64_t program_key,
+                          gptrs_hip_tensor* const* inputs, size_t n_in, gptrs_hip_tensor** outputs, size_t n_out) {
+    return gptrs_hip_run_program_donate(b, program_json, json_len, program_key, inputs, nullptr, n_in, outputs, n_out);
+}
+
+int gptrs_hip_execute_instruction(gptrs_hip_backend* b, const char* instruction_json, size_t json_len,
+                                  gptrs_hip_tensor* const* inputs, size_t n_in, gptrs_hip_tensor** output) {
+    return guarded([&] {
+        if (!b || !instruction_json || !output) gptrs::fail_exec("null argument");
+        // Wrap the instruction into a one-instruction program whose parameters are the Value
+        // operands in order of appearance.
+        gptrs::Json j;
+        try {
+            j = gptrs::JsonParser(instruction_json, json_len).parse();
+        } catch (const gptrs::JsonError& e) {
+            gptrs::fail_spec(e.what());
+        }
+        std::string params, ids;
+        size_t nv = 0;
+        try {
+            for (auto& od : j.at("operands").as_array())
+                if (const gptrs::Json* v = od.find("Value")) {
+                    if (nv >= n_in) gptrs::fail_exec("execute_instruction: fewer inputs than Value operands");
+                    const gptrs::Spec& s = inputs[nv]->spec;
+                    std::string dims;
+                    for (size_t i = 0; i < s.dims.size(); ++i) dims += (i ? "," : "") + std::string("{\"Static\":") + std::to_string(s.dims[i]) + "}";
+                    params += (nv ? "," : "") + std::string("{\"Tensor\":{\"dtype\":\"") + gptrs::dtype_name(s.dtype) + "\",\"shape\":{\"dims\":[" + dims + "]}}}";
+                    ids += (nv ? "," : "") + std::to_string(v->as_int());
+                    ++nv;
+                }
+        } catch (const gptrs::JsonError& e) {
+            gptrs::fail_spec(e.what());
+        }
+        if (nv != n_in) gptrs::fail_exec("execute_instruction: input count does not match Value operands");
+        // result type = the instruction's own output
+        const char* p = strstr(instruction_json, "\"output\"");
+        if (!p) gptrs::fail_spec("json error: missing field `output`");
+        const char* colon = strchr(p, ':');
+        int depth = 0;
+        const char* q = colon + 1;
+        const char* start = nullptr;
+        const char* end_all = instruction_json + json_len;
+        for (; q < end_all; ++q) {
+            if (*q == '{') { if (!depth) start = q; ++depth; }
+            else if (*q == '}') { --depth; if (!depth) { ++q; break; } }
+        }
+        if (!start) gptrs::fail_spec("json error: malformed `output`");
+        const std::string out_type(start, q);
+        const std::string prog = std::string("{\"spec_version\":\"ptir.v0.4\",\"entry\":\"main\",\"functions\":[{\"name\":\"main\",\"parameters\":[") +
+                                 params + "],\"parameter_ids\":[" + ids + "],\"results\":[" + out_type + "],\"body\":[" +
+                                 std::string(instruction_json, json_len) + "],\"hints\":[],\"result_ids\":[" +
+                                 std::to_string(j.at("id").as_int()) + "]}],\"regions\":[]}";
+        std::lock_guard<std::mutex> g(b->impl.mu);
+        b->impl.run_program(prog.data(), prog.size(), 0, inputs, nullptr, n_in, output, 1);
+    });
+}
+
+int gptrs_hip_param_get(gptrs_hip_backend* b, const uint8_t id[16], gptrs_hip_tensor** out) {
+    return guarded([&] {
+        if (!b || !id || !out) gptrs::fail_exec("null argument");
+        std::array<uint8_t, 16> key;
+        memcpy(key.data(), id, 16);
+        std::lock_guard<std::mutex> g(b->impl.mu);
+        *out = b->impl.param_get(key);
+    });
+}
+
+int gptrs_hip_param_set(gptrs_hip_backend* b, const uint8_t id[16], gptrs_hip_tensor* t) {
+    return guarded([&] {
+        if (!b || !id || !t) gptrs::fail_exec("null argument");
+        std::array<uint8_t, 16> key;
+        memcpy(key.data(), id, 16);
+        std::lock_guard<std::mutex> g(b->impl.mu);
+        b->impl.param_set(key, t);
+    });
+}
+
+int gptrs_hip_supports_decode_sampling(const gptrs_hip_backend*, float temperature, int has_top_k, int has_random_u) {
+    if (has_top_k) return 0;
+    return temperature <= 0.0f || has_random_u ? 1 : 0;
+}
+
+int gptrs_hip_sample_decode_token(gptrs_hip_backend* b, const gptrs_hip_tensor* logits, float temperature, int has_top_k,
+                                  int has_random_u, float random_u, int64_t* token_out) {
+    return guarded([&] {
+        if (!b || !logits || !token_out) gptrs::fail_exec("null argument");
+        std::lock_guard<std::mutex> g(b->impl.mu);
+        *token_out = b->impl.sample(logits, temperature, has_top_k != 0, has_random_u != 0, random_u);
+    });
+}
+
+const char* gptrs_hip_last_error(void) { return g_last_error.c_str(); }
+
+int gptrs_hip_synchronize(gptrs_hip_backend* b) {
+    return guarded([&] {
+        if (!b) gptrs::fail_exec("null argument");
+        std::lock_guard<std::mutex> g(b->impl.mu);
+        b->impl.synchronize();
+    });
+}
+
+int gptrs_hip_set_option(gptrs_hip_backend* b, const char* name, int64_t value) {
+    return guarded([&] {
+        if (!b || !name) gptrs::fail_exec("null argument");
+        std::lock_guard<std::mutex> g(b->impl.mu);
+        if (!strcmp(name, "fusion")) b->impl.opt_fusion = value != 0;
+        else gptrs::fail_spec(std::string("unknown option `") + name + "`");
+    });
+}
+
+int64_t gptrs_hip_counter(const gptrs_hip_backend* b, const char* name) {
+    if (!b || !name) return -1;
+    const Backend& i = b->impl;
+    if (!strcmp(name, "kernel_launches")) return i.n_launches;
+    if (!strcmp(name, "programs_compiled")) return i.n_compiled;
+    if (!strcmp(name, "program_cache_hits")) return i.n_cache_hits;
+    if (!strcmp(name, "fused_ops")) return i.n_fused;
+    if (!strcmp(name, "bytes_allocated")) return i.bytes_allocated();
+    if (!strcmp(name, "inplace_updates")) return i.n_inplace;
+    if (!strcmp(name, "last_program_launches")) return i.last_launches;
+    return -1;
+}
+
+}  // extern "C"

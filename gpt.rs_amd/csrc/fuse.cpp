@@ -1,0 +1,763 @@
+// Backend optimizer pass: recognises the exact instruction sequences the reference's functionals
+// emit (crates/gpt-rs/src/ops/functional/*.rs) and rewrites each to one fused instruction.
+// The reference's Triton backend does the same job with #[ptir_pattern] views
+// (crates/gpt-rs-backend-triton/src/optimizer/layer_norm_fusion.rs:30-97); here the matcher runs
+// inside the executor on the program it is handed, so it needs no front-end support.
+//
+// Matching is structural on the def-use graph, rooted at the last instruction of a sequence.
+// A fused instruction takes over the root's value id; the sequence's interior instructions are
+// left in place and removed by dead-code elimination when nothing else reads them, so a value the
+// caller also asked for (e.g. layer_norm's mean) is still produced by the generic path.
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+
+#include "kernels.hpp"
+#include "runtime.hpp"
+
+namespace gptrs {
+namespace {
+
+struct Fuser {
+    Function& fn;
+    std::vector<int> def;   // value id -> body index, -1 for parameters
+    int fused = 0;
+
+    explicit Fuser(Function& f) : fn(f) { reindex(); }
+
+    void reindex() {
+        def.assign(fn.max_value_id + 1, -1);
+        for (size_t i = 0; i < fn.body.size(); ++i)
+            if (!fn.body[i].dead)
+                for (int id : fn.body[i].out_ids) def[id] = (int)i;
+    }
+    const Instr* producer(int v) const {
+        if (v < 0 || v >= (int)def.size() || def[v] < 0) return nullptr;
+        return &fn.body[def[v]];
+    }
+    const Spec* spec_of(int v) const {
+        if (v < 0) return nullptr;
+        if (const Instr* p = producer(v)) {
+            for (size_t i = 0; i < p->out_ids.size(); ++i)
+                if (p->out_ids[i] == v) return &p->out_specs[i];
+            return nullptr;
+        }
+        for (size_t i = 0; i < fn.param_ids.size(); ++i)
+            if (fn.param_ids[i] == v) return &fn.param_specs[i];
+        return nullptr;
+    }
+    // Looks through instructions that do not change the value: identity Slice / BroadcastTo /
+    // Transpose / Reshape-to-same-shape (the front end's canonicaliser removes these,
+    // crates/gpt-rs/src/backend/pipeline.rs:74-119) and StopGradient.
+    int strip(int v) const {
+        for (;;) {
+            const Instr* p = producer(v);
+            if (!p || p->operands.empty() || p->operands[0].value < 0) return v;
+            const Spec* in = spec_of(p->operands[0].value);
+            if (!in) return v;
+            bool ident = false;
+            switch (p->op) {
+                case OpKind::StopGradient: ident = true; break;
+                case OpKind::Reshape: case OpKind::BroadcastTo: ident = in->dims == p->out_specs[0].dims; break;
+                case OpKind::Slice:
+                    ident = in->dims == p->out_specs[0].dims;
+                    for (auto s : p->a) ident = ident && s == 0;
+                    break;
+                case OpKind::Transpose:
+                    ident = true;
+                    for (size_t i = 0; i < p->a.size(); ++i) ident = ident && p->a[i] == (int64_t)i;
+                    break;
+                default: break;
+            }
+            if (!ident) return v;
+            v = p->operands[0].value;
+        }
+    }
+    const Instr* prod(int v) const { return producer(strip(v)); }
+
+    // ---- small matchers; every `v` is stripped first
+    bool binary(int v, BinaryOp op, int& a, int& b) const {
+        const Instr* p = prod(v);
+        if (!p || p->op != OpKind::Binary || p->binary != op || p->scalar_rhs) return false;
+        a = p->operands[0].value;
+        b = p->operands[1].value;
+        return a >= 0 && b >= 0;
+    }
+    bool unary(int v, UnaryOp op, int& a) const {
+        const Instr* p = prod(v);
+        if (!p || p->op != OpKind::Unary || p->unary != op) return false;
+        a = p->operands[0].value;
+        return a >= 0;
+    }
+    bool bcast(int v, int& src) const {  // a real (non-identity) broadcast of a value
+        const Instr* p = prod(v);
+        if (!p || p->op != OpKind::BroadcastTo) return false;
+        src = p->operands[0].value;
+        return src >= 0;
+    }
+    bool reduce_last(int v, ReduceKind kind, int& src) const {
+        const Instr* p = prod(v);
+        if (!p || p->op != OpKind::Reduce || p->reduce != kind || !p->keepdims || p->a.size() != 1) return false;
+        src = p->operands[0].value;
+        const Spec* s = spec_of(src);
+        if (!s || s->rank() < 1) return false;
+        int64_t ax = p->a[0] < 0 ? p->a[0] + s->rank() : p->a[0];
+        return ax == s->rank() - 1;
+    }
+    static bool literal_scalar(const Literal& l, float& out) {
+        if (l.spec.count() != 1) return false;
+        if (l.spec.dtype == DType::F32) { memcpy(&out, l.bytes.data(), 4); return true; }
+        if (l.spec.dtype == DType::BF16) {
+            uint16_t b; memcpy(&b, l.bytes.data(), 2);
+            uint32_t u = (uint32_t)b << 16; memcpy(&out, &u, 4); return true;
+        }
+        return false;
+    }
+    // BroadcastTo(...BroadcastTo(Literal scalar)) chains (crates/gpt-rs/src/ops/ptir/graph.rs:757-793)
+    bool scalar(int v, float& out) const {
+        for (int depth = 0; depth < 4; ++depth) {
+            const Instr* p = producer(v);
+            if (!p) return false;
+            if (p->op == OpKind::Constant) return literal_scalar(fn.literals[p->literal], out);
+            if (p->op != OpKind::BroadcastTo && p->op != OpKind::Reshape) return false;
+            const Operand& o = p->operands[0];
+            if (o.value < 0) return literal_scalar(fn.literals[o.literal], out);
+            v = o.value;
+        }
+        return false;
+    }
+    // Add/Mul in either operand order: `pred(x)` picks which side is which
+    template <typename F>
+    bool binary_comm(int v, BinaryOp op, int& first, int& second, F is_second) const {
+        int a, b;
+        if (!binary(v, op, a, b)) return false;
+        if (is_second(b)) { first = a; second = b; return true; }
+        if (is_second(a)) { first = b; second = a; return true; }
+        return false;
+    }
+    bool vector_bcast_last(int v, int64_t n, int& vec) const {  // BroadcastTo(x[n]) along the last axis
+        int src;
+        if (!bcast(v, src)) return false;
+        const Spec* s = spec_of(src);
+        if (!s || s->rank() != 1 || s->dims[0] != n) return false;
+        vec = src;
+        return true;
+    }
+    bool slice(int v, int& src, std::vector<int64_t>& starts, std::vector<int64_t>& sizes) const {
+        const Instr* p = producer(v);  // not stripped: identity slices are handled by callers via strip()
+        if (!p || p->op != OpKind::Slice) return false;
+        src = p->operands[0].value;
+        starts = p->a;
+        sizes = p->b;
+        return src >= 0;
+    }
+    bool reshape_of(int v, int& src) const {
+        const Instr* p = producer(v);
+        if (!p || p->op != OpKind::Reshape) return false;
+        src = p->operands[0].value;
+        return src >= 0;
+    }
+    bool transpose102(int v, int& src) const {
+        const Instr* p = producer(v);
+        if (!p || p->op != OpKind::Transpose || p->a != std::vector<int64_t>{1, 0, 2}) return false;
+        src = p->operands[0].value;
+        return src >= 0;
+    }
+
+    // Replace the instruction that defines `root_v` by `ni` (placed where the root was).
+    void replace_root(int root_v, Instr ni) {
+        const int idx = def[root_v];
+        ni.dead = false;
+        fn.body[idx] = std::move(ni);
+        ++fused;
+    }
+    void kill(int v) {  // mark the (non-root) producer of a secondary output dead
+        if (def[v] >= 0) fn.body[def[v]].dead = true;
+    }
+
+    // ---------------------------------------------------------------- elementwise sequences
+    bool m_softmax(int v, int& x) const {  // ops/functional/common.rs:22-31
+        int e, sb, s, e2, sh, xx, mb, m, x2;
+        if (!binary(v, BinaryOp::Div, e, sb)) return false;
+        if (!bcast(sb, s) || !reduce_last(s, ReduceKind::Sum, e2) || strip(e2) != strip(e)) return false;
+        if (!unary(e, UnaryOp::Exp, sh) || !binary(sh, BinaryOp::Sub, xx, mb)) return false;
+        if (!bcast(mb, m) || !reduce_last(m, ReduceKind::Max, x2) || strip(x2) != strip(xx)) return false;
+        x = xx;
+        return true;
+    }
+    bool m_gelu(int v, int& x, float (&lit)[3]) const {  // activation.rs:96-113
+        int half, op, xa, l0, er, l2, sc, xb, l1;
+        if (!binary(v, BinaryOp::Mul, half, op)) return false;
+        if (!binary(half, BinaryOp::Mul, xa, l0) || !scalar(l0, lit[0])) return false;
+        if (!binary(op, BinaryOp::Add, er, l2) || !scalar(l2, lit[2])) return false;
+        if (!unary(er, UnaryOp::Erf, sc) || !binary(sc, BinaryOp::Div, xb, l1) || !scalar(l1, lit[1])) return false;
+        if (strip(xa) != strip(xb)) return false;
+        x = xa;
+        return true;
+    }
+    bool m_silu(int v, int& g) const {  // activation.rs:119-134
+        int ga, d, e, l1, n, gb, lm;
+        float one, neg;
+        if (!binary(v, BinaryOp::Div, ga, d)) return false;
+        if (!binary(d, BinaryOp::Add, e, l1) || !scalar(l1, one) || one != 1.0f) return false;
+        if (!unary(e, UnaryOp::Exp, n) || !binary(n, BinaryOp::Mul, gb, lm) || !scalar(lm, neg) || neg != -1.0f) return false;
+        if (strip(ga) != strip(gb)) return false;
+        g = ga;
+        return true;
+    }
+    bool m_layer_norm(int v, int& x, int& gamma, int& beta, float& inv_n, float& eps) const {  // normalization.rs:123-174
+        const Spec* os = spec_of(v);
+        if (!os || os->rank() < 1) return false;
+        const int64_t n = os->dims.back();
+        int t, bb, nrm, gb, cen, isb, is, ve, vm, eb, vs, ic, sq, c1, c2, xx, mb, mean, s, ic2, x2;
+        float inv2;
+        auto is_vec = [&](int q) { int tmp; return vector_bcast_last(q, n, tmp); };
+        if (!binary_comm(v, BinaryOp::Add, t, bb, is_vec) || !vector_bcast_last(bb, n, beta)) return false;
+        if (!binary_comm(t, BinaryOp::Mul, nrm, gb, is_vec) || !vector_bcast_last(gb, n, gamma)) return false;
+        if (!binary(nrm, BinaryOp::Mul, cen, isb) || !bcast(isb, is) || !unary(is, UnaryOp::Rsqrt, ve)) return false;
+        if (!binary(ve, BinaryOp::Add, vm, eb) || !scalar(eb, eps)) return false;
+        if (!binary(vm, BinaryOp::Mul, vs, ic) || !scalar(ic, inv_n)) return false;
+        if (!reduce_last(vs, ReduceKind::Sum, sq) || !binary(sq, BinaryOp::Mul, c1, c2)) return false;
+        if (strip(c1) != strip(cen) || strip(c2) != strip(cen)) return false;
+        if (!binary(cen, BinaryOp::Sub, xx, mb) || !bcast(mb, mean)) return false;
+        if (!binary(mean, BinaryOp::Mul, s, ic2) || !scalar(ic2, inv2) || inv2 != inv_n) return false;
+        if (!reduce_last(s, ReduceKind::Sum, x2) || strip(x2) != strip(xx)) return false;
+        x = xx;
+        return true;
+    }
+    bool m_rms_norm(int v, int& x, int& gamma, float& inv_n, float& eps) const {  // normalization.rs:183-217
+        const Spec* os = spec_of(v);
+        if (!os || os->rank() < 1) return false;
+        const int64_t n = os->dims.back();
+        int nrm, gb, xx, irb, ir, t, ms, eb, s, ic, sq, x1, x2;
+        auto is_vec = [&](int q) { int tmp; return vector_bcast_last(q, n, tmp); };
+        if (!binary_comm(v, BinaryOp::Mul, nrm, gb, is_vec) || !vector_bcast_last(gb, n, gamma)) return false;
+        if (!binary(nrm, BinaryOp::Mul, xx, irb) || !bcast(irb, ir) || !unary(ir, UnaryOp::Rsqrt, t)) return false;
+        if (!binary(t, BinaryOp::Add, ms, eb) || !scalar(eb, eps)) return false;
+        if (!binary(ms, BinaryOp::Mul, s, ic) || !scalar(ic, inv_n)) return false;
+        if (!reduce_last(s, ReduceKind::Sum, sq) || !binary(sq, BinaryOp::Mul, x1, x2)) return false;
+        if (strip(x1) != strip(xx) || strip(x2) != strip(xx)) return false;
+        x = xx;
+        return true;
+    }
+
+    Instr make(OpKind op, const char* name, std::vector<int> ins, int out_id, const Spec& out_spec) const {
+        Instr ni;
+        ni.op = op;
+        ni.op_name = name;
+        for (int v : ins) { Operand o; o.value = v; ni.operands.push_back(o); }
+        ni.out_ids = {out_id};
+        ni.out_specs = {out_spec};
+        return ni;
+    }
+
+    // Roots are visited last-to-first so a larger sequence claims its instructions before a
+    // smaller one nested inside it can (layer_norm contains an rms_norm-shaped tail; swiglu
+    // contains silu).
+    void pass_elementwise() {
+        for (int i = (int)fn.body.size() - 1; i >= 0; --i) {
+            Instr& in = fn.body[i];
+            if (in.dead || in.op != OpKind::Binary || in.scalar_rhs) continue;
+            const int v = in.out_ids[0];
+            const Spec out = in.out_specs[0];
+            if (!dtype_is_float(out.dtype)) continue;
+            int x, g, b, u;
+            float inv_n, eps, lit[3];
+            if (in.binary == BinaryOp::Div && m_softmax(v, x)) {
+                replace_root(v, make(OpKind::FSoftmax, "fused.softmax", {x}, v, out));
+            } else if (in.binary == BinaryOp::Add && m_layer_norm(v, x, g, b, inv_n, eps)) {
+                Instr ni = make(OpKind::FLayerNorm, "fused.layer_norm", {x, g, b}, v, out);
+                ni.scale = inv_n; ni.eps = eps;
+                replace_root(v, ni);
+            } else if (in.binary == BinaryOp::Mul && m_rms_norm(v, x, g, inv_n, eps)) {
+                Instr ni = make(OpKind::FRmsNorm, "fused.rms_norm", {x, g}, v, out);
+                ni.scale = inv_n; ni.eps = eps;
+                replace_root(v, ni);
+            } else if (in.binary == BinaryOp::Mul && m_gelu(v, x, lit)) {
+                Instr ni = make(OpKind::FGelu, "fused.gelu", {x}, v, out);
+                ni.fparam[0] = lit[0]; ni.fparam[1] = lit[1]; ni.fparam[2] = lit[2];
+                replace_root(v, ni);
+            } else if (in.binary == BinaryOp::Mul) {
+                int a = in.operands[0].value, c = in.operands[1].value;
+                if (a >= 0 && c >= 0 && m_silu(a, g)) { u = c; replace_root(v, make(OpKind::FSwiglu, "fused.swiglu", {g, u}, v, out)); }
+            } else if (in.binary == BinaryOp::Div && m_silu(v, g)) {
+                replace_root(v, make(OpKind::FSilu, "fused.silu", {g}, v, out));
+            }
+        }
+    }
+
+    // ---------------------------------------------------------------- RoPE on packed QKV
+    // rotary.rs:430-536.  Matches one head group: v == Reshape([T, H*Dh])(Transpose[1,0,2](rotated))
+    bool m_rope_group(int v, int& qkv, int64_t& col, int64_t& heads, int64_t& dh, int64_t& half, int& cos, int& sin) const {
+        int tr, rot;
+        if (!reshape_of(strip(v), tr) || !transpose102(strip(tr), rot)) return false;
+        rot = strip(rot);
+        const Instr* cat = producer(rot);
+        if (!cat || cat->op != OpKind::Concat || cat->axis != 2 || cat->operands.size() != 2) return false;
+        int fr = cat->operands[0].value, sr = cat->operands[1].value;
+        int pass = -1;
+        {   // partial rotary: Concat(2)(Concat(2)(fr, sr), pass)
+            const Instr* inner = producer(strip(fr));
+            if (inner && inner->op == OpKind::Concat && inner->axis == 2 && inner->operands.size() == 2) {
+                pass = sr;
+                fr = inner->operands[0].value;
+                sr = inner->operands[1].value;
+            }
+        }
+        int m1, m2, m3, m4, a1, c1, b1, s1, b2, c2, a2, s2;
+        if (!binary(fr, BinaryOp::Sub, m1, m2) || !binary(sr, BinaryOp::Add, m3, m4)) return false;
+        if (!binary(m1, BinaryOp::Mul, a1, c1) || !binary(m2, BinaryOp::Mul, b1, s1)) return false;
+        if (!binary(m3, BinaryOp::Mul, b2, c2) || !binary(m4, BinaryOp::Mul, a2, s2)) return false;
+        if (strip(a1) != strip(a2) || strip(b1) != strip(b2) || strip(c1) != strip(c2) || strip(s1) != strip(s2)) return false;
+        // a = Slice(xr,[0,0,0],[H,T,half]), b = Slice(xr,[0,0,half],[H,T,half])
+        int xa, xb;
+        std::vector<int64_t> st, sz, st2, sz2;
+        if (!slice(strip(a1), xa, st, sz) || !slice(strip(b1), xb, st2, sz2)) return false;
+        if (sz.size() != 3 || sz != sz2 || st != std::vector<int64_t>{0, 0, 0}) return false;
+        heads = sz[0];
+        const int64_t T = sz[1];
+        half = sz[2];
+        if (st2 != std::vector<int64_t>{0, 0, half}) return false;
+        int xh = strip(xa);  // xr (identity slice when rotary_dim == head_dim) or a real slice of xh
+        if (strip(xb) != xh) return false;
+        {
+            int src; std::vector<int64_t> s3, z3;
+            if (slice(xh, src, s3, z3)) {
+                if (s3 != std::vector<int64_t>{0, 0, 0} || z3 != std::vector<int64_t>{heads, T, 2 * half}) return false;
+                xh = strip(src);
+            }
+        }
+        const Spec* xs = spec_of(xh);
+        if (!xs || xs->rank() != 3 || xs->dims[0] != heads || xs->dims[1] != T) return false;
+        dh = xs->dims[2];
+        if (2 * half > dh) return false;
+        if (pass >= 0) {
+            int ps; std::vector<int64_t> s4, z4;
+            if (!slice(strip(pass), ps, s4, z4) || strip(ps) != xh) return false;
+            if (s4 != std::vector<int64_t>{0, 0, 2 * half} || z4 != std::vector<int64_t>{heads, T, dh - 2 * half}) return false;
+        } else if (2 * half != dh) {
+            return false;
+        }
+        // xh = Transpose[1,0,2](Reshape([T,H,dh])(Slice(qkv,[0,col],[T,H*dh])))
+        int rs, sl, q;
+        std::vector<int64_t> s5, z5;
+        if (!transpose102(xh, rs) || !reshape_of(strip(rs), sl)) return false;
+        const Spec* rss = spec_of(strip(rs));
+        if (!rss || rss->dims != std::vector<int64_t>{T, heads, dh}) return false;
+        if (!slice(sl, q, s5, z5) || s5.size() != 2 || s5[0] != 0 || z5 != std::vector<int64_t>{T, heads * dh}) return false;
+        qkv = q;
+        col = s5[1];
+        // cos/sin: BroadcastTo([H,T,half])(Reshape([1,T,half])(cos))
+        auto table = [&](int cv, int& tab) {
+            int r;
+            const Instr* p = producer(strip(cv));
+            if (!p) return false;
+            if (p->op == OpKind::BroadcastTo) {
+                if (p->out_specs[0].dims != std::vector<int64_t>{heads, T, half}) return false;
+                r = p->operands[0].value;
+            } else {
+                r = strip(cv);  // heads == 1: the broadcast is an identity
+            }
+            if (r < 0) return false;
+            int src;
+            if (!reshape_of(strip(r), src)) return false;
+            const Spec* ts = spec_of(src);
+            if (!ts || ts->dims != std::vector<int64_t>{T, half}) return false;
+            tab = src;
+            return true;
+        };
+        return table(c1, cos) && table(s1, sin);
+    }
+
+    void pass_rope() {
+        for (size_t i = 0; i < fn.body.size(); ++i) {
+            Instr& in = fn.body[i];
+            if (in.dead || in.op != OpKind::Concat || in.axis != 1 || in.operands.size() != 3) continue;
+            const Spec out = in.out_specs[0];
+            if (out.rank() != 2 || !dtype_is_float(out.dtype)) continue;
+            const int qv = in.operands[0].value, kv = in.operands[1].value, vv = in.operands[2].value;
+            if (qv < 0 || kv < 0 || vv < 0) continue;
+            int qkv_q, qkv_k, cq, sq, ck, sk;
+            int64_t colq, hq, dq, halfq, colk, hk, dk, halfk;
+            if (!m_rope_group(qv, qkv_q, colq, hq, dq, halfq, cq, sq)) continue;
+            if (!m_rope_group(kv, qkv_k, colk, hk, dk, halfk, ck, sk)) continue;
+            if (qkv_q != qkv_k || cq != ck || sq != sk || dq != dk || halfq != halfk) continue;
+            if (colq != 0 || colk != hq * dq) continue;
+            int vsrc; std::vector<int64_t> s, z;
+            if (!slice(strip(vv), vsrc, s, z) || vsrc != qkv_q) continue;
+            const int64_t T = out.dims[0];
+            if (s != std::vector<int64_t>{0, (hq + hk) * dq} || z != std::vector<int64_t>{T, hk * dq}) continue;
+            const Spec* qs = spec_of(qkv_q);
+            if (!qs || qs->dims != out.dims || out.dims[1] != (hq + 2 * hk) * dq) continue;
+            Instr ni = make(OpKind::FRope, "fused.rope_qkv_packed", {qkv_q, cq, sq}, in.out_ids[0], out);
+            ni.n_q = hq; ni.n_kv = hk; ni.head_dim = dq; ni.rot_half = halfq;
+            replace_root(in.out_ids[0], ni);
+        }
+    }
+
+    // ---------------------------------------------------------------- attention
+    // Walks Reshape / BroadcastTo([Hkv,g,L,Dh]) / Reshape back to the [Hkv, L, Dh] source of a
+    // grouped K or V operand (attention.rs:703-711).
+    bool group_source(int v, int64_t hq, int64_t L, int64_t dh, int& src, int64_t& hkv) const {
+        int64_t g = 1;
+        for (int depth = 0; depth < 6; ++depth) {
+            v = strip(v);
+            const Spec* s = spec_of(v);
+            if (!s) return false;
+            const Instr* p = producer(v);
+            if (p && p->op == OpKind::Reshape) { v = p->operands[0].value; if (v < 0) return false; continue; }
+            if (p && p->op == OpKind::BroadcastTo) {
+                const Spec* is = spec_of(p->operands[0].value);
+                const Spec& os = p->out_specs[0];
+                if (!is || os.rank() != 4 || is->rank() != 4 || is->dims[1] != 1 || is->dims[0] != os.dims[0] ||
+                    is->dims[2] != L || is->dims[3] != dh || os.dims[2] != L || os.dims[3] != dh)
+                    return false;
+                g = os.dims[1];
+                v = p->operands[0].value;
+                continue;
+            }
+            if (s->rank() == 3 && s->dims[1] == L && s->dims[2] == dh && s->dims[0] * g == hq) {
+                src = v;
+                hkv = s->dims[0];
+                return true;
+            }
+            return false;
+        }
+        return false;
+    }
+    bool is_dot(int v, std::vector<int64_t> bl, std::vector<int64_t> br, std::vector<int64_t> cl, std::vector<int64_t> cr,
+                int& a, int& b) const {
+        const Instr* p = producer(strip(v));
+        if (!p || p->op != OpKind::Dot || p->a != bl || p->b != br || p->c != cl || p->d != cr) return false;
+        a = p->operands[0].value;
+        b = p->operands[1].value;
+        return a >= 0 && b >= 0;
+    }
+    // select(qpos >= pos, 0, -big): returns the compare's operands
+    bool m_mask_select(int v, int& lhs, int& rhs) const {
+        const Instr* p = producer(strip(v));
+        if (!p || p->op != OpKind::Select) return false;
+        const Instr* c = producer(strip(p->operands[0].value));
+        float z, ng;
+        if (!c || c->op != OpKind::Compare || c->cmp != CmpOp::GreaterEqual) return false;
+        if (p->operands[1].value < 0 || p->operands[2].value < 0) return false;
+        if (!scalar(p->operands[1].value, z) || !scalar(p->operands[2].value, ng)) return false;
+        // the kernels drop masked terms outright, exact only while exp(mask + s - max) underflows to 0
+        if (z != 0.0f || !(ng <= -1e8f)) return false;
+        lhs = c->operands[0].value;
+        rhs = c->operands[1].value;
+        return lhs >= 0 && rhs >= 0;
+    }
+    bool is_iota(int v, int64_t axis) const {
+        const Instr* p = producer(strip(v));
+        return p && p->op == OpKind::Iota && p->axis == axis;
+    }
+    // packed-QKV column block: Reshape(dims)(Slice(qkv,[0,col],[T,width])), optionally transposed
+    bool m_qkv_block(int v, bool transposed, int& qkv, int64_t& col, int64_t& width) const {
+        v = strip(v);
+        if (transposed) { int t; if (!transpose102(v, t)) return false; v = strip(t); }
+        int sl;
+        if (!reshape_of(v, sl)) return false;
+        std::vector<int64_t> s, z;
+        if (!slice(strip(sl), qkv, s, z) || s.size() != 2 || s[0] != 0) return false;
+        col = s[1];
+        width = z[1];
+        return true;
+    }
+
+    static bool decode_kernel_ok(DType dt, int64_t hq, int64_t hkv, int64_t dh) {
+        const int64_t vec = 16 / (int64_t)dtype_size(dt);
+        if (dh % vec || dh > 256) return false;
+        const int64_t lpr = dh / vec;
+        if (lpr > 64 || (lpr & (lpr - 1))) return false;
+        const int64_t g = hq / hkv;
+        return g == 1 || g == 2 || g == 4 || g == 8;
+    }
+
+    void pass_attention() {
+        for (size_t i = 0; i < fn.body.size(); ++i) {
+            Instr& in = fn.body[i];
+            if (in.dead || in.op != OpKind::Reshape) continue;
+            const Spec out = in.out_specs[0];
+            if (out.rank() != 2 || !dtype_is_float(out.dtype) || in.operands[0].value < 0) continue;
+            const int64_t T = out.dims[0];
+            int c = strip(in.operands[0].value);
+            bool prefill = false;
+            { int t; if (transpose102(c, t)) { prefill = true; c = strip(t); } }
+            int P, Vg;
+            if (!is_dot(c, {0}, {0}, {2}, {1}, P, Vg)) continue;
+            const Spec* cs = spec_of(c);
+            if (!cs || cs->rank() != 3 || cs->dims[1] != T) continue;
+            const int64_t hq = cs->dims[0], dh = cs->dims[2];
+            if (out.dims[1] != hq * dh) continue;
+            const Instr* sm = producer(strip(P));
+            if (!sm || sm->op != OpKind::FSoftmax) continue;
+            const int S3 = sm->operands[0].value;
+            const Spec* ss = spec_of(S3);
+            if (!ss || ss->rank() != 3) continue;
+            const int64_t L = ss->dims[2];  // keys attended (capacity in decode, T in prefill)
+            int S2, mk, S, scb, Q, Kg;
+            float scale;
+            auto is_mask = [&](int q) { const Instr* p = producer(strip(q)); return p && p->op == OpKind::BroadcastTo; };
+            if (!binary_comm(S3, BinaryOp::Add, S2, mk, is_mask)) continue;
+            if (!binary(S2, BinaryOp::Mul, S, scb) || !scalar(scb, scale)) continue;
+            if (!is_dot(S, {0}, {0}, {2}, {2}, Q, Kg)) continue;
+            int Ksrc, Vsrc;
+            int64_t hkv, hkv2;
+            if (!group_source(Kg, hq, L, dh, Ksrc, hkv) || !group_source(Vg, hq, L, dh, Vsrc, hkv2) || hkv != hkv2) continue;
+            // mask: BroadcastTo chain down to the Select
+            int mv = mk;
+            for (int d = 0; d < 3; ++d) { int src; if (bcast(mv, src)) mv = src; else break; }
+            int cl, cr;
+            if (!m_mask_select(mv, cl, cr)) continue;
+            int qkv, qkv2, qkv3;
+            int64_t col, width;
+            if (!prefill) {
+                if (T != 1) continue;
+                // K' = DynamicUpdateSlice(cacheK, Reshape(Slice(qkv)), update_starts), same for V'
+                const Instr* ku = producer(strip(Ksrc));
+                const Instr* vu = producer(strip(Vsrc));
+                if (!ku || !vu || ku->op != OpKind::DynamicUpdateSlice || vu->op != OpKind::DynamicUpdateSlice) continue;
+                if (ku->operands[2].value < 0 || ku->operands[2].value != vu->operands[2].value) continue;
+                if (ku->a != std::vector<int64_t>{hkv, 1, dh} || vu->a != ku->a) continue;
+                const int cache_k = ku->operands[0].value, cache_v = vu->operands[0].value;
+                if (cache_k < 0 || cache_v < 0 || ku->operands[1].value < 0 || vu->operands[1].value < 0) continue;
+                if (!m_qkv_block(Q, false, qkv, col, width) || col != 0 || width != hq * dh) continue;
+                if (!m_qkv_block(ku->operands[1].value, false, qkv2, col, width) || qkv2 != qkv || col != hq * dh || width != hkv * dh) continue;
+                if (!m_qkv_block(vu->operands[1].value, false, qkv3, col, width) || qkv3 != qkv || col != (hq + hkv) * dh || width != hkv * dh) continue;
+                const Spec* qs = spec_of(qkv);
+                if (!qs || qs->dims != std::vector<int64_t>{1, (hq + 2 * hkv) * dh}) continue;
+                // mask compare: BroadcastTo([C])(DynamicSlice{[1]}(iota, query_start)) >= iota
+                int qp, ds_src;
+                if (!is_iota(cr, 0) || !bcast(cl, qp)) continue;
+                const Instr* dsl = producer(strip(qp));
+                if (!dsl || dsl->op != OpKind::DynamicSlice || dsl->a != std::vector<int64_t>{1}) continue;
+                ds_src = dsl->operands[0].value;
+                if (ds_src < 0 || !is_iota(ds_src, 0) || dsl->operands[1].value < 0) continue;
+                const Spec* ios = spec_of(strip(ds_src));
+                if (!ios || ios->dims != std::vector<int64_t>{L}) continue;
+                if (!decode_kernel_ok(out.dtype, hq, hkv, dh)) continue;
+                const int kout = ku->out_ids[0], vout = vu->out_ids[0];
+                Instr ni = make(OpKind::FAttnDecode, "fused.attention_decode_cache",
+                                {qkv, cache_k, cache_v, ku->operands[2].value, dsl->operands[1].value}, in.out_ids[0], out);
+                ni.out_ids = {in.out_ids[0], kout, vout};
+                ni.out_specs = {out, ku->out_specs[0], vu->out_specs[0]};
+                ni.n_q = hq; ni.n_kv = hkv; ni.head_dim = dh; ni.scale = scale;
+                kill(kout);
+                kill(vout);
+                replace_root(in.out_ids[0], ni);
+                reindex();
+            } else {
+                if (L != T || dh > 256) continue;
+                if (!is_iota(cl, 0) || !is_iota(cr, 1)) continue;
+                const Spec* i0 = spec_of(strip(cl));
+                if (!i0 || i0->dims != std::vector<int64_t>{T, T}) continue;
+                if (!m_qkv_block(Q, true, qkv, col, width) || col != 0 || width != hq * dh) continue;
+                if (!m_qkv_block(Ksrc, true, qkv2, col, width) || qkv2 != qkv || col != hq * dh || width != hkv * dh) continue;
+                if (!m_qkv_block(Vsrc, true, qkv3, col, width) || qkv3 != qkv || col != (hq + hkv) * dh || width != hkv * dh) continue;
+                const Spec* qs = spec_of(qkv);
+                if (!qs || qs->dims != std::vector<int64_t>{T, (hq + 2 * hkv) * dh}) continue;
+                if (hq % hkv) continue;
+                Instr ni = make(OpKind::FAttnPrefill, "fused.attention_prefill", {qkv}, in.out_ids[0], out);
+                ni.n_q = hq; ni.n_kv = hkv; ni.head_dim = dh; ni.scale = scale;
+                replace_root(in.out_ids[0], ni);
+            }
+        }
+    }
+
+    // ---------------------------------------------------------------- linear layers
+    std::vector<int> count_uses() const {
+        std::vector<int> uses(fn.max_value_id + 1, 0);
+        for (auto& in : fn.body)
+            if (!in.dead)
+                for (auto& o : in.operands)
+                    if (o.value >= 0) ++uses[o.value];
+        for (int r : fn.result_ids) ++uses[r];
+        return uses;
+    }
+
+    void pass_linear() {
+        // 1. x[M,K] . W[K,N] -> FLinear
+        for (auto& in : fn.body) {
+            if (in.dead || in.op != OpKind::Dot) continue;
+            if (!in.a.empty() || !in.b.empty() || in.c != std::vector<int64_t>{1} || in.d != std::vector<int64_t>{0}) continue;
+            if (in.operands[0].value < 0 || in.operands[1].value < 0) continue;
+            const Spec* l = spec_of(in.operands[0].value);
+            const Spec* r = spec_of(in.operands[1].value);
+            if (!l || !r || l->rank() != 2 || r->rank() != 2 || !dtype_is_float(l->dtype)) continue;
+            in.op = OpKind::FLinear;
+            in.op_name = "fused.linear";
+            in.act = 0;
+            ++fused;
+        }
+        reindex();
+        // 2. epilogues, each absorbed only when the linear's value has no other reader
+        bool changed = true;
+        while (changed) {
+            changed = false;
+            const std::vector<int> uses = count_uses();
+            for (size_t i = 0; i < fn.body.size() && !changed; ++i) {
+                Instr& in = fn.body[i];
+                if (in.dead) continue;
+                const int v = in.out_ids[0];
+                auto linear_of = [&](int q) -> Instr* {
+                    if (q < 0 || def[q] < 0) return nullptr;
+                    Instr* p = &fn.body[def[q]];
+                    return (p->op == OpKind::FLinear && !p->dead && uses[q] == 1) ? p : nullptr;
+                };
+                if (in.op == OpKind::Binary && in.binary == BinaryOp::Add && !in.scalar_rhs) {
+                    const int a = in.operands[0].value, b = in.operands[1].value;
+                    if (a < 0 || b < 0) continue;
+                    // bias: Add(linear, BroadcastTo(b[N]))  (tensor_ops.rs:42-56)
+                    Instr* lin = linear_of(a);
+                    int vec;
+                    if (lin && !lin->has_bias && !lin->has_residual && lin->act == 0 &&
+                        vector_bcast_last(b, in.out_specs[0].dims.back(), vec)) {
+                        Instr ni = *lin;
+                        Operand o; o.value = vec;
+                        ni.operands.push_back(o);
+                        ni.has_bias = true;
+                        ni.out_ids = {v};
+                        lin->dead = true;
+                        fn.body[i] = ni;
+                        reindex();
+                        changed = true;
+                        continue;
+                    }
+                    // residual: Add(linear, r) or Add(r, linear)
+                    for (int side = 0; side < 2 && !changed; ++side) {
+                        Instr* l2 = linear_of(side == 0 ? a : b);
+                        const int other = side == 0 ? b : a;
+                        if (!l2 || l2->has_residual || l2->act == 2) continue;
+                        if (def[other] >= 0 && def[other] > def[l2->out_ids[0]]) {
+                            // the residual is produced after the linear: fine, the fused op sits at the Add
+                        }
+                        const Spec* os = spec_of(other);
+                        if (!os || *os != in.out_specs[0]) continue;
+                        Instr ni = *l2;
+                        Operand o; o.value = other;
+                        ni.operands.push_back(o);
+                        ni.has_residual = true;
+                        ni.out_ids = {v};
+                        l2->dead = true;
+                        fn.body[i] = ni;
+                        reindex();
+                        changed = true;
+                    }
+                } else if (in.op == OpKind::FGelu) {
+                    Instr* lin = linear_of(in.operands[0].value);
+                    if (lin && lin->act == 0 && !lin->has_residual && in.fparam[0] == 0.5f && in.fparam[1] == 1.41421354f &&
+                        in.fparam[2] == 1.0f) {
+                        Instr ni = *lin;
+                        ni.act = 1;
+                        ni.out_ids = {v};
+                        lin->dead = true;
+                        fn.body[i] = ni;
+                        reindex();
+                        changed = true;
+                    }
+                } else if (in.op == OpKind::FSwiglu) {
+                    Instr* lg = linear_of(in.operands[0].value);
+                    Instr* lu = linear_of(in.operands[1].value);
+                    if (lg && lu && lg != lu && lg->act == 0 && lu->act == 0 && !lg->has_bias && !lu->has_bias &&
+                        !lg->has_residual && !lu->has_residual && lg->operands[0].value == lu->operands[0].value) {
+                        const Spec* wg = spec_of(lg->operands[1].value);
+                        const Spec* wu = spec_of(lu->operands[1].value);
+                        if (wg && wu && *wg == *wu) {
+                            Instr ni = *lg;
+                            ni.operands.push_back(lu->operands[1]);
+                            ni.act = 2;
+                            ni.out_ids = {v};
+                            lg->dead = true;
+                            lu->dead = true;
+                            fn.body[i] = ni;
+                            reindex();
+                            changed = true;
+                        }
+                    }
+                }
+            }
+        }
+    }
+
+    // Binary ops whose rhs is a broadcast scalar literal read the scalar as a kernel argument.
+    void pass_scalar_rhs() {
+        for (auto& in : fn.body) {
+            if (in.dead || in.op != OpKind::Binary || in.scalar_rhs) continue;
+            const int b = in.operands[1].value;
+            float val;
+            if (b < 0 || !scalar(b, val)) continue;
+            const Instr* p = producer(b);
+            if (!p || p->op != OpKind::BroadcastTo) continue;
+            in.scalar_rhs = true;
+            in.scalar_val = val;
+            in.operands.resize(1);
+        }
+    }
+
+    void dce() {
+        std::vector<bool> live(fn.max_value_id + 1, false);
+        for (int r : fn.result_ids) live[r] = true;
+        for (int i = (int)fn.body.size() - 1; i >= 0; --i) {
+            Instr& in = fn.body[i];
+            if (in.dead) continue;
+            bool any = false;
+            for (int id : in.out_ids) any = any || live[id];
+            if (!any) { in.dead = true; continue; }
+            for (auto& o : in.operands)
+                if (o.value >= 0) live[o.value] = true;
+        }
+        reindex();
+    }
+
+    // Stable topological order: a fused instruction sits at its root's position, which can be
+    // before the producer of an operand that the original sequence only read later.
+    void toposort() {
+        const size_t n = fn.body.size();
+        std::vector<bool> placed_val(fn.max_value_id + 1, false);
+        for (int p : fn.param_ids) placed_val[p] = true;
+        std::vector<bool> done(n, false);
+        std::vector<Instr> order;
+        order.reserve(n);
+        size_t remaining = 0;
+        for (auto& in : fn.body) if (!in.dead) ++remaining;
+        while (remaining) {
+            bool progress = false;
+            for (size_t i = 0; i < n; ++i) {
+                if (done[i] || fn.body[i].dead) continue;
+                bool ready = true;
+                for (auto& o : fn.body[i].operands)
+                    if (o.value >= 0 && !placed_val[o.value]) { ready = false; break; }
+                if (!ready) continue;
+                for (int id : fn.body[i].out_ids) placed_val[id] = true;
+                order.push_back(fn.body[i]);
+                done[i] = true;
+                --remaining;
+                progress = true;
+            }
+            if (!progress) fail_exec("operand value missing");
+        }
+        fn.body = std::move(order);
+        reindex();
+    }
+};
+
+}  // namespace
+
+int fuse_function(Function& fn) {
+    Fuser f(fn);
+    f.dce();
+    f.pass_elementwise();
+    f.dce();
+    f.pass_rope();
+    f.pass_attention();
+    f.dce();
+    f.pass_linear();
+    f.dce();
+    f.pass_scalar_rhs();
+    f.dce();
+    f.toposort();
+    return f.fused;
+}
+
+}  // namespace gptrs

@@ -1,0 +1,131 @@
+// Launchers for the HIP kernels (gfx950).  Plain-pointer interfaces; all launches are
+// asynchronous on the given stream.  Shapes are validated by the executor before any call.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace gptrs {
+namespace k {
+
+constexpr int kMaxRank = 6;
+
+// dst[dst_off + sum c_i*dst_stride_i] = src[src_off + sum c_i*src_stride_i] over `dims`.
+// Strides in elements.  dyn: 0 static; 1 = add clamp(starts[i],0,dyn_max[i])*dyn_stride[i] to the
+// SOURCE offset (DynamicSlice, cpu.rs:804-820); 2 = to the DEST offset (DynamicUpdateSlice).
+struct CopyDesc {
+    int rank = 0;
+    int dyn = 0;
+    int64_t total = 0;
+    int64_t dst_off = 0, src_off = 0;
+    int64_t dims[kMaxRank] = {};
+    int64_t dst_stride[kMaxRank] = {};
+    int64_t src_stride[kMaxRank] = {};
+    int dyn_rank = 0;
+    int64_t dyn_max[kMaxRank] = {};
+    int64_t dyn_stride[kMaxRank] = {};
+};
+void copy_strided(hipStream_t s, void* dst, const void* src, int elem_size, const CopyDesc& d, const int32_t* starts);
+
+// Up to 256 payload bytes travel as kernel arguments: an upload with no staging buffer and
+// no host synchronisation (token ids, positions, update_starts, RoPE rows).
+struct SmallPayload { uint32_t w[64]; };
+void store_small(hipStream_t s, void* dst, const SmallPayload& p, int nbytes);
+void fill_zero(hipStream_t s, void* dst, size_t nbytes);
+
+// dtype: 0 f32, 2 bf16 (tags of include/gptrs_hip.h).  Math in f32, output rounded to dtype.
+void unary(hipStream_t s, int dtype, int op, const void* x, void* y, int64_t n);
+void binary(hipStream_t s, int dtype, int op, const void* a, const void* b, void* y, int64_t n);
+// b is a scalar (broadcast literal) -- used when the rhs is BroadcastTo(scalar literal)
+void binary_scalar(hipStream_t s, int dtype, int op, const void* a, float b, void* y, int64_t n);
+void compare(hipStream_t s, int dtype, int op, const void* a, const void* b, uint8_t* y, int64_t n);
+void select(hipStream_t s, int elem_size, const uint8_t* p, const void* t, const void* f, void* y, int64_t n);
+void cast(hipStream_t s, int src_dtype, int dst_dtype, const void* x, void* y, int64_t n);
+void iota(hipStream_t s, int32_t* y, int64_t outer, int64_t axis_len, int64_t inner);
+// x viewed as [outer][axis_len][inner]; kind 0 sum 1 max 2 min; f32 accumulation
+void reduce(hipStream_t s, int dtype, int kind, const void* x, void* y, int64_t outer, int64_t axis_len, int64_t inner);
+// rows of `table` ([vocab][inner] elements of elem_size) by si32 index; an out-of-range index
+// zero-fills the row and raises *err_flag (checked at the next synchronising call)
+void take(hipStream_t s, int elem_size, const void* table, const int32_t* idx, void* y, int64_t n_idx,
+          int64_t vocab, int64_t inner, int* err_flag);
+
+// C[b][m][n] = sum_k A[b][m][k] * B[b][k][n]; element strides given per operand; f32 accumulate.
+struct DotDesc {
+    int64_t batch, m, n, k;
+    int64_t a_sb, a_sm, a_sk;
+    int64_t b_sb, b_sk, b_sn;
+    int64_t c_sb, c_sm;  // C is [b][m][n] with n contiguous
+};
+void dot_generic(hipStream_t s, int dtype, const void* a, const void* b, void* c, const DotDesc& d);
+
+// last row of [rows][vocab] logits; ties -> smallest index; result (int64) written to *out
+void argmax_last_row(hipStream_t s, int dtype, const void* logits, int64_t rows, int64_t vocab, int64_t* out,
+                     float* scratch_val, int32_t* scratch_idx, int scratch_cap);
+// temperature sampling with a caller-supplied uniform u (inverse-CDF over softmax(logits/T))
+void sample_temperature_last_row(hipStream_t s, int dtype, const void* logits, int64_t rows, int64_t vocab,
+                                 float temperature, float u, int64_t* out);
+
+// ---- fused kernels (kernels_fused.hip) --------------------------------------------------
+// y[r] = LN(x[r]) * gamma + beta over the last axis, two-pass (mean, then centred variance):
+// ops/functional/normalization.rs:123-174.  inv_n is the f32-rounded 1/N multiplier.
+void layer_norm(hipStream_t s, int dtype, const void* x, const void* gamma, const void* beta, void* y,
+                int64_t rows, int64_t n, float inv_n, float eps);
+// y = x * rsqrt(mean(x^2)+eps) * gamma: normalization.rs:183-217
+void rms_norm(hipStream_t s, int dtype, const void* x, const void* gamma, void* y, int64_t rows, int64_t n,
+              float inv_n, float eps);
+void softmax_rows(hipStream_t s, int dtype, const void* x, void* y, int64_t rows, int64_t n);
+void gelu(hipStream_t s, int dtype, const void* x, void* y, int64_t n, float half, float inv_div, float one);
+void swiglu(hipStream_t s, int dtype, const void* gate, const void* up, void* y, int64_t n);  // up==nullptr: silu
+
+// Linear layer y[M,N] = act(x[M,K] . W[K,N] + bias) (+ residual), W row-major [in,out]
+// (nn/layers/linear.rs:50-71).  act: 0 none, 1 exact-erf gelu.  w2 != nullptr: SwiGLU pair,
+// y = silu(x.W) * (x.W2).  Picks a bandwidth-bound GEMV kernel for small M and an MFMA tile
+// kernel for large M.  `ws` is a scratch buffer of at least linear_workspace_bytes().
+struct LinearArgs {
+    int dtype;
+    const void* x; const void* w; const void* w2; const void* bias; const void* residual;
+    void* y;
+    int64_t m, k, n;
+    int act;
+    void* ws; size_t ws_bytes;
+    int* counters;  // >= kLinearCounters zero-initialised ints, left zero by every launch
+};
+constexpr int kLinearCounters = 4096;
+size_t linear_workspace_bytes(int dtype, int64_t m, int64_t k, int64_t n, bool dual);
+void linear(hipStream_t s, const LinearArgs& a);
+
+// Rotate-half RoPE on packed [T, Q|K|V] rows (ops/functional/rotary.rs:430-536).
+void rope_packed(hipStream_t s, int dtype, const void* qkv, const void* cos, const void* sin, void* out,
+                 int64_t t, int64_t n_q, int64_t n_kv, int64_t head_dim, int64_t half);
+
+// Decode attention over a fixed-capacity cache (ops/functional/attention.rs:657-779), T = 1.
+// Appends this step's K/V rows at clamp(update_starts[1]) into k_out/v_out (which already hold
+// the previous cache contents: either the donated buffers or a copy) and attends over positions
+// 0..=query_start[0].
+struct AttnDecodeArgs {
+    int dtype;
+    const void* qkv;            // [1, (n_q + 2 n_kv) * head_dim]
+    void* k_cache; void* v_cache;  // [n_kv, capacity, head_dim], updated in place
+    const int32_t* update_starts;  // si32[3]
+    const int32_t* query_start;    // si32[1]
+    void* ctx;                  // [1, n_q * head_dim]
+    int64_t n_q, n_kv, head_dim, capacity;
+    float scale;
+    void* ws; size_t ws_bytes;
+};
+size_t attn_decode_workspace_bytes(int64_t n_q, int64_t head_dim, int64_t capacity);
+void attn_decode(hipStream_t s, const AttnDecodeArgs& a);
+
+// Prefill causal attention (ops/functional/attention.rs:443-522): packed qkv [T, P] ->
+// ctx [T, n_q*head_dim], and K/V in cache layout [n_kv, T, head_dim].
+struct AttnPrefillArgs {
+    int dtype;
+    const void* qkv;
+    void* ctx; void* k_out; void* v_out;
+    int64_t t, n_q, n_kv, head_dim;
+    float scale;
+};
+void attn_prefill(hipStream_t s, const AttnPrefillArgs& a);
+
+}  // namespace k
+}  // namespace gptrs

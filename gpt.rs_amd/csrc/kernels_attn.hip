@@ -1,0 +1,293 @@
+// Causal attention kernels for the two sequences the reference emits:
+//   * attention_decode_cache (crates/gpt-rs/src/ops/functional/attention.rs:657-779), T = 1
+//   * attention without cache (attention.rs:443-522), prefill
+// Both compute softmax((q.k) * scale + mask) . v with the additive -1e9 mask replaced by its
+// exact f32 effect: masked positions contribute exactly 0 (exp underflows), so only positions
+// <= the query position are visited.  GQA: query head h reads kv head h / group.
+#include "kernels.hpp"
+#include "device_utils.hpp"
+
+namespace gptrs {
+namespace k {
+
+static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p, int64_t i);
+template <> __device__ __forceinline__ float ldf<float>(const float* p, int64_t i) { return p[i]; }
+template <> __device__ __forceinline__ float ldf<bf16_t>(const bf16_t* p, int64_t i) { return bf16_to_f32(p[i]); }
+template <typename T> __device__ __forceinline__ void stf(T* p, int64_t i, float v);
+template <> __device__ __forceinline__ void stf<float>(float* p, int64_t i, float v) { p[i] = v; }
+template <> __device__ __forceinline__ void stf<bf16_t>(bf16_t* p, int64_t i, float v) { p[i] = f32_to_bf16(v); }
+
+template <typename T> struct Vec16;
+template <> struct Vec16<float> {
+    static constexpr int N = 4;
+    static __device__ __forceinline__ void load(const float* p, float (&o)[4]) {
+        const float4 v = *reinterpret_cast<const float4*>(p);
+        o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+    }
+};
+template <> struct Vec16<bf16_t> {
+    static constexpr int N = 8;
+    static __device__ __forceinline__ void load(const bf16_t* p, float (&o)[8]) {
+        const uint4 v = *reinterpret_cast<const uint4*>(p);
+        o[0] = bf16lo(v.x); o[1] = bf16hi(v.x); o[2] = bf16lo(v.y); o[3] = bf16hi(v.y);
+        o[4] = bf16lo(v.z); o[5] = bf16hi(v.z); o[6] = bf16lo(v.w); o[7] = bf16hi(v.w);
+    }
+};
+
+__device__ __forceinline__ int64_t clamp_i64(int64_t v, int64_t lo, int64_t hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+// ------------------------------------------------------------------------------ decode
+// grid (n_kv, nsplit), 256 threads.  A cache row (head_dim elements) is read by LPR lanes with one
+// 16-byte load each, so a wave streams 64/LPR positions at a time; every such lane-group keeps
+// its own online-softmax state for the G query heads of this kv head.  States are merged by
+// shuffles inside the wave, through LDS across the four waves, and across splits by
+// attn_decode_combine_kernel.
+template <typename T, int G>
+__global__ __launch_bounds__(256) void attn_decode_kernel(const T* __restrict__ qkv, T* __restrict__ kc,
+                                                          T* __restrict__ vc, const int32_t* __restrict__ us,
+                                                          const int32_t* __restrict__ qs, T* __restrict__ ctx,
+                                                          float* __restrict__ ws, int n_q, int n_kv, int dh,
+                                                          int64_t cap, float scale, int64_t chunk, int nsplit) {
+    constexpr int VEC = Vec16<T>::N;
+    const int lpr = dh / VEC;          // lanes per cache row (power of two, <= 64)
+    const int rpw = 64 / lpr;          // rows per wave-iteration
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int sub = lane / lpr, li = lane % lpr;
+    const int nstream = 4 * rpw, sid = wave * rpw + sub;
+    const int kvh = blockIdx.x, split = blockIdx.y;
+
+    const int64_t qpos = clamp_i64(qs[0], 0, cap - 1);   // DynamicSlice clamp (cpu.rs:804-820)
+    const int64_t upd = clamp_i64(us[1], 0, cap - 1);    // DynamicUpdateSlice clamp on the position axis
+    const T* knew = qkv + (int64_t)n_q * dh + (int64_t)kvh * dh;
+    const T* vnew = qkv + (int64_t)(n_q + n_kv) * dh + (int64_t)kvh * dh;
+
+    // append this step's row (exactly one block per kv head owns position `upd`)
+    if (upd / chunk == split) {
+        for (int d = threadIdx.x; d < dh; d += 256) {
+            kc[((int64_t)kvh * cap + upd) * dh + d] = knew[d];
+            vc[((int64_t)kvh * cap + upd) * dh + d] = vnew[d];
+        }
+    }
+
+    const int64_t p0 = (int64_t)split * chunk;
+    int64_t p1 = p0 + chunk;
+    if (p1 > qpos + 1) p1 = qpos + 1;
+
+    float qf[G][VEC];
+#pragma unroll
+    for (int g = 0; g < G; ++g) Vec16<T>::load(qkv + (int64_t)(kvh * G + g) * dh + li * VEC, qf[g]);
+
+    float m[G], l[G], o[G][VEC];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        m[g] = -INFINITY; l[g] = 0.f;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) o[g][v] = 0.f;
+    }
+
+    for (int64_t p = p0 + sid; p < p1; p += nstream) {
+        float kf[VEC], vf[VEC];
+        if (p == upd) {
+            Vec16<T>::load(knew + li * VEC, kf);
+            Vec16<T>::load(vnew + li * VEC, vf);
+        } else {
+            Vec16<T>::load(kc + ((int64_t)kvh * cap + p) * dh + li * VEC, kf);
+            Vec16<T>::load(vc + ((int64_t)kvh * cap + p) * dh + li * VEC, vf);
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            float s = 0.f;
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) s += qf[g][v] * kf[v];
+            for (int off = 1; off < lpr; off <<= 1) s += __shfl_xor(s, off, 64);
+            s *= scale;
+            const float mn = fmaxf(m[g], s);
+            const float corr = expf(m[g] - mn);
+            const float pe = expf(s - mn);
+            l[g] = l[g] * corr + pe;
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) o[g][v] = o[g][v] * corr + pe * vf[v];
+            m[g] = mn;
+        }
+    }
+
+    // merge the rpw lane-groups of this wave
+    for (int off = lpr; off < 64; off <<= 1) {
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const float om = __shfl_xor(m[g], off, 64);
+            const float ol = __shfl_xor(l[g], off, 64);
+            const float mn = fmaxf(m[g], om);
+            const float ca = mn == -INFINITY ? 0.f : expf(m[g] - mn);
+            const float cb = mn == -INFINITY ? 0.f : expf(om - mn);
+            l[g] = l[g] * ca + ol * cb;
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) {
+                const float ov = __shfl_xor(o[g][v], off, 64);
+                o[g][v] = o[g][v] * ca + ov * cb;
+            }
+            m[g] = mn;
+        }
+    }
+
+    // merge the four waves through LDS
+    __shared__ float sm[4][G], sl[4][G];
+    __shared__ float so[4][G][256];
+    if (sub == 0) {
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            if (li == 0) { sm[wave][g] = m[g]; sl[wave][g] = l[g]; }
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) so[wave][g][li * VEC + v] = o[g][v];
+        }
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < G * dh; idx += 256) {
+        const int g = idx / dh, d = idx % dh;
+        float mn = fmaxf(fmaxf(sm[0][g], sm[1][g]), fmaxf(sm[2][g], sm[3][g]));
+        float L = 0.f, O = 0.f;
+        if (mn != -INFINITY) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const float c = expf(sm[w][g] - mn);
+                L += sl[w][g] * c;
+                O += so[w][g][d] * c;
+            }
+        }
+        const int h = kvh * G + g;
+        if (nsplit == 1) {
+            stf(ctx, (int64_t)h * dh + d, O / L);
+        } else {
+            float* rec = ws + ((int64_t)h * nsplit + split) * (dh + 2);
+            if (d == 0) { rec[0] = mn; rec[1] = L; }
+            rec[2 + d] = O;
+        }
+    }
+}
+
+template <typename T>
+__global__ void attn_decode_combine_kernel(const float* __restrict__ ws, T* __restrict__ ctx, int dh, int nsplit) {
+    const int h = blockIdx.x;
+    const float* base = ws + (int64_t)h * nsplit * (dh + 2);
+    float mn = -INFINITY;
+    for (int s = 0; s < nsplit; ++s) mn = fmaxf(mn, base[(int64_t)s * (dh + 2)]);
+    for (int d = threadIdx.x; d < dh; d += blockDim.x) {
+        float L = 0.f, O = 0.f;
+        for (int s = 0; s < nsplit; ++s) {
+            const float* rec = base + (int64_t)s * (dh + 2);
+            if (rec[0] == -INFINITY) continue;
+            const float c = expf(rec[0] - mn);
+            L += rec[1] * c;
+            O += rec[2 + d] * c;
+        }
+        stf(ctx, (int64_t)h * dh + d, O / L);
+    }
+}
+
+static int decode_splits(int64_t n_kv, int64_t cap) {
+    int64_t by_len = cdiv(cap, 64);
+    int64_t by_fill = 512 / (n_kv > 0 ? n_kv : 1);
+    if (by_fill < 1) by_fill = 1;
+    int64_t s = by_len < by_fill ? by_len : by_fill;
+    return (int)(s < 1 ? 1 : s);
+}
+size_t attn_decode_workspace_bytes(int64_t n_q, int64_t head_dim, int64_t capacity) {
+    // n_kv >= 1, so 512 splits bounds every launch geometry
+    int64_t s = cdiv(capacity, 64);
+    if (s > 512) s = 512;
+    return (size_t)n_q * (size_t)s * (size_t)(head_dim + 2) * sizeof(float);
+}
+
+template <typename T>
+static void attn_decode_t(hipStream_t s, const AttnDecodeArgs& a) {
+    const int nsplit = decode_splits(a.n_kv, a.capacity);
+    const int64_t chunk = cdiv(a.capacity, nsplit);
+    dim3 grid((unsigned)a.n_kv, (unsigned)nsplit);
+    const int g = (int)(a.n_q / a.n_kv);
+#define GPTRS_LAUNCH(G)                                                                                          \
+    attn_decode_kernel<T, G><<<grid, 256, 0, s>>>((const T*)a.qkv, (T*)a.k_cache, (T*)a.v_cache, a.update_starts,    \
+        a.query_start, (T*)a.ctx, (float*)a.ws, (int)a.n_q, (int)a.n_kv, (int)a.head_dim, a.capacity, a.scale, chunk, nsplit)
+    switch (g) {
+        case 1: GPTRS_LAUNCH(1); break;
+        case 2: GPTRS_LAUNCH(2); break;
+        case 4: GPTRS_LAUNCH(4); break;
+        default: GPTRS_LAUNCH(8); break;
+    }
+#undef GPTRS_LAUNCH
+    if (nsplit > 1) {
+        const int block = a.head_dim <= 64 ? 64 : (a.head_dim <= 128 ? 128 : 256);
+        attn_decode_combine_kernel<T><<<(unsigned)a.n_q, block, 0, s>>>((const float*)a.ws, (T*)a.ctx, (int)a.head_dim, nsplit);
+    }
+}
+void attn_decode(hipStream_t s, const AttnDecodeArgs& a) {
+    if (a.dtype == 0) attn_decode_t<float>(s, a);
+    else attn_decode_t<bf16_t>(s, a);
+}
+
+// ------------------------------------------------------------------------------ prefill
+// grid (ceil(T/4), n_q), 256 threads: one wave per query row.  Keys are visited 64 at a time
+// (one per lane) with an online softmax; the P.V update then walks the chunk with the lanes
+// spread over head_dim so V rows are read coalesced.
+template <typename T>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(const T* __restrict__ qkv, T* __restrict__ ctx, int64_t t,
+                                                           int n_q, int n_kv, int dh, float scale) {
+    __shared__ float qsm[4][256];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t i = (int64_t)blockIdx.x * 4 + wave;
+    const int h = blockIdx.y;
+    const int kvh = h / (n_q / n_kv);
+    const int64_t P = (int64_t)(n_q + 2 * n_kv) * dh;
+    const int64_t koff = (int64_t)n_q * dh + (int64_t)kvh * dh;
+    const int64_t voff = (int64_t)(n_q + n_kv) * dh + (int64_t)kvh * dh;
+    if (i < t)
+        for (int d = lane; d < dh; d += 64) qsm[wave][d] = ldf(qkv, i * P + (int64_t)h * dh + d);
+    __syncthreads();
+    if (i >= t) return;
+    float m = -INFINITY, l = 0.f;
+    float o[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int64_t j0 = 0; j0 <= i; j0 += 64) {
+        const int64_t j = j0 + lane;
+        float s = -INFINITY;
+        if (j <= i) {
+            const T* kr = qkv + j * P + koff;
+            float acc = 0.f;
+            for (int d = 0; d < dh; ++d) acc += qsm[wave][d] * ldf(kr, d);
+            s = acc * scale;
+        }
+        const float mn = fmaxf(m, wave_max(s));
+        const float corr = expf(m - mn);
+        const float pe = j <= i ? expf(s - mn) : 0.f;
+        l = l * corr + wave_sum(pe);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) o[c] *= corr;
+        const int cnt = (int)((i - j0 + 1) < 64 ? (i - j0 + 1) : 64);
+        for (int jj = 0; jj < cnt; ++jj) {
+            const float pj = __shfl(pe, jj, 64);
+            const T* vr = qkv + (j0 + jj) * P + voff;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int d = lane + 64 * c;
+                if (d < dh) o[c] += pj * ldf(vr, d);
+            }
+        }
+        m = mn;
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const int d = lane + 64 * c;
+        if (d < dh) stf(ctx, i * (int64_t)n_q * dh + (int64_t)h * dh + d, o[c] / l);
+    }
+}
+void attn_prefill(hipStream_t s, const AttnPrefillArgs& a) {
+    if (a.t <= 0) return;
+    dim3 grid((unsigned)cdiv(a.t, 4), (unsigned)a.n_q);
+    if (a.dtype == 0)
+        attn_prefill_kernel<float><<<grid, 256, 0, s>>>((const float*)a.qkv, (float*)a.ctx, a.t, (int)a.n_q, (int)a.n_kv, (int)a.head_dim, a.scale);
+    else
+        attn_prefill_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)a.qkv, (bf16_t*)a.ctx, a.t, (int)a.n_q, (int)a.n_kv, (int)a.head_dim, a.scale);
+}
+
+}  // namespace k
+}  // namespace gptrs

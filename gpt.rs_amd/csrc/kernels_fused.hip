@@ -1,0 +1,234 @@
+// Fused kernels for the functional sequences of the LM path: row norms, softmax, GELU/SwiGLU,
+// packed RoPE.  Each replaces an exact PTIR op sequence emitted by
+// crates/gpt-rs/src/ops/functional/*.rs; math is f32 with one rounding to the output dtype.
+#include "kernels.hpp"
+#include "device_utils.hpp"
+
+namespace gptrs {
+namespace k {
+
+static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+template <typename T> __device__ __forceinline__ float ldf(const T* p, int64_t i);
+template <> __device__ __forceinline__ float ldf<float>(const float* p, int64_t i) { return p[i]; }
+template <> __device__ __forceinline__ float ldf<bf16_t>(const bf16_t* p, int64_t i) { return bf16_to_f32(p[i]); }
+template <typename T> __device__ __forceinline__ void stf(T* p, int64_t i, float v);
+template <> __device__ __forceinline__ void stf<float>(float* p, int64_t i, float v) { p[i] = v; }
+template <> __device__ __forceinline__ void stf<bf16_t>(bf16_t* p, int64_t i, float v) { p[i] = f32_to_bf16(v); }
+
+// ------------------------------------------------------------------------------ layer_norm
+// normalization.rs:123-174: mean = sum*(1/N); c = x-mean; var = sum(c*c)*(1/N); y = c*rsqrt(var+eps)*g+b
+// One block per row; the row stays in registers between the passes (up to 16 values/thread).
+template <typename T, int PER>
+__global__ void layer_norm_kernel(const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta,
+                                  T* __restrict__ y, int64_t n, float inv_n, float eps) {
+    __shared__ float red[16];
+    const T* row = x + (int64_t)blockIdx.x * n;
+    T* out = y + (int64_t)blockIdx.x * n;
+    float v[PER];
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int64_t i = threadIdx.x + (int64_t)j * blockDim.x;
+        v[j] = i < n ? ldf(row, i) : 0.f;
+        s += v[j];
+    }
+    const float mean = block_sum(s, red) * inv_n;
+    float q = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int64_t i = threadIdx.x + (int64_t)j * blockDim.x;
+        const float c = i < n ? v[j] - mean : 0.f;
+        v[j] = c;
+        q += c * c;
+    }
+    const float var = block_sum(q, red) * inv_n;
+    const float inv_std = 1.0f / sqrtf(var + eps);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int64_t i = threadIdx.x + (int64_t)j * blockDim.x;
+        if (i < n) stf(out, i, (v[j] * inv_std) * ldf(gamma, i) + ldf(beta, i));
+    }
+}
+// rows longer than 16*blockDim: re-read from memory on each pass
+template <typename T>
+__global__ void layer_norm_long_kernel(const T* __restrict__ x, const T* __restrict__ gamma, const T* __restrict__ beta,
+                                       T* __restrict__ y, int64_t n, float inv_n, float eps) {
+    __shared__ float red[16];
+    const T* row = x + (int64_t)blockIdx.x * n;
+    T* out = y + (int64_t)blockIdx.x * n;
+    float s = 0.f;
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) s += ldf(row, i);
+    const float mean = block_sum(s, red) * inv_n;
+    float q = 0.f;
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) { const float c = ldf(row, i) - mean; q += c * c; }
+    const float inv_std = 1.0f / sqrtf(block_sum(q, red) * inv_n + eps);
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x)
+        stf(out, i, ((ldf(row, i) - mean) * inv_std) * ldf(gamma, i) + ldf(beta, i));
+}
+
+template <typename T>
+static void layer_norm_t(hipStream_t s, const T* x, const T* g, const T* b, T* y, int64_t rows, int64_t n, float inv_n,
+                         float eps) {
+    const int block = n <= 256 ? 64 : 256;
+    const int64_t per = cdiv(n, block);
+    const unsigned grid = (unsigned)rows;
+    if (per <= 4) layer_norm_kernel<T, 4><<<grid, block, 0, s>>>(x, g, b, y, n, inv_n, eps);
+    else if (per <= 16) layer_norm_kernel<T, 16><<<grid, block, 0, s>>>(x, g, b, y, n, inv_n, eps);
+    else layer_norm_long_kernel<T><<<grid, 1024, 0, s>>>(x, g, b, y, n, inv_n, eps);
+}
+void layer_norm(hipStream_t s, int dtype, const void* x, const void* gamma, const void* beta, void* y, int64_t rows,
+                int64_t n, float inv_n, float eps) {
+    if (rows <= 0 || n <= 0) return;
+    if (dtype == 0) layer_norm_t<float>(s, (const float*)x, (const float*)gamma, (const float*)beta, (float*)y, rows, n, inv_n, eps);
+    else layer_norm_t<bf16_t>(s, (const bf16_t*)x, (const bf16_t*)gamma, (const bf16_t*)beta, (bf16_t*)y, rows, n, inv_n, eps);
+}
+
+// ------------------------------------------------------------------------------ rms_norm
+// normalization.rs:183-217: y = (x * rsqrt(sum(x*x)*(1/N) + eps)) * gamma
+template <typename T, int PER>
+__global__ void rms_norm_kernel(const T* __restrict__ x, const T* __restrict__ gamma, T* __restrict__ y, int64_t n,
+                                float inv_n, float eps) {
+    __shared__ float red[16];
+    const T* row = x + (int64_t)blockIdx.x * n;
+    T* out = y + (int64_t)blockIdx.x * n;
+    float v[PER];
+    float q = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int64_t i = threadIdx.x + (int64_t)j * blockDim.x;
+        v[j] = i < n ? ldf(row, i) : 0.f;
+        q += v[j] * v[j];
+    }
+    const float inv_rms = 1.0f / sqrtf(block_sum(q, red) * inv_n + eps);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int64_t i = threadIdx.x + (int64_t)j * blockDim.x;
+        if (i < n) stf(out, i, (v[j] * inv_rms) * ldf(gamma, i));
+    }
+}
+template <typename T>
+__global__ void rms_norm_long_kernel(const T* __restrict__ x, const T* __restrict__ gamma, T* __restrict__ y, int64_t n,
+                                     float inv_n, float eps) {
+    __shared__ float red[16];
+    const T* row = x + (int64_t)blockIdx.x * n;
+    T* out = y + (int64_t)blockIdx.x * n;
+    float q = 0.f;
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) { const float v = ldf(row, i); q += v * v; }
+    const float inv_rms = 1.0f / sqrtf(block_sum(q, red) * inv_n + eps);
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) stf(out, i, (ldf(row, i) * inv_rms) * ldf(gamma, i));
+}
+template <typename T>
+static void rms_norm_t(hipStream_t s, const T* x, const T* g, T* y, int64_t rows, int64_t n, float inv_n, float eps) {
+    const int block = n <= 256 ? 64 : 256;
+    const int64_t per = cdiv(n, block);
+    if (per <= 4) rms_norm_kernel<T, 4><<<(unsigned)rows, block, 0, s>>>(x, g, y, n, inv_n, eps);
+    else if (per <= 16) rms_norm_kernel<T, 16><<<(unsigned)rows, block, 0, s>>>(x, g, y, n, inv_n, eps);
+    else rms_norm_long_kernel<T><<<(unsigned)rows, 1024, 0, s>>>(x, g, y, n, inv_n, eps);
+}
+void rms_norm(hipStream_t s, int dtype, const void* x, const void* gamma, void* y, int64_t rows, int64_t n, float inv_n,
+              float eps) {
+    if (rows <= 0 || n <= 0) return;
+    if (dtype == 0) rms_norm_t<float>(s, (const float*)x, (const float*)gamma, (float*)y, rows, n, inv_n, eps);
+    else rms_norm_t<bf16_t>(s, (const bf16_t*)x, (const bf16_t*)gamma, (bf16_t*)y, rows, n, inv_n, eps);
+}
+
+// ------------------------------------------------------------------------------ softmax
+// common.rs:22-31: e = exp(x - max); y = e / sum(e)   (true division)
+template <typename T>
+__global__ void softmax_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t n) {
+    __shared__ float red[16];
+    const T* row = x + (int64_t)blockIdx.x * n;
+    T* out = y + (int64_t)blockIdx.x * n;
+    float mx = -INFINITY;
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) mx = fmaxf(mx, ldf(row, i));
+    mx = block_max(mx, red);
+    float sum = 0.f;
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) sum += expf(ldf(row, i) - mx);
+    sum = block_sum(sum, red);
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) stf(out, i, expf(ldf(row, i) - mx) / sum);
+}
+void softmax_rows(hipStream_t s, int dtype, const void* x, void* y, int64_t rows, int64_t n) {
+    if (rows <= 0 || n <= 0) return;
+    const int block = n <= 64 ? 64 : (n <= 2048 ? 256 : 1024);
+    if (dtype == 0) softmax_kernel<float><<<(unsigned)rows, block, 0, s>>>((const float*)x, (float*)y, n);
+    else softmax_kernel<bf16_t><<<(unsigned)rows, block, 0, s>>>((const bf16_t*)x, (bf16_t*)y, n);
+}
+
+// ------------------------------------------------------------------------------ activations
+// activation.rs:96-113: (x*0.5) * (erf(x / sqrt2) + 1); the three literals come from the program
+template <typename T>
+__global__ void gelu_kernel(const T* __restrict__ x, T* __restrict__ y, int64_t n, float half, float div, float one) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        const float v = ldf(x, i);
+        stf(y, i, (v * half) * (erff(v / div) + one));
+    }
+}
+void gelu(hipStream_t s, int dtype, const void* x, void* y, int64_t n, float half, float div, float one) {
+    if (n <= 0) return;
+    const unsigned g = (unsigned)(cdiv(n, 256) > 16384 ? 16384 : cdiv(n, 256));
+    if (dtype == 0) gelu_kernel<float><<<g, 256, 0, s>>>((const float*)x, (float*)y, n, half, div, one);
+    else gelu_kernel<bf16_t><<<g, 256, 0, s>>>((const bf16_t*)x, (bf16_t*)y, n, half, div, one);
+}
+// activation.rs:141-162: (g / (1 + exp(g * -1))) * u
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gate, const T* __restrict__ up, T* __restrict__ y, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        const float g = ldf(gate, i);
+        float r = g / (1.0f + expf(g * -1.0f));
+        if (up) r *= ldf(up, i);
+        stf(y, i, r);
+    }
+}
+void swiglu(hipStream_t s, int dtype, const void* gate, const void* up, void* y, int64_t n) {
+    if (n <= 0) return;
+    const unsigned g = (unsigned)(cdiv(n, 256) > 16384 ? 16384 : cdiv(n, 256));
+    if (dtype == 0) swiglu_kernel<float><<<g, 256, 0, s>>>((const float*)gate, (const float*)up, (float*)y, n);
+    else swiglu_kernel<bf16_t><<<g, 256, 0, s>>>((const bf16_t*)gate, (const bf16_t*)up, (bf16_t*)y, n);
+}
+
+// ------------------------------------------------------------------------------ RoPE
+// rotary.rs:430-536 on packed rows [T, Q|K|V]: for each Q/K head and j < half:
+//   out[j]      = a*cos[t,j] - b*sin[t,j]      (a = x[j], b = x[j+half])
+//   out[j+half] = b*cos[t,j] + a*sin[t,j]
+// columns >= 2*half of a head and all of V pass through.
+template <typename T>
+__global__ void rope_kernel(const T* __restrict__ qkv, const T* __restrict__ cs, const T* __restrict__ sn,
+                            T* __restrict__ out, int64_t t, int64_t qk_cols, int64_t total_cols, int64_t head_dim,
+                            int64_t half) {
+    const int64_t total = t * total_cols;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t row = idx / total_cols, col = idx % total_cols;
+        float r;
+        if (col < qk_cols) {
+            const int64_t d = col % head_dim;
+            if (d < half) {
+                const float a = ldf(qkv, idx), b = ldf(qkv, idx + half);
+                r = a * ldf(cs, row * half + d) - b * ldf(sn, row * half + d);
+            } else if (d < 2 * half) {
+                const int64_t j = d - half;
+                const float b = ldf(qkv, idx), a = ldf(qkv, idx - half);
+                r = b * ldf(cs, row * half + j) + a * ldf(sn, row * half + j);
+            } else {
+                r = ldf(qkv, idx);
+            }
+        } else {
+            r = ldf(qkv, idx);
+        }
+        stf(out, idx, r);
+    }
+}
+void rope_packed(hipStream_t s, int dtype, const void* qkv, const void* cos, const void* sin, void* out, int64_t t,
+                 int64_t n_q, int64_t n_kv, int64_t head_dim, int64_t half) {
+    const int64_t qk_cols = (n_q + n_kv) * head_dim, total_cols = (n_q + 2 * n_kv) * head_dim;
+    const int64_t total = t * total_cols;
+    if (total <= 0) return;
+    const unsigned g = (unsigned)(cdiv(total, 256) > 16384 ? 16384 : cdiv(total, 256));
+    if (dtype == 0)
+        rope_kernel<float><<<g, 256, 0, s>>>((const float*)qkv, (const float*)cos, (const float*)sin, (float*)out, t, qk_cols, total_cols, head_dim, half);
+    else
+        rope_kernel<bf16_t><<<g, 256, 0, s>>>((const bf16_t*)qkv, (const bf16_t*)cos, (const bf16_t*)sin, (bf16_t*)out, t, qk_cols, total_cols, head_dim, half);
+}
+
+}  // namespace k
+}  // namespace gptrs

@@ -1,0 +1,873 @@
+// Program -> Plan: validate every instruction against docs/backend.md, decide where each SSA
+// value lives (input, donated-in-place, output buffer, workspace slice, constant block) and
+// precompute one launch descriptor per instruction.  run_step() issues the launches.
+#include <algorithm>
+#include <cstring>
+#include <functional>
+
+#include "runtime.hpp"
+
+namespace gptrs {
+
+static constexpr size_t kAlign = 256;
+static size_t align_up(size_t n) { return (n + kAlign - 1) / kAlign * kAlign; }
+
+static std::vector<int64_t> row_major_strides(const std::vector<int64_t>& dims) {
+    std::vector<int64_t> s(dims.size(), 1);
+    for (int i = (int)dims.size() - 2; i >= 0; --i) s[i] = s[i + 1] * dims[i + 1];
+    return s;
+}
+
+// Build a CopyDesc over `dims` with the given element strides, merging adjacent dims that are
+// contiguous on both sides and dropping extent-1 dims.
+static k::CopyDesc make_copy(const std::vector<int64_t>& dims, const std::vector<int64_t>& dst_stride,
+                             const std::vector<int64_t>& src_stride, int64_t dst_off, int64_t src_off) {
+    std::vector<int64_t> d, ds, ss;
+    for (size_t i = 0; i < dims.size(); ++i) {
+        if (dims[i] == 1) continue;
+        if (!d.empty() && ds.back() == dst_stride[i] * dims[i] && ss.back() == src_stride[i] * dims[i]) {
+            d.back() *= dims[i];
+            ds.back() = dst_stride[i];
+            ss.back() = src_stride[i];
+        } else {
+            d.push_back(dims[i]);
+            ds.push_back(dst_stride[i]);
+            ss.push_back(src_stride[i]);
+        }
+    }
+    if ((int)d.size() > k::kMaxRank) fail_unimpl("copy", "rank above 6 after collapsing");
+    k::CopyDesc c;
+    c.rank = (int)d.size();
+    c.total = 1;
+    for (size_t i = 0; i < d.size(); ++i) {
+        c.dims[i] = d[i];
+        c.dst_stride[i] = ds[i];
+        c.src_stride[i] = ss[i];
+        c.total *= d[i];
+    }
+    for (auto x : dims) if (x == 0) c.total = 0;
+    c.dst_off = dst_off;
+    c.src_off = src_off;
+    return c;
+}
+
+// Reinterpret a copy of `es`-byte elements as words `f` times wider when every run allows it.
+static bool can_widen(const k::CopyDesc& c, int f) {
+    if (c.total == 0 || c.rank == 0) return false;
+    const int last = c.rank - 1;
+    bool ok = c.dst_stride[last] == 1 && c.src_stride[last] == 1 && c.dims[last] % f == 0 && c.dst_off % f == 0 &&
+              c.src_off % f == 0;
+    for (int i = 0; i < last && ok; ++i) ok = c.dst_stride[i] % f == 0 && c.src_stride[i] % f == 0;
+    for (int i = 0; i < c.dyn_rank && ok; ++i) ok = c.dyn_stride[i] % f == 0;
+    return ok;
+}
+static void apply_widen(k::CopyDesc& c, int f) {
+    const int last = c.rank - 1;
+    c.dims[last] /= f;
+    c.total /= f;
+    c.dst_off /= f;
+    c.src_off /= f;
+    for (int i = 0; i < last; ++i) { c.dst_stride[i] /= f; c.src_stride[i] /= f; }
+    for (int i = 0; i < c.dyn_rank; ++i) c.dyn_stride[i] /= f;
+}
+// Widens every piece of one op to a common word size; returns the element size to launch with.
+// (Device buffers are 256-byte aligned, so element offsets decide alignment.)
+static int widen_copies(std::vector<k::CopyDesc>& cs, int es) {
+    for (int w : {16, 8, 4, 2}) {
+        if (w <= es || w % es) continue;
+        const int f = w / es;
+        bool ok = true;
+        for (auto& c : cs) ok = ok && (c.total == 0 || can_widen(c, f));
+        if (!ok) continue;
+        for (auto& c : cs) if (c.total) apply_widen(c, f);
+        return w;
+    }
+    return es;
+}
+
+static int64_t norm_axis(int64_t axis, int rank, const char* op) {
+    if (axis < 0) axis += rank;
+    if (axis < 0 || axis >= rank) fail_exec(std::string(op) + " axis out of range");
+    return axis;
+}
+
+namespace {
+struct Builder {
+    Plan& plan;
+    const std::vector<bool>& donated;
+    std::vector<int> use_count;      // per root value
+    std::vector<int> last_use;       // per root value: last step index that reads it
+    std::vector<int> def_step;       // per root value
+    std::vector<size_t> lit_offset;  // literal index -> const offset
+
+    Builder(Plan& p, const std::vector<bool>& d) : plan(p), donated(d) {}
+
+    const Spec& spec_of(const Instr& in, size_t i) {
+        const Operand& o = in.operands[i];
+        if (o.value >= 0) {
+            if (o.value >= (int)plan.values.size() || !plan.values[o.value].defined) fail_exec("operand value missing");
+            return plan.values[o.value].spec;
+        }
+        return plan.fn.literals[o.literal].spec;
+    }
+    int root(int v) const {
+        while (plan.values[v].root != v) v = plan.values[v].root;
+        return v;
+    }
+    size_t const_add(const std::vector<uint8_t>& bytes) {
+        size_t off = align_up(plan.const_host.size());
+        plan.const_host.resize(off + std::max<size_t>(bytes.size(), 1), 0);
+        if (!bytes.empty()) memcpy(plan.const_host.data() + off, bytes.data(), bytes.size());
+        return off;
+    }
+    void define(int id, const Spec& s) {
+        if (id < 0) fail_exec("negative value id");
+        if (id >= (int)plan.values.size()) plan.values.resize(id + 1);
+        if (plan.values[id].defined) fail_exec("value id defined twice");
+        plan.values[id].spec = s;
+        plan.values[id].root = id;
+        plan.values[id].defined = true;
+    }
+
+    void validate(Instr& in);
+    void build();
+    void describe(Step& st);
+};
+}  // namespace
+
+static void expect(bool c, const std::string& msg) {
+    if (!c) fail_exec(msg);
+}
+
+// Shape/dtype rules per op (docs/backend.md "Operation reference"; messages follow cpu.rs).
+void Builder::validate(Instr& in) {
+    const Spec& out = in.out_specs[0];
+    auto same_shape = [&](size_t a, size_t b, const char* what) {
+        expect(spec_of(in, a).dims == spec_of(in, b).dims, std::string(what) + " size mismatch");
+    };
+    switch (in.op) {
+        case OpKind::Constant:
+            expect(plan.fn.literals[in.literal].spec == out, "constant output spec mismatch");
+            break;
+        case OpKind::Unary: {
+            const Spec& x = spec_of(in, 0);
+            expect(dtype_is_float(x.dtype), "elementwise unary only supports f32/bf16 tensors");
+            expect(x == out, "elementwise unary output spec mismatch");
+            break;
+        }
+        case OpKind::Binary: {
+            const Spec& a = spec_of(in, 0);
+            if (in.scalar_rhs) {  // rhs folded to a kernel argument by the fusion pass
+                expect(dtype_is_float(a.dtype) && a == out, "elementwise binary output spec mismatch");
+                break;
+            }
+            const Spec& b = spec_of(in, 1);
+            expect(a.dtype == b.dtype && dtype_is_float(a.dtype), "elementwise binary only supports f32/bf16 tensors of one dtype");
+            same_shape(0, 1, "elementwise");
+            expect(a == out, "elementwise binary output spec mismatch");
+            break;
+        }
+        case OpKind::Compare: {
+            const Spec& a = spec_of(in, 0);
+            const Spec& b = spec_of(in, 1);
+            expect(a.dtype == b.dtype && (a.dtype == DType::SI32 || dtype_is_float(a.dtype)), "compare supports si32/f32/bf16 tensors");
+            same_shape(0, 1, "compare");
+            expect(out.dtype == DType::I1 && out.dims == a.dims, "compare output must be i1 of the operand shape");
+            break;
+        }
+        case OpKind::Select: {
+            const Spec& p = spec_of(in, 0);
+            const Spec& t = spec_of(in, 1);
+            const Spec& f = spec_of(in, 2);
+            expect(p.dtype == DType::I1 && t.dtype == f.dtype, "select dtype combination unsupported");
+            expect(p.dims == t.dims && t.dims == f.dims && t == out, "select shape mismatch");
+            break;
+        }
+        case OpKind::Cast:
+            expect(spec_of(in, 0).dims == out.dims, "cast shape mismatch");
+            break;
+        case OpKind::StopGradient:
+            expect(spec_of(in, 0) == out, "stop_gradient output spec mismatch");
+            break;
+        case OpKind::Reshape: {
+            const Spec& x = spec_of(in, 0);
+            expect(x.dtype == out.dtype && x.count() == out.count(), "reshape element count mismatch");
+            break;
+        }
+        case OpKind::Transpose: {
+            const Spec& x = spec_of(in, 0);
+            expect((int)in.a.size() == x.rank() && x.dtype == out.dtype && out.rank() == x.rank(), "transpose perm rank mismatch");
+            std::vector<bool> seen(x.rank(), false);
+            for (int i = 0; i < x.rank(); ++i) {
+                const int64_t p = in.a[i];
+                expect(p >= 0 && p < x.rank() && !seen[p], "transpose perm is not a permutation");
+                seen[p] = true;
+                expect(out.dims[i] == x.dims[p], "transpose output shape mismatch");
+            }
+            break;
+        }
+        case OpKind::BroadcastTo: {
+            const Spec& x = spec_of(in, 0);
+            expect(x.dtype == out.dtype, "broadcast_to dtype mismatch");
+            if (x.rank() > out.rank()) fail_spec("broadcast_to: input rank exceeds result rank");
+            const int pad = out.rank() - x.rank();
+            for (int i = 0; i < x.rank(); ++i)
+                if (x.dims[i] != out.dims[pad + i] && x.dims[i] != 1)
+                    fail_spec("broadcast_to: shapes " + x.str() + " and " + out.str() + " are not broadcast-compatible");
+            break;
+        }
+        case OpKind::Slice: {
+            const Spec& x = spec_of(in, 0);
+            expect((int)in.a.size() == x.rank() && (int)in.b.size() == x.rank(), "slice starts/sizes must match rank");
+            for (int i = 0; i < x.rank(); ++i) expect(in.a[i] >= 0 && in.b[i] >= 0 && in.a[i] + in.b[i] <= x.dims[i], "slice exceeds bounds");
+            expect(out.dtype == x.dtype && out.dims == in.b, "slice output shape mismatch");
+            break;
+        }
+        case OpKind::Concat: {
+            const Spec& x0 = spec_of(in, 0);
+            in.axis = norm_axis(in.axis, x0.rank(), "concat");
+            int64_t total = 0;
+            for (size_t i = 0; i < in.operands.size(); ++i) {
+                const Spec& x = spec_of(in, i);
+                expect(x.dtype == x0.dtype && x.rank() == x0.rank(), "concat dtype/rank mismatch");
+                for (int d = 0; d < x.rank(); ++d)
+                    if (d != in.axis) expect(x.dims[d] == x0.dims[d], "concat shape mismatch off the concat axis");
+                total += x.dims[in.axis];
+            }
+            expect(out.dtype == x0.dtype && out.rank() == x0.rank() && out.dims[in.axis] == total, "concat output shape mismatch");
+            break;
+        }
+        case OpKind::Iota:
+            expect(out.dtype == DType::SI32, "iota only supports si32");
+            expect(in.axis >= 0 && in.axis < out.rank(), "iota axis out of range");
+            break;
+        case OpKind::Take: {
+            const Spec& x = spec_of(in, 0);
+            const Spec& idx = spec_of(in, 1);
+            expect(x.rank() >= 1, "take requires rank >= 1");
+            expect(idx.dtype == DType::SI32, "take indices must be si32");
+            std::vector<int64_t> want = idx.dims;
+            want.insert(want.end(), x.dims.begin() + 1, x.dims.end());
+            expect(out.dtype == x.dtype && out.dims == want, "take output shape mismatch");
+            break;
+        }
+        case OpKind::DynamicSlice: {
+            const Spec& x = spec_of(in, 0);
+            const Spec& st = spec_of(in, 1);
+            expect((int)in.a.size() == x.rank(), "dynamic_slice sizes length must match input rank");
+            expect(st.dtype == DType::SI32, "dynamic_slice starts must be si32");
+            expect(st.rank() == 1 && st.dims[0] == x.rank(), "dynamic_slice starts must be 1-D of length equal to rank");
+            for (int i = 0; i < x.rank(); ++i)
+                if (in.a[i] > x.dims[i]) fail_spec("dynamic_slice size exceeds dimension");
+            expect(out.dtype == x.dtype && out.dims == in.a, "dynamic_slice output shape mismatch");
+            break;
+        }
+        case OpKind::DynamicUpdateSlice: {
+            const Spec& x = spec_of(in, 0);
+            const Spec& u = spec_of(in, 1);
+            const Spec& st = spec_of(in, 2);
+            expect(x.dtype == u.dtype, "dynamic_update_slice dtype mismatch");
+            expect(u.rank() == x.rank() && in.a == u.dims, "dynamic_update_slice sizes must match update shape");
+            expect(st.dtype == DType::SI32 && st.rank() == 1 && st.dims[0] == x.rank(), "dynamic_update_slice starts must be si32[rank]");
+            for (int i = 0; i < x.rank(); ++i)
+                if (u.dims[i] > x.dims[i]) fail_spec("dynamic_update_slice update exceeds base dimension");
+            expect(out == x, "dynamic_update_slice output spec mismatch");
+            break;
+        }
+        case OpKind::Reduce: {
+            const Spec& x = spec_of(in, 0);
+            expect(dtype_is_float(x.dtype), "reduce only supports f32/bf16 tensors");
+            if (in.a.size() != 1) fail_exec("reduce currently supports single axis");
+            in.a[0] = norm_axis(in.a[0], x.rank(), "reduce");
+            std::vector<int64_t> want;
+            for (int i = 0; i < x.rank(); ++i) {
+                if (i == in.a[0]) { if (in.keepdims) want.push_back(1); }
+                else want.push_back(x.dims[i]);
+            }
+            expect(out.dtype == x.dtype && out.dims == want, "reduce output shape mismatch");
+            break;
+        }
+        case OpKind::Dot: {
+            const Spec& l = spec_of(in, 0);
+            const Spec& r = spec_of(in, 1);
+            expect(l.dtype == r.dtype && dtype_is_float(l.dtype), "dot_general only supports f32/bf16 tensors of one dtype");
+            expect(in.a.size() == in.b.size(), "dot_general batch dimension mismatch");
+            expect(in.c.size() == in.d.size(), "dot_general dimension mismatch");
+            auto check_axes = [&](const std::vector<int64_t>& ax, int rank) {
+                for (auto a : ax) expect(a >= 0 && a < rank, "dot_general axis out of range");
+            };
+            check_axes(in.a, l.rank()); check_axes(in.c, l.rank());
+            check_axes(in.b, r.rank()); check_axes(in.d, r.rank());
+            for (size_t i = 0; i < in.a.size(); ++i) expect(l.dims[in.a[i]] == r.dims[in.b[i]], "dot_general batch dimension mismatch");
+            for (size_t i = 0; i < in.c.size(); ++i) expect(l.dims[in.c[i]] == r.dims[in.d[i]], "dot_general dimension mismatch on contraction");
+            std::vector<int64_t> want;
+            std::vector<int64_t> bl = in.a;
+            std::sort(bl.begin(), bl.end());
+            for (auto a : bl) want.push_back(l.dims[a]);
+            auto has = [](const std::vector<int64_t>& v, int64_t x) { return std::find(v.begin(), v.end(), x) != v.end(); };
+            for (int i = 0; i < l.rank(); ++i) if (!has(in.a, i) && !has(in.c, i)) want.push_back(l.dims[i]);
+            for (int i = 0; i < r.rank(); ++i) if (!has(in.b, i) && !has(in.d, i)) want.push_back(r.dims[i]);
+            expect(out.dtype == l.dtype && out.dims == want, "dot_general output shape mismatch");
+            break;
+        }
+        case OpKind::CustomCall:
+            // docs/backend.md:581-582: unknown targets MUST answer Unimplemented
+            fail_unimpl("custom_call", "unknown target `" + in.target + "`");
+        case OpKind::Unsupported:
+            fail_unimpl(in.op_name, "operation not supported in the hip backend");
+        default:
+            break;  // fused ops are produced from already-validated sequences
+    }
+}
+
+// Element strides of `src` broadcast (right-aligned) to `out_rank` dims: 0 where it repeats.
+static std::vector<int64_t> broadcast_strides(const Spec& src, const Spec& out) {
+    std::vector<int64_t> s = row_major_strides(src.dims), r(out.rank(), 0);
+    const int pad = out.rank() - src.rank();
+    for (int i = 0; i < src.rank(); ++i) r[pad + i] = src.dims[i] == 1 ? 0 : s[i];
+    return r;
+}
+
+// One group of dot axes as a single (extent, stride), or false when they do not collapse.
+static bool collapse_axes(const Spec& s, const std::vector<int64_t>& axes, int64_t& extent, int64_t& stride) {
+    const auto st = row_major_strides(s.dims);
+    extent = 1;
+    stride = 1;
+    std::vector<std::pair<int64_t, int64_t>> ds;  // (dim, stride), skipping extent-1 axes
+    for (auto a : axes) {
+        extent *= s.dims[a];
+        if (s.dims[a] != 1) ds.push_back({s.dims[a], st[a]});
+    }
+    if (ds.empty()) { stride = 0; return true; }
+    for (size_t i = 0; i + 1 < ds.size(); ++i)
+        if (ds[i].second != ds[i + 1].second * ds[i + 1].first) return false;
+    stride = ds.back().second;
+    return true;
+}
+
+void Builder::describe(Step& st) {
+    Instr& in = st.in;
+    const Spec& out = in.out_specs[0];
+    const auto out_strides = row_major_strides(out.dims);
+    auto es_of = [&](const Spec& s) { return (int)dtype_size(s.dtype); };
+    switch (in.op) {
+        case OpKind::BroadcastTo: {
+            const Spec& x = spec_of(in, 0);
+            st.copies.push_back(make_copy(out.dims, out_strides, broadcast_strides(x, out), 0, 0));
+            st.elem_size = widen_copies(st.copies, es_of(out));
+            break;
+        }
+        case OpKind::Slice: {
+            const Spec& x = spec_of(in, 0);
+            const auto xs = row_major_strides(x.dims);
+            int64_t off = 0;
+            for (int i = 0; i < x.rank(); ++i) off += in.a[i] * xs[i];
+            st.copies.push_back(make_copy(out.dims, out_strides, xs, 0, off));
+            st.elem_size = widen_copies(st.copies, es_of(out));
+            break;
+        }
+        case OpKind::Transpose: {
+            const Spec& x = spec_of(in, 0);
+            const auto xs = row_major_strides(x.dims);
+            std::vector<int64_t> ss(x.rank());
+            for (int i = 0; i < x.rank(); ++i) ss[i] = xs[in.a[i]];
+            st.copies.push_back(make_copy(out.dims, out_strides, ss, 0, 0));
+            st.elem_size = widen_copies(st.copies, es_of(out));
+            break;
+        }
+        case OpKind::Concat: {
+            int64_t along = 0;
+            for (size_t i = 0; i < in.operands.size(); ++i) {
+                const Spec& x = spec_of(in, i);
+                st.copies.push_back(make_copy(x.dims, out_strides, row_major_strides(x.dims), along * out_strides[in.axis], 0));
+                along += x.dims[in.axis];
+            }
+            st.elem_size = widen_copies(st.copies, es_of(out));
+            break;
+        }
+        case OpKind::DynamicSlice: {
+            const Spec& x = spec_of(in, 0);
+            const auto xs = row_major_strides(x.dims);
+            k::CopyDesc c = make_copy(out.dims, out_strides, xs, 0, 0);
+            c.dyn = 1;
+            c.dyn_rank = x.rank();
+            if (x.rank() > k::kMaxRank) fail_unimpl("dynamic_slice", "rank above 6");
+            for (int i = 0; i < x.rank(); ++i) { c.dyn_max[i] = x.dims[i] - in.a[i]; c.dyn_stride[i] = xs[i]; }
+            st.copies.push_back(c);
+            st.elem_size = widen_copies(st.copies, es_of(out));
+            break;
+        }
+        case OpKind::DynamicUpdateSlice: {
+            const Spec& x = spec_of(in, 0);
+            const Spec& u = spec_of(in, 1);
+            const auto xs = row_major_strides(x.dims);
+            k::CopyDesc c = make_copy(u.dims, xs, row_major_strides(u.dims), 0, 0);
+            c.dyn = 2;
+            c.dyn_rank = x.rank();
+            if (x.rank() > k::kMaxRank) fail_unimpl("dynamic_update_slice", "rank above 6");
+            for (int i = 0; i < x.rank(); ++i) { c.dyn_max[i] = x.dims[i] - u.dims[i]; c.dyn_stride[i] = xs[i]; }
+            st.copies.push_back(c);
+            st.elem_size = widen_copies(st.copies, es_of(out));
+            break;
+        }
+        case OpKind::Iota: {
+            st.outer = 1; st.inner = 1;
+            for (int i = 0; i < in.axis; ++i) st.outer *= out.dims[i];
+            for (int i = (int)in.axis + 1; i < out.rank(); ++i) st.inner *= out.dims[i];
+            st.axis_len = out.dims[in.axis];
+            break;
+        }
+        case OpKind::Reduce: {
+            const Spec& x = spec_of(in, 0);
+            const int ax = (int)in.a[0];
+            st.outer = 1; st.inner = 1;
+            for (int i = 0; i < ax; ++i) st.outer *= x.dims[i];
+            for (int i = ax + 1; i < x.rank(); ++i) st.inner *= x.dims[i];
+            st.axis_len = x.dims[ax];
+            break;
+        }
+        case OpKind::Take: {
+            const Spec& x = spec_of(in, 0);
+            st.outer = spec_of(in, 1).count();
+            st.axis_len = x.dims[0];
+            st.inner = x.dims[0] ? x.count() / x.dims[0] : 0;
+            break;
+        }
+        case OpKind::Dot: {
+            const Spec& l = spec_of(in, 0);
+            const Spec& r = spec_of(in, 1);
+            auto has = [](const std::vector<int64_t>& v, int64_t x) { return std::find(v.begin(), v.end(), x) != v.end(); };
+            // batch axes sorted as the reference does (cpu.rs:2166-2169); pair them up accordingly
+            std::vector<std::pair<int64_t, int64_t>> bp;
+            for (size_t i = 0; i < in.a.size(); ++i) bp.push_back({in.a[i], in.b[i]});
+            std::vector<int64_t> bl = in.a, br = in.b;
+            std::sort(bl.begin(), bl.end());
+            std::sort(br.begin(), br.end());
+            std::vector<int64_t> lf, rf;
+            for (int i = 0; i < l.rank(); ++i) if (!has(in.a, i) && !has(in.c, i)) lf.push_back(i);
+            for (int i = 0; i < r.rank(); ++i) if (!has(in.b, i) && !has(in.d, i)) rf.push_back(i);
+            k::DotDesc& d = st.dot;
+            int64_t e;
+            bool lok = collapse_axes(l, bl, d.batch, d.a_sb) & collapse_axes(l, lf, d.m, d.a_sm) & collapse_axes(l, in.c, d.k, d.a_sk);
+            bool rok = collapse_axes(r, br, e, d.b_sb) & collapse_axes(r, in.d, e, d.b_sk) & collapse_axes(r, rf, d.n, d.b_sn);
+            d.c_sb = d.m * d.n;
+            d.c_sm = d.n;
+            const size_t es = dtype_size(l.dtype);
+            size_t scratch = 0;
+            if (!lok) {  // repack lhs as [batch][m][k]
+                std::vector<int64_t> order = bl;
+                order.insert(order.end(), lf.begin(), lf.end());
+                order.insert(order.end(), in.c.begin(), in.c.end());
+                const auto ls = row_major_strides(l.dims);
+                std::vector<int64_t> dims, ss;
+                for (auto a : order) { dims.push_back(l.dims[a]); ss.push_back(ls[a]); }
+                st.pack_l = make_copy(dims, row_major_strides(dims), ss, 0, 0);
+                st.lhs_pack = true;
+                st.pack_l_off = scratch;
+                scratch += align_up((size_t)l.count() * es);
+                d.a_sb = d.m * d.k; d.a_sm = d.k; d.a_sk = 1;
+            }
+            if (!rok) {  // repack rhs as [batch][k][n]
+                std::vector<int64_t> order = br;
+                order.insert(order.end(), in.d.begin(), in.d.end());
+                order.insert(order.end(), rf.begin(), rf.end());
+                const auto rs = row_major_strides(r.dims);
+                std::vector<int64_t> dims, ss;
+                for (auto a : order) { dims.push_back(r.dims[a]); ss.push_back(rs[a]); }
+                st.pack_r = make_copy(dims, row_major_strides(dims), ss, 0, 0);
+                st.rhs_pack = true;
+                st.pack_r_off = scratch;
+                scratch += align_up((size_t)r.count() * es);
+                d.b_sb = d.k * d.n; d.b_sk = d.n; d.b_sn = 1;
+            }
+            st.scratch_bytes = scratch;
+            break;
+        }
+        case OpKind::FLinear: {
+            const Spec& x = spec_of(in, 0);
+            const Spec& w = spec_of(in, 1);
+            st.scratch_bytes = k::linear_workspace_bytes((int)x.dtype, x.dims[0], x.dims[1], w.dims[1], in.act == 2);
+            break;
+        }
+        case OpKind::FAttnDecode: {
+            const Spec& ck = spec_of(in, 1);
+            st.scratch_bytes = k::attn_decode_workspace_bytes(in.n_q, in.head_dim, ck.dims[1]);
+            break;
+        }
+        default:
+            break;
+    }
+}
+
+void Builder::build() {
+    Function& fn = plan.fn;
+    plan.values.assign(fn.max_value_id + 1, ValueInfo{});
+    if (fn.param_ids.size() != donated.size()) fail_exec("entry input arity mismatch");
+    for (size_t i = 0; i < fn.param_ids.size(); ++i) define(fn.param_ids[i], fn.param_specs[i]);
+
+    // literals -> const block
+    lit_offset.resize(fn.literals.size());
+    for (size_t i = 0; i < fn.literals.size(); ++i) lit_offset[i] = const_add(fn.literals[i].bytes);
+
+    // pass 1: validate, define values, record aliasing
+    for (auto& in : fn.body) {
+        if (in.dead) continue;
+        for (size_t i = 0; i < in.operands.size(); ++i) (void)spec_of(in, i);
+        validate(in);
+        for (size_t o = 0; o < in.out_ids.size(); ++o) define(in.out_ids[o], in.out_specs[o]);
+        const bool alias = in.op == OpKind::Reshape || in.op == OpKind::StopGradient ||
+                           (in.op == OpKind::Cast && spec_of(in, 0).dtype == in.out_specs[0].dtype);
+        if (alias && in.operands[0].value >= 0) plan.values[in.out_ids[0]].root = root(in.operands[0].value);
+    }
+    for (size_t i = 0; i < fn.result_ids.size(); ++i) {
+        const int id = fn.result_ids[i];
+        if (id < 0 || id >= (int)plan.values.size() || !plan.values[id].defined) fail_exec("missing function result value");
+        if (plan.values[id].spec != fn.result_specs[i]) fail_exec("function result spec mismatch");
+    }
+
+    // pass 2: steps
+    const int nv = (int)plan.values.size();
+    use_count.assign(nv, 0);
+    last_use.assign(nv, -1);
+    def_step.assign(nv, -1);
+    plan.storage.assign(nv, RootStorage{});
+    for (auto& in : fn.body) {
+        if (in.dead) continue;
+        const bool alias = plan.values[in.out_ids[0]].root != in.out_ids[0];
+        if (in.op == OpKind::Constant) {
+            RootStorage& rs = plan.storage[in.out_ids[0]];
+            rs.kind = Storage::Const;
+            rs.offset = lit_offset[in.literal];
+            continue;
+        }
+        if (alias) continue;  // pure view: no work
+        Step st;
+        st.in = in;
+        for (auto& o : in.operands) {
+            st.src.push_back(o.value);
+            st.src_const.push_back(o.value < 0 ? lit_offset[o.literal] : 0);
+        }
+        st.dst = in.out_ids;
+        describe(st);
+        const int idx = (int)plan.steps.size();
+        for (int v : st.src)
+            if (v >= 0) { const int r = root(v); ++use_count[r]; last_use[r] = idx; }
+        for (int v : st.dst) def_step[v] = idx;
+        plan.steps.push_back(std::move(st));
+    }
+    const int n_steps = (int)plan.steps.size();
+
+    // storage classes
+    for (size_t i = 0; i < fn.param_ids.size(); ++i) {
+        RootStorage& rs = plan.storage[fn.param_ids[i]];
+        rs.kind = Storage::Input;
+        rs.index = (int)i;
+    }
+    std::vector<int> input_of_root(nv, -1);
+    for (size_t i = 0; i < fn.param_ids.size(); ++i) input_of_root[fn.param_ids[i]] = (int)i;
+    std::vector<bool> root_is_result(nv, false);
+    for (int id : fn.result_ids) root_is_result[root(id)] = true;
+
+    // results -> output buffers (shared when several results alias one root)
+    std::map<int, int> out_buf_of_root;
+    plan.out_buffer_of_result.assign(fn.result_ids.size(), -1);
+    plan.result_input_alias.assign(fn.result_ids.size(), -1);
+    auto new_out_buffer = [&](int r) {
+        const int ob = (int)plan.out_buffer_bytes.size();
+        plan.out_buffer_bytes.push_back(std::max<size_t>(plan.values[r].spec.bytes(), 1));
+        plan.out_buffer_inplace_input.push_back(-1);
+        out_buf_of_root[r] = ob;
+        plan.storage[r].kind = Storage::Output;
+        plan.storage[r].index = ob;
+        return ob;
+    };
+    for (size_t i = 0; i < fn.result_ids.size(); ++i) {
+        const int r = root(fn.result_ids[i]);
+        if (plan.storage[r].kind == Storage::Input) { plan.result_input_alias[i] = plan.storage[r].index; continue; }
+        if (plan.storage[r].kind == Storage::Const) {
+            // a constant returned directly: give it an output buffer filled by a copy step
+            fail_unimpl("constant", "returning a Constant as a function result");
+        }
+        auto it = out_buf_of_root.find(r);
+        plan.out_buffer_of_result[i] = it != out_buf_of_root.end() ? it->second : new_out_buffer(r);
+    }
+
+    // in-place updates on donated inputs
+    for (auto& st : plan.steps) {
+        std::vector<std::pair<int, int>> pairs;  // (base operand slot, output slot)
+        if (st.in.op == OpKind::DynamicUpdateSlice) pairs = {{0, 0}};
+        if (st.in.op == OpKind::FAttnDecode) pairs = {{1, 1}, {2, 2}};
+        bool all_inplace = !pairs.empty();
+        for (auto& pr : pairs) {
+            const int bv = st.src[pr.first];
+            bool ok = bv >= 0;
+            int br = ok ? root(bv) : -1;
+            ok = ok && input_of_root[br] >= 0 && donated[input_of_root[br]] && use_count[br] == 1 && !root_is_result[br];
+            const int ov = st.dst[pr.second];
+            ok = ok && plan.storage[ov].kind == Storage::Output;  // the updated cache is a program result
+            if (ok) {
+                // a second in-place claim on one input would alias two outputs
+                for (int ip : plan.out_buffer_inplace_input) ok = ok && ip != input_of_root[br];
+            }
+            if (ok) {
+                plan.out_buffer_inplace_input[plan.storage[ov].index] = input_of_root[br];
+            } else {
+                all_inplace = false;
+            }
+        }
+        st.copy_base = !all_inplace;  // informational: run_step compares pointers
+    }
+
+    // workspace: temps by liveness (first-fit over a free list), plus per-step scratch
+    struct Block { size_t off, size; };
+    std::vector<Block> free_list;
+    size_t high = 0;
+    auto ws_alloc = [&](size_t bytes) {
+        bytes = align_up(std::max<size_t>(bytes, 1));
+        for (size_t i = 0; i < free_list.size(); ++i) {
+            if (free_list[i].size >= bytes) {
+                const size_t off = free_list[i].off;
+                free_list[i].off += bytes;
+                free_list[i].size -= bytes;
+                if (!free_list[i].size) free_list.erase(free_list.begin() + i);
+                return off;
+            }
+        }
+        const size_t off = high;
+        high += bytes;
+        return off;
+    };
+    auto ws_free = [&](size_t off, size_t bytes) {
+        bytes = align_up(std::max<size_t>(bytes, 1));
+        free_list.push_back({off, bytes});
+        std::sort(free_list.begin(), free_list.end(), [](const Block& a, const Block& b) { return a.off < b.off; });
+        for (size_t i = 0; i + 1 < free_list.size();) {
+            if (free_list[i].off + free_list[i].size == free_list[i + 1].off) {
+                free_list[i].size += free_list[i + 1].size;
+                free_list.erase(free_list.begin() + i + 1);
+            } else {
+                ++i;
+            }
+        }
+    };
+    std::vector<std::vector<int>> dying(n_steps);
+    for (int v = 0; v < nv; ++v)
+        if (plan.values[v].defined && plan.values[v].root == v && def_step[v] >= 0 && plan.storage[v].kind == Storage::Temp)
+            dying[std::max(last_use[v], def_step[v])].push_back(v);
+    for (int s = 0; s < n_steps; ++s) {
+        Step& st = plan.steps[s];
+        for (int v : st.dst) {
+            RootStorage& rs = plan.storage[v];
+            if (rs.kind != Storage::Temp) continue;
+            rs.bytes = std::max<size_t>(plan.values[v].spec.bytes(), 1);
+            rs.offset = ws_alloc(rs.bytes);
+        }
+        if (st.scratch_bytes) {
+            st.scratch_off = ws_alloc(st.scratch_bytes);
+            ws_free(st.scratch_off, st.scratch_bytes);
+        }
+        for (int v : dying[s]) ws_free(plan.storage[v].offset, plan.storage[v].bytes);
+    }
+    plan.workspace_bytes = high;
+}
+
+void build_plan(Plan& plan, const std::vector<bool>& donated) {
+    Builder b(plan, donated);
+    b.build();
+}
+
+// ------------------------------------------------------------------------------ execution
+static inline const void* src_ptr(const Step& st, const ExecCtx& cx, size_t i) {
+    return st.src[i] >= 0 ? cx.ptr[st.src[i]] : (const void*)(cx.consts + st.src_const[i]);
+}
+
+void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
+    const Instr& in = st.in;
+    const Spec& out = in.out_specs[0];
+    void* dst = cx.ptr[st.dst[0]];
+    hipStream_t s = cx.stream;
+    auto in_spec = [&](size_t i) -> const Spec& {
+        return st.src[i] >= 0 ? plan.values[st.src[i]].spec : plan.fn.literals[in.operands[i].literal].spec;
+    };
+    switch (in.op) {
+        case OpKind::BroadcastTo:
+        case OpKind::Slice:
+        case OpKind::Transpose:
+            k::copy_strided(s, dst, src_ptr(st, cx, 0), st.elem_size, st.copies[0], nullptr);
+            ++cx.launches;
+            break;
+        case OpKind::Concat:
+            for (size_t i = 0; i < st.copies.size(); ++i) {
+                k::copy_strided(s, dst, src_ptr(st, cx, i), st.elem_size, st.copies[i], nullptr);
+                ++cx.launches;
+            }
+            break;
+        case OpKind::DynamicSlice:
+            k::copy_strided(s, dst, src_ptr(st, cx, 0), st.elem_size, st.copies[0], (const int32_t*)src_ptr(st, cx, 1));
+            ++cx.launches;
+            break;
+        case OpKind::DynamicUpdateSlice: {
+            const void* base = src_ptr(st, cx, 0);
+            if (dst != base && out.bytes()) {
+                GPTRS_HIP_CHECK(hipMemcpyAsync(dst, base, out.bytes(), hipMemcpyDeviceToDevice, s));
+                ++cx.launches;
+            }
+            k::copy_strided(s, dst, src_ptr(st, cx, 1), st.elem_size, st.copies[0], (const int32_t*)src_ptr(st, cx, 2));
+            ++cx.launches;
+            break;
+        }
+        case OpKind::Unary:
+            k::unary(s, (int)out.dtype, (int)in.unary, src_ptr(st, cx, 0), dst, out.count());
+            ++cx.launches;
+            break;
+        case OpKind::Binary:
+            if (in.scalar_rhs) k::binary_scalar(s, (int)out.dtype, (int)in.binary, src_ptr(st, cx, 0), in.scalar_val, dst, out.count());
+            else k::binary(s, (int)out.dtype, (int)in.binary, src_ptr(st, cx, 0), src_ptr(st, cx, 1), dst, out.count());
+            ++cx.launches;
+            break;
+        case OpKind::Compare:
+            k::compare(s, (int)in_spec(0).dtype, (int)in.cmp, src_ptr(st, cx, 0), src_ptr(st, cx, 1), (uint8_t*)dst, out.count());
+            ++cx.launches;
+            break;
+        case OpKind::Select:
+            k::select(s, (int)dtype_size(out.dtype), (const uint8_t*)src_ptr(st, cx, 0), src_ptr(st, cx, 1), src_ptr(st, cx, 2), dst, out.count());
+            ++cx.launches;
+            break;
+        case OpKind::Cast:
+            k::cast(s, (int)in_spec(0).dtype, (int)out.dtype, src_ptr(st, cx, 0), dst, out.count());
+            ++cx.launches;
+            break;
+        case OpKind::Iota:
+            k::iota(s, (int32_t*)dst, st.outer, st.axis_len, st.inner);
+            ++cx.launches;
+            break;
+        case OpKind::Reduce:
+            k::reduce(s, (int)out.dtype, (int)in.reduce, src_ptr(st, cx, 0), dst, st.outer, st.axis_len, st.inner);
+            ++cx.launches;
+            break;
+        case OpKind::Take:
+            k::take(s, (int)dtype_size(out.dtype), src_ptr(st, cx, 0), (const int32_t*)src_ptr(st, cx, 1), dst, st.outer,
+                    st.axis_len, st.inner, cx.err_flag);
+            ++cx.launches;
+            break;
+        case OpKind::Dot: {
+            const void* a = src_ptr(st, cx, 0);
+            const void* b = src_ptr(st, cx, 1);
+            const int es = (int)dtype_size(out.dtype);
+            if (st.lhs_pack) {
+                void* p = cx.ws + st.scratch_off + st.pack_l_off;
+                k::copy_strided(s, p, a, es, st.pack_l, nullptr);
+                a = p;
+                ++cx.launches;
+            }
+            if (st.rhs_pack) {
+                void* p = cx.ws + st.scratch_off + st.pack_r_off;
+                k::copy_strided(s, p, b, es, st.pack_r, nullptr);
+                b = p;
+                ++cx.launches;
+            }
+            k::dot_generic(s, (int)out.dtype, a, b, dst, st.dot);
+            ++cx.launches;
+            break;
+        }
+        case OpKind::FLayerNorm: {
+            const Spec& x = in_spec(0);
+            const int64_t n = x.dims.back();
+            k::layer_norm(s, (int)out.dtype, src_ptr(st, cx, 0), src_ptr(st, cx, 1), src_ptr(st, cx, 2), dst, n ? x.count() / n : 0, n, in.scale, in.eps);
+            ++cx.launches;
+            break;
+        }
+        case OpKind::FRmsNorm: {
+            const Spec& x = in_spec(0);
+            const int64_t n = x.dims.back();
+            k::rms_norm(s, (int)out.dtype, src_ptr(st, cx, 0), src_ptr(st, cx, 1), dst, n ? x.count() / n : 0, n, in.scale, in.eps);
+            ++cx.launches;
+            break;
+        }
+        case OpKind::FSoftmax: {
+            const int64_t n = out.dims.back();
+            k::softmax_rows(s, (int)out.dtype, src_ptr(st, cx, 0), dst, n ? out.count() / n : 0, n);
+            ++cx.launches;
+            break;
+        }
+        case OpKind::FGelu:
+            k::gelu(s, (int)out.dtype, src_ptr(st, cx, 0), dst, out.count(), in.fparam[0], in.fparam[1], in.fparam[2]);
+            ++cx.launches;
+            break;
+        case OpKind::FSilu:
+            k::swiglu(s, (int)out.dtype, src_ptr(st, cx, 0), nullptr, dst, out.count());
+            ++cx.launches;
+            break;
+        case OpKind::FSwiglu:
+            k::swiglu(s, (int)out.dtype, src_ptr(st, cx, 0), src_ptr(st, cx, 1), dst, out.count());
+            ++cx.launches;
+            break;
+        case OpKind::FLinear: {
+            const Spec& x = in_spec(0);
+            const Spec& w = in_spec(1);
+            k::LinearArgs a{};
+            a.dtype = (int)out.dtype;
+            a.x = src_ptr(st, cx, 0);
+            a.w = src_ptr(st, cx, 1);
+            size_t i = 2;
+            if (in.act == 2) a.w2 = src_ptr(st, cx, i++);
+            if (in.has_bias) a.bias = src_ptr(st, cx, i++);
+            if (in.has_residual) a.residual = src_ptr(st, cx, i++);
+            a.y = dst;
+            a.m = x.dims[0]; a.k = x.dims[1]; a.n = w.dims[1];
+            a.act = in.act == 1 ? 1 : 0;
+            a.ws = cx.ws + st.scratch_off;
+            a.ws_bytes = st.scratch_bytes;
+            a.counters = cx.counters;
+            k::linear(s, a);
+            cx.launches += (in.act == 2 && a.m > 16) ? 3 : 1;
+            break;
+        }
+        case OpKind::FRope: {
+            const Spec& x = in_spec(0);
+            k::rope_packed(s, (int)out.dtype, src_ptr(st, cx, 0), src_ptr(st, cx, 1), src_ptr(st, cx, 2), dst, x.dims[0],
+                           in.n_q, in.n_kv, in.head_dim, in.rot_half);
+            ++cx.launches;
+            break;
+        }
+        case OpKind::FAttnDecode: {
+            const Spec& ck = in_spec(1);
+            void* kout = cx.ptr[st.dst[1]];
+            void* vout = cx.ptr[st.dst[2]];
+            const void* kin = src_ptr(st, cx, 1);
+            const void* vin = src_ptr(st, cx, 2);
+            if (kout != kin) { GPTRS_HIP_CHECK(hipMemcpyAsync(kout, kin, ck.bytes(), hipMemcpyDeviceToDevice, s)); ++cx.launches; }
+            if (vout != vin) { GPTRS_HIP_CHECK(hipMemcpyAsync(vout, vin, ck.bytes(), hipMemcpyDeviceToDevice, s)); ++cx.launches; }
+            k::AttnDecodeArgs a{};
+            a.dtype = (int)out.dtype;
+            a.qkv = src_ptr(st, cx, 0);
+            a.k_cache = kout; a.v_cache = vout;
+            a.update_starts = (const int32_t*)src_ptr(st, cx, 3);
+            a.query_start = (const int32_t*)src_ptr(st, cx, 4);
+            a.ctx = dst;
+            a.n_q = in.n_q; a.n_kv = in.n_kv; a.head_dim = in.head_dim; a.capacity = ck.dims[1];
+            a.scale = in.scale;
+            a.ws = cx.ws + st.scratch_off;
+            a.ws_bytes = st.scratch_bytes;
+            k::attn_decode(s, a);
+            cx.launches += 2;
+            break;
+        }
+        case OpKind::FAttnPrefill: {
+            const Spec& x = in_spec(0);
+            k::AttnPrefillArgs a{};
+            a.dtype = (int)out.dtype;
+            a.qkv = src_ptr(st, cx, 0);
+            a.ctx = dst;
+            a.t = x.dims[0]; a.n_q = in.n_q; a.n_kv = in.n_kv; a.head_dim = in.head_dim;
+            a.scale = in.scale;
+            k::attn_prefill(s, a);
+            ++cx.launches;
+            break;
+        }
+        default:
+            fail_unimpl(in.op_name, "no kernel bound to this operation");
+    }
+}
+
+}  // namespace gptrs

@@ -1,0 +1,134 @@
+// PTIR (ptir.v0.4) program model as the executor sees it, parsed from the serde-JSON
+// wire form of crates/gpt-rs/src/backend/spec.rs:644-817.
+#pragma once
+#include <cstdint>
+#include <map>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "json.hpp"
+
+namespace gptrs {
+
+// Error kinds map 1:1 onto BackendError (spec.rs:1224-1228).
+enum class ErrKind { Spec = 1, Unimplemented = 2, Execution = 3 };
+struct BackendError : std::runtime_error {
+    ErrKind kind;
+    BackendError(ErrKind k, const std::string& m) : std::runtime_error(m), kind(k) {}
+};
+[[noreturn]] inline void fail_spec(const std::string& m) { throw BackendError(ErrKind::Spec, m); }
+[[noreturn]] inline void fail_unimpl(const std::string& op, const std::string& why) {
+    throw BackendError(ErrKind::Unimplemented, op + " is not implemented: " + why);
+}
+[[noreturn]] inline void fail_exec(const std::string& m) {
+    throw BackendError(ErrKind::Execution, "backend execution failure: " + m);
+}
+
+// Tags shared with include/gptrs_hip.h.
+enum class DType : uint32_t { F32 = 0, F16 = 1, BF16 = 2, SI32 = 3, I1 = 4, SI8 = 5, UI8 = 6, Invalid = 99 };
+
+inline size_t dtype_size(DType d) {
+    switch (d) {
+        case DType::F32: case DType::SI32: return 4;
+        case DType::F16: case DType::BF16: return 2;
+        case DType::I1: case DType::SI8: case DType::UI8: return 1;
+        default: return 0;
+    }
+}
+inline const char* dtype_name(DType d) {
+    switch (d) {
+        case DType::F32: return "F32"; case DType::F16: return "F16"; case DType::BF16: return "Bf16";
+        case DType::SI32: return "Si32"; case DType::I1: return "I1"; case DType::SI8: return "Si8";
+        case DType::UI8: return "Ui8"; default: return "?";
+    }
+}
+inline bool dtype_is_float(DType d) { return d == DType::F32 || d == DType::BF16; }
+DType parse_dtype(const std::string& name);  // throws Spec error on dtypes the backend does not execute
+
+struct Spec {
+    DType dtype = DType::F32;
+    std::vector<int64_t> dims;
+    int64_t count() const {
+        int64_t n = 1;
+        for (auto d : dims) n *= d;
+        return n;
+    }
+    size_t bytes() const { return (size_t)count() * dtype_size(dtype); }
+    int rank() const { return (int)dims.size(); }
+    bool operator==(const Spec& o) const { return dtype == o.dtype && dims == o.dims; }
+    bool operator!=(const Spec& o) const { return !(*this == o); }
+    std::string str() const;
+};
+
+struct Literal {
+    Spec spec;
+    std::vector<uint8_t> bytes;
+};
+
+enum class OpKind {
+    Constant, Unary, Binary, Dot, Reduce, Compare, Select, Cast, StopGradient, Reshape, Transpose,
+    BroadcastTo, Slice, Concat, Iota, Take, DynamicSlice, DynamicUpdateSlice, CustomCall,
+    // fused forms produced by the executor's pattern pass (never present on the wire)
+    FLayerNorm, FRmsNorm, FSoftmax, FGelu, FSilu, FSwiglu, FLinear, FRope, FAttnDecode, FAttnPrefill,
+    FEmbed,
+    Unsupported
+};
+enum class UnaryOp { Neg, Abs, Exp, Log, Tanh, Erf, Rsqrt, Reciprocal };
+enum class BinaryOp { Add, Sub, Mul, Div, Maximum, Minimum };
+enum class ReduceKind { Sum, Max, Min };
+enum class CmpOp { Less, LessEqual, Equal, GreaterEqual, Greater, NotEqual };
+
+struct Operand {
+    int value = -1;    // SSA value id, or -1 when literal
+    int literal = -1;  // index into Function::literals
+};
+
+struct Instr {
+    OpKind op = OpKind::Unsupported;
+    std::string op_name;             // wire name, for error messages
+    std::vector<Operand> operands;
+    std::vector<int> out_ids;        // one on the wire; fused ops may define several
+    std::vector<Spec> out_specs;
+    bool dead = false;
+
+    // attributes (only those of `op` are meaningful)
+    UnaryOp unary{};
+    BinaryOp binary{};
+    ReduceKind reduce{};
+    CmpOp cmp{};
+    std::vector<int64_t> a, b, c, d;  // dot: batch_lhs, batch_rhs, contract_lhs, contract_rhs
+                                      // slice: a=starts b=sizes; transpose: a=perm; reduce: a=axes
+                                      // dyn ops: a=sizes
+    int64_t axis = 0;                 // concat / iota axis
+    bool keepdims = true;
+    int literal = -1;                 // Constant payload
+    std::string target;               // CustomCall
+    std::map<std::string, Json> attrs;
+    // fused-op parameters
+    float eps = 0.f, scale = 0.f;
+    int64_t n_q = 0, n_kv = 0, head_dim = 0, rot_half = 0;
+    int act = 0;                      // FLinear epilogue: 0 none, 1 gelu, 2 swiglu (dual weights)
+    bool has_bias = false, has_residual = false;
+    float fparam[4] = {0.f, 0.f, 0.f, 0.f};  // FGelu: half, divisor, one
+    bool scalar_rhs = false;                 // Binary whose rhs is a broadcast scalar literal
+    float scalar_val = 0.f;
+};
+
+struct Function {
+    std::string name;
+    std::vector<int> param_ids;
+    std::vector<Spec> param_specs;
+    std::vector<int> result_ids;
+    std::vector<Spec> result_specs;
+    std::vector<Instr> body;
+    std::vector<Literal> literals;
+    int max_value_id = 0;
+};
+
+// Parses `Program` JSON and returns the entry function.  Enforces spec_version
+// (spec.rs:844-856), static shapes, single tensor outputs (cpu.rs:257-266).
+Function parse_program(const char* json, size_t len);
+Instr parse_instruction(const Json& j, Function& fn);
+
+}  // namespace gptrs

@@ -1,0 +1,187 @@
+// Host runtime of the hip PTIR backend: device buffers, tensor handles, the stable-id parameter
+// memo and compiled-program (plan) cache.  One Backend owns one device and one HIP stream; every
+// kernel, copy and readback is ordered on that stream.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <array>
+#include <atomic>
+#include <list>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "kernels.hpp"
+#include "ptir.hpp"
+
+namespace gptrs {
+
+#define GPTRS_HIP_CHECK(expr)                                                                      \
+    do {                                                                                           \
+        hipError_t e_ = (expr);                                                                    \
+        if (e_ != hipSuccess)                                                                      \
+            ::gptrs::fail_exec(std::string(#expr) + " failed: " + hipGetErrorString(e_));          \
+    } while (0)
+
+class Backend;
+
+// Size-bucketed cache of device allocations (the reference's Triton backend keeps the same kind
+// of cache, crates/gpt-rs-backend-triton/src/device.rs:727-751).  Blocks are only ever used on the
+// backend's single stream, so a freed block may be handed out again immediately.
+class DevicePool {
+  public:
+    void* alloc(size_t bytes, size_t* cap_out);
+    void release(void* p, size_t cap);
+    void trim();  // return every cached block to the driver
+    size_t bytes_allocated = 0;
+
+  private:
+    static size_t bucket(size_t n);
+    std::unordered_map<size_t, std::vector<void*>> free_;
+};
+
+struct Buffer {
+    void* ptr = nullptr;
+    size_t cap = 0;
+    Backend* owner = nullptr;
+    ~Buffer();
+};
+using BufferP = std::shared_ptr<Buffer>;
+
+}  // namespace gptrs
+
+// The opaque handle type of include/gptrs_hip.h.
+struct gptrs_hip_tensor {
+    std::atomic<int> refs{1};
+    gptrs::Spec spec;
+    gptrs::BufferP buf;
+    bool consumed = false;  // donated to a run_program call
+    void* data() const { return buf ? buf->ptr : nullptr; }
+};
+
+namespace gptrs {
+
+// ---- compiled program -------------------------------------------------------------------
+enum class Storage { Input, Temp, Output, Const, InPlace };
+
+struct ValueInfo {
+    Spec spec;
+    int root = -1;  // value whose storage this one aliases (itself when it owns storage)
+    bool defined = false;
+};
+
+struct RootStorage {
+    Storage kind = Storage::Temp;
+    int index = 0;       // Input: input position; Output: output-buffer index; InPlace: input position
+    size_t offset = 0;   // Temp: byte offset in the workspace; Const: offset in the const block
+    size_t bytes = 0;
+};
+
+struct Step {
+    Instr in;                      // attributes (operands resolved below)
+    std::vector<int> src;          // operand value ids (-1 for literal operands)
+    std::vector<size_t> src_const; // const-block offset for literal operands
+    std::vector<int> dst;          // output value ids
+    // precomputed launch descriptors
+    std::vector<k::CopyDesc> copies;  // strided copies (one per concat operand, etc.)
+    int elem_size = 0;
+    k::DotDesc dot{};
+    int64_t outer = 0, axis_len = 0, inner = 0;
+    float scalar = 0.f;
+    bool rhs_scalar = false;
+    size_t scratch_off = 0, scratch_bytes = 0;  // per-step scratch inside the workspace
+    bool copy_base = false;        // DynamicUpdateSlice / FAttnDecode: copy base -> out first
+    bool lhs_pack = false, rhs_pack = false;    // Dot: operands repacked into scratch first
+    k::CopyDesc pack_l{}, pack_r{};
+    size_t pack_l_off = 0, pack_r_off = 0;
+};
+
+struct Plan {
+    Function fn;
+    std::vector<ValueInfo> values;          // indexed by value id
+    std::vector<RootStorage> storage;       // indexed by value id (meaningful for roots)
+    std::vector<Step> steps;
+    std::vector<int> out_buffer_of_result;  // result position -> output buffer index (or -1: aliases an input)
+    std::vector<int> result_input_alias;    // result position -> input position it aliases, or -1
+    std::vector<size_t> out_buffer_bytes;
+    std::vector<int> out_buffer_inplace_input;  // output buffer index -> donated input position or -1
+    size_t workspace_bytes = 0;
+    BufferP workspace;
+    BufferP consts;
+    std::vector<uint8_t> const_host;
+    int fused_ops = 0;
+    int launches_estimate = 0;
+};
+
+struct IdHash {
+    size_t operator()(const std::array<uint8_t, 16>& a) const {
+        size_t h = 1469598103934665603ull;
+        for (auto b : a) h = (h ^ b) * 1099511628211ull;
+        return h;
+    }
+};
+
+class Backend {
+  public:
+    explicit Backend(int device);
+    ~Backend();
+
+    gptrs_hip_tensor* materialize(const Spec& spec, const void* host, size_t nbytes);
+    void to_literal(const gptrs_hip_tensor* t, void* dst, size_t cap);
+    void run_program(const char* json, size_t len, uint64_t key, gptrs_hip_tensor* const* inputs,
+                     const uint8_t* donate, size_t n_in, gptrs_hip_tensor** outputs, size_t n_out);
+    gptrs_hip_tensor* param_get(const std::array<uint8_t, 16>& id);
+    void param_set(const std::array<uint8_t, 16>& id, gptrs_hip_tensor* t);
+    int64_t sample(const gptrs_hip_tensor* logits, float temperature, bool has_top_k, bool has_u, float u);
+    void synchronize();
+    void check_device_errors();
+
+    BufferP new_buffer(size_t bytes);
+    void release_block(void* p, size_t cap) { pool_.release(p, cap); }
+
+    std::mutex mu;
+    hipStream_t stream = nullptr;
+    int device = 0;
+    bool opt_fusion = true;
+    // counters
+    int64_t n_launches = 0, n_compiled = 0, n_cache_hits = 0, n_fused = 0, n_inplace = 0, last_launches = 0;
+    int64_t bytes_allocated() const { return (int64_t)pool_.bytes_allocated; }
+
+  private:
+    std::shared_ptr<Plan> get_plan(const char* json, size_t len, uint64_t key, const uint8_t* donate, size_t n_in);
+    void execute(Plan& plan, gptrs_hip_tensor* const* inputs, const uint8_t* donate, gptrs_hip_tensor** outputs);
+
+    DevicePool pool_;
+    std::unordered_map<std::array<uint8_t, 16>, gptrs_hip_tensor*, IdHash> params_;
+    std::list<std::pair<uint64_t, std::shared_ptr<Plan>>> plan_lru_;
+    std::unordered_map<uint64_t, std::list<std::pair<uint64_t, std::shared_ptr<Plan>>>::iterator> plan_index_;
+    // device-side helpers
+    int* d_err_flag_ = nullptr;
+    int* d_counters_ = nullptr;
+    float* d_argmax_val_ = nullptr;
+    int32_t* d_argmax_idx_ = nullptr;
+    int64_t* d_token_ = nullptr;
+    void* h_pinned_ = nullptr;  // 64 bytes of pinned host memory for readbacks
+};
+
+// fuse.cpp: canonicalise + pattern-fuse the entry function in place.  Returns the number of fused ops.
+int fuse_function(Function& fn);
+// plan.cpp: validate every instruction, assign storage and build launch descriptors.
+void build_plan(Plan& plan, const std::vector<bool>& donated);
+// plan.cpp: run one step with resolved pointers.
+struct ExecCtx {
+    Backend* be;
+    hipStream_t stream;
+    std::vector<void*> ptr;  // per value id
+    char* ws;
+    char* consts;
+    int* err_flag;
+    int* counters;
+    int64_t launches = 0;
+};
+void run_step(const Plan& plan, const Step& st, ExecCtx& cx);
+
+}  // namespace gptrs

@@ -1,0 +1,577 @@
+"""GPT-2 and Ministral model drivers and the greedy Generator, generic over a backend.
+
+Host-side mirror of crates/gpt-rs/src/model/{gpt,ministral}.rs, nn/layers/*.rs and
+inference/{generate,sampler}.rs: each forward call captures the whole model into ONE
+PTIR program (as the reference's lazy GraphArena does, ops/graph/arena.rs:340-375),
+caches it by shape (plan cache, ops/graph/plan.rs:20-29) and hands it to
+`backend.run_program`.  Weights are program inputs fed from the backend's parameter
+memo; per-step scalars (token ids, positions, update_starts, query_start, RoPE rows)
+are tiny uploads, exactly the reference's calling convention.
+
+`backend` is any object with the PortableBackend surface (spec.rs:1287-1349):
+materialize / to_literal / run_program / param_resolver / sample_decode_token.
+"""
+from __future__ import annotations
+
+import hashlib
+import itertools
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+from . import functional as F
+from .ptir import FunctionBuilder, Program, Tensor, TensorSpec, f32_to_bf16_bits
+
+
+def decode_cache_capacity(required_len: int, max_len: int) -> int:
+    """model/gpt.rs:940-943: next power of two, capped at the context length."""
+    bucket = 1
+    while bucket < max(required_len, 1):
+        bucket *= 2
+    return min(bucket, max_len)
+
+
+@dataclass
+class DecodeKvCache:
+    """ops/functional/attention.rs:100-126: fixed-capacity [Hkv, capacity, Dh] + active len."""
+
+    keys: object
+    values: object
+    len: int
+    capacity: int
+
+
+def _np_to_bytes(arr: np.ndarray, dtype: str) -> bytes:
+    if dtype == "Bf16":
+        return f32_to_bf16_bits(np.asarray(arr, np.float32)).astype("<u2").tobytes()
+    if dtype == "F32":
+        return np.ascontiguousarray(arr, dtype="<f4").tobytes()
+    if dtype == "Si32":
+        return np.ascontiguousarray(arr, dtype="<i4").tobytes()
+    raise ValueError(dtype)
+
+
+def param_id(namespace: str, name: str) -> bytes:
+    """Stable 16-byte parameter key.  The reference derives it with blake3
+    (crates/gpt-rs/src/params.rs:29-48); only stability and uniqueness matter to a
+    backend's memo, so this build uses blake2b-128 over the same inputs."""
+    base = hashlib.blake2b(name.encode(), digest_size=16).digest()
+    return hashlib.blake2b(b"gpt-rs:param-key:v1" + namespace.encode() + base, digest_size=16).digest()
+
+
+class _ModelBase:
+    """Shared plumbing: parameter registration, program cache, tiny uploads."""
+
+    namespace = "model"
+
+    _instances = itertools.count()
+
+    def __init__(self, backend, dtype: str):
+        self.backend = backend
+        self.dtype = dtype
+        # one memo namespace per model instance (the reference namespaces by model handle)
+        self.namespace = f"{type(self).namespace}#{next(_ModelBase._instances)}"
+        self.param_names: List[str] = []
+        self.param_specs: Dict[str, TensorSpec] = {}
+        self._programs: Dict[tuple, Tuple[Program, dict]] = {}
+        self._param_handles: Optional[list] = None
+
+    # -- parameters ------------------------------------------------------------------
+    def set_param(self, name: str, array: np.ndarray, dtype: Optional[str] = None):
+        """runtime/loader.rs:234-239: materialize once, store under the stable id."""
+        dtype = dtype or self.dtype
+        spec = TensorSpec(dtype, array.shape)
+        handle = self.backend.materialize(spec, _np_to_bytes(array, dtype))
+        self.backend.param_resolver().set(param_id(self.namespace, name), handle)
+        if name not in self.param_specs:
+            self.param_names.append(name)
+        self.param_specs[name] = spec
+        self._param_handles = None
+
+    def param_handle(self, name: str):
+        h = self.backend.param_resolver().get(param_id(self.namespace, name))
+        if h is None:
+            raise KeyError(f"parameter {name} not materialized")
+        return h
+
+    def _declare_params(self, fb: FunctionBuilder) -> Dict[str, Tensor]:
+        return {n: fb.param(self.param_specs[n].dtype, self.param_specs[n].dims) for n in self.param_names}
+
+    def _upload_i32(self, values: Sequence[int]):
+        arr = np.asarray(values, dtype=np.int32)
+        return self.backend.materialize(TensorSpec("Si32", arr.shape), arr.tobytes())
+
+    def _zeros(self, dims):
+        return self.backend.materialize(TensorSpec(self.dtype, dims), None)
+
+    def _run(self, program: Program, args: list, donate: Optional[list] = None):
+        if self._param_handles is None:   # Param inputs are fed by stable id (arena.rs:1163-1168)
+            self._param_handles = [self.param_handle(n) for n in self.param_names]
+        params = self._param_handles
+        don = None
+        if donate is not None:
+            don = list(donate) + [False] * len(params)
+        return self.backend.run_program(program, list(args) + params, don)
+
+
+# ================================================================================ GPT-2
+@dataclass
+class GptConfig:
+    """model/gpt.rs GptConfig."""
+
+    vocab_size: int = 50257
+    context_length: int = 1024
+    embed_dim: int = 768
+    num_layers: int = 12
+    num_heads: int = 12
+    mlp_ratio: int = 4
+    eps: float = 1e-5
+
+    def attention_config(self) -> F.AttentionConfig:
+        return F.AttentionConfig(self.embed_dim, self.num_heads, self.num_heads, self.embed_dim // self.num_heads)
+
+
+class Gpt(_ModelBase):
+    """model/gpt.rs: learned positions, pre-LN blocks with biases, final LN, lm_head[d,V]."""
+
+    namespace = "gpt"
+
+    def __init__(self, config: GptConfig, backend, dtype: str = "F32"):
+        super().__init__(backend, dtype)
+        self.config = config
+        self.attn = config.attention_config()
+
+    @classmethod
+    def random(cls, config: GptConfig, backend, seed: int = 0, dtype: str = "F32", std: float = 0.02) -> "Gpt":
+        """Shapes and constant inits of Gpt::random (model/gpt.rs:128-208); the random
+        stream is numpy's PCG64, not Rust's StdRng."""
+        m = cls(config, backend, dtype)
+        rng = np.random.default_rng(seed)
+        d, hid = config.embed_dim, config.embed_dim * config.mlp_ratio
+
+        def rn(*shape):
+            return (rng.standard_normal(shape, dtype=np.float32) * np.float32(std)).astype(np.float32)
+
+        m.set_param("tok_embeddings.weight", rn(config.vocab_size, d))
+        m.set_param("pos_embeddings", rn(config.context_length, d))
+        for i in range(config.num_layers):
+            p = f"blocks.{i}."
+            m.set_param(p + "ln_1.gamma", np.ones(d, np.float32))
+            m.set_param(p + "ln_1.beta", np.zeros(d, np.float32))
+            m.set_param(p + "attention.w_qkv", rn(d, 3 * d))
+            m.set_param(p + "attention.b_qkv", np.zeros(3 * d, np.float32))
+            m.set_param(p + "attention.w_out", rn(d, d))
+            m.set_param(p + "attention.b_out", np.zeros(d, np.float32))
+            m.set_param(p + "ln_2.gamma", np.ones(d, np.float32))
+            m.set_param(p + "ln_2.beta", np.zeros(d, np.float32))
+            m.set_param(p + "feed_forward.w_in", rn(d, hid))
+            m.set_param(p + "feed_forward.b_in", np.zeros(hid, np.float32))
+            m.set_param(p + "feed_forward.w_out", rn(hid, d))
+            m.set_param(p + "feed_forward.b_out", np.zeros(d, np.float32))
+        m.set_param("final_ln.gamma", np.ones(d, np.float32))
+        m.set_param("final_ln.beta", np.zeros(d, np.float32))
+        m.set_param("lm_head", rn(d, config.vocab_size))
+        return m
+
+    @property
+    def num_layers(self): return self.config.num_layers
+    @property
+    def context_length(self): return self.config.context_length
+
+    # -- graph pieces ----------------------------------------------------------------
+    def _block_tail(self, P, i, x, attn_ctx):
+        p = f"blocks.{i}."
+        eps = self.config.eps
+        attn_out = F.linear(attn_ctx, P[p + "attention.w_out"], P[p + "attention.b_out"])
+        residual = attn_out + x                               # model/gpt.rs:81-97: attn_output.add(x)
+        normed2, *_ = F.layer_norm(residual, P[p + "ln_2.gamma"], P[p + "ln_2.beta"], eps)
+        hidden = F.linear(normed2, P[p + "feed_forward.w_in"], P[p + "feed_forward.b_in"])
+        act = F.gelu(hidden)
+        ff = F.linear(act, P[p + "feed_forward.w_out"], P[p + "feed_forward.b_out"])
+        return ff + residual
+
+    def _build(self, seq: int, capacity: int, decode: bool, batch: int = 1) -> Tuple[Program, dict]:
+        """One program for the whole forward (model/gpt.rs:585-751)."""
+        key = (seq, capacity, decode, batch)
+        if key in self._programs:
+            return self._programs[key]
+        cfg, L = self.config, self.config.num_layers
+        hkv, dh = self.attn.num_key_value_heads, self.attn.kv_head_dim
+        fb = FunctionBuilder("main", self.dtype)
+        rows = seq * batch
+        tok = fb.param("Si32", [rows])
+        pos = fb.param("Si32", [rows])
+        layout = {"args": ["tokens", "positions"]}
+        if decode:
+            upd = fb.param("Si32", [3])
+            qst = fb.param("Si32", [1])
+            layout["args"] += ["update_starts", "query_start"]
+            caches = [[(fb.param(self.dtype, [hkv, capacity, dh]), fb.param(self.dtype, [hkv, capacity, dh]))
+                       for _ in range(L)] for _ in range(batch)]
+        else:
+            start_zeros = fb.param("Si32", [3])
+            layout["args"] += ["start_zeros"]
+            bases = [[(fb.param(self.dtype, [hkv, capacity, dh]), fb.param(self.dtype, [hkv, capacity, dh]))
+                      for _ in range(L)] for _ in range(batch)]
+        layout["n_args"] = len(fb.params)
+        P = self._declare_params(fb)
+
+        tok_emb = F.embedding_lookup(P["tok_embeddings.weight"], tok)
+        pos_emb = F.embedding_lookup(P["pos_embeddings"], pos)
+        hidden = tok_emb + pos_emb
+        new_caches = [[None] * L for _ in range(batch)]
+        for i in range(L):
+            p = f"blocks.{i}."
+            normed, *_ = F.layer_norm(hidden, P[p + "ln_1.gamma"], P[p + "ln_1.beta"], cfg.eps)
+            qkv = F.linear(normed, P[p + "attention.w_qkv"], P[p + "attention.b_qkv"])
+            ctxs = []
+            for b in range(batch):
+                qkv_b = qkv if batch == 1 else qkv.slice([b * seq, 0], [seq, qkv.dims[1]])
+                if decode:
+                    ck, cv = caches[b][i]
+                    ctx, k2, v2 = F.attention_decode_cache(self.attn, qkv_b, ck, cv, upd, qst)
+                else:
+                    ctx, k, v = F.attention(self.attn, qkv_b, None)
+                    kb, vb = bases[b][i]
+                    k2 = F.dynamic_update_slice_into(kb, k, start_zeros)   # model/gpt.rs:712-730
+                    v2 = F.dynamic_update_slice_into(vb, v, start_zeros)
+                new_caches[b][i] = (k2, v2)
+                ctxs.append(ctx)
+            ctx_all = ctxs[0] if batch == 1 else Tensor.concat(0, ctxs)
+            hidden = self._block_tail(P, i, hidden, ctx_all)
+        normalized, *_ = F.layer_norm(hidden, P["final_ln.gamma"], P["final_ln.beta"], cfg.eps)
+        logits = normalized.matmul(P["lm_head"])
+        results = []
+        for b in range(batch):
+            for i in range(L):
+                results += list(new_caches[b][i])
+        results.append(logits)
+        fb.set_results(results)
+        prog = Program(fb)
+        self._programs[key] = (prog, layout)
+        return prog, layout
+
+    # -- forward -----------------------------------------------------------------------
+    def forward_with_decode_cache(self, tokens: Sequence[int], position_offset: int,
+                                  caches: List[Optional[DecodeKvCache]], fixed_capacity: Optional[int] = None):
+        """model/gpt.rs:585-751.  Returns the logits handle [T, V]; `caches` is updated in place."""
+        return self.forward_batch([list(tokens)], position_offset, [caches], fixed_capacity)
+
+    def forward_batch(self, token_rows: List[List[int]], position_offset: int,
+                      caches: List[List[Optional[DecodeKvCache]]], fixed_capacity: Optional[int] = None):
+        """Independent sequences sharing the weights: row-stacked hidden states, one M=B*T
+        GEMM per linear, per-sequence attention.  The reference has no batch dimension
+        (ops/functional/attention.rs:189-203); with one row this is exactly its path."""
+        cfg = self.config
+        batch, seq = len(token_rows), len(token_rows[0])
+        if seq == 0:
+            raise ValueError("token sequence must contain at least one element")
+        if any(len(r) != seq for r in token_rows):
+            raise ValueError("all sequences of a batch must have equal length")
+        total = position_offset + seq
+        if total > cfg.context_length:
+            raise ValueError(f"token sequence length {total} exceeds model context length {cfg.context_length}")
+        for row in token_rows:
+            for t in row:
+                if not 0 <= t < cfg.vocab_size:
+                    raise ValueError(f"token index {t} out of range")
+        if any(len(c) != cfg.num_layers for c in caches):
+            raise ValueError(f"expected {cfg.num_layers} cache slots (one per layer)")
+        if fixed_capacity is not None:
+            if not 0 < fixed_capacity <= cfg.context_length or fixed_capacity < total:
+                raise ValueError(f"decode cache capacity {fixed_capacity} invalid for sequence length {total}")
+            capacity = fixed_capacity
+        else:
+            capacity = decode_cache_capacity(total, cfg.context_length)
+        have = caches[0][0] is not None
+        if have and caches[0][0].capacity < capacity:
+            self._grow_caches(caches, capacity)
+        if have and (seq != 1):
+            raise ValueError("decode with an existing cache supports one token per sequence")
+        L = cfg.num_layers
+        prog, _ = self._build(seq, capacity, have, batch)
+        toks = [t for row in token_rows for t in row]
+        poss = [position_offset + j for _ in range(batch) for j in range(seq)]
+        args = [self._upload_i32(toks), self._upload_i32(poss)]
+        if have:
+            for c in caches:
+                for slot in c:
+                    if slot.len != position_offset:
+                        raise ValueError(f"decode cache length {slot.len} must match position offset {position_offset}")
+            args += [self._upload_i32([0, position_offset, 0]), self._upload_i32([position_offset])]
+            kv = [h for c in caches for slot in c for h in (slot.keys, slot.values)]
+        else:
+            hkv, dh = self.attn.num_key_value_heads, self.attn.kv_head_dim
+            args.append(self._upload_i32([0, 0, 0]))
+            kv = [self._zeros([hkv, capacity, dh]) for _ in range(2 * L * batch)]
+        donate = [False] * len(args) + [True] * len(kv)       # old caches are dropped (gpt.rs:738-747)
+        outs = self._run(prog, args + kv, donate)
+        it = iter(outs[:-1])
+        for b in range(batch):
+            for i in range(L):
+                k, v = next(it), next(it)
+                caches[b][i] = DecodeKvCache(k, v, total, capacity)
+        return outs[-1]
+
+    def _grow_caches(self, caches, capacity: int):
+        """model/gpt.rs:626-657: copy each layer's cache into a larger zero buffer."""
+        hkv, dh = self.attn.num_key_value_heads, self.attn.kv_head_dim
+        old_cap = caches[0][0].capacity
+        key = ("grow", old_cap, capacity)
+        if key not in self._programs:
+            fb = FunctionBuilder("main", self.dtype)
+            base = fb.param(self.dtype, [hkv, capacity, dh])
+            old = fb.param(self.dtype, [hkv, old_cap, dh])
+            st = fb.param("Si32", [3])
+            fb.set_results([F.dynamic_update_slice_into(base, old, st)])
+            self._programs[key] = (Program(fb), {})
+        prog = self._programs[key][0]
+        st = self._upload_i32([0, 0, 0])
+        for c in caches:
+            for i, slot in enumerate(c):
+                k = self.backend.run_program(prog, [self._zeros([hkv, capacity, dh]), slot.keys, st], [True, False, False])[0]
+                v = self.backend.run_program(prog, [self._zeros([hkv, capacity, dh]), slot.values, st], [True, False, False])[0]
+                c[i] = DecodeKvCache(k, v, slot.len, capacity)
+
+
+# ================================================================================ Ministral
+@dataclass
+class MinistralConfig:
+    """model/ministral.rs MinistralConfig."""
+
+    vocab_size: int = 131072
+    context_length: int = 4096
+    embed_dim: int = 3072
+    num_layers: int = 26
+    num_heads: int = 32
+    num_kv_heads: int = 8
+    head_dim: int = 128
+    ffn_dim: int = 9216
+    rotary_dim: int = 128
+    rope_theta: float = 1e6
+    eps: float = 1e-5
+
+    def attention_config(self) -> F.AttentionConfig:
+        return F.AttentionConfig(self.embed_dim, self.num_heads, self.num_kv_heads, self.head_dim)
+
+
+class Ministral(_ModelBase):
+    """model/ministral.rs: RMSNorm, packed-QKV RoPE from host tables, GQA, SwiGLU, no biases,
+    untied lm_head."""
+
+    namespace = "ministral"
+
+    def __init__(self, config: MinistralConfig, backend, dtype: str = "Bf16"):
+        super().__init__(backend, dtype)
+        self.config = config
+        self.attn = config.attention_config()
+        self.rope = F.RopeConfig(config.rotary_dim, config.rope_theta, None)
+
+    @classmethod
+    def random(cls, config: MinistralConfig, backend, seed: int = 0, dtype: str = "Bf16", std: float = 0.02):
+        m = cls(config, backend, dtype)
+        rng = np.random.default_rng(seed)
+        d, a = config.embed_dim, config.attention_config()
+
+        def rn(*shape):
+            out = rng.standard_normal(shape, dtype=np.float32)
+            out *= np.float32(std)
+            return out
+
+        m.set_param("tok_embeddings.weight", rn(config.vocab_size, d))
+        for i in range(config.num_layers):
+            p = f"blocks.{i}."
+            m.set_param(p + "norm_1.gamma", np.ones(d, np.float32))
+            m.set_param(p + "attention.w_qkv", rn(d, a.total_projection_dim))
+            m.set_param(p + "attention.w_out", rn(a.query_projection_dim, d))
+            m.set_param(p + "norm_2.gamma", np.ones(d, np.float32))
+            m.set_param(p + "feed_forward.w_gate", rn(d, config.ffn_dim))
+            m.set_param(p + "feed_forward.w_up", rn(d, config.ffn_dim))
+            m.set_param(p + "feed_forward.w_down", rn(config.ffn_dim, d))
+        m.set_param("final_norm.gamma", np.ones(d, np.float32))
+        m.set_param("lm_head", rn(d, config.vocab_size))
+        return m
+
+    @property
+    def num_layers(self): return self.config.num_layers
+    @property
+    def context_length(self): return self.config.context_length
+
+    def _linear(self, P, name: str, x: Tensor) -> Tensor:
+        """nn/layers/linear.rs:50-71 without bias.  Subclasses swap in quantized weights."""
+        return F.linear(x, P[name])
+
+    def _build(self, seq: int, capacity: int, decode: bool, batch: int = 1) -> Tuple[Program, dict]:
+        key = (seq, capacity, decode, batch)
+        if key in self._programs:
+            return self._programs[key]
+        cfg, L = self.config, self.config.num_layers
+        hkv, dh = self.attn.num_key_value_heads, self.attn.kv_head_dim
+        half = cfg.rotary_dim // 2
+        fb = FunctionBuilder("main", self.dtype)
+        rows = seq * batch
+        tok = fb.param("Si32", [rows])
+        cos = fb.param(self.dtype, [seq, half])
+        sin = fb.param(self.dtype, [seq, half])
+        layout = {"args": ["tokens", "cos", "sin"]}
+        if decode:
+            upd = fb.param("Si32", [3])
+            qst = fb.param("Si32", [1])
+            caches = [[(fb.param(self.dtype, [hkv, capacity, dh]), fb.param(self.dtype, [hkv, capacity, dh]))
+                       for _ in range(L)] for _ in range(batch)]
+        else:
+            start_zeros = fb.param("Si32", [3])
+            bases = [[(fb.param(self.dtype, [hkv, capacity, dh]), fb.param(self.dtype, [hkv, capacity, dh]))
+                      for _ in range(L)] for _ in range(batch)]
+        layout["n_args"] = len(fb.params)
+        P = self._declare_params(fb)
+
+        hidden = F.embedding_lookup(P["tok_embeddings.weight"], tok)
+        new_caches = [[None] * L for _ in range(batch)]
+        for i in range(L):
+            p = f"blocks.{i}."
+            normed, *_ = F.rms_norm(hidden, P[p + "norm_1.gamma"], cfg.eps)
+            qkv = self._linear(P, p + "attention.w_qkv", normed)
+            ctxs = []
+            for b in range(batch):
+                qkv_b = qkv if batch == 1 else qkv.slice([b * seq, 0], [seq, qkv.dims[1]])
+                qkv_b = F.apply_rope_qkv_packed(self.attn, qkv_b, cos, sin)   # ministral.rs:166-201
+                if decode:
+                    ck, cv = caches[b][i]
+                    ctx, k2, v2 = F.attention_decode_cache(self.attn, qkv_b, ck, cv, upd, qst)
+                else:
+                    ctx, k, v = F.attention(self.attn, qkv_b, None)
+                    kb, vb = bases[b][i]
+                    k2 = F.dynamic_update_slice_into(kb, k, start_zeros)
+                    v2 = F.dynamic_update_slice_into(vb, v, start_zeros)
+                new_caches[b][i] = (k2, v2)
+                ctxs.append(ctx)
+            ctx_all = ctxs[0] if batch == 1 else Tensor.concat(0, ctxs)
+            attn_out = self._linear(P, p + "attention.w_out", ctx_all)
+            residual = attn_out + hidden
+            normed2, *_ = F.rms_norm(residual, P[p + "norm_2.gamma"], cfg.eps)
+            gate = self._linear(P, p + "feed_forward.w_gate", normed2)     # nn/layers/feed_forward.rs GatedFeedForward
+            up = self._linear(P, p + "feed_forward.w_up", normed2)
+            act = F.swiglu(gate, up)
+            ff = self._linear(P, p + "feed_forward.w_down", act)
+            hidden = ff + residual
+        normalized, *_ = F.rms_norm(hidden, P["final_norm.gamma"], cfg.eps)
+        logits = normalized.matmul(P["lm_head"])
+        results = []
+        for b in range(batch):
+            for i in range(L):
+                results += list(new_caches[b][i])
+        results.append(logits)
+        fb.set_results(results)
+        prog = Program(fb)
+        self._programs[key] = (prog, layout)
+        return prog, layout
+
+    def forward_with_decode_cache(self, tokens, position_offset, caches, fixed_capacity=None):
+        """model/ministral.rs:613-766."""
+        return self.forward_batch([list(tokens)], position_offset, [caches], fixed_capacity)
+
+    def forward_batch(self, token_rows, position_offset, caches, fixed_capacity=None):
+        cfg = self.config
+        batch, seq = len(token_rows), len(token_rows[0])
+        if seq == 0:
+            raise ValueError("token sequence must contain at least one element")
+        if any(len(r) != seq for r in token_rows):
+            raise ValueError("all sequences of a batch must have equal length")
+        total = position_offset + seq
+        if total > cfg.context_length:
+            raise ValueError(f"token sequence length {total} exceeds model context length {cfg.context_length}")
+        if fixed_capacity is not None:
+            if not 0 < fixed_capacity <= cfg.context_length or fixed_capacity < total:
+                raise ValueError(f"decode cache capacity {fixed_capacity} invalid for sequence length {total}")
+            capacity = fixed_capacity
+        else:
+            capacity = decode_cache_capacity(total, cfg.context_length)
+        have = caches[0][0] is not None
+        if have and caches[0][0].capacity < capacity:
+            Gpt._grow_caches(self, caches, capacity)
+        if have and seq != 1:
+            raise ValueError("decode with an existing cache supports one token per sequence")
+        L = cfg.num_layers
+        prog, _ = self._build(seq, capacity, have, batch)
+        cos, sin = F.rotary_cos_sin_cache_slice(position_offset, seq, self.rope)   # ministral.rs:253-261
+        half = cfg.rotary_dim // 2
+        toks = [t for row in token_rows for t in row]
+        args = [self._upload_i32(toks),
+                self.backend.materialize(TensorSpec(self.dtype, [seq, half]), _np_to_bytes(cos, self.dtype)),
+                self.backend.materialize(TensorSpec(self.dtype, [seq, half]), _np_to_bytes(sin, self.dtype))]
+        if have:
+            args += [self._upload_i32([0, position_offset, 0]), self._upload_i32([position_offset])]
+            kv = [h for c in caches for slot in c for h in (slot.keys, slot.values)]
+        else:
+            hkv, dh = self.attn.num_key_value_heads, self.attn.kv_head_dim
+            args.append(self._upload_i32([0, 0, 0]))
+            kv = [self._zeros([hkv, capacity, dh]) for _ in range(2 * L * batch)]
+        donate = [False] * len(args) + [True] * len(kv)
+        outs = self._run(prog, args + kv, donate)
+        it = iter(outs[:-1])
+        for b in range(batch):
+            for i in range(L):
+                k, v = next(it), next(it)
+                caches[b][i] = DecodeKvCache(k, v, total, capacity)
+        return outs[-1]
+
+
+# ================================================================================ Generator
+class Generator:
+    """Greedy generation loop (crates/gpt-rs/src/inference/generate.rs:37-203).
+
+    With `device_sampling` the token comes from backend.sample_decode_token (spec.rs:1333-1348)
+    and only 8 bytes cross PCIe per step; otherwise the last logits row is read back and
+    arg-maxed on the host (sampler.rs:96-103).
+    """
+
+    def __init__(self, model, prompt: Sequence[int], kv_cache_capacity: Optional[int] = None,
+                 device_sampling: bool = True):
+        if len(prompt) == 0:
+            raise ValueError("prompt must be non-empty")
+        self.model = model
+        self.tokens = list(prompt)
+        self.capacity = kv_cache_capacity
+        self.device_sampling = device_sampling
+        self.caches: List[Optional[DecodeKvCache]] = [None] * model.num_layers
+        self.window_start = max(0, len(self.tokens) - model.context_length)
+        context = self.tokens[self.window_start:]
+        self.logits = model.forward_with_decode_cache(context, 0, self.caches, self.capacity)
+        self.processed_len = len(context)
+
+    def _sample(self) -> int:
+        be = self.model.backend
+        if self.device_sampling:
+            tok = be.sample_decode_token(self.logits, temperature=0.0)
+            if tok is not None:
+                return tok
+        row = be.to_numpy(self.logits)[-1]
+        return int(np.argmax(row))
+
+    def step(self) -> int:
+        nxt = self._sample()
+        self.tokens.append(nxt)
+        if self.processed_len >= self.model.context_length:
+            # generate.rs:127-134: slide the window and rebuild the caches
+            self.caches = [None] * self.model.num_layers
+            self.window_start = len(self.tokens) - self.model.context_length
+            context = self.tokens[self.window_start:]
+            self.logits = self.model.forward_with_decode_cache(context, 0, self.caches, self.capacity)
+            self.processed_len = len(context)
+        else:
+            self.logits = self.model.forward_with_decode_cache([nxt], self.processed_len, self.caches, self.capacity)
+            self.processed_len += 1
+        return nxt
+
+    def step_final(self) -> int:
+        nxt = self._sample()
+        self.tokens.append(nxt)
+        return nxt
+
+    def generate(self, max_new_tokens: int) -> List[int]:
+        out = []
+        for i in range(max_new_tokens):
+            out.append(self.step() if i + 1 < max_new_tokens else self.step_final())
+        return out

@@ -1,0 +1,147 @@
+/*
+ * gptrs_hip.h -- C ABI of the MI355X (gfx950) PTIR backend, libgptrs_hip.so.
+ *
+ * One entry point per method of the reference's `PortableBackend` trait
+ * (crates/gpt-rs/src/backend/spec.rs:1287-1349) plus the `ParamResolver` pair
+ * (crates/gpt-rs/src/backend/param_resolver.rs:11-50).  A Rust shim crate binds these
+ * with `extern "C"` and implements the trait over them; nothing here exposes torch,
+ * HIP or C++ types.
+ *
+ * Return codes select the `BackendError` variant (spec.rs:1224-1228):
+ *   0 ok, 1 SpecViolation, 2 Unimplemented, 3 Execution.
+ * `gptrs_hip_last_error` returns the message of the calling thread's last failure.
+ *
+ * Threading: every entry point may be called from any thread (`Send + Sync`,
+ * spec.rs:1287); calls on one backend are serialised internally.
+ */
+#ifndef GPTRS_HIP_H
+#define GPTRS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GPTRS_HIP_OK 0
+#define GPTRS_HIP_ERR_SPEC 1
+#define GPTRS_HIP_ERR_UNIMPLEMENTED 2
+#define GPTRS_HIP_ERR_EXECUTION 3
+
+/* dtype tags: 0..4 are the reference C backend's PtirTensor tags
+ * (crates/gpt-rs-backend-c/src/codegen/mod.rs:71-75); 5..7 extend them. */
+#define GPTRS_HIP_F32 0u
+#define GPTRS_HIP_F16 1u
+#define GPTRS_HIP_BF16 2u
+#define GPTRS_HIP_SI32 3u
+#define GPTRS_HIP_I1 4u
+#define GPTRS_HIP_SI8 5u
+#define GPTRS_HIP_UI8 6u
+
+typedef struct gptrs_hip_backend gptrs_hip_backend;
+typedef struct gptrs_hip_tensor gptrs_hip_tensor;
+
+/* Same field order as the reference C backend's PtirTensor minus the data pointer
+ * (crates/gpt-rs-backend-c/src/codegen/mod.rs:64-69): a TensorSpec (spec.rs:210-232)
+ * with static dims. */
+typedef struct {
+    uint32_t dtype;
+    uint32_t rank;
+    const int64_t* dims;
+} gptrs_hip_tensor_desc;
+
+/* Backend construction: the registry constructor `register_portable_backend("hip", ctor)`
+ * (crates/gpt-rs/src/backend/registry.rs:246-260) calls this once per backend instance. */
+int gptrs_hip_create(int device, gptrs_hip_backend** out);
+void gptrs_hip_destroy(gptrs_hip_backend* b);
+
+/* PortableBackend::backend_name (spec.rs:1291): returns "hip". */
+const char* gptrs_hip_backend_name(const gptrs_hip_backend* b);
+
+/* PortableBackend::materialize (spec.rs:1311): TensorInit::Literal when host_bytes is
+ * non-NULL (row-major little-endian, nbytes must equal the spec's byte length),
+ * TensorInit::Zeroed when it is NULL. */
+int gptrs_hip_materialize(gptrs_hip_backend* b, const gptrs_hip_tensor_desc* desc,
+                          const void* host_bytes, size_t nbytes, gptrs_hip_tensor** out);
+
+/* PortableBackend::to_literal (spec.rs:1314): copies the tensor to host memory.
+ * cap must be at least the tensor's byte length. */
+int gptrs_hip_to_literal(gptrs_hip_backend* b, const gptrs_hip_tensor* t, void* host_dst, size_t cap);
+
+/* TensorHandle: Clone / Drop (spec.rs:1288).  Handles are reference counted. */
+void gptrs_hip_tensor_retain(gptrs_hip_tensor* t);
+void gptrs_hip_tensor_release(gptrs_hip_tensor* t);
+
+/* Spec of a handle (what `DeviceTensor::tensor_spec` carries on the Rust side).
+ * dims_out receives up to dims_cap extents; returns the rank, or -1 on a NULL handle. */
+int gptrs_hip_tensor_spec(const gptrs_hip_tensor* t, uint32_t* dtype_out, int64_t* dims_out, size_t dims_cap);
+
+/* PortableBackend::run_program (spec.rs:1324; call site ops/graph/arena.rs:1014).
+ * program_json: serde-JSON text of `Program` (spec.rs:799-807).  program_key: any
+ * non-zero 64-bit key that identifies this text (PlanKey.hash, arena.rs:993); the parsed,
+ * fused and planned form is cached under it.  0 disables the cache.
+ * inputs follow `function.parameter_ids`, outputs follow `function.result_ids`;
+ * n_out must equal the number of results.  Each output is a new handle owned by the
+ * caller.  Inputs are left unchanged. */
+int gptrs_hip_run_program(gptrs_hip_backend* b, const char* program_json, size_t json_len,
+                          uint64_t program_key, gptrs_hip_tensor* const* inputs, size_t n_in,
+                          gptrs_hip_tensor** outputs, size_t n_out);
+
+/* run_program with buffer donation: donate[i] != 0 tells the backend that the caller
+ * drops input i right after the call (what the models do with the previous step's KV
+ * caches, crates/gpt-rs/src/model/gpt.rs:738-747), so a DynamicUpdateSlice of it may
+ * write in place.  A donated handle is consumed: it stays releasable, but reading it
+ * afterwards is an Execution error.  donate may be NULL (no donation). */
+int gptrs_hip_run_program_donate(gptrs_hip_backend* b, const char* program_json, size_t json_len,
+                                 uint64_t program_key, gptrs_hip_tensor* const* inputs,
+                                 const uint8_t* donate, size_t n_in,
+                                 gptrs_hip_tensor** outputs, size_t n_out);
+
+/* PortableBackend::execute_instruction (spec.rs:1317): one Instruction as JSON, operands
+ * positional (literal operands are taken from the JSON). */
+int gptrs_hip_execute_instruction(gptrs_hip_backend* b, const char* instruction_json, size_t json_len,
+                                  gptrs_hip_tensor* const* inputs, size_t n_in, gptrs_hip_tensor** output);
+
+/* ParamResolver::get / set (param_resolver.rs:11-19): stable u128 id, little-endian.
+ * get stores NULL in *out when the id is unknown; a returned handle is retained for
+ * the caller.  set retains the handle for the memo. */
+int gptrs_hip_param_get(gptrs_hip_backend* b, const uint8_t id[16], gptrs_hip_tensor** out);
+int gptrs_hip_param_set(gptrs_hip_backend* b, const uint8_t id[16], gptrs_hip_tensor* t);
+
+/* PortableBackend::supports_decode_sampling (spec.rs:1333): 1 for greedy
+ * (temperature <= 0) and for temperature sampling with a caller-supplied uniform
+ * random_u and no top_k; 0 otherwise. */
+int gptrs_hip_supports_decode_sampling(const gptrs_hip_backend* b, float temperature, int has_top_k,
+                                       int has_random_u);
+
+/* PortableBackend::sample_decode_token (spec.rs:1341): samples from the LAST row of a
+ * [rows, vocab] (or [vocab]) logits tensor on the device; 8 bytes cross PCIe.
+ * Greedy ties go to the smallest index (docs/backend.md:270).  *token_out = -1 means
+ * Ok(None): the request is not served here and the host sampler must run. */
+int gptrs_hip_sample_decode_token(gptrs_hip_backend* b, const gptrs_hip_tensor* logits, float temperature,
+                                  int has_top_k, int has_random_u, float random_u, int64_t* token_out);
+
+/* Message of the calling thread's most recent non-zero return (BackendError Display). */
+const char* gptrs_hip_last_error(void);
+
+/* Blocks until all work queued by this backend has finished (used around timed regions;
+ * to_literal and sample_decode_token synchronise by themselves). */
+int gptrs_hip_synchronize(gptrs_hip_backend* b);
+
+/* Execution options: name in {"fusion", "graphs", "trace"}; value 0/1.  "fusion" = rewrite
+ * matched functional sequences to fused kernels (on by default; off = one generic kernel
+ * per instruction, the reference harness's "optimizer off" leg,
+ * crates/gpt-rs-backend-tests/src/torch_parity/harness.rs:494-511). */
+int gptrs_hip_set_option(gptrs_hip_backend* b, const char* name, int64_t value);
+
+/* Counters since creation (the reference's cache_event / WorkStats fields,
+ * crates/gpt-rs/src/ops/graph/arena.rs:1201-1243): name in {"kernel_launches",
+ * "programs_compiled", "program_cache_hits", "fused_ops", "bytes_allocated",
+ * "inplace_updates", "last_program_launches"}.  Unknown names return -1. */
+int64_t gptrs_hip_counter(const gptrs_hip_backend* b, const char* name);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GPTRS_HIP_H */

@@ -1,0 +1,345 @@
+"""GPU parity, op by op: every PTIR op the LM path emits, HIP vs the CPU oracle on identical
+seeded inputs.  Integer / index ops must be bit-exact; float ops within the reference suite's
+tolerance (5e-4 + 1e-4*max, torch_parity/common.rs:14-15).  Shapes follow the reference's
+parity-case catalogue (crates/gpt-rs-backend-tests/src/lib.rs:99-261)."""
+import numpy as np
+import pytest
+
+from parity import FunctionBuilder, Program, assert_close, check_program, hip_run, oracle_run
+from gptrs_amd import functional as F
+from gptrs_amd.ptir import Tensor
+
+pytestmark = pytest.mark.gpu
+
+
+def rng_uniform(seed, shape, lo=-1.0, hi=1.0):
+    return np.random.default_rng(seed).uniform(lo, hi, size=shape).astype(np.float32)
+
+
+def prog(build, param_specs):
+    fb = FunctionBuilder("main")
+    params = [fb.param(dt, dims) for dt, dims in param_specs]
+    res = build(fb, *params)
+    fb.set_results(list(res) if isinstance(res, (list, tuple)) else [res])
+    return Program(fb)
+
+
+# ------------------------------------------------------------------ reference-held vectors
+def test_smoke_matmul_golden(hip):
+    # crates/gpt-rs-backend-tests/src/smoke.rs:12-24
+    p = prog(lambda fb, a, b: a.matmul(b), [("F32", [2, 2]), ("F32", [2, 2])])
+    out = hip_run(hip, p, [np.array([[1, 2], [3, 4]], np.float32), np.array([[5, 6], [7, 8]], np.float32)])[0]
+    assert out.reshape(-1).tolist() == [19.0, 22.0, 43.0, 50.0]
+
+
+@pytest.mark.parametrize("start,expect", [(-3, [1, 2]), (9, [4, 5]), (2, [3, 4])])
+def test_dynamic_slice_clamp_golden(hip, start, expect):
+    # crates/gpt-rs-backend-triton/tests/dynamic_ops_gpu.rs:35-70
+    p = prog(lambda fb, x, s: x.dynamic_slice(s, [2]), [("F32", [5]), ("Si32", [1])])
+    out = hip_run(hip, p, [np.array([1, 2, 3, 4, 5], np.float32), np.array([start], np.int32)])[0]
+    assert out.tolist() == [float(v) for v in expect]
+
+
+def test_dynamic_slice_si32_golden(hip):
+    p = prog(lambda fb, x, s: x.dynamic_slice(s, [2]), [("Si32", [5]), ("Si32", [1])])
+    out = hip_run(hip, p, [np.array([10, 20, 30, 40, 50], np.int32), np.array([7], np.int32)])[0]
+    assert out.tolist() == [40, 50]
+
+
+@pytest.mark.parametrize("start,expect", [(-2, [99, 88, 12, 13, 14]), (8, [10, 11, 12, 99, 88])])
+def test_dynamic_update_slice_clamp_golden(hip, start, expect):
+    # crates/gpt-rs-backend-triton/tests/dynamic_ops_gpu.rs:72-104
+    p = prog(lambda fb, x, u, s: x.dynamic_update_slice(u, s, [2]), [("F32", [5]), ("F32", [2]), ("Si32", [1])])
+    out = hip_run(hip, p, [np.array([10, 11, 12, 13, 14], np.float32), np.array([99, 88], np.float32),
+                           np.array([start], np.int32)])[0]
+    assert out.tolist() == [float(v) for v in expect]
+
+
+def test_scalar_broadcast_add_golden(hip):
+    # crates/gpt-rs/tests/graph_cache_stability.rs:95-131, lazy_graph.rs:100-132
+    x = np.array([1, 2, 3, 4], np.float32)
+    assert hip_run(hip, prog(lambda fb, a: a + 1.0, [("F32", [4])]), [x])[0].tolist() == [2, 3, 4, 5]
+    assert hip_run(hip, prog(lambda fb, a: a + 2.0, [("F32", [4])]), [x])[0].tolist() == [3, 4, 5, 6]
+    p = prog(lambda fb, a, b: a + b, [("F32", [4]), ("F32", [4])])
+    assert hip_run(hip, p, [np.array([2, 4, 6, 8], np.float32), np.ones(4, np.float32)])[0].tolist() == [3, 5, 7, 9]
+
+
+def test_greedy_sample_golden(hip):
+    # crates/gpt-rs-backend-triton/tests/decode_sampling.rs:6-20
+    from gptrs_amd.ptir import TensorSpec
+    h = hip.materialize(TensorSpec("F32", [1, 4]), np.array([[-1.0, 0.1, 2.5, 0.4]], np.float32))
+    assert hip.sample_decode_token(h, temperature=0.0) == 2
+    assert hip.supports_decode_sampling(0.0) and not hip.supports_decode_sampling(1.0, top_k=5)
+
+
+# ------------------------------------------------------------------ layout / index ops (bit-exact)
+@pytest.mark.parametrize("dtype", ["F32", "Bf16", "Si32"])
+def test_layout_ops_exact(hip, dtype):
+    r = np.random.default_rng(11)
+    x = r.integers(-100, 100, size=(3, 4, 6)).astype(np.float32)
+
+    def build(fb, a):
+        s = a.slice([1, 0, 2], [2, 3, 4])
+        t = a.transpose([2, 0, 1])
+        rs = a.reshape([6, 12])
+        c = Tensor.concat(1, [a, a.slice([0, 1, 0], [3, 2, 6])])
+        b = a.slice([0, 0, 0], [3, 1, 6]).broadcast_to([2, 3, 4, 6])
+        return [s, t, rs, c, b]
+
+    check_program(hip, prog(build, [(dtype, [3, 4, 6])]), [x], atol=0, rtol=0)
+
+
+def test_iota_compare_select_cast_exact(hip):
+    def build(fb, x, y):
+        i0 = fb.iota([5, 7], 0)
+        i1 = fb.iota([5, 7], 1)
+        ge = i0.greater_equal(i1)
+        sel = Tensor.select(ge, x, y)
+        return [i0, i1, ge, sel, ge.cast("Si32"), i1.cast("F32"), x.cast("Si32"), ge.cast("F32"), i0.compare(i1, "NotEqual")]
+
+    x = rng_uniform(1, (5, 7), -300, 300)
+    y = rng_uniform(2, (5, 7))
+    check_program(hip, prog(build, [("F32", [5, 7]), ("F32", [5, 7])]), [x, y], atol=0, rtol=0)
+
+
+def test_cast_saturation_and_nan(hip):
+    x = np.array([1.9, -1.9, 3e9, -3e9, np.nan, 0.0, -0.0, 1e-30], np.float32)
+    check_program(hip, prog(lambda fb, a: [a.cast("Si32"), a.cast("I1"), a.cast("Bf16")], [("F32", [8])]), [x], atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("vocab,embed,seq", [(64, 32, 16), (32, 8, 5), (32, 128, 8)])
+def test_take_embedding_exact(hip, vocab, embed, seq):
+    w = rng_uniform(3, (vocab, embed))
+    idx = np.random.default_rng(4).integers(0, vocab, size=seq).astype(np.int32)
+    idx[-1] = idx[0]  # duplicate indices
+    check_program(hip, prog(lambda fb, t, i: F.embedding_lookup(t, i), [("F32", [vocab, embed]), ("Si32", [seq])]),
+                  [w, idx], atol=0, rtol=0)
+
+
+def test_take_out_of_range_is_an_execution_error(hip):
+    from gptrs_amd.backend import BackendError
+    p = prog(lambda fb, t, i: t.take(i), [("F32", [8, 4]), ("Si32", [2])])
+    with pytest.raises(BackendError) as ei:
+        hip_run(hip, p, [np.zeros((8, 4), np.float32), np.array([1, 8], np.int32)])
+    assert ei.value.kind == "execution" and "out of bounds" in str(ei.value)
+
+
+def test_dynamic_ops_rank3_exact(hip):
+    base = rng_uniform(5, (4, 16, 8))
+    upd = rng_uniform(6, (4, 1, 8))
+    for pos in (0, 7, 15, 40, -3):
+        st = np.array([0, pos, 0], np.int32)
+        p = prog(lambda fb, b, u, s: [b.dynamic_update_slice(u, s, [4, 1, 8]), b.dynamic_slice(s, [4, 2, 8])],
+                 [("F32", [4, 16, 8]), ("F32", [4, 1, 8]), ("Si32", [3])])
+        check_program(hip, p, [base, upd, st], atol=0, rtol=0)
+
+
+# ------------------------------------------------------------------ float ops
+MATMUL_SHAPES = [(1, 1, 1), (1, 5, 3), (4, 5, 1), (7, 13, 9), (33, 65, 31), (8, 1, 8), (1, 16, 17), (64, 128, 32)]
+
+
+@pytest.mark.parametrize("m,k,n", MATMUL_SHAPES)
+@pytest.mark.parametrize("dtype", ["F32", "Bf16"])
+def test_matmul(hip, m, k, n, dtype):
+    # torch_parity/matmul.rs:78-115
+    a, b = rng_uniform(7, (m, k)), rng_uniform(8, (k, n))
+    tol = dict(atol=5e-4, rtol=1e-4) if dtype == "F32" else dict(atol=2e-2, rtol=2e-2)
+    check_program(hip, prog(lambda fb, x, y: x.matmul(y), [(dtype, [m, k]), (dtype, [k, n])]), [a, b], **tol)
+
+
+@pytest.mark.parametrize("b,m,k,n", [(1, 4, 5, 2), (2, 7, 13, 9), (8, 4, 8, 4), (3, 33, 65, 31)])
+def test_matmul_batched(hip, b, m, k, n):
+    a, c = rng_uniform(9, (b, m, k)), rng_uniform(10, (b, k, n))
+    check_program(hip, prog(lambda fb, x, y: x.matmul(y), [("F32", [b, m, k]), ("F32", [b, k, n])]), [a, c])
+
+
+def test_dot_general_attention_contractions(hip):
+    q, kk, v = rng_uniform(1, (4, 3, 8)), rng_uniform(2, (4, 5, 8)), rng_uniform(3, (4, 5, 8))
+
+    def build(fb, a, b, c):
+        s = a.dot_general(b, [0], [2], [2])
+        return [s, s.dot_general(c, [0], [2], [1])]
+
+    check_program(hip, prog(build, [("F32", [4, 3, 8]), ("F32", [4, 5, 8]), ("F32", [4, 5, 8])]), [q, kk, v])
+
+
+def test_dot_general_non_collapsible_operands(hip):
+    # contraction over two non-adjacent lhs axes forces the repack path
+    a, b = rng_uniform(1, (3, 4, 5)), rng_uniform(2, (3, 5, 6))
+    p = prog(lambda fb, x, y: x.dot_general(y, [], [0, 2], [0, 1]), [("F32", [3, 4, 5]), ("F32", [3, 5, 6])])
+    check_program(hip, p, [a, b])
+
+
+@pytest.mark.parametrize("shape", [(3, 2, 4), (2, 1), (3, 2), (2, 7), (4, 128), (2, 3, 8), (2, 4, 32), (1, 3, 257), (4, 768)])
+@pytest.mark.parametrize("dtype", ["F32", "Bf16"])
+def test_softmax(hip, shape, dtype):
+    x = rng_uniform(12, shape, -3, 3)
+    tol = dict() if dtype == "F32" else dict(atol=1e-2, rtol=2e-2)
+    check_program(hip, prog(lambda fb, a: F.softmax_last_axis(a), [(dtype, list(shape))]), [x], **tol)
+
+
+def test_softmax_extreme_and_constant(hip):
+    x = rng_uniform(13, (4, 16), -80, 80)
+    check_program(hip, prog(lambda fb, a: F.softmax_last_axis(a), [("F32", [4, 16])]), [x], atol=5e-3, rtol=5e-3)
+    c = np.full((2, 3, 17), 0.25, np.float32)
+    out = check_program(hip, prog(lambda fb, a: F.softmax_last_axis(a), [("F32", [2, 3, 17])]), [c])
+    assert np.allclose(out[0].sum(-1), 1.0, atol=1e-6)
+
+
+@pytest.mark.parametrize("shape,lo,hi", [((6,), -1, 1), ((256,), -1, 1), ((4, 16), -1, 1), ((2, 3, 8), -1, 1), ((256,), -10, 10)])
+def test_gelu(hip, shape, lo, hi):
+    x = rng_uniform(14, shape, lo, hi)
+    check_program(hip, prog(lambda fb, a: F.gelu(a), [("F32", list(shape))]), [x])
+
+
+def test_silu_and_swiglu(hip):
+    check_program(hip, prog(lambda fb, a: F.silu(a), [("F32", [3, 17])]), [rng_uniform(15, (3, 17), -40, 40)])
+    g, u = rng_uniform(16, (5, 19), -10, 10), rng_uniform(17, (5, 19))
+    check_program(hip, prog(lambda fb, a, b: F.swiglu(a, b), [("F32", [5, 19]), ("F32", [5, 19])]), [g, u])
+    check_program(hip, prog(lambda fb, a, b: F.swiglu(a, b), [("Bf16", [5, 19]), ("Bf16", [5, 19])]), [g, u], atol=5e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("shape", [(3, 4), (2, 5, 8), (1, 16, 64), (2, 3, 4, 5)])
+def test_add_bias(hip, shape):
+    x, b = rng_uniform(18, shape), rng_uniform(19, (shape[-1],))
+    check_program(hip, prog(lambda fb, a, c: F.add_bias(a, c), [("F32", list(shape)), ("F32", [shape[-1]])]), [x, b])
+
+
+@pytest.mark.parametrize("shape,eps", [((2, 3, 4), 1e-5), ((2, 3, 1), 1e-5), ((2, 3, 13), 1e-5), ((2, 4, 256), 1e-5), ((1, 8), 1e-5),
+                                       ((2, 3, 17), 1e-3), ((4, 768), 1e-5), ((3, 3072), 1e-5), ((2, 5000), 1e-5)])
+def test_layer_norm_all_outputs(hip, shape, eps):
+    # checks out, normalized, mean, inv_std like torch_parity/functional_ops.rs
+    n = shape[-1]
+    x, g, b = rng_uniform(20, shape), rng_uniform(21, (n,)), rng_uniform(22, (n,))
+    p = prog(lambda fb, a, c, d: list(F.layer_norm(a, c, d, eps)), [("F32", list(shape)), ("F32", [n]), ("F32", [n])])
+    check_program(hip, p, [x, g, b], atol=2e-3 if n == 1 else 5e-4)
+    p1 = prog(lambda fb, a, c, d: F.layer_norm(a, c, d, eps)[0], [("F32", list(shape)), ("F32", [n]), ("F32", [n])])
+    check_program(hip, p1, [x, g, b])
+
+
+def test_layer_norm_constant_input_gives_beta(hip):
+    x = np.full((2, 3, 17), 0.5, np.float32)
+    g, b = rng_uniform(1, (17,)), rng_uniform(2, (17,))
+    p = prog(lambda fb, a, c, d: F.layer_norm(a, c, d, 1e-5)[0], [("F32", [2, 3, 17]), ("F32", [17]), ("F32", [17])])
+    out = check_program(hip, p, [x, g, b])[0]
+    assert np.allclose(out, np.broadcast_to(b, out.shape), atol=1e-6)
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 4), (5, 16), (1, 3072), (8, 3072)])
+@pytest.mark.parametrize("dtype", ["F32", "Bf16"])
+def test_rms_norm(hip, shape, dtype):
+    n = shape[-1]
+    x, g = rng_uniform(23, shape), rng_uniform(24, (n,))
+    tol = dict() if dtype == "F32" else dict(atol=3e-2, rtol=2e-2)
+    p = prog(lambda fb, a, c: F.rms_norm(a, c, 1e-5)[0], [(dtype, list(shape)), (dtype, [n])])
+    check_program(hip, p, [x, g], **tol)
+
+
+@pytest.mark.parametrize("hq,hkv,dh,rot,seq", [(4, 4, 8, 8, 5), (4, 2, 8, 4, 3), (8, 2, 16, 16, 1), (4, 1, 8, 6, 4)])
+def test_rope_packed(hip, hq, hkv, dh, rot, seq):
+    cfg = F.AttentionConfig(hq * dh, hq, hkv, dh)
+    cos, sin = F.rotary_cos_sin_cache_slice(3, seq, F.RopeConfig(rot, 10000.0))
+    qkv = rng_uniform(25, (seq, cfg.total_projection_dim))
+    p = prog(lambda fb, a, c, s: F.apply_rope_qkv_packed(cfg, a, c, s),
+             [("F32", [seq, cfg.total_projection_dim]), ("F32", [seq, rot // 2]), ("F32", [seq, rot // 2])])
+    out = check_program(hip, p, [qkv, cos, sin])[0]
+    # rotation preserves the norm of each (first, second) pair; V passes through untouched
+    assert np.array_equal(out[:, (hq + hkv) * dh:], qkv[:, (hq + hkv) * dh:])
+
+
+@pytest.mark.parametrize("hq,hkv,dh,seq", [(3, 3, 2, 4), (2, 2, 4, 1), (4, 4, 8, 8), (4, 4, 1, 3), (4, 1, 4, 5), (4, 2, 8, 6), (8, 2, 16, 33)])
+def test_attention_prefill(hip, hq, hkv, dh, seq):
+    # torch_parity/attention.rs: seq4/embed6/H3, seq1 embed8 H2, seq8 embed32 H4, head_dim 1, MQA, GQA
+    cfg = F.AttentionConfig(hq * dh, hq, hkv, dh)
+    qkv = rng_uniform(26, (seq, cfg.total_projection_dim))
+    p = prog(lambda fb, a: list(F.attention(cfg, a, None)), [("F32", [seq, cfg.total_projection_dim])])
+    check_program(hip, p, [qkv])
+
+
+def test_attention_with_concat_cache(hip):
+    cfg = F.AttentionConfig(16, 4, 2, 4)
+    qkv = rng_uniform(27, (3, cfg.total_projection_dim))
+    ck, cv = rng_uniform(28, (2, 4, 4)), rng_uniform(29, (2, 4, 4))
+    p = prog(lambda fb, a, k, v: list(F.attention(cfg, a, (k, v))),
+             [("F32", [3, cfg.total_projection_dim]), ("F32", [2, 4, 4]), ("F32", [2, 4, 4])])
+    check_program(hip, p, [qkv, ck, cv])
+
+
+@pytest.mark.parametrize("dtype", ["F32", "Bf16"])
+@pytest.mark.parametrize("hq,hkv,dh,cap", [(4, 4, 8, 16), (4, 2, 8, 32), (8, 2, 16, 128), (12, 12, 64, 128), (32, 8, 128, 256), (4, 4, 1, 8), (6, 2, 4, 16)])
+def test_attention_decode_cache(hip, dtype, hq, hkv, dh, cap):
+    cfg = F.AttentionConfig(hq * dh, hq, hkv, dh)
+    P = cfg.total_projection_dim
+    specs = [(dtype, [1, P]), (dtype, [hkv, cap, dh]), (dtype, [hkv, cap, dh]), ("Si32", [3]), ("Si32", [1])]
+    p = prog(lambda fb, a, k, v, us, qs: list(F.attention_decode_cache(cfg, a, k, v, us, qs)), specs)
+    tol = dict() if dtype == "F32" else dict(atol=3e-2, rtol=3e-2)
+    for pos in (0, 1, cap // 2, cap - 1):
+        qkv = rng_uniform(30 + pos, (1, P))
+        ck, cv = rng_uniform(31, (hkv, cap, dh)), rng_uniform(32, (hkv, cap, dh))
+        # stale garbage beyond the valid length must not matter (capacity-independence)
+        ck[:, pos + 1:], cv[:, pos + 1:] = 1e3, -1e3
+        check_program(hip, p, [qkv, ck, cv, np.array([0, pos, 0], np.int32), np.array([pos], np.int32)], **tol)
+
+
+def test_decode_equals_prefill_row(hip):
+    # attention_prefill4_decode3 == full (crates/gpt-rs-backend-tests/src/lib.rs:231-232)
+    cfg = F.AttentionConfig(32, 4, 2, 8)
+    P, T, cap = cfg.total_projection_dim, 7, 16
+    qkv = rng_uniform(40, (T, P))
+    full = prog(lambda fb, a: list(F.attention(cfg, a, None)), [("F32", [T, P])])
+    ctx_full, k_full, v_full = hip_run(hip, full, [qkv])
+    dec = prog(lambda fb, a, k, v, us, qs: list(F.attention_decode_cache(cfg, a, k, v, us, qs)),
+               [("F32", [1, P]), ("F32", [2, cap, 8]), ("F32", [2, cap, 8]), ("Si32", [3]), ("Si32", [1])])
+    ck = np.zeros((2, cap, 8), np.float32)
+    cv = np.zeros((2, cap, 8), np.float32)
+    ck[:, :4], cv[:, :4] = k_full[:, :4], v_full[:, :4]
+    for pos in range(4, T):
+        ctx, ck, cv = hip_run(hip, dec, [qkv[pos:pos + 1], ck, cv, np.array([0, pos, 0], np.int32), np.array([pos], np.int32)])
+        assert_close(ctx[0], ctx_full[pos], what=f"decode row {pos}")
+    assert_close(ck[:, :T], k_full)
+
+
+# ------------------------------------------------------------------ error surface
+def test_unknown_custom_call_is_unimplemented(hip):
+    from gptrs_amd.backend import BackendError
+    from gptrs_amd.ptir import TensorSpec
+    p = prog(lambda fb, a: fb.custom_call("gpt_rs.nobody.knows.v1", [a], TensorSpec("F32", [4])), [("F32", [4])])
+    with pytest.raises(BackendError) as ei:
+        hip_run(hip, p, [np.zeros(4, np.float32)])
+    assert ei.value.kind == "unimplemented"
+
+
+def test_wrong_spec_version_and_arity(hip):
+    from gptrs_amd.backend import BackendError
+    from gptrs_amd.ptir import TensorSpec
+    p = prog(lambda fb, a: a + 1.0, [("F32", [4])])
+    js = p.json_bytes.replace(b"ptir.v0.4", b"ptir.v0.3")
+    h = hip.materialize(TensorSpec("F32", [4]), np.zeros(4, np.float32))
+    with pytest.raises(BackendError) as ei:
+        hip.run_program_json(js, 0, [h], 1)
+    assert ei.value.kind == "spec"
+    with pytest.raises(BackendError) as ei:
+        hip.run_program_json(p.json_bytes, 0, [h, h], 1)
+    assert "arity" in str(ei.value)
+    h2 = hip.materialize(TensorSpec("F32", [5]), np.zeros(5, np.float32))
+    with pytest.raises(BackendError):
+        hip.run_program_json(p.json_bytes, 0, [h2], 1)
+
+
+def test_inputs_unchanged_without_donation(hip):
+    from gptrs_amd.ptir import TensorSpec
+    p = prog(lambda fb, b, u, s: b.dynamic_update_slice(u, s, [2]), [("F32", [5]), ("F32", [2]), ("Si32", [1])])
+    base = hip.materialize(TensorSpec("F32", [5]), np.arange(5, dtype=np.float32))
+    upd = hip.materialize(TensorSpec("F32", [2]), np.array([9, 9], np.float32))
+    st = hip.materialize(TensorSpec("Si32", [1]), np.array([1], np.int32))
+    out = hip.run_program(p, [base, upd, st])[0]
+    assert hip.to_numpy(out).tolist() == [0, 9, 9, 3, 4]
+    assert hip.to_numpy(base).tolist() == [0, 1, 2, 3, 4]
+    # donated: the update happens in place and the input handle is consumed
+    before = hip.counter("inplace_updates")
+    out2 = hip.run_program(p, [base, upd, st], [True, False, False])[0]
+    assert hip.to_numpy(out2).tolist() == [0, 9, 9, 3, 4]
+    assert hip.counter("inplace_updates") == before + 1
+    from gptrs_amd.backend import BackendError
+    with pytest.raises(BackendError):
+        hip.to_numpy(base)
