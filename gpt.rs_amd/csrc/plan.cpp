@@ -392,7 +392,7 @@ void Builder::describe(Step& st) {
             c.dyn = 1;
             c.dyn_rank = x.rank();
             if (x.rank() > k::kMaxRank) fail_unimpl("dynamic_slice", "rank above 6");
-            for (int i = 0; i < x.rank(); ++i) { c.dyn_max[i] = x.dims[i] - in.a[i]; c.dyn_stride[i] = xs[i]; }
+            for (int i = 0; i < x.rank(); ++i) { c.dyn_max[i] = x.dims[i] - in.a[i]; c.dyn_stride[i] = c.dyn_max[i] ? xs[i] : 0; }
             st.copies.push_back(c);
             st.elem_size = widen_copies(st.copies, es_of(out));
             break;
@@ -405,7 +405,7 @@ void Builder::describe(Step& st) {
             c.dyn = 2;
             c.dyn_rank = x.rank();
             if (x.rank() > k::kMaxRank) fail_unimpl("dynamic_update_slice", "rank above 6");
-            for (int i = 0; i < x.rank(); ++i) { c.dyn_max[i] = x.dims[i] - u.dims[i]; c.dyn_stride[i] = xs[i]; }
+            for (int i = 0; i < x.rank(); ++i) { c.dyn_max[i] = x.dims[i] - u.dims[i]; c.dyn_stride[i] = c.dyn_max[i] ? xs[i] : 0; }
             st.copies.push_back(c);
             st.elem_size = widen_copies(st.copies, es_of(out));
             break;
