@@ -1,0 +1,191 @@
+#!/usr/bin/env python3
+"""Decode throughput of the HIP PTIR backend on one MI355X.
+
+Workload (BASELINE.json configs[3], batch 1): Ministral-3B-shaped decoder, bf16, random-init
+N(0, 0.02) weights from a seed, prompt of 1024 random token ids, greedy decode with a
+fixed-capacity KV cache.  One "step" = one decode token: upload of the per-step scalars, one
+`run_program` over the whole model, on-device argmax and the 8-byte token readback -- the
+reference's decode-steady protocol (crates/gpt-rs-cli/src/main.rs:976-1051).
+
+Prints ONE JSON line; `value` = tokens/s with all weights and the KV cache resident in HBM.
+`roofline` covers the dominant kernel family (the linear-layer GEMV launches): algorithmic bytes
+(every weight element once + activations in/out) over the HIP-event time of those launches on
+the backend's stream.  `cpu_baseline` times the reference C backend's own GEMV kernels
+(oracle/_ref, built from the reference checkout) on one host core over a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+import __graft_entry__ as entry  # noqa: E402
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def algorithmic_bytes_per_step(cfg, dtype_bytes: int, cache_len: int) -> int:
+    """Minimum HBM traffic of one decode token: every weight once, the valid KV once, the new KV
+    row and the logits written once."""
+    a = cfg.attention_config()
+    per_layer = (cfg.embed_dim * a.total_projection_dim + a.query_projection_dim * cfg.embed_dim
+                 + 3 * cfg.embed_dim * cfg.ffn_dim + 2 * cfg.embed_dim)
+    weights = cfg.num_layers * per_layer + cfg.embed_dim + cfg.embed_dim * cfg.vocab_size
+    kv_row = cfg.num_layers * 2 * cfg.num_kv_heads * cfg.head_dim
+    return dtype_bytes * (weights + kv_row * (cache_len + 1) + cfg.vocab_size + cfg.embed_dim)
+
+
+def cpu_baseline(cfg, seconds_budget: float = 25.0):
+    """Reference C kernels (gpt_rs_c_matmul_f32_cached_b, GEMV path, packed-B cache warm) on one
+    core, f32 (the reference executes no bf16).  Sample: ONE layer's five weight matrices plus a
+    1/8 column slice of lm_head; a token = 26 layers + the full lm_head, extrapolated linearly."""
+    ref_dir = os.path.join(ROOT, "oracle", "_ref")
+    flags = open("/proc/cpuinfo").read()
+    name = "libgptrs_c_ref_avx512.so" if (" avx512f" in flags and " fma" in flags) else "libgptrs_c_ref_avx2.so"
+    path = os.path.join(ref_dir, name)
+    if not os.path.exists(path):
+        return None
+    lib = ctypes.CDLL(path)
+    fp = ctypes.POINTER(ctypes.c_float)
+    lib.gptrs_ref_cache_new.restype = ctypes.c_void_p
+    lib.gptrs_ref_cache_free.argtypes = [ctypes.c_void_p]
+    lib.gptrs_ref_matmul_f32_cached.argtypes = [fp, fp, fp, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_void_p]
+    a = cfg.attention_config()
+    d, f = cfg.embed_dim, cfg.ffn_dim
+    head_cols = cfg.vocab_size // 8
+    shapes = [(d, a.total_projection_dim), (a.query_projection_dim, d), (d, f), (d, f), (f, d), (d, head_cols)]
+    rng = np.random.default_rng(0)
+    mats, caches, xs, ys = [], [], [], []
+    for k, n in shapes:
+        w = rng.standard_normal((k, n), dtype=np.float32)
+        w *= np.float32(0.02)
+        mats.append(w)
+        caches.append(lib.gptrs_ref_cache_new())
+        xs.append(rng.standard_normal((1, k), dtype=np.float32))
+        ys.append(np.empty((1, n), np.float32))
+
+    def call(i):
+        k, n = shapes[i]
+        lib.gptrs_ref_matmul_f32_cached(xs[i].ctypes.data_as(fp), mats[i].ctypes.data_as(fp), ys[i].ctypes.data_as(fp), 1, n, k, caches[i])
+
+    for i in range(len(shapes)):
+        call(i)  # packs B once (gpt_rs_c_prepare warms this cache in the reference)
+    t_layer, t_head, reps = 0.0, 0.0, 0
+    t_start = time.perf_counter()
+    while reps < 3 or (time.perf_counter() - t_start < seconds_budget / 3 and reps < 20):
+        t0 = time.perf_counter()
+        for i in range(5):
+            call(i)
+        t1 = time.perf_counter()
+        call(5)
+        t2 = time.perf_counter()
+        t_layer += t1 - t0
+        t_head += t2 - t1
+        reps += 1
+    for c in caches:
+        lib.gptrs_ref_cache_free(c)
+    t_token = cfg.num_layers * t_layer / reps + 8 * t_head / reps
+    return {"value": round(1.0 / t_token, 4), "unit": "tokens/s", "cores": 1, "kind": "reference",
+            "sample": f"{reps} reps of one layer's 5 f32 GEMVs + 1/8 of lm_head through {name} "
+                      f"(gpt_rs_c_matmul_f32_cached_b, m=1, packed-B cache warm); token time = 26 layers + "
+                      f"8 head slices; non-GEMV ops excluded"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=224)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--prompt", type=int, default=1024)
+    ap.add_argument("--layers", type=int, default=26, help="debug only: fewer layers is NOT the benchmark config")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (no collectives, no sharding); --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    entry.load_package()
+    from gptrs_amd import models
+    from gptrs_amd.backend import HipBackend
+
+    be = HipBackend(0)
+    cfg = models.MinistralConfig(num_layers=args.layers)
+    total_len = args.prompt + args.warmup + args.steps + 1
+    capacity = max(1280, (total_len + 255) // 256 * 256)
+    if capacity > cfg.context_length:
+        raise SystemExit(f"prompt + warmup + steps = {total_len} exceeds the context length {cfg.context_length}")
+    t0 = time.perf_counter()
+    model = models.Ministral.random(cfg, be, seed=5, dtype="Bf16")
+    t_init = time.perf_counter() - t0
+    prompt = np.random.default_rng(6).integers(0, cfg.vocab_size, args.prompt).tolist()
+
+    # prefill (reported separately, crates/gpt-rs-cli/src/main.rs:900-935): first call compiles the plan
+    gen = models.Generator(model, prompt, kv_cache_capacity=capacity)
+    be.synchronize()
+    t0 = time.perf_counter()
+    gen = models.Generator(model, prompt, kv_cache_capacity=capacity)
+    be.synchronize()
+    t_prefill = time.perf_counter() - t0
+
+    for _ in range(args.warmup):
+        gen.step()
+    be.synchronize()
+    start_len = gen.processed_len
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        gen.step()
+    be.synchronize()
+    elapsed = time.perf_counter() - t0
+    launches = be.counter("last_program_launches")
+
+    # second pass over fresh steps with every linear launch bracketed by HIP events
+    prof_steps = min(32, capacity - gen.processed_len - 1)
+    roof = None
+    if prof_steps > 0:
+        be.set_option("profile", 1)
+        for _ in range(prof_steps):
+            gen.step()
+        t_ns = be.counter("linear_time_ns")
+        calls = be.counter("linear_calls")
+        nbytes = be.counter("linear_bytes")
+        be.set_option("profile", 0)
+        if t_ns > 0:
+            achieved = nbytes / (t_ns * 1e-9) / 1e9
+            roof = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                    "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                    "kernel": "gemv_kernel<bf16> (+gemv_reduce_kernel): all linear layers of a decode step",
+                    "launches": calls, "avg_launch_us": round(t_ns / max(calls, 1) / 1e3, 2),
+                    "bytes_per_launch": round(nbytes / max(calls, 1))}
+
+    mid_len = start_len + args.steps // 2
+    step_bytes = algorithmic_bytes_per_step(cfg, 2, mid_len)
+    ms_per_step = elapsed / args.steps * 1e3
+    out = {
+        "metric": "decode tokens/s, Ministral-3B-shape bf16 batch 1 (HBM GB/s as % of 8 TB/s in hbm_frac)",
+        "value": round(args.steps / elapsed, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "ministral-3b-shape bf16 decode, batch 1, prompt 1024, greedy, KV capacity %d" % capacity,
+                   "layers": cfg.num_layers, "d_model": cfg.embed_dim, "heads": cfg.num_heads, "kv_heads": cfg.num_kv_heads,
+                   "head_dim": cfg.head_dim, "ffn": cfg.ffn_dim, "vocab": cfg.vocab_size, "cache_len_mid": mid_len},
+        "hbm_gbps": round(step_bytes / (elapsed / args.steps) / 1e9, 1),
+        "hbm_frac": round(step_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS, 4),
+        "algorithmic_bytes_per_step": step_bytes,
+        "launches_per_step": launches,
+        "prefill_ms": round(t_prefill * 1e3, 2), "prefill_tokens": args.prompt,
+        "weight_init_s": round(t_init, 1),
+        "roofline": roof,
+        "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(cfg),
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

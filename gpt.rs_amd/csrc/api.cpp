@@ -68,6 +68,7 @@ Backend::Backend(int dev) : device(dev) {
 Backend::~Backend() {
     (void)hipSetDevice(device);
     if (stream) (void)hipStreamSynchronize(stream);
+    try { profile_collect(); } catch (...) {}
     for (auto& kv : params_) {
         if (kv.second->refs.fetch_sub(1) == 1) delete kv.second;
     }
@@ -82,6 +83,24 @@ Backend::~Backend() {
     (void)hipFree(d_token_);
     if (h_pinned_) (void)hipHostFree(h_pinned_);
     if (stream) (void)hipStreamDestroy(stream);
+}
+
+void Backend::profile_collect() {
+    if (prof_events.empty()) return;
+    GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
+    for (auto& pr : prof_events) {
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, pr.first, pr.second) == hipSuccess) prof_linear_ns += (double)ms * 1e6;
+        (void)hipEventDestroy(pr.first);
+        (void)hipEventDestroy(pr.second);
+    }
+    prof_events.clear();
+}
+void Backend::profile_reset() {
+    profile_collect();
+    prof_linear_ns = 0.0;
+    prof_linear_calls = 0;
+    prof_linear_bytes = 0;
 }
 
 BufferP Backend::new_buffer(size_t bytes) {
@@ -269,6 +288,7 @@ void Backend::execute(Plan& plan, gptrs_hip_tensor* const* inputs, const uint8_t
     cx.consts = plan.consts ? (char*)plan.consts->ptr : nullptr;
     cx.err_flag = d_err_flag_;
     cx.counters = d_counters_;
+    cx.profile = opt_profile;
     cx.ptr.assign(plan.values.size(), nullptr);
     for (size_t v = 0; v < plan.values.size(); ++v) {
         if (!plan.values[v].defined) continue;
@@ -530,12 +550,22 @@ int gptrs_hip_set_option(gptrs_hip_backend* b, const char* name, int64_t value) 
         if (!b || !name) gptrs::fail_exec("null argument");
         std::lock_guard<std::mutex> g(b->impl.mu);
         if (!strcmp(name, "fusion")) b->impl.opt_fusion = value != 0;
+        else if (!strcmp(name, "profile")) { b->impl.profile_reset(); b->impl.opt_profile = value != 0; }
         else gptrs::fail_spec(std::string("unknown option `") + name + "`");
     });
 }
 
 int64_t gptrs_hip_counter(const gptrs_hip_backend* b, const char* name) {
     if (!b || !name) return -1;
+    if (!strncmp(name, "linear_", 7)) {
+        Backend& m = const_cast<Backend&>(b->impl);
+        std::lock_guard<std::mutex> g(m.mu);
+        try { m.profile_collect(); } catch (...) { return -1; }
+        if (!strcmp(name, "linear_time_ns")) return (int64_t)m.prof_linear_ns;
+        if (!strcmp(name, "linear_calls")) return m.prof_linear_calls;
+        if (!strcmp(name, "linear_bytes")) return m.prof_linear_bytes;
+        return -1;
+    }
     const Backend& i = b->impl;
     if (!strcmp(name, "kernel_launches")) return i.n_launches;
     if (!strcmp(name, "programs_compiled")) return i.n_compiled;

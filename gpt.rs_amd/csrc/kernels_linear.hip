@@ -3,8 +3,8 @@
 //
 //  * M <= 16  (decode): HBM-bound GEMV.  Lanes run along N so every wave load is a run of
 //    contiguous 16-byte words of one weight row; K is split across the 16 row-groups of a block
-//    and across blockIdx.y; partial sums meet in LDS, then (split-K) in a scratch buffer whose
-//    last-arriving block sums the slices in a fixed order, so results are run-to-run identical.
+//    and across blockIdx.y; partial sums meet in LDS, then (split-K) in a scratch buffer that a
+//    small second kernel sums in a fixed order, so results are run-to-run identical.
 //  * M > 16   (prefill): tiled GEMM (gemm_tiled below; MFMA tiles live in kernels_mfma.hip).
 #include "kernels.hpp"
 #include "device_utils.hpp"
@@ -59,10 +59,9 @@ __global__ __launch_bounds__(256) void gemv_kernel(const T* __restrict__ x, cons
     constexpr int LN = VEC == 1 ? 64 : 16;  // lanes along N
     constexpr int RG = 256 / LN;            // row groups per block
     constexpr int CT = LN * VEC;            // columns per block
-    constexpr int U = 4;                    // rows in flight per thread
+    constexpr int U = MT >= 16 ? 2 : 4;      // rows in flight per thread
     __shared__ float xs[MT][kGemvKT];
     __shared__ float red[RG][CT + 1];
-    __shared__ int s_ticket;
 
     const int cn = threadIdx.x % LN, rg = threadIdx.x / LN;
     const int64_t col = (int64_t)blockIdx.x * CT + (int64_t)cn * VEC;
@@ -90,28 +89,27 @@ __global__ __launch_bounds__(256) void gemv_kernel(const T* __restrict__ x, cons
             for (int64_t r0 = rg; r0 < kt; r0 += RG * U) {
                 float wv[U][VEC];
                 float wv2[DUAL ? U : 1][VEC];
+                // all U loads are issued before any is consumed; rows past the end re-read the last
+                // valid row and are multiplied by zero
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
                     const int64_t r = r0 + (int64_t)u * RG;
-                    if (r < kt) {
-                        RowVec<T, VEC>::load(w + (k0 + r) * N + col, wv[u]);
-                        if (DUAL) RowVec<T, VEC>::load(w2 + (k0 + r) * N + col, wv2[u]);
-                    } else {
-#pragma unroll
-                        for (int v = 0; v < VEC; ++v) { wv[u][v] = 0.f; if (DUAL) wv2[u][v] = 0.f; }
-                    }
+                    const int64_t rc = r < kt ? r : kt - 1;
+                    RowVec<T, VEC>::load(w + (k0 + rc) * N + col, wv[u]);
+                    if (DUAL) RowVec<T, VEC>::load(w2 + (k0 + rc) * N + col, wv2[u]);
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
                     const int64_t r = r0 + (int64_t)u * RG;
-                    const int rr = r < kt ? (int)r : 0;
+                    const bool live = r < kt;
+                    const int rr = live ? (int)r : 0;
 #pragma unroll
                     for (int m = 0; m < MT; ++m) {
-                        const float xv = xs[m][rr];
+                        const float xv = live ? xs[m][rr] : 0.f;
 #pragma unroll
                         for (int v = 0; v < VEC; ++v) {
-                            acc[m][v] += xv * wv[u][v];
-                            if (DUAL) acc2[m][v] += xv * wv2[u][v];
+                            acc[m][v] = __builtin_fmaf(xv, wv[u][v], acc[m][v]);
+                            if (DUAL) acc2[m][v] = __builtin_fmaf(xv, wv2[u][v], acc2[m][v]);
                         }
                     }
                 }
@@ -119,11 +117,15 @@ __global__ __launch_bounds__(256) void gemv_kernel(const T* __restrict__ x, cons
         }
     }
 
-    // ---- meet the RG row-groups in LDS, one output row at a time
+    // ---- meet the RG row-groups in LDS, one output row at a time.  The loops over m are fully
+    // unrolled (static register indices); rows m >= M leave through a block-uniform branch.
     const int t = threadIdx.x;
     const int64_t ocol = (int64_t)blockIdx.x * CT + t;
-    for (int m = 0; m < M; ++m) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        if (m >= M) break;
         float tot = 0.f, tot2 = 0.f;
+#pragma unroll
         for (int pass = 0; pass < (DUAL ? 2 : 1); ++pass) {
             __syncthreads();
 #pragma unroll
@@ -147,29 +149,28 @@ __global__ __launch_bounds__(256) void gemv_kernel(const T* __restrict__ x, cons
             }
         }
     }
-    if (S == 1) return;
+}
 
-    // ---- split-K: the last block to arrive for this column tile sums the S slices in order
-    __threadfence();
-    __syncthreads();
-    if (t == 0) s_ticket = atomicAdd(&counters[blockIdx.x], 1);
-    __syncthreads();
-    if (s_ticket != S - 1) return;
-    __threadfence();
-    if (t < CT && ocol < N) {
-        for (int m = 0; m < M; ++m) {
-            float tot = 0.f, tot2 = 0.f;
-            for (int sidx = 0; sidx < S; ++sidx) {
-                tot += __hip_atomic_load(&partial[((int64_t)sidx * M + m) * N + ocol], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (DUAL)
-                    tot2 += __hip_atomic_load(&partial[((int64_t)(S + sidx) * M + m) * N + ocol], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-            const float b = bias ? ldf(bias, ocol) : 0.f;
-            const float r = residual ? ldf(residual, (int64_t)m * N + ocol) : 0.f;
-            stf(y, (int64_t)m * N + ocol, finish(tot, tot2, DUAL, act, b, residual != nullptr, r));
+// Split-K epilogue: sums the S slices in a fixed order (run-to-run identical results) and applies
+// bias / activation / residual.  A separate launch, because a grid-wide "last block finishes"
+// scheme needs device-scope fences, and on this multi-XCD part each such fence writes back and
+// invalidates a whole L2: measured ~90 us per GEMV, against ~3 us for this kernel.
+template <typename T, bool DUAL>
+__global__ void gemv_reduce_kernel(const float* __restrict__ partial, const T* __restrict__ bias,
+                                   const T* __restrict__ residual, T* __restrict__ y, int M, int64_t N, int S, int act) {
+    const int64_t total = (int64_t)M * N;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t col = idx % N;
+        float tot = 0.f, tot2 = 0.f;
+#pragma unroll 8
+        for (int sidx = 0; sidx < S; ++sidx) {
+            tot += partial[(int64_t)sidx * total + idx];
+            if (DUAL) tot2 += partial[(int64_t)(S + sidx) * total + idx];
         }
+        const float b = bias ? ldf(bias, col) : 0.f;
+        const float r = residual ? ldf(residual, idx) : 0.f;
+        stf(y, idx, finish(tot, tot2, DUAL, act, b, residual != nullptr, r));
     }
-    if (t == 0) counters[blockIdx.x] = 0;  // ready for the next launch on this stream
 }
 
 // Launch geometry shared by linear() and linear_workspace_bytes().
@@ -209,6 +210,14 @@ static void launch_gemv(hipStream_t s, const LinearArgs& a, const GemvPlan& p, f
     else
         gemv_kernel<T, VEC, MT, false><<<grid, 256, 0, s>>>((const T*)a.x, (const T*)a.w, nullptr, (const T*)a.bias,
             (const T*)a.residual, (T*)a.y, partial, counters, (int)a.m, a.k, a.n, p.kc, a.act);
+    if (p.splits > 1) {
+        const int64_t total = a.m * a.n;
+        const unsigned g = (unsigned)(cdiv(total, 256) > 2048 ? 2048 : cdiv(total, 256));
+        if (a.w2)
+            gemv_reduce_kernel<T, true><<<g, 256, 0, s>>>(partial, (const T*)a.bias, (const T*)a.residual, (T*)a.y, (int)a.m, a.n, p.splits, a.act);
+        else
+            gemv_reduce_kernel<T, false><<<g, 256, 0, s>>>(partial, (const T*)a.bias, (const T*)a.residual, (T*)a.y, (int)a.m, a.n, p.splits, a.act);
+    }
 }
 template <typename T, int VEC>
 static void launch_gemv_m(hipStream_t s, const LinearArgs& a, const GemvPlan& p, float* partial, int* counters) {

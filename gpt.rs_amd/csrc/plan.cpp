@@ -819,7 +819,20 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
             a.ws = cx.ws + st.scratch_off;
             a.ws_bytes = st.scratch_bytes;
             a.counters = cx.counters;
+            hipEvent_t e0 = nullptr, e1 = nullptr;
+            if (cx.profile) {
+                GPTRS_HIP_CHECK(hipEventCreate(&e0));
+                GPTRS_HIP_CHECK(hipEventCreate(&e1));
+                GPTRS_HIP_CHECK(hipEventRecord(e0, s));
+            }
             k::linear(s, a);
+            if (cx.profile) {
+                GPTRS_HIP_CHECK(hipEventRecord(e1, s));
+                cx.be->prof_events.emplace_back(e0, e1);
+                ++cx.be->prof_linear_calls;
+                // algorithmic bytes: activations in, every weight once, result out
+                cx.be->prof_linear_bytes += (int64_t)dtype_size(out.dtype) * (a.m * a.k + a.k * a.n * (a.w2 ? 2 : 1) + a.m * a.n);
+            }
             cx.launches += (in.act == 2 && a.m > 16) ? 3 : 1;
             break;
         }

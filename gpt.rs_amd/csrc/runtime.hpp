@@ -146,6 +146,13 @@ class Backend {
     hipStream_t stream = nullptr;
     int device = 0;
     bool opt_fusion = true;
+    // opt-in timing of the linear-layer launches with HIP events on the execution stream
+    bool opt_profile = false;
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> prof_events;
+    int64_t prof_linear_calls = 0, prof_linear_bytes = 0;
+    double prof_linear_ns = 0.0;
+    void profile_reset();
+    void profile_collect();  // synchronises, folds pending event pairs into prof_linear_ns
     // counters
     int64_t n_launches = 0, n_compiled = 0, n_cache_hits = 0, n_fused = 0, n_inplace = 0, last_launches = 0;
     int64_t bytes_allocated() const { return (int64_t)pool_.bytes_allocated; }
@@ -181,6 +188,7 @@ struct ExecCtx {
     int* err_flag;
     int* counters;
     int64_t launches = 0;
+    bool profile = false;
 };
 void run_step(const Plan& plan, const Step& st, ExecCtx& cx);
 

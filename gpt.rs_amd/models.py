@@ -15,6 +15,7 @@ from __future__ import annotations
 
 import hashlib
 import itertools
+import os
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -83,6 +84,14 @@ class _ModelBase:
         dtype = dtype or self.dtype
         spec = TensorSpec(dtype, array.shape)
         handle = self.backend.materialize(spec, _np_to_bytes(array, dtype))
+        self.backend.param_resolver().set(param_id(self.namespace, name), handle)
+        if name not in self.param_specs:
+            self.param_names.append(name)
+        self.param_specs[name] = spec
+        self._param_handles = None
+
+    def set_param_bytes(self, name: str, spec: TensorSpec, data: bytes):
+        handle = self.backend.materialize(spec, data)
         self.backend.param_resolver().set(param_id(self.namespace, name), handle)
         if name not in self.param_specs:
             self.param_names.append(name)
@@ -370,27 +379,43 @@ class Ministral(_ModelBase):
 
     @classmethod
     def random(cls, config: MinistralConfig, backend, seed: int = 0, dtype: str = "Bf16", std: float = 0.02):
+        """Shapes and constant inits of Ministral::random (model/ministral.rs:262-330).  Every
+        tensor draws from its own numpy stream SeedSequence([seed, index]), so the weights do not
+        depend on the order or the number of worker threads that generate them."""
+        from concurrent.futures import ThreadPoolExecutor
         m = cls(config, backend, dtype)
-        rng = np.random.default_rng(seed)
         d, a = config.embed_dim, config.attention_config()
-
-        def rn(*shape):
-            out = rng.standard_normal(shape, dtype=np.float32)
-            out *= np.float32(std)
-            return out
-
-        m.set_param("tok_embeddings.weight", rn(config.vocab_size, d))
+        plan = [("tok_embeddings.weight", (config.vocab_size, d), "randn")]
         for i in range(config.num_layers):
             p = f"blocks.{i}."
-            m.set_param(p + "norm_1.gamma", np.ones(d, np.float32))
-            m.set_param(p + "attention.w_qkv", rn(d, a.total_projection_dim))
-            m.set_param(p + "attention.w_out", rn(a.query_projection_dim, d))
-            m.set_param(p + "norm_2.gamma", np.ones(d, np.float32))
-            m.set_param(p + "feed_forward.w_gate", rn(d, config.ffn_dim))
-            m.set_param(p + "feed_forward.w_up", rn(d, config.ffn_dim))
-            m.set_param(p + "feed_forward.w_down", rn(config.ffn_dim, d))
-        m.set_param("final_norm.gamma", np.ones(d, np.float32))
-        m.set_param("lm_head", rn(d, config.vocab_size))
+            plan += [(p + "norm_1.gamma", (d,), "ones"),
+                     (p + "attention.w_qkv", (d, a.total_projection_dim), "randn"),
+                     (p + "attention.w_out", (a.query_projection_dim, d), "randn"),
+                     (p + "norm_2.gamma", (d,), "ones"),
+                     (p + "feed_forward.w_gate", (d, config.ffn_dim), "randn"),
+                     (p + "feed_forward.w_up", (d, config.ffn_dim), "randn"),
+                     (p + "feed_forward.w_down", (config.ffn_dim, d), "randn")]
+        plan += [("final_norm.gamma", (d,), "ones"), ("lm_head", (d, config.vocab_size), "randn")]
+
+        def make(idx):
+            name, shape, kind = plan[idx]
+            if kind == "ones":
+                arr = np.ones(shape, np.float32)
+            else:
+                arr = np.random.default_rng(np.random.SeedSequence([seed, idx])).standard_normal(shape, dtype=np.float32)
+                arr *= np.float32(std)
+            return name, shape, _np_to_bytes(arr, dtype)
+
+        workers = max(1, min(16, (os.cpu_count() or 1)))
+        with ThreadPoolExecutor(max_workers=workers) as ex:
+            # bounded look-ahead keeps at most a few tensors of host memory in flight
+            pending, nxt = [], 0
+            while nxt < len(plan) or pending:
+                while nxt < len(plan) and len(pending) < 2 * workers:
+                    pending.append(ex.submit(make, nxt))
+                    nxt += 1
+                name, shape, data = pending.pop(0).result()
+                m.set_param_bytes(name, TensorSpec(dtype, shape), data)
         return m
 
     @property

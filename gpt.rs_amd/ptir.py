@@ -30,10 +30,11 @@ FLOAT_DTYPES = ("F32", "Bf16", "F16", "F64")
 def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
     """Round-to-nearest-even f32 -> bf16 bit pattern (uint16). NaN stays NaN."""
     x = np.asarray(x, dtype=np.float32, order="C")
-    u = x.reshape(-1).view(np.uint32).astype(np.uint64)
-    rounded = (u + 0x7FFF + ((u >> 16) & 1)) >> 16
-    nan = np.isnan(x)
+    u = x.reshape(-1).view(np.uint32)
+    # uint32 arithmetic wraps only for negative NaNs, which the NaN fix-up below overrides
+    rounded = (u + (np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1)))) >> np.uint32(16)
     out = rounded.astype(np.uint16).reshape(x.shape)
+    nan = np.isnan(x)
     if np.any(nan):
         out = np.where(nan, np.uint16(0x7FC0), out)
     return out

@@ -129,16 +129,20 @@ const char* gptrs_hip_last_error(void);
  * to_literal and sample_decode_token synchronise by themselves). */
 int gptrs_hip_synchronize(gptrs_hip_backend* b);
 
-/* Execution options: name in {"fusion", "graphs", "trace"}; value 0/1.  "fusion" = rewrite
- * matched functional sequences to fused kernels (on by default; off = one generic kernel
- * per instruction, the reference harness's "optimizer off" leg,
- * crates/gpt-rs-backend-tests/src/torch_parity/harness.rs:494-511). */
+/* Execution options: name in {"fusion", "profile"}; value 0/1.  "fusion" = rewrite matched
+ * functional sequences to fused kernels (on by default; off = one generic kernel per
+ * instruction, the reference harness's "optimizer off" leg,
+ * crates/gpt-rs-backend-tests/src/torch_parity/harness.rs:494-511).  "profile" = bracket every
+ * linear-layer launch with HIP events on the execution stream (the per-op ns/calls counters the
+ * reference C backend exports, crates/gpt-rs-backend-c/src/lib.rs:587-671); setting it resets
+ * the linear_* counters. */
 int gptrs_hip_set_option(gptrs_hip_backend* b, const char* name, int64_t value);
 
 /* Counters since creation (the reference's cache_event / WorkStats fields,
  * crates/gpt-rs/src/ops/graph/arena.rs:1201-1243): name in {"kernel_launches",
  * "programs_compiled", "program_cache_hits", "fused_ops", "bytes_allocated",
- * "inplace_updates", "last_program_launches"}.  Unknown names return -1. */
+ * "inplace_updates", "last_program_launches", and with the "profile" option "linear_time_ns",
+ * "linear_calls", "linear_bytes" (these three synchronise)}.  Unknown names return -1. */
 int64_t gptrs_hip_counter(const gptrs_hip_backend* b, const char* name);
 
 #ifdef __cplusplus
