@@ -22,7 +22,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import numpy as np
 
 from . import functional as F
-from .ptir import FunctionBuilder, Program, Tensor, TensorSpec, f32_to_bf16_bits
+from .ptir import FunctionBuilder, Program, Tensor, TensorSpec, bf16_bits_to_f32, f32_to_bf16_bits
 
 
 def decode_cache_capacity(required_len: int, max_len: int) -> int:
@@ -378,10 +378,13 @@ class Ministral(_ModelBase):
         self.rope = F.RopeConfig(config.rotary_dim, config.rope_theta, None)
 
     @classmethod
-    def random(cls, config: MinistralConfig, backend, seed: int = 0, dtype: str = "Bf16", std: float = 0.02):
+    def random(cls, config: MinistralConfig, backend, seed: int = 0, dtype: str = "Bf16", std: float = 0.02,
+               bf16_values: bool = False):
         """Shapes and constant inits of Ministral::random (model/ministral.rs:262-330).  Every
         tensor draws from its own numpy stream SeedSequence([seed, index]), so the weights do not
-        depend on the order or the number of worker threads that generate them."""
+        depend on the order or the number of worker threads that generate them.  `bf16_values`
+        rounds the draws to bf16-representable values whatever the storage dtype, so an f32
+        model can be given exactly the weights of a bf16 one."""
         from concurrent.futures import ThreadPoolExecutor
         m = cls(config, backend, dtype)
         d, a = config.embed_dim, config.attention_config()
@@ -404,6 +407,8 @@ class Ministral(_ModelBase):
             else:
                 arr = np.random.default_rng(np.random.SeedSequence([seed, idx])).standard_normal(shape, dtype=np.float32)
                 arr *= np.float32(std)
+                if bf16_values and dtype != "Bf16":
+                    arr = bf16_bits_to_f32(f32_to_bf16_bits(arr))
             return name, shape, _np_to_bytes(arr, dtype)
 
         workers = max(1, min(16, (os.cpu_count() or 1)))

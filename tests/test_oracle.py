@@ -1,0 +1,413 @@
+"""CPU tests that pin the oracle (oracle/ptir_oracle.py) before anything is compared against it:
+reference-held vectors, brute force, float64 / torch routines, the reference C kernels, and
+invariants chosen so that a dropped term, wrong sign or transposed operand fails."""
+import ctypes
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import __graft_entry__ as entry
+from parity import FunctionBuilder, Program, oracle_run
+from gptrs_amd import functional as F
+from gptrs_amd.ptir import Tensor
+
+po = entry.load_oracle()
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def prog(build, param_specs, dtype="F32"):
+    fb = FunctionBuilder("main", dtype)
+    params = [fb.param(dt, dims) for dt, dims in param_specs]
+    res = build(fb, *params)
+    fb.set_results(list(res) if isinstance(res, (list, tuple)) else [res])
+    return Program(fb)
+
+
+def U(seed, shape, lo=-1.0, hi=1.0):
+    return np.random.default_rng(seed).uniform(lo, hi, size=shape).astype(np.float32)
+
+
+def close(a, e, atol=5e-4, rtol=1e-4):
+    a, e = np.asarray(a, np.float64), np.asarray(e, np.float64)
+    assert a.shape == e.shape
+    assert np.all(np.abs(a - e) <= atol + rtol * np.maximum(np.abs(a), np.abs(e))), np.max(np.abs(a - e))
+
+
+# ---------------------------------------------------------------- vectors held by the reference
+def test_matmul_golden():  # crates/gpt-rs-backend-tests/src/smoke.rs:12-24
+    p = prog(lambda fb, a, b: a.matmul(b), [("F32", [2, 2]), ("F32", [2, 2])])
+    out = oracle_run(p, [np.array([[1, 2], [3, 4]], np.float32), np.array([[5, 6], [7, 8]], np.float32)])[0]
+    assert out.reshape(-1).tolist() == [19.0, 22.0, 43.0, 50.0]
+
+
+def test_dynamic_slice_and_update_golden():  # crates/gpt-rs-backend-triton/tests/dynamic_ops_gpu.rs:35-104
+    ds = prog(lambda fb, x, s: x.dynamic_slice(s, [2]), [("F32", [5]), ("Si32", [1])])
+    x = np.array([1, 2, 3, 4, 5], np.float32)
+    assert oracle_run(ds, [x, np.array([-3], np.int32)])[0].tolist() == [1, 2]
+    assert oracle_run(ds, [x, np.array([9], np.int32)])[0].tolist() == [4, 5]
+    dsi = prog(lambda fb, x, s: x.dynamic_slice(s, [2]), [("Si32", [5]), ("Si32", [1])])
+    assert oracle_run(dsi, [np.array([10, 20, 30, 40, 50], np.int32), np.array([7], np.int32)])[0].tolist() == [40, 50]
+    du = prog(lambda fb, x, u, s: x.dynamic_update_slice(u, s, [2]), [("F32", [5]), ("F32", [2]), ("Si32", [1])])
+    b, u = np.array([10, 11, 12, 13, 14], np.float32), np.array([99, 88], np.float32)
+    assert oracle_run(du, [b, u, np.array([-2], np.int32)])[0].tolist() == [99, 88, 12, 13, 14]
+    assert oracle_run(du, [b, u, np.array([8], np.int32)])[0].tolist() == [10, 11, 12, 99, 88]
+
+
+def test_scalar_broadcast_add_golden():  # crates/gpt-rs/tests/graph_cache_stability.rs:95-131, lazy_graph.rs:100-132
+    x = np.array([1, 2, 3, 4], np.float32)
+    assert oracle_run(prog(lambda fb, a: a + 1.0, [("F32", [4])]), [x])[0].tolist() == [2, 3, 4, 5]
+    assert oracle_run(prog(lambda fb, a: a + 2.0, [("F32", [4])]), [x])[0].tolist() == [3, 4, 5, 6]
+    p = prog(lambda fb, a, b: a + b, [("F32", [4]), ("F32", [4])])
+    assert oracle_run(p, [np.array([2, 4, 6, 8], np.float32), np.ones(4, np.float32)])[0].tolist() == [3, 5, 7, 9]
+
+
+def test_greedy_argmax_golden():  # crates/gpt-rs-backend-triton/tests/decode_sampling.rs:6-20
+    assert po.argmax_first(np.array([-1.0, 0.1, 2.5, 0.4], np.float32)) == 2
+    assert po.argmax_first(np.array([1.0, 3.0, 3.0], np.float32)) == 1  # smallest index on ties
+
+
+# ---------------------------------------------------------------- index ops vs brute force
+def test_index_ops_brute_force():
+    x = np.arange(2 * 3 * 4, dtype=np.float32).reshape(2, 3, 4)
+
+    def build(fb, a):
+        return [a.slice([0, 1, 1], [2, 2, 3]), a.transpose([2, 0, 1]), a.reshape([4, 6]),
+                Tensor.concat(2, [a, a.slice([0, 0, 0], [2, 3, 2])]),
+                a.slice([0, 0, 0], [2, 1, 4]).broadcast_to([2, 5, 4])]
+
+    s, t, r, c, b = oracle_run(prog(build, [("F32", [2, 3, 4])]), [x])
+    for i in range(2):
+        for j in range(2):
+            for k in range(3):
+                assert s[i, j, k] == x[i, j + 1, k + 1]
+    for i in range(4):
+        for j in range(2):
+            for k in range(3):
+                assert t[i, j, k] == x[j, k, i]
+    assert r.reshape(-1).tolist() == x.reshape(-1).tolist()
+    assert c.shape == (2, 3, 6) and np.array_equal(c[:, :, 4:], x[:, :, :2]) and np.array_equal(c[:, :, :4], x)
+    for j in range(5):
+        assert np.array_equal(b[:, j, :], x[:, 0, :])
+
+
+def test_iota_compare_select_take_cast():
+    def build(fb, x, idx, tab):
+        i0, i1 = fb.iota([3, 4], 0), fb.iota([3, 4], 1)
+        ge = i0.greater_equal(i1)
+        return [i0, i1, ge, Tensor.select(ge, x, x * 2.0), tab.take(idx), x.cast("Si32"), ge.cast("F32")]
+
+    x = np.array([[1.9, -1.9, 3e9, -3e9], [np.nan, 0.5, -0.5, 7], [1, 2, 3, 4]], np.float32)
+    idx = np.array([2, 0, 2], np.int32)
+    tab = np.arange(12, dtype=np.float32).reshape(3, 4)
+    i0, i1, ge, sel, tk, ci, gf = oracle_run(prog(build, [("F32", [3, 4]), ("Si32", [3]), ("F32", [3, 4])]), [x, idx, tab])
+    assert i0.tolist() == [[0] * 4, [1] * 4, [2] * 4] and i1.tolist() == [[0, 1, 2, 3]] * 3
+    assert ge.tolist() == [[1, 0, 0, 0], [1, 1, 0, 0], [1, 1, 1, 0]]
+    assert sel[0, 0] == x[0, 0] and sel[0, 1] == x[0, 1] * 2
+    assert np.array_equal(tk, tab[[2, 0, 2]])
+    # docs/backend.md:96-102: trunc toward zero, saturate, NaN -> 0
+    assert ci[0].tolist() == [1, -1, 2147483647, -2147483648] and ci[1, 0] == 0
+    assert gf.tolist() == [[1, 0, 0, 0], [1, 1, 0, 0], [1, 1, 1, 0]]
+
+
+def test_take_out_of_range_raises():
+    p = prog(lambda fb, t, i: t.take(i), [("F32", [4, 2]), ("Si32", [1])])
+    with pytest.raises(po.OracleError) as ei:
+        oracle_run(p, [np.zeros((4, 2), np.float32), np.array([4], np.int32)])
+    assert ei.value.kind == "execution"
+
+
+# ---------------------------------------------------------------- dot_general
+@pytest.mark.parametrize("m,k,n", [(1, 1, 1), (1, 5, 3), (7, 13, 9), (33, 65, 31), (1, 768, 2304)])
+def test_dot_vs_float64(m, k, n):
+    a, b = U(1, (m, k)), U(2, (k, n))
+    out = oracle_run(prog(lambda fb, x, y: x.matmul(y), [("F32", [m, k]), ("F32", [k, n])]), [a, b])[0]
+    close(out, a.astype(np.float64) @ b.astype(np.float64))
+
+
+def test_dot_is_sequential_f32_accumulation():
+    # cpu.rs:2196-2225: sum += a*b in k order, in f32 -- bit-exact against a Python loop
+    a, b = U(3, (2, 37)), U(4, (37, 3))
+    out = oracle_run(prog(lambda fb, x, y: x.matmul(y), [("F32", [2, 37]), ("F32", [37, 3])]), [a, b])[0]
+    for i in range(2):
+        for j in range(3):
+            s = np.float32(0)
+            for p in range(37):
+                s = np.float32(s + np.float32(a[i, p] * b[p, j]))
+            assert out[i, j] == s
+
+
+def test_dot_general_batched_and_transposed_operand():
+    q, kk = U(5, (4, 3, 8)), U(6, (4, 5, 8))
+    out = oracle_run(prog(lambda fb, a, b: a.dot_general(b, [0], [2], [2]), [("F32", [4, 3, 8]), ("F32", [4, 5, 8])]), [q, kk])[0]
+    close(out, np.einsum("hmd,hnd->hmn", q.astype(np.float64), kk.astype(np.float64)))
+
+
+def _ref_lib():
+    flags = open("/proc/cpuinfo").read()
+    name = "libgptrs_c_ref_avx512.so" if " avx512f" in flags else "libgptrs_c_ref_avx2.so"
+    path = os.path.join(ROOT, "oracle", "_ref", name)
+    if not os.path.exists(path):
+        pytest.skip("oracle/_ref not built (reference checkout not mounted)")
+    lib = ctypes.CDLL(path)
+    fp = ctypes.POINTER(ctypes.c_float)
+    lib.gptrs_ref_matmul_f32.argtypes = [fp, fp, fp, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_size_t]
+    return lib, fp
+
+
+@pytest.mark.parametrize("m,k,n", [(2, 2, 2), (1, 768, 2304), (8, 768, 3072), (64, 3072, 768), (7, 13, 9)])
+def test_dot_vs_reference_c_kernels(m, k, n):
+    """The oracle's dot_general against gpt_rs_c_matmul_f32 compiled from the reference checkout."""
+    lib, fp = _ref_lib()
+    a, b = U(7, (m, k)), U(8, (k, n))
+    if (m, k, n) == (2, 2, 2):
+        a, b = np.array([[1, 2], [3, 4]], np.float32), np.array([[5, 6], [7, 8]], np.float32)
+    c = np.empty((m, n), np.float32)
+    lib.gptrs_ref_matmul_f32(a.ctypes.data_as(fp), b.ctypes.data_as(fp), c.ctypes.data_as(fp), m, n, k)
+    if (m, k, n) == (2, 2, 2):
+        assert c.reshape(-1).tolist() == [19.0, 22.0, 43.0, 50.0]
+    out = oracle_run(prog(lambda fb, x, y: x.matmul(y), [("F32", [m, k]), ("F32", [k, n])]), [a, b])[0]
+    close(out, c, atol=1e-4, rtol=1e-4)
+
+
+# ---------------------------------------------------------------- functionals vs torch CPU
+@pytest.mark.parametrize("shape", [(2, 3, 4), (2, 3, 13), (2, 4, 256), (1, 8), (4, 768)])
+def test_layer_norm_vs_torch(shape):
+    n = shape[-1]
+    x, g, b = U(9, shape), U(10, (n,)), U(11, (n,))
+    out, normalized, mean, inv_std = oracle_run(
+        prog(lambda fb, a, c, d: list(F.layer_norm(a, c, d, 1e-5)), [("F32", list(shape)), ("F32", [n]), ("F32", [n])]), [x, g, b])
+    tx = torch.from_numpy(x).double()
+    ref = torch.nn.functional.layer_norm(tx, (n,), torch.from_numpy(g).double(), torch.from_numpy(b).double(), 1e-5)
+    close(out, ref.numpy())
+    close(mean[..., 0], tx.mean(-1).numpy())
+    close(inv_std[..., 0], (1.0 / torch.sqrt(tx.var(-1, unbiased=False) + 1e-5)).numpy(), atol=1e-3, rtol=1e-3)
+    close(normalized, ((tx - tx.mean(-1, keepdim=True)) / torch.sqrt(tx.var(-1, unbiased=False, keepdim=True) + 1e-5)).numpy())
+
+
+def test_rms_norm_vs_closed_form():
+    x, g = U(12, (3, 64)), U(13, (64,))
+    out = oracle_run(prog(lambda fb, a, c: F.rms_norm(a, c, 1e-5)[0], [("F32", [3, 64]), ("F32", [64])]), [x, g])[0]
+    x64 = x.astype(np.float64)
+    close(out, x64 / np.sqrt((x64 ** 2).mean(-1, keepdims=True) + 1e-5) * g)
+
+
+@pytest.mark.parametrize("shape,lo,hi,tol", [((3, 2, 4), -1, 1, 5e-4), ((4, 128), -1, 1, 5e-4), ((1, 3, 257), -1, 1, 5e-4), ((4, 16), -80, 80, 5e-3)])
+def test_softmax_vs_torch(shape, lo, hi, tol):
+    x = U(14, shape, lo, hi)
+    out = oracle_run(prog(lambda fb, a: F.softmax_last_axis(a), [("F32", list(shape))]), [x])[0]
+    close(out, torch.softmax(torch.from_numpy(x).double(), -1).numpy(), atol=tol, rtol=tol)
+    assert np.allclose(out.sum(-1), 1.0, atol=1e-5)
+
+
+def test_gelu_silu_swiglu_vs_torch():
+    x = U(15, (256,), -10, 10)
+    out = oracle_run(prog(lambda fb, a: F.gelu(a), [("F32", [256])]), [x])[0]
+    close(out, torch.nn.functional.gelu(torch.from_numpy(x).double(), approximate="none").numpy())
+    x = U(16, (3, 17), -40, 40)
+    out = oracle_run(prog(lambda fb, a: F.silu(a), [("F32", [3, 17])]), [x])[0]
+    close(out, torch.nn.functional.silu(torch.from_numpy(x).double()).numpy())
+    g, u = U(17, (5, 19), -10, 10), U(18, (5, 19))
+    out = oracle_run(prog(lambda fb, a, b: F.swiglu(a, b), [("F32", [5, 19]), ("F32", [5, 19])]), [g, u])[0]
+    close(out, (torch.nn.functional.silu(torch.from_numpy(g).double()) * torch.from_numpy(u).double()).numpy())
+
+
+# ---------------------------------------------------------------- RoPE
+def test_rope_tables_closed_form():
+    cos, sin = F.rotary_cos_sin_cache_slice(5, 3, F.RopeConfig(8, 10000.0))
+    for p in range(3):
+        for i in range(4):
+            ang = (5 + p) * 10000.0 ** (-(2.0 * i) / 8.0)
+            assert abs(cos[p, i] - math.cos(ang)) < 1e-5 and abs(sin[p, i] - math.sin(ang)) < 1e-5
+    c0, s0 = F.rotary_cos_sin_cache_slice(0, 1, F.RopeConfig(8, 1e6))
+    assert np.all(c0 == 1.0) and np.all(s0 == 0.0)
+
+
+@pytest.mark.parametrize("hq,hkv,dh,rot", [(4, 4, 8, 8), (4, 2, 8, 4), (2, 1, 16, 6)])
+def test_rope_vs_rotate_half_formula(hq, hkv, dh, rot):
+    # torch_parity/rotary_ops.rs: x*cos + rotate_half(x)*sin on the first `rot` dims of each head
+    cfg = F.AttentionConfig(hq * dh, hq, hkv, dh)
+    seq, P = 5, cfg.total_projection_dim
+    cos, sin = F.rotary_cos_sin_cache_slice(2, seq, F.RopeConfig(rot, 10000.0))
+    qkv = U(19, (seq, P))
+    out = oracle_run(prog(lambda fb, a, c, s: F.apply_rope_qkv_packed(cfg, a, c, s),
+                          [("F32", [seq, P]), ("F32", [seq, rot // 2]), ("F32", [seq, rot // 2])]), [qkv, cos, sin])[0]
+    exp = qkv.astype(np.float64).copy()
+    half = rot // 2
+    for h in range(hq + hkv):
+        blk = qkv[:, h * dh:(h + 1) * dh].astype(np.float64)
+        a, b = blk[:, :half], blk[:, half:rot]
+        exp[:, h * dh:h * dh + half] = a * cos - b * sin
+        exp[:, h * dh + half:h * dh + rot] = b * cos + a * sin
+    close(out, exp)
+    # rotation preserves each pair's norm; position 0 is the identity; V untouched
+    n_in = np.hypot(qkv[:, :half], qkv[:, half:rot])
+    n_out = np.hypot(out[:, :half], out[:, half:rot])
+    assert np.allclose(n_in, n_out, atol=1e-5)
+    assert np.array_equal(out[:, (hq + hkv) * dh:], qkv[:, (hq + hkv) * dh:])
+
+
+# ---------------------------------------------------------------- attention vs the torch formula
+def torch_attention(qkv, cfg):
+    # torch_parity/attention.rs:13-58: /sqrt(Dh), tril mask with -inf, softmax, repeat_interleave for GQA
+    t = torch.from_numpy(qkv).double()
+    T = t.shape[0]
+    hq, hkv, dh = cfg.num_query_heads, cfg.num_key_value_heads, cfg.head_dim
+    q = t[:, :hq * dh].reshape(T, hq, dh).transpose(0, 1)
+    k = t[:, hq * dh:(hq + hkv) * dh].reshape(T, hkv, dh).transpose(0, 1)
+    v = t[:, (hq + hkv) * dh:].reshape(T, hkv, dh).transpose(0, 1)
+    kg, vg = k.repeat_interleave(hq // hkv, 0), v.repeat_interleave(hq // hkv, 0)
+    s = q @ kg.transpose(1, 2) / math.sqrt(dh)
+    s = s.masked_fill(~torch.tril(torch.ones(T, T, dtype=torch.bool)), float("-inf"))
+    ctx = torch.softmax(s, -1) @ vg
+    return ctx.transpose(0, 1).reshape(T, hq * dh).numpy(), k.numpy(), v.numpy()
+
+
+@pytest.mark.parametrize("hq,hkv,dh,seq", [(3, 3, 2, 4), (2, 2, 4, 1), (4, 4, 8, 8), (4, 4, 1, 3), (4, 1, 4, 5), (4, 2, 8, 6)])
+def test_attention_prefill_vs_torch(hq, hkv, dh, seq):
+    cfg = F.AttentionConfig(hq * dh, hq, hkv, dh)
+    qkv = U(20, (seq, cfg.total_projection_dim))
+    ctx, k, v = oracle_run(prog(lambda fb, a: list(F.attention(cfg, a, None)), [("F32", [seq, cfg.total_projection_dim])]), [qkv])
+    e_ctx, e_k, e_v = torch_attention(qkv, cfg)
+    close(ctx, e_ctx)
+    assert np.array_equal(k, e_k.astype(np.float32)) and np.array_equal(v, e_v.astype(np.float32))
+
+
+def test_decode_cache_equals_full_attention_and_ignores_stale_rows():
+    cfg = F.AttentionConfig(32, 4, 2, 8)
+    P, T, cap = cfg.total_projection_dim, 6, 16
+    qkv = U(21, (T, P))
+    e_ctx, e_k, e_v = torch_attention(qkv, cfg)
+    dec = prog(lambda fb, a, k, v, us, qs: list(F.attention_decode_cache(cfg, a, k, v, us, qs)),
+               [("F32", [1, P]), ("F32", [2, cap, 8]), ("F32", [2, cap, 8]), ("Si32", [3]), ("Si32", [1])])
+    ck = np.full((2, cap, 8), 123.0, np.float32)  # stale garbage everywhere
+    cv = np.full((2, cap, 8), -77.0, np.float32)
+    for pos in range(T):
+        ctx, ck, cv = oracle_run(dec, [qkv[pos:pos + 1], ck, cv, np.array([0, pos, 0], np.int32), np.array([pos], np.int32)])
+        close(ctx[0], e_ctx[pos])
+    assert np.array_equal(ck[:, :T], e_k.astype(np.float32))
+
+
+# ---------------------------------------------------------------- whole model invariants
+def test_tiny_gpt_kv_cache_greedy_equals_full_context_greedy():
+    # crates/gpt-rs-backend-tests/src/smoke.rs:43-82 (config at :45-53), 16 steps
+    from gptrs_amd import models
+    from oracle_backend import OracleBackend
+    cfg = models.GptConfig(vocab_size=64, context_length=32, embed_dim=32, num_layers=2, num_heads=4, mlp_ratio=2)
+    be = OracleBackend()
+    m = models.Gpt.random(cfg, be, seed=7, std=0.2)
+    prompt = [3, 17, 42, 5]
+    cached = models.Generator(m, prompt).generate(16)
+    cur, full = list(prompt), []
+    for _ in range(16):
+        caches = [None] * cfg.num_layers
+        t = int(np.argmax(be.to_numpy(m.forward_with_decode_cache(cur, 0, caches, None))[-1]))
+        full.append(t)
+        cur.append(t)
+    assert cached == full
+
+
+def test_tiny_gpt_logits_vs_independent_torch_model():
+    """GPT-2 forward written directly in torch (float64) from model/gpt.rs's wiring."""
+    from gptrs_amd import models
+    from oracle_backend import OracleBackend
+    cfg = models.GptConfig(vocab_size=64, context_length=32, embed_dim=32, num_layers=2, num_heads=4, mlp_ratio=2)
+    be = OracleBackend()
+    m = models.Gpt.random(cfg, be, seed=3, std=0.2)
+    toks = [5, 9, 1, 33, 60]
+    caches = [None] * cfg.num_layers
+    logits = be.to_numpy(m.forward_with_decode_cache(toks, 0, caches, None))
+    W = {n: torch.from_numpy(be.to_numpy(m.param_handle(n)).copy()).double() for n in m.param_names}
+    x = W["tok_embeddings.weight"][toks] + W["pos_embeddings"][:len(toks)]
+    T, d, H = len(toks), cfg.embed_dim, cfg.num_heads
+    for i in range(cfg.num_layers):
+        p = f"blocks.{i}."
+        h = torch.nn.functional.layer_norm(x, (d,), W[p + "ln_1.gamma"], W[p + "ln_1.beta"], cfg.eps)
+        qkv = h @ W[p + "attention.w_qkv"] + W[p + "attention.b_qkv"]
+        q, k, v = [t.reshape(T, H, d // H).transpose(0, 1) for t in qkv.split(d, dim=1)]
+        s = q @ k.transpose(1, 2) / math.sqrt(d // H)
+        s = s.masked_fill(~torch.tril(torch.ones(T, T, dtype=torch.bool)), float("-inf"))
+        ctx = (torch.softmax(s, -1) @ v).transpose(0, 1).reshape(T, d)
+        x = ctx @ W[p + "attention.w_out"] + W[p + "attention.b_out"] + x
+        h = torch.nn.functional.layer_norm(x, (d,), W[p + "ln_2.gamma"], W[p + "ln_2.beta"], cfg.eps)
+        ff = torch.nn.functional.gelu(h @ W[p + "feed_forward.w_in"] + W[p + "feed_forward.b_in"])
+        x = ff @ W[p + "feed_forward.w_out"] + W[p + "feed_forward.b_out"] + x
+    x = torch.nn.functional.layer_norm(x, (d,), W["final_ln.gamma"], W["final_ln.beta"], cfg.eps)
+    close(logits, (x @ W["lm_head"]).numpy(), atol=1e-4, rtol=1e-4)
+
+
+def test_tiny_ministral_logits_vs_independent_torch_model():
+    """Ministral forward (RMSNorm, rotate-half RoPE, GQA, SwiGLU) written directly in torch."""
+    from gptrs_amd import models
+    from oracle_backend import OracleBackend
+    cfg = models.MinistralConfig(vocab_size=64, context_length=32, embed_dim=16, num_layers=2, num_heads=4,
+                                 num_kv_heads=2, head_dim=4, ffn_dim=48, rotary_dim=4, rope_theta=10000.0)
+    be = OracleBackend()
+    m = models.Ministral.random(cfg, be, seed=3, dtype="F32", std=0.2)
+    toks = [5, 9, 1, 33, 60, 2]
+    caches = [None] * cfg.num_layers
+    logits = be.to_numpy(m.forward_with_decode_cache(toks, 0, caches, None))
+    W = {n: torch.from_numpy(be.to_numpy(m.param_handle(n)).copy()).double() for n in m.param_names}
+    T, hq, hkv, dh = len(toks), cfg.num_heads, cfg.num_kv_heads, cfg.head_dim
+    inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, cfg.rotary_dim, 2).double() / cfg.rotary_dim))
+    ang = torch.arange(T).double()[:, None] * inv[None, :]
+    cos, sin = torch.cos(ang), torch.sin(ang)
+
+    def rms(v, g):
+        return v / torch.sqrt((v * v).mean(-1, keepdim=True) + cfg.eps) * g
+
+    def rope(t, heads):
+        t = t.reshape(T, heads, dh)
+        a, b = t[..., :cfg.rotary_dim // 2], t[..., cfg.rotary_dim // 2:cfg.rotary_dim]
+        out = torch.cat([a * cos[:, None] - b * sin[:, None], b * cos[:, None] + a * sin[:, None], t[..., cfg.rotary_dim:]], -1)
+        return out.transpose(0, 1)
+
+    x = W["tok_embeddings.weight"][toks]
+    for i in range(cfg.num_layers):
+        p = f"blocks.{i}."
+        qkv = rms(x, W[p + "norm_1.gamma"]) @ W[p + "attention.w_qkv"]
+        q = rope(qkv[:, :hq * dh], hq)
+        k = rope(qkv[:, hq * dh:(hq + hkv) * dh], hkv).repeat_interleave(hq // hkv, 0)
+        v = qkv[:, (hq + hkv) * dh:].reshape(T, hkv, dh).transpose(0, 1).repeat_interleave(hq // hkv, 0)
+        s = q @ k.transpose(1, 2) / math.sqrt(dh)
+        s = s.masked_fill(~torch.tril(torch.ones(T, T, dtype=torch.bool)), float("-inf"))
+        ctx = (torch.softmax(s, -1) @ v).transpose(0, 1).reshape(T, hq * dh)
+        x = ctx @ W[p + "attention.w_out"] + x
+        h = rms(x, W[p + "norm_2.gamma"])
+        x = (torch.nn.functional.silu(h @ W[p + "feed_forward.w_gate"]) * (h @ W[p + "feed_forward.w_up"])) @ W[p + "feed_forward.w_down"] + x
+    close(logits, (rms(x, W["final_norm.gamma"]) @ W["lm_head"]).numpy(), atol=1e-4, rtol=1e-4)
+
+
+# ---------------------------------------------------------------- bf16 + quantization definitions
+def test_bf16_rounding_matches_torch():
+    x = np.concatenate([U(22, (4096,), -3, 3), np.array([0.0, -0.0, 1.0, 1.00390625, 1.01171875, 3.3895314e38, np.inf, -np.inf], np.float32)])
+    ours = po.round_bf16(x)
+    ref = torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()
+    assert np.array_equal(ours, ref)
+    from gptrs_amd.ptir import f32_to_bf16_bits, bf16_bits_to_f32
+    assert np.array_equal(bf16_bits_to_f32(f32_to_bf16_bits(x)), ref)
+    assert np.isnan(po.round_bf16(np.array([np.nan], np.float32))[0])
+
+
+def test_bf16_program_rounds_every_op_output():
+    x = U(23, (4, 8))
+    out = oracle_run(prog(lambda fb, a: (a * a + 1.0), [("Bf16", [4, 8])], dtype="Bf16"), [x])[0]
+    xb = po.round_bf16(x)
+    assert np.array_equal(out, po.round_bf16(po.round_bf16(xb * xb) + np.float32(1.0)))
+
+
+def test_int8_and_int4_pack_round_trip():
+    w = U(24, (256, 24), -0.05, 0.05)
+    q, s = po.quantize_int8_per_channel(w)
+    assert q.dtype == np.int8 and np.abs(q).max() == 127
+    assert np.max(np.abs(po.dequantize_int8(q, s) - w)) <= 0.51 * s.max() + 1e-7
+    pk, s4 = po.quantize_int4_g128(w)
+    assert pk.shape == (128, 24) and s4.shape == (2, 24)
+    deq = po.dequantize_int4_g128(pk, s4)
+    assert np.max(np.abs(deq - w)) <= 0.51 * s4.max() + 1e-7
+    # nibble order: low nibble is the even row
+    lo = int(pk[0, 0] & 0xF)
+    lo = lo - 16 if lo > 7 else lo
+    assert lo == int(np.clip(np.rint(w[0, 0] / s4[0, 0]), -7, 7))
