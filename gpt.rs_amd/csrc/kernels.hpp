@@ -93,7 +93,6 @@ struct LinearArgs {
 constexpr int kLinearCounters = 4096;
 size_t linear_workspace_bytes(int dtype, int64_t m, int64_t k, int64_t n, bool dual);
 void linear(hipStream_t s, const LinearArgs& a);
-
 // Rotate-half RoPE on packed [T, Q|K|V] rows (ops/functional/rotary.rs:430-536).
 void rope_packed(hipStream_t s, int dtype, const void* qkv, const void* cos, const void* sin, void* out,
                  int64_t t, int64_t n_q, int64_t n_kv, int64_t head_dim, int64_t half);

@@ -36,6 +36,8 @@ template <> struct Vec16<bf16_t> {
     }
 };
 
+constexpr int kMaxDecodeSplits = 512;
+
 __device__ __forceinline__ int64_t clamp_i64(int64_t v, int64_t lo, int64_t hi) { return v < lo ? lo : (v > hi ? hi : v); }
 
 // ------------------------------------------------------------------------------ decode
@@ -87,15 +89,27 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const T* __restrict__ 
         for (int v = 0; v < VEC; ++v) o[g][v] = 0.f;
     }
 
-    for (int64_t p = p0 + sid; p < p1; p += nstream) {
-        float kf[VEC], vf[VEC];
-        if (p == upd) {
-            Vec16<T>::load(knew + li * VEC, kf);
-            Vec16<T>::load(vnew + li * VEC, vf);
-        } else {
-            Vec16<T>::load(kc + ((int64_t)kvh * cap + p) * dh + li * VEC, kf);
-            Vec16<T>::load(vc + ((int64_t)kvh * cap + p) * dh + li * VEC, vf);
+    // Two positions per lane-group are loaded before either is consumed (the kernel is bound by
+    // load latency, not bandwidth); a position past the end re-reads a valid row and is skipped.
+    for (int64_t base = p0 + sid; base < p1; base += 2 * nstream) {
+        float kf2[2][VEC], vf2[2][VEC];
+        bool live[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int64_t p = base + (int64_t)j * nstream;
+            live[j] = p < p1;
+            const int64_t pc = live[j] ? p : base;
+            const bool fresh = pc == upd;
+            const T* kr = fresh ? knew : kc + ((int64_t)kvh * cap + pc) * dh;
+            const T* vr = fresh ? vnew : vc + ((int64_t)kvh * cap + pc) * dh;
+            Vec16<T>::load(kr + li * VEC, kf2[j]);
+            Vec16<T>::load(vr + li * VEC, vf2[j]);
         }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+        if (!live[j]) continue;
+        const float (&kf)[VEC] = kf2[j];
+        const float (&vf)[VEC] = vf2[j];
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             float s = 0.f;
@@ -110,6 +124,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const T* __restrict__ 
 #pragma unroll
             for (int v = 0; v < VEC; ++v) o[g][v] = o[g][v] * corr + pe * vf[v];
             m[g] = mn;
+        }
         }
     }
 
@@ -169,41 +184,60 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const T* __restrict__ 
 
 template <typename T>
 __global__ void attn_decode_combine_kernel(const float* __restrict__ ws, T* __restrict__ ctx, int dh, int nsplit) {
+    // per-split weights exp(m_s - max) are computed once into LDS; the slice loads of the output
+    // loop are then independent of each other
+    __shared__ float wgt[kMaxDecodeSplits];
+    __shared__ float red[16];
     const int h = blockIdx.x;
     const float* base = ws + (int64_t)h * nsplit * (dh + 2);
     float mn = -INFINITY;
-    for (int s = 0; s < nsplit; ++s) mn = fmaxf(mn, base[(int64_t)s * (dh + 2)]);
+    for (int s = threadIdx.x; s < nsplit; s += blockDim.x) {
+        const float ms = base[(int64_t)s * (dh + 2)];
+        wgt[s] = ms;
+        mn = fmaxf(mn, ms);
+    }
+    mn = block_max(mn, red);
+    float lsum = 0.f;
+    for (int s = threadIdx.x; s < nsplit; s += blockDim.x) {
+        const float ms = wgt[s];
+        const float c = ms == -INFINITY ? 0.f : expf(ms - mn);
+        wgt[s] = c;
+        lsum += base[(int64_t)s * (dh + 2) + 1] * c;
+    }
+    const float L = block_sum(lsum, red);  // also orders the wgt[] writes before the reads below
     for (int d = threadIdx.x; d < dh; d += blockDim.x) {
-        float L = 0.f, O = 0.f;
-        for (int s = 0; s < nsplit; ++s) {
-            const float* rec = base + (int64_t)s * (dh + 2);
-            if (rec[0] == -INFINITY) continue;
-            const float c = expf(rec[0] - mn);
-            L += rec[1] * c;
-            O += rec[2 + d] * c;
-        }
+        float O = 0.f;
+#pragma unroll 8
+        for (int s = 0; s < nsplit; ++s) O += base[(int64_t)s * (dh + 2) + 2 + d] * wgt[s];
         stf(ctx, (int64_t)h * dh + d, O / L);
     }
 }
 
-static int decode_splits(int64_t n_kv, int64_t cap) {
-    int64_t by_len = cdiv(cap, 64);
-    int64_t by_fill = 512 / (n_kv > 0 ? n_kv : 1);
-    if (by_fill < 1) by_fill = 1;
-    int64_t s = by_len < by_fill ? by_len : by_fill;
-    return (int)(s < 1 ? 1 : s);
+// Launch geometry shared by attn_decode() and attn_decode_workspace_bytes(): chunks of two
+// positions per lane-group, capped at kMaxDecodeSplits splits.
+static void decode_geometry(int dtype, int64_t dh, int64_t cap, int* nsplit, int64_t* chunk) {
+    const int64_t vec = dtype == 0 ? 4 : 8;
+    const int64_t lpr = dh / vec > 0 ? dh / vec : 1;
+    const int64_t nstream = 4 * (64 / lpr);
+    int64_t c = 2 * nstream;
+    if (cdiv(cap, c) > kMaxDecodeSplits) c = cdiv(cdiv(cap, kMaxDecodeSplits), 2 * nstream) * 2 * nstream;
+    *chunk = c;
+    *nsplit = (int)cdiv(cap, c);
 }
 size_t attn_decode_workspace_bytes(int64_t n_q, int64_t head_dim, int64_t capacity) {
-    // n_kv >= 1, so 512 splits bounds every launch geometry
-    int64_t s = cdiv(capacity, 64);
-    if (s > 512) s = 512;
-    return (size_t)n_q * (size_t)s * (size_t)(head_dim + 2) * sizeof(float);
+    int ns0, ns2;
+    int64_t c;
+    decode_geometry(0, head_dim, capacity, &ns0, &c);
+    decode_geometry(2, head_dim, capacity, &ns2, &c);
+    const int ns = ns0 > ns2 ? ns0 : ns2;
+    return (size_t)n_q * (size_t)ns * (size_t)(head_dim + 2) * sizeof(float);
 }
 
 template <typename T>
 static void attn_decode_t(hipStream_t s, const AttnDecodeArgs& a) {
-    const int nsplit = decode_splits(a.n_kv, a.capacity);
-    const int64_t chunk = cdiv(a.capacity, nsplit);
+    int nsplit;
+    int64_t chunk;
+    decode_geometry(a.dtype, a.head_dim, a.capacity, &nsplit, &chunk);
     dim3 grid((unsigned)a.n_kv, (unsigned)nsplit);
     const int g = (int)(a.n_q / a.n_kv);
 #define GPTRS_LAUNCH(G)                                                                                          \

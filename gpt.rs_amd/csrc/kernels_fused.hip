@@ -70,7 +70,7 @@ __global__ void layer_norm_long_kernel(const T* __restrict__ x, const T* __restr
 template <typename T>
 static void layer_norm_t(hipStream_t s, const T* x, const T* g, const T* b, T* y, int64_t rows, int64_t n, float inv_n,
                          float eps) {
-    const int block = n <= 256 ? 64 : 256;
+    const int block = n <= 256 ? 64 : (n <= 1024 ? 256 : 1024);  // decode has ONE row: spread it over many lanes
     const int64_t per = cdiv(n, block);
     const unsigned grid = (unsigned)rows;
     if (per <= 4) layer_norm_kernel<T, 4><<<grid, block, 0, s>>>(x, g, b, y, n, inv_n, eps);
@@ -120,7 +120,7 @@ __global__ void rms_norm_long_kernel(const T* __restrict__ x, const T* __restric
 }
 template <typename T>
 static void rms_norm_t(hipStream_t s, const T* x, const T* g, T* y, int64_t rows, int64_t n, float inv_n, float eps) {
-    const int block = n <= 256 ? 64 : 256;
+    const int block = n <= 256 ? 64 : (n <= 1024 ? 256 : 1024);  // decode has ONE row: spread it over many lanes
     const int64_t per = cdiv(n, block);
     if (per <= 4) rms_norm_kernel<T, 4><<<(unsigned)rows, block, 0, s>>>(x, g, y, n, inv_n, eps);
     else if (per <= 16) rms_norm_kernel<T, 16><<<(unsigned)rows, block, 0, s>>>(x, g, y, n, inv_n, eps);

@@ -806,7 +806,7 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
             const Spec& x = in_spec(0);
             const Spec& w = in_spec(1);
             k::LinearArgs a{};
-            a.dtype = (int)out.dtype;
+            a.dtype = (int)x.dtype;
             a.x = src_ptr(st, cx, 0);
             a.w = src_ptr(st, cx, 1);
             size_t i = 2;
@@ -831,7 +831,7 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
                 cx.be->prof_events.emplace_back(e0, e1);
                 ++cx.be->prof_linear_calls;
                 // algorithmic bytes: activations in, every weight once, result out
-                cx.be->prof_linear_bytes += (int64_t)dtype_size(out.dtype) * (a.m * a.k + a.k * a.n * (a.w2 ? 2 : 1) + a.m * a.n);
+                cx.be->prof_linear_bytes += (int64_t)dtype_size(x.dtype) * (a.m * a.k + a.k * a.n * (a.w2 ? 2 : 1) + a.m * a.n);
             }
             cx.launches += (in.act == 2 && a.m > 16) ? 3 : 1;
             break;
