@@ -75,6 +75,7 @@ Backend::~Backend() {
     params_.clear();
     plan_index_.clear();
     plan_lru_.clear();
+    tiled_cache_.clear();
     pool_.trim();
     (void)hipFree(d_err_flag_);
     (void)hipFree(d_counters_);
@@ -107,7 +108,25 @@ BufferP Backend::new_buffer(size_t bytes) {
     auto b = std::make_shared<Buffer>();
     b->ptr = pool_.alloc(bytes, &b->cap);
     b->owner = this;
+    b->id = next_buffer_id_++;
     return b;
+}
+
+BufferP Backend::tiled_weights(const BufferP& src, DType dtype, int64_t k, int64_t n) {
+    auto it = tiled_cache_.find(src->id);
+    if (it != tiled_cache_.end()) {
+        if (it->second.src.lock() == src) return it->second.tiled;
+        tiled_cache_.erase(it);
+    }
+    if (tiled_cache_.size() >= 64 && (tiled_cache_.size() & 63) == 0) {  // drop entries whose source died
+        for (auto e = tiled_cache_.begin(); e != tiled_cache_.end();)
+            e = e->second.src.expired() ? tiled_cache_.erase(e) : std::next(e);
+    }
+    BufferP t = new_buffer(k::tiled_weight_bytes((int)dtype, k, n));
+    k::tile_weights(stream, (int)dtype, src->ptr, t->ptr, k, n);
+    tiled_cache_[src->id] = Derived{src, t};
+    ++n_tiled_built;
+    return t;
 }
 
 gptrs_hip_tensor* Backend::materialize(const Spec& spec, const void* host, size_t nbytes) {
@@ -289,6 +308,8 @@ void Backend::execute(Plan& plan, gptrs_hip_tensor* const* inputs, const uint8_t
     cx.err_flag = d_err_flag_;
     cx.counters = d_counters_;
     cx.profile = opt_profile;
+    cx.input_bufs.resize(n_in);
+    for (size_t i = 0; i < n_in; ++i) cx.input_bufs[i] = inputs[i]->buf;
     cx.ptr.assign(plan.values.size(), nullptr);
     for (size_t v = 0; v < plan.values.size(); ++v) {
         if (!plan.values[v].defined) continue;
@@ -319,7 +340,10 @@ void Backend::execute(Plan& plan, gptrs_hip_tensor* const* inputs, const uint8_t
         outputs[i] = t;
     }
     for (size_t ip = 0; ip < n_in; ++ip)
-        if (inplace_ok[ip]) inputs[ip]->consumed = true;
+        if (inplace_ok[ip]) {
+            inputs[ip]->consumed = true;
+            inputs[ip]->buf->id = next_buffer_id_++;  // contents changed: derived copies are stale
+        }
 }
 
 void Backend::run_program(const char* json, size_t len, uint64_t key, gptrs_hip_tensor* const* inputs,
@@ -573,6 +597,7 @@ int64_t gptrs_hip_counter(const gptrs_hip_backend* b, const char* name) {
     if (!strcmp(name, "fused_ops")) return i.n_fused;
     if (!strcmp(name, "bytes_allocated")) return i.bytes_allocated();
     if (!strcmp(name, "inplace_updates")) return i.n_inplace;
+    if (!strcmp(name, "derived_weights_built")) return i.n_tiled_built;
     if (!strcmp(name, "last_program_launches")) return i.last_launches;
     return -1;
 }

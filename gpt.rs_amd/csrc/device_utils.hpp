@@ -23,10 +23,24 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
     return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
 }
 
+// Sum over the 64 lanes of a wave, result in every lane.  Cross-lane moves use DPP modifiers
+// (register-to-register, VALU rate) instead of ds_bpermute: 16 x 6 bpermutes per thread at the end of
+// a GEMV block kept the LDS pipe busy for ~4 us.  Steps: xor 1 and xor 2 inside quads, mirrored
+// halves of 8 and 16 lanes, then lane 15 / lane 31 of the previous rows broadcast into rows 1,3 /
+// 2,3; lane 63 then holds the total and is read back as a scalar.
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
+    int x = __float_as_int(v);
+#define GPTRS_DPP_ADD(ctrl, row_mask)                                                                         \
+    x = __float_as_int(__int_as_float(x) +                                                                     \
+                       __int_as_float(__builtin_amdgcn_update_dpp(0, x, (ctrl), (row_mask), 0xf, false)))
+    GPTRS_DPP_ADD(0xB1, 0xf);   // quad_perm [1,0,3,2]
+    GPTRS_DPP_ADD(0x4E, 0xf);   // quad_perm [2,3,0,1]
+    GPTRS_DPP_ADD(0x141, 0xf);  // row_half_mirror
+    GPTRS_DPP_ADD(0x140, 0xf);  // row_mirror
+    GPTRS_DPP_ADD(0x142, 0xa);  // row_bcast:15 into rows 1 and 3
+    GPTRS_DPP_ADD(0x143, 0xc);  // row_bcast:31 into rows 2 and 3
+#undef GPTRS_DPP_ADD
+    return __int_as_float(__builtin_amdgcn_readlane(x, 63));
 }
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll

@@ -680,6 +680,54 @@ struct Fuser {
         }
     }
 
+    // Decode-sized linears whose weights are program inputs run over the column-tiled weight copy;
+    // an RMSNorm feeding only such linears is folded into them (every block reads the whole row of x
+    // anyway, so the row statistic is free).
+    void pass_tiled_linear() {
+        auto is_param = [&](int v) { return v >= 0 && def[v] < 0 && spec_of(v) != nullptr; };
+        for (auto& in : fn.body) {
+            if (in.dead || in.op != OpKind::FLinear) continue;
+            const Spec* xs = spec_of(in.operands[0].value);
+            const Spec* ws = spec_of(in.operands[1].value);
+            if (!xs || !ws) continue;
+            const int64_t M = xs->dims[0];
+            if (!k::gemv_tiled_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1])) continue;
+            if (!is_param(in.operands[1].value)) continue;
+            if (in.act == 2 && (!is_param(in.operands[2].value) || M > 8)) continue;
+            in.tiled = true;
+        }
+        const std::vector<int> uses = count_uses();
+        std::vector<bool> is_result(fn.max_value_id + 1, false);
+        for (int r : fn.result_ids) is_result[r] = true;
+        for (size_t i = 0; i < fn.body.size(); ++i) {
+            Instr& nrm = fn.body[i];
+            if (nrm.dead || nrm.op != OpKind::FRmsNorm) continue;
+            const int nv = nrm.out_ids[0];
+            if (is_result[nv] || nrm.out_specs[0].rank() != 2) continue;
+            std::vector<Instr*> cons;
+            int found = 0;
+            for (auto& c : fn.body) {
+                if (c.dead) continue;
+                for (size_t o = 0; o < c.operands.size(); ++o) {
+                    if (c.operands[o].value != nv) continue;
+                    ++found;
+                    if (c.op == OpKind::FLinear && c.tiled && !c.norm && o == 0) cons.push_back(&c);
+                }
+            }
+            if (cons.empty() || (int)cons.size() != found || found != uses[nv]) continue;
+            for (Instr* c : cons) {
+                c->operands[0] = nrm.operands[0];
+                c->operands.push_back(nrm.operands[1]);
+                c->norm = true;
+                c->eps = nrm.eps;
+                c->scale = nrm.scale;
+            }
+            nrm.dead = true;
+            ++fused;
+        }
+        reindex();
+    }
+
     // Binary ops whose rhs is a broadcast scalar literal read the scalar as a kernel argument.
     void pass_scalar_rhs() {
         for (auto& in : fn.body) {
@@ -753,6 +801,8 @@ int fuse_function(Function& fn) {
     f.pass_attention();
     f.dce();
     f.pass_linear();
+    f.dce();
+    f.pass_tiled_linear();
     f.dce();
     f.pass_scalar_rhs();
     f.dce();

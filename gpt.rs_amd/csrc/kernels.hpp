@@ -93,6 +93,22 @@ struct LinearArgs {
 constexpr int kLinearCounters = 4096;
 size_t linear_workspace_bytes(int dtype, int64_t m, int64_t k, int64_t n, bool dual);
 void linear(hipStream_t s, const LinearArgs& a);
+// Decode GEMV (M <= 16) over a column-tiled copy of the weights, Wt[tile][k][v] with
+// v = column % (16 bytes / element size): no split-K, one launch per linear layer.  gamma != nullptr
+// fuses a preceding RMSNorm (x is then the un-normalised row; inv_n, eps as in rms_norm()).
+struct TiledLinearArgs {
+    int dtype;
+    const void* x; const void* wt; const void* wt2; const void* gamma; const void* bias; const void* residual;
+    void* y;
+    int64_t m, k, n;
+    int act;
+    float inv_n, eps;
+};
+size_t tiled_weight_bytes(int dtype, int64_t k, int64_t n);
+void tile_weights(hipStream_t s, int dtype, const void* w, void* wt, int64_t k, int64_t n);
+bool gemv_tiled_supported(int dtype, int64_t m, int64_t k, int64_t n);
+void gemv_tiled(hipStream_t s, const TiledLinearArgs& a);
+
 // Rotate-half RoPE on packed [T, Q|K|V] rows (ops/functional/rotary.rs:430-536).
 void rope_packed(hipStream_t s, int dtype, const void* qkv, const void* cos, const void* sin, void* out,
                  int64_t t, int64_t n_q, int64_t n_kv, int64_t head_dim, int64_t half);

@@ -99,6 +99,7 @@ struct Builder {
     std::vector<int> last_use;       // per root value: last step index that reads it
     std::vector<int> def_step;       // per root value
     std::vector<size_t> lit_offset;  // literal index -> const offset
+    std::vector<int> param_pos;      // value id -> input position, -1 when not a function parameter
 
     Builder(Plan& p, const std::vector<bool>& d) : plan(p), donated(d) {}
 
@@ -486,7 +487,18 @@ void Builder::describe(Step& st) {
         case OpKind::FLinear: {
             const Spec& x = spec_of(in, 0);
             const Spec& w = spec_of(in, 1);
-            st.scratch_bytes = k::linear_workspace_bytes((int)x.dtype, x.dims[0], x.dims[1], w.dims[1], in.act == 2);
+            if (in.tiled) {
+                auto pos = [&](size_t op) {
+                    const int v = in.operands[op].value;
+                    const int p = v >= 0 && v < (int)param_pos.size() ? param_pos[v] : -1;
+                    if (p < 0) fail_exec("tiled linear: weight operand is not a program input");
+                    return p;
+                };
+                st.tiled_w_input = pos(1);
+                if (in.act == 2) st.tiled_w2_input = pos(2);
+            } else {
+                st.scratch_bytes = k::linear_workspace_bytes((int)x.dtype, x.dims[0], x.dims[1], w.dims[1], in.act == 2);
+            }
             break;
         }
         case OpKind::FAttnDecode: {
@@ -504,6 +516,8 @@ void Builder::build() {
     plan.values.assign(fn.max_value_id + 1, ValueInfo{});
     if (fn.param_ids.size() != donated.size()) fail_exec("entry input arity mismatch");
     for (size_t i = 0; i < fn.param_ids.size(); ++i) define(fn.param_ids[i], fn.param_specs[i]);
+    param_pos.assign(plan.values.size(), -1);
+    for (size_t i = 0; i < fn.param_ids.size(); ++i) param_pos[fn.param_ids[i]] = (int)i;
 
     // literals -> const block
     lit_offset.resize(fn.literals.size());
@@ -805,6 +819,41 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
         case OpKind::FLinear: {
             const Spec& x = in_spec(0);
             const Spec& w = in_spec(1);
+            if (in.tiled) {
+                k::TiledLinearArgs ta{};
+                ta.dtype = (int)x.dtype;
+                ta.x = src_ptr(st, cx, 0);
+                ta.m = x.dims[0]; ta.k = x.dims[1]; ta.n = w.dims[1];
+                BufferP wt = cx.be->tiled_weights(cx.input_bufs[st.tiled_w_input], x.dtype, ta.k, ta.n);
+                BufferP wt2;
+                ta.wt = wt->ptr;
+                size_t oi = 2;
+                if (in.act == 2) {
+                    wt2 = cx.be->tiled_weights(cx.input_bufs[st.tiled_w2_input], x.dtype, ta.k, ta.n);
+                    ta.wt2 = wt2->ptr;
+                    ++oi;
+                }
+                if (in.has_bias) ta.bias = src_ptr(st, cx, oi++);
+                if (in.has_residual) ta.residual = src_ptr(st, cx, oi++);
+                if (in.norm) { ta.gamma = src_ptr(st, cx, oi++); ta.inv_n = in.scale; ta.eps = in.eps; }
+                ta.y = dst;
+                ta.act = in.act == 1 ? 1 : 0;
+                hipEvent_t e0 = nullptr, e1 = nullptr;
+                if (cx.profile) {
+                    GPTRS_HIP_CHECK(hipEventCreate(&e0));
+                    GPTRS_HIP_CHECK(hipEventCreate(&e1));
+                    GPTRS_HIP_CHECK(hipEventRecord(e0, s));
+                }
+                k::gemv_tiled(s, ta);
+                if (cx.profile) {
+                    GPTRS_HIP_CHECK(hipEventRecord(e1, s));
+                    cx.be->prof_events.emplace_back(e0, e1);
+                    ++cx.be->prof_linear_calls;
+                    cx.be->prof_linear_bytes += (int64_t)dtype_size(x.dtype) * (ta.m * ta.k + ta.k * ta.n * (ta.wt2 ? 2 : 1) + ta.m * ta.n);
+                }
+                ++cx.launches;
+                break;
+            }
             k::LinearArgs a{};
             a.dtype = (int)x.dtype;
             a.x = src_ptr(st, cx, 0);

@@ -47,6 +47,7 @@ struct Buffer {
     void* ptr = nullptr;
     size_t cap = 0;
     Backend* owner = nullptr;
+    uint64_t id = 0;  // identity of the CONTENTS: fresh per allocation, bumped when updated in place
     ~Buffer();
 };
 using BufferP = std::shared_ptr<Buffer>;
@@ -95,6 +96,7 @@ struct Step {
     size_t scratch_off = 0, scratch_bytes = 0;  // per-step scratch inside the workspace
     bool copy_base = false;        // DynamicUpdateSlice / FAttnDecode: copy base -> out first
     bool lhs_pack = false, rhs_pack = false;    // Dot: operands repacked into scratch first
+    int tiled_w_input = -1, tiled_w2_input = -1;  // FLinear over column-tiled weights: input positions of W, W2
     k::CopyDesc pack_l{}, pack_r{};
     size_t pack_l_off = 0, pack_r_off = 0;
 };
@@ -140,6 +142,10 @@ class Backend {
     void check_device_errors();
 
     BufferP new_buffer(size_t bytes);
+    // Column-tiled copy of a weight tensor (kernels_gemv_tiled.hip), built on first use and kept while
+    // the source buffer lives: the backend-side memo of derived weight formats.
+    BufferP tiled_weights(const BufferP& src, DType dtype, int64_t k, int64_t n);
+    int64_t n_tiled_built = 0;
     void release_block(void* p, size_t cap) { pool_.release(p, cap); }
 
     std::mutex mu;
@@ -172,6 +178,9 @@ class Backend {
     int32_t* d_argmax_idx_ = nullptr;
     int64_t* d_token_ = nullptr;
     void* h_pinned_ = nullptr;  // 64 bytes of pinned host memory for readbacks
+    struct Derived { std::weak_ptr<Buffer> src; BufferP tiled; };
+    std::unordered_map<uint64_t, Derived> tiled_cache_;
+    uint64_t next_buffer_id_ = 1;
 };
 
 // fuse.cpp: canonicalise + pattern-fuse the entry function in place.  Returns the number of fused ops.
@@ -189,6 +198,7 @@ struct ExecCtx {
     int* counters;
     int64_t launches = 0;
     bool profile = false;
+    std::vector<BufferP> input_bufs;  // per input position
 };
 void run_step(const Plan& plan, const Step& st, ExecCtx& cx);
 
