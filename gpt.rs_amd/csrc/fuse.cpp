@@ -565,6 +565,29 @@ struct Fuser {
         }
     }
 
+    // Decode attention reads Q and the new K row straight from the projection; a packed-QKV RoPE
+    // that feeds only that attention is applied on load (and to the appended cache row) instead
+    // of in a kernel of its own.
+    void pass_rope_into_attention() {
+        const std::vector<int> uses = count_uses();
+        for (auto& at : fn.body) {
+            if (at.dead || at.op != OpKind::FAttnDecode || at.rot_half > 0) continue;
+            const int qv = at.operands[0].value;
+            if (qv < 0 || def[qv] < 0 || uses[qv] != 1) continue;
+            Instr& rp = fn.body[def[qv]];
+            if (rp.op != OpKind::FRope || rp.dead) continue;
+            const int64_t vec = 16 / (int64_t)dtype_size(at.out_specs[0].dtype);
+            if (rp.rot_half % vec || rp.head_dim != at.head_dim || rp.n_q != at.n_q || rp.n_kv != at.n_kv) continue;
+            at.operands[0] = rp.operands[0];
+            at.operands.push_back(rp.operands[1]);
+            at.operands.push_back(rp.operands[2]);
+            at.rot_half = rp.rot_half;
+            rp.dead = true;
+            ++fused;
+        }
+        reindex();
+    }
+
     // ---------------------------------------------------------------- linear layers
     std::vector<int> count_uses() const {
         std::vector<int> uses(fn.max_value_id + 1, 0);
@@ -799,6 +822,8 @@ int fuse_function(Function& fn) {
     f.dce();
     f.pass_rope();
     f.pass_attention();
+    f.dce();
+    f.pass_rope_into_attention();
     f.dce();
     f.pass_linear();
     f.dce();

@@ -127,6 +127,9 @@ struct AttnDecodeArgs {
     int64_t n_q, n_kv, head_dim, capacity;
     float scale;
     void* ws; size_t ws_bytes;
+    // optional fused RoPE of Q and of the appended K row (qkv is then the pre-RoPE projection):
+    // cos/sin rows [rot_half] of this position; requires rot_half % (16 / element size) == 0
+    const void* cos; const void* sin; int64_t rot_half;
 };
 size_t attn_decode_workspace_bytes(int64_t n_q, int64_t head_dim, int64_t capacity);
 void attn_decode(hipStream_t s, const AttnDecodeArgs& a);

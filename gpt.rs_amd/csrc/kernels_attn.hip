@@ -40,6 +40,49 @@ constexpr int kMaxDecodeSplits = 512;
 
 __device__ __forceinline__ int64_t clamp_i64(int64_t v, int64_t lo, int64_t hi) { return v < lo ? lo : (v > hi ? hi : v); }
 
+// Rotate-half RoPE (ops/functional/rotary.rs:430-536) applied while loading VEC consecutive dims
+// [c0, c0+VEC) of one head: dims below `half` pair with dim+half, the next `half` dims pair with
+// dim-half, dims >= 2*half pass through.  Needs half % VEC == 0 so a chunk never straddles a
+// boundary.  The result is rounded to T, the value a stored post-RoPE row would hold.
+template <typename T>
+__device__ __forceinline__ void load_roped(const T* __restrict__ head, int c0, int half, const T* __restrict__ cs,
+                                           const T* __restrict__ sn, float (&out)[Vec16<T>::N]) {
+    constexpr int VEC = Vec16<T>::N;
+    float own[VEC];
+    Vec16<T>::load(head + c0, own);
+    if (c0 >= 2 * half) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) out[v] = own[v];
+        return;
+    }
+    const bool first = c0 < half;
+    float other[VEC], c[VEC], s[VEC];
+    Vec16<T>::load(head + (first ? c0 + half : c0 - half), other);
+    const int j0 = first ? c0 : c0 - half;
+    Vec16<T>::load(cs + j0, c);
+    Vec16<T>::load(sn + j0, s);
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+        // first half: a*cos - b*sin with (a,b) = (own, other); second half: b*cos + a*sin with (b,a) = (own, other)
+        const float r = first ? own[v] * c[v] - other[v] * s[v] : own[v] * c[v] + other[v] * s[v];
+        T tmp;
+        stf(&tmp, 0, r);
+        out[v] = ldf(&tmp, 0);
+    }
+}
+template <typename T>
+__device__ __forceinline__ T roped_elem(const T* __restrict__ head, int d, int half, const T* __restrict__ cs,
+                                        const T* __restrict__ sn) {
+    if (d >= 2 * half) return head[d];
+    const bool first = d < half;
+    const int j = first ? d : d - half;
+    const float own = ldf(head, d), other = ldf(head, first ? d + half : d - half);
+    const float r = first ? own * ldf(cs, j) - other * ldf(sn, j) : own * ldf(cs, j) + other * ldf(sn, j);
+    T tmp;
+    stf(&tmp, 0, r);
+    return tmp;
+}
+
 // ------------------------------------------------------------------------------ decode
 // grid (n_kv, nsplit), 256 threads.  A cache row (head_dim elements) is read by LPR lanes with one
 // 16-byte load each, so a wave streams 64/LPR positions at a time; every such lane-group keeps
@@ -51,7 +94,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const T* __restrict__ 
                                                           T* __restrict__ vc, const int32_t* __restrict__ us,
                                                           const int32_t* __restrict__ qs, T* __restrict__ ctx,
                                                           float* __restrict__ ws, int n_q, int n_kv, int dh,
-                                                          int64_t cap, float scale, int64_t chunk, int nsplit) {
+                                                          int64_t cap, float scale, int64_t chunk, int nsplit,
+                                                          const T* __restrict__ cs, const T* __restrict__ sn, int half) {
     constexpr int VEC = Vec16<T>::N;
     const int lpr = dh / VEC;          // lanes per cache row (power of two, <= 64)
     const int rpw = 64 / lpr;          // rows per wave-iteration
@@ -68,7 +112,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const T* __restrict__ 
     // append this step's row (exactly one block per kv head owns position `upd`)
     if (upd / chunk == split) {
         for (int d = threadIdx.x; d < dh; d += 256) {
-            kc[((int64_t)kvh * cap + upd) * dh + d] = knew[d];
+            kc[((int64_t)kvh * cap + upd) * dh + d] = cs ? roped_elem<T>(knew, d, half, cs, sn) : knew[d];
             vc[((int64_t)kvh * cap + upd) * dh + d] = vnew[d];
         }
     }
@@ -79,7 +123,11 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const T* __restrict__ 
 
     float qf[G][VEC];
 #pragma unroll
-    for (int g = 0; g < G; ++g) Vec16<T>::load(qkv + (int64_t)(kvh * G + g) * dh + li * VEC, qf[g]);
+    for (int g = 0; g < G; ++g) {
+        const T* qh = qkv + (int64_t)(kvh * G + g) * dh;
+        if (cs) load_roped<T>(qh, li * VEC, half, cs, sn, qf[g]);
+        else Vec16<T>::load(qh + li * VEC, qf[g]);
+    }
 
     float m[G], l[G], o[G][VEC];
 #pragma unroll
@@ -102,7 +150,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const T* __restrict__ 
             const bool fresh = pc == upd;
             const T* kr = fresh ? knew : kc + ((int64_t)kvh * cap + pc) * dh;
             const T* vr = fresh ? vnew : vc + ((int64_t)kvh * cap + pc) * dh;
-            Vec16<T>::load(kr + li * VEC, kf2[j]);
+            if (cs && fresh) load_roped<T>(knew, li * VEC, half, cs, sn, kf2[j]);
+            else Vec16<T>::load(kr + li * VEC, kf2[j]);
             Vec16<T>::load(vr + li * VEC, vf2[j]);
         }
 #pragma unroll
@@ -242,7 +291,8 @@ static void attn_decode_t(hipStream_t s, const AttnDecodeArgs& a) {
     const int g = (int)(a.n_q / a.n_kv);
 #define GPTRS_LAUNCH(G)                                                                                          \
     attn_decode_kernel<T, G><<<grid, 256, 0, s>>>((const T*)a.qkv, (T*)a.k_cache, (T*)a.v_cache, a.update_starts,    \
-        a.query_start, (T*)a.ctx, (float*)a.ws, (int)a.n_q, (int)a.n_kv, (int)a.head_dim, a.capacity, a.scale, chunk, nsplit)
+        a.query_start, (T*)a.ctx, (float*)a.ws, (int)a.n_q, (int)a.n_kv, (int)a.head_dim, a.capacity, a.scale, chunk, nsplit, \
+        (const T*)a.cos, (const T*)a.sin, (int)a.rot_half)
     switch (g) {
         case 1: GPTRS_LAUNCH(1); break;
         case 2: GPTRS_LAUNCH(2); break;
