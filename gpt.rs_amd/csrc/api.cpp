@@ -1,4 +1,5 @@
 // Backend implementation and the extern "C" surface declared in include/gptrs_hip.h.
+#include <algorithm>
 #include <cstring>
 
 #include "../../include/gptrs_hip.h"
@@ -118,6 +119,7 @@ BufferP Backend::tiled_weights(const BufferP& src, DType dtype, int64_t k, int64
         if (it->second.src.lock() == src) return it->second.tiled;
         tiled_cache_.erase(it);
     }
+    if (capturing) fail_exec("derived weight copy missing while recording a graph");
     if (tiled_cache_.size() >= 64 && (tiled_cache_.size() & 63) == 0) {  // drop entries whose source died
         for (auto e = tiled_cache_.begin(); e != tiled_cache_.end();)
             e = e->second.src.expired() ? tiled_cache_.erase(e) : std::next(e);
@@ -251,6 +253,7 @@ std::shared_ptr<Plan> Backend::get_plan(const char* json, size_t len, uint64_t k
     }
     if (opt_fusion) plan->fused_ops = fuse_function(plan->fn);
     build_plan(*plan, don);
+    plan->cacheable = key != 0;
     if (plan->workspace_bytes) plan->workspace = new_buffer(plan->workspace_bytes);
     if (!plan->const_host.empty()) {
         plan->consts = new_buffer(plan->const_host.size());
@@ -268,6 +271,91 @@ std::shared_ptr<Plan> Backend::get_plan(const char* json, size_t len, uint64_t k
         }
     }
     return plan;
+}
+
+Plan::~Plan() {
+    for (auto& g : graphs) {
+        if (g.exec) (void)hipGraphExecDestroy(g.exec);
+        if (g.graph) (void)hipGraphDestroy(g.graph);
+    }
+}
+
+// Steady-state decode runs the same plan over the same addresses every step (weights and KV caches
+// stay put, the pool hands the small per-step buffers back in the same order).  Such a step is
+// recorded once by stream capture and replayed with one hipGraphLaunch.  An address set is recorded
+// the second time it is seen, after an eager run has built every derived weight copy, so nothing is
+// allocated while recording.  Returns false when the caller must run the steps eagerly.
+bool Backend::run_graphed(Plan& plan, ExecCtx& cx, const std::vector<BufferP>& out_bufs) {
+    constexpr size_t kMaxGraphs = 8, kSeenRing = 32;
+    if (!opt_graphs || opt_profile || !plan.cacheable || plan.steps.size() < 4) return false;
+    if (plan.graph_builds >= 16 && plan.graph_hits < 4 * plan.graph_builds) return false;  // addresses never settle
+    std::vector<uint64_t> key;
+    key.reserve(cx.input_bufs.size() + out_bufs.size() + 8);
+    for (const auto& b : cx.input_bufs) key.push_back((uint64_t)(uintptr_t)b->ptr);
+    for (const auto& b : out_bufs) key.push_back((uint64_t)(uintptr_t)b->ptr);
+    for (const Step& st : plan.steps) {
+        if (st.tiled_w_input >= 0) key.push_back(cx.input_bufs[st.tiled_w_input]->id);
+        if (st.tiled_w2_input >= 0) key.push_back(cx.input_bufs[st.tiled_w2_input]->id);
+    }
+    for (auto& g : plan.graphs)
+        if (g.key == key) {
+            GPTRS_HIP_CHECK(hipGraphLaunch(g.exec, stream));
+            g.last_use = ++plan.graph_clock;
+            ++plan.graph_hits;
+            ++n_graph_launches;
+            cx.launches = g.launches;
+            return true;
+        }
+    uint64_t h = 1469598103934665603ull;
+    for (uint64_t v : key) h = (h ^ v) * 1099511628211ull;
+    if (std::find(plan.seen_keys.begin(), plan.seen_keys.end(), h) == plan.seen_keys.end()) {
+        if (plan.seen_keys.size() < kSeenRing) plan.seen_keys.push_back(h);
+        else plan.seen_keys[plan.runs % kSeenRing] = h;
+        return false;
+    }
+    // record
+    PlanGraph pg;
+    pg.key = std::move(key);
+    GPTRS_HIP_CHECK(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+    capturing = true;
+    std::string err;
+    try {
+        for (const Step& st : plan.steps) run_step(plan, st, cx);
+    } catch (const std::exception& e) {
+        err = e.what();
+    }
+    capturing = false;
+    hipError_t ec = hipStreamEndCapture(stream, &pg.graph);
+    if (!err.empty() || ec != hipSuccess || !pg.graph) {
+        if (pg.graph) (void)hipGraphDestroy(pg.graph);
+        (void)hipGetLastError();
+        plan.graph_builds += 4;  // a plan that cannot be recorded stops trying soon
+        cx.launches = 0;
+        return false;
+    }
+    ec = hipGraphInstantiate(&pg.exec, pg.graph, nullptr, nullptr, 0);
+    if (ec != hipSuccess) {
+        (void)hipGraphDestroy(pg.graph);
+        (void)hipGetLastError();
+        plan.graph_builds += 4;
+        cx.launches = 0;
+        return false;
+    }
+    pg.launches = cx.launches;
+    pg.last_use = ++plan.graph_clock;
+    ++plan.graph_builds;
+    ++n_graphs_built;
+    if (plan.graphs.size() >= kMaxGraphs) {
+        auto lru = std::min_element(plan.graphs.begin(), plan.graphs.end(),
+                                    [](const PlanGraph& a, const PlanGraph& b) { return a.last_use < b.last_use; });
+        (void)hipGraphExecDestroy(lru->exec);
+        (void)hipGraphDestroy(lru->graph);
+        plan.graphs.erase(lru);
+    }
+    GPTRS_HIP_CHECK(hipGraphLaunch(pg.exec, stream));
+    ++n_graph_launches;
+    plan.graphs.push_back(std::move(pg));
+    return true;
 }
 
 void Backend::execute(Plan& plan, gptrs_hip_tensor* const* inputs, const uint8_t* donate, gptrs_hip_tensor** outputs) {
@@ -324,7 +412,9 @@ void Backend::execute(Plan& plan, gptrs_hip_tensor* const* inputs, const uint8_t
             case Storage::InPlace: break;
         }
     }
-    for (const Step& st : plan.steps) run_step(plan, st, cx);
+    if (!run_graphed(plan, cx, out_bufs))
+        for (const Step& st : plan.steps) run_step(plan, st, cx);
+    ++plan.runs;
     {
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) fail_exec(std::string("kernel launch failed: ") + hipGetErrorString(e));
@@ -574,6 +664,7 @@ int gptrs_hip_set_option(gptrs_hip_backend* b, const char* name, int64_t value) 
         if (!b || !name) gptrs::fail_exec("null argument");
         std::lock_guard<std::mutex> g(b->impl.mu);
         if (!strcmp(name, "fusion")) b->impl.opt_fusion = value != 0;
+        else if (!strcmp(name, "graphs")) b->impl.opt_graphs = value != 0;
         else if (!strcmp(name, "profile")) { b->impl.profile_reset(); b->impl.opt_profile = value != 0; }
         else gptrs::fail_spec(std::string("unknown option `") + name + "`");
     });
@@ -599,6 +690,8 @@ int64_t gptrs_hip_counter(const gptrs_hip_backend* b, const char* name) {
     if (!strcmp(name, "inplace_updates")) return i.n_inplace;
     if (!strcmp(name, "derived_weights_built")) return i.n_tiled_built;
     if (!strcmp(name, "last_program_launches")) return i.last_launches;
+    if (!strcmp(name, "graph_launches")) return i.n_graph_launches;
+    if (!strcmp(name, "graphs_built")) return i.n_graphs_built;
     return -1;
 }
 

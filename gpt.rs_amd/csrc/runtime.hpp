@@ -27,6 +27,7 @@ namespace gptrs {
     } while (0)
 
 class Backend;
+struct ExecCtx;
 
 // Size-bucketed cache of device allocations (the reference's Triton backend keeps the same kind
 // of cache, crates/gpt-rs-backend-triton/src/device.rs:727-751).  Blocks are only ever used on the
@@ -101,7 +102,22 @@ struct Step {
     size_t pack_l_off = 0, pack_r_off = 0;
 };
 
+// A captured replay of one plan for one set of buffer addresses.
+struct PlanGraph {
+    std::vector<uint64_t> key;  // input/output addresses + content ids of the weights read through derived copies
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    uint64_t last_use = 0;
+    int64_t launches = 0;
+};
+
 struct Plan {
+    ~Plan();
+    bool cacheable = false;                 // lives in the plan LRU (program_key != 0)
+    std::vector<PlanGraph> graphs;
+    std::vector<uint64_t> seen_keys;        // hashes of address sets executed eagerly so far (ring)
+    int64_t graph_builds = 0, graph_hits = 0, runs = 0;
+    uint64_t graph_clock = 0;
     Function fn;
     std::vector<ValueInfo> values;          // indexed by value id
     std::vector<RootStorage> storage;       // indexed by value id (meaningful for roots)
@@ -152,6 +168,10 @@ class Backend {
     hipStream_t stream = nullptr;
     int device = 0;
     bool opt_fusion = true;
+    // replay steady-state programs (same plan, same buffer addresses) as captured HIP graphs
+    bool opt_graphs = true;
+    bool capturing = false;
+    int64_t n_graph_launches = 0, n_graphs_built = 0;
     // opt-in timing of the linear-layer launches with HIP events on the execution stream
     bool opt_profile = false;
     std::vector<std::pair<hipEvent_t, hipEvent_t>> prof_events;
@@ -166,6 +186,7 @@ class Backend {
   private:
     std::shared_ptr<Plan> get_plan(const char* json, size_t len, uint64_t key, const uint8_t* donate, size_t n_in);
     void execute(Plan& plan, gptrs_hip_tensor* const* inputs, const uint8_t* donate, gptrs_hip_tensor** outputs);
+    bool run_graphed(Plan& plan, ExecCtx& cx, const std::vector<BufferP>& out_bufs);
 
     DevicePool pool_;
     std::unordered_map<std::array<uint8_t, 16>, gptrs_hip_tensor*, IdHash> params_;

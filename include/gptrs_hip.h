@@ -135,13 +135,16 @@ int gptrs_hip_synchronize(gptrs_hip_backend* b);
  * crates/gpt-rs-backend-tests/src/torch_parity/harness.rs:494-511).  "profile" = bracket every
  * linear-layer launch with HIP events on the execution stream (the per-op ns/calls counters the
  * reference C backend exports, crates/gpt-rs-backend-c/src/lib.rs:587-671); setting it resets
- * the linear_* counters. */
+ * the linear_* counters.  "graphs" (default 1) = replay a cached program that runs again over the
+ * same buffer addresses as a recorded HIP graph, one launch per program instead of one per kernel
+ * (no counterpart in the reference: its backends launch op by op). */
 int gptrs_hip_set_option(gptrs_hip_backend* b, const char* name, int64_t value);
 
 /* Counters since creation (the reference's cache_event / WorkStats fields,
  * crates/gpt-rs/src/ops/graph/arena.rs:1201-1243): name in {"kernel_launches",
  * "programs_compiled", "program_cache_hits", "fused_ops", "bytes_allocated",
- * "inplace_updates", "last_program_launches", and with the "profile" option "linear_time_ns",
+ * "inplace_updates", "last_program_launches", "derived_weights_built" (column-tiled weight copies
+ * made for the decode GEMV), "graph_launches", "graphs_built", and with the "profile" option "linear_time_ns",
  * "linear_calls", "linear_bytes" (these three synchronise)}.  Unknown names return -1. */
 int64_t gptrs_hip_counter(const gptrs_hip_backend* b, const char* name);
 

@@ -108,6 +108,33 @@ def test_decode_launch_count_and_inplace_cache(hip):
     assert hip.counter("last_program_launches") <= 3 + 10 * MID_MINISTRAL.num_layers
 
 
+def test_graph_replay_matches_eager_every_step(hip):
+    """A decode step that runs again over the same buffer addresses is replayed as a recorded HIP
+    graph.  Every replay must give the bytes the eager launches give, with readbacks (host
+    synchronisation) and eager work (materialize, sampling) between replays."""
+    m = models.Ministral.random(MID_MINISTRAL, hip, seed=4, dtype="Bf16")
+    hip.set_option("graphs", 0)
+    try:
+        gen = models.Generator(m, PROMPT, kv_cache_capacity=64)
+        eager = []
+        for _ in range(24):
+            gen.step()
+            eager.append(hip.to_numpy(gen.logits).copy())
+    finally:
+        hip.set_option("graphs", 1)
+    before = hip.counter("graph_launches")
+    gen = models.Generator(m, PROMPT, kv_cache_capacity=64)
+    for i in range(24):
+        gen.step()
+        got = hip.to_numpy(gen.logits)
+        assert got.tobytes() == eager[i].tobytes(), f"step {i}"
+    assert hip.counter("graph_launches") - before >= 12
+    # a prefill over the same plan cache still runs (eagerly) and agrees
+    gen2 = models.Generator(m, PROMPT, kv_cache_capacity=64)
+    gen2.step()
+    assert hip.to_numpy(gen2.logits).tobytes() == eager[0].tobytes()
+
+
 def test_batched_decode_matches_single_sequences(hip):
     cfg = TINY_GPT
     m = models.Gpt.random(cfg, hip, seed=21, std=0.2)
