@@ -113,8 +113,9 @@ BufferP Backend::new_buffer(size_t bytes) {
     return b;
 }
 
-BufferP Backend::tiled_weights(const BufferP& src, DType dtype, int64_t k, int64_t n) {
-    auto it = tiled_cache_.find(src->id);
+BufferP Backend::derived_weights(const BufferP& src, int kind, DType dtype, int64_t k, int64_t n) {
+    const uint64_t ckey = src->id * 2 + (uint64_t)kind;
+    auto it = tiled_cache_.find(ckey);
     if (it != tiled_cache_.end()) {
         if (it->second.src.lock() == src) return it->second.tiled;
         tiled_cache_.erase(it);
@@ -124,9 +125,15 @@ BufferP Backend::tiled_weights(const BufferP& src, DType dtype, int64_t k, int64
         for (auto e = tiled_cache_.begin(); e != tiled_cache_.end();)
             e = e->second.src.expired() ? tiled_cache_.erase(e) : std::next(e);
     }
-    BufferP t = new_buffer(k::tiled_weight_bytes((int)dtype, k, n));
-    k::tile_weights(stream, (int)dtype, src->ptr, t->ptr, k, n);
-    tiled_cache_[src->id] = Derived{src, t};
+    BufferP t;
+    if (kind == 0) {
+        t = new_buffer(k::tiled_weight_bytes((int)dtype, k, n));
+        k::tile_weights(stream, (int)dtype, src->ptr, t->ptr, k, n);
+    } else {
+        t = new_buffer(k::mfma_weight_bytes((int)dtype, k, n));
+        k::mfma_pack_weights(stream, (int)dtype, src->ptr, t->ptr, k, n);
+    }
+    tiled_cache_[ckey] = Derived{src, t};
     ++n_tiled_built;
     return t;
 }

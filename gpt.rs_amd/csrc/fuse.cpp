@@ -714,9 +714,14 @@ struct Fuser {
             const Spec* ws = spec_of(in.operands[1].value);
             if (!xs || !ws) continue;
             const int64_t M = xs->dims[0];
-            if (!k::gemv_tiled_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1])) continue;
             if (!is_param(in.operands[1].value)) continue;
-            if (in.act == 2 && (!is_param(in.operands[2].value) || M > 8)) continue;
+            if (in.act == 2 && !is_param(in.operands[2].value)) continue;
+            if (k::mfma_gemm_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1])) {
+                in.mfma = true;
+                continue;
+            }
+            if (!k::gemv_tiled_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1])) continue;
+            if (in.act == 2 && M > 8) continue;
             in.tiled = true;
         }
         const std::vector<int> uses = count_uses();

@@ -109,6 +109,19 @@ void tile_weights(hipStream_t s, int dtype, const void* w, void* wt, int64_t k, 
 bool gemv_tiled_supported(int dtype, int64_t m, int64_t k, int64_t n);
 void gemv_tiled(hipStream_t s, const TiledLinearArgs& a);
 
+// Prefill GEMM (M > 16, bf16) on the matrix cores over a k-grouped copy of the weights,
+// Wk8[K/8][Npad][8] (kernels_mfma.hip).  wk2 != nullptr: SwiGLU pair.
+struct MfmaLinearArgs {
+    const void* x; const void* wk; const void* wk2; const void* bias; const void* residual;
+    void* y;
+    int64_t m, k, n;
+    int act;
+};
+size_t mfma_weight_bytes(int dtype, int64_t k, int64_t n);
+void mfma_pack_weights(hipStream_t s, int dtype, const void* w, void* out, int64_t k, int64_t n);
+bool mfma_gemm_supported(int dtype, int64_t m, int64_t k, int64_t n);
+void mfma_gemm(hipStream_t s, const MfmaLinearArgs& a);
+
 // Rotate-half RoPE on packed [T, Q|K|V] rows (ops/functional/rotary.rs:430-536).
 void rope_packed(hipStream_t s, int dtype, const void* qkv, const void* cos, const void* sin, void* out,
                  int64_t t, int64_t n_q, int64_t n_kv, int64_t head_dim, int64_t half);

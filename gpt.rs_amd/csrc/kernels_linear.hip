@@ -286,16 +286,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const T* __restrict__ x
     }
 }
 
-bool mfma_gemm_supported(int dtype, int64_t m, int64_t k, int64_t n);
-void mfma_gemm(hipStream_t s, int dtype, const void* x, const void* w, const void* bias, const void* residual, void* y,
-               int64_t m, int64_t k, int64_t n, int act);
-
 static void gemm_any(hipStream_t s, int dtype, const void* x, const void* w, const void* bias, const void* residual,
                      void* y, int64_t m, int64_t k, int64_t n, int act) {
-    if (mfma_gemm_supported(dtype, m, k, n)) {
-        mfma_gemm(s, dtype, x, w, bias, residual, y, m, k, n, act);
-        return;
-    }
     dim3 grid((unsigned)cdiv(n, 64), (unsigned)cdiv(m, 64));
     if (dtype == 0)
         gemm_tiled_kernel<float><<<grid, 256, 0, s>>>((const float*)x, (const float*)w, (const float*)bias, (const float*)residual, (float*)y, m, k, n, act);

@@ -1,13 +1,236 @@
-// MFMA tile GEMM for prefill-sized linears (M > 16).  Filled in by mfma_gemm(); until a shape is
-// supported the caller falls back to the LDS-tiled FMA kernel in kernels_linear.hip.
+// MFMA tile GEMM for prefill-sized linear layers (M > 16), bf16 in / f32 accumulate / bf16 out.
+//
+// v_mfma_f32_32x32x16_bf16 wants, per lane, 8 consecutive k of ONE row (A) or ONE column (B).
+// Activations x[M,K] are row-major, so A fragments are plain 16-byte loads.  Weights are stored
+// [in,out] row-major (nn/layers/linear.rs:50-71), the wrong way round for B, so the GEMM reads a
+// derived copy Wk8[K/8][Npad][8] (8 consecutive k of a column are adjacent; Npad = N rounded up to
+// the 128-column block tile, zero filled) that the backend builds once per weight and keeps beside
+// the original.  With it a block's B tile is, per group of 8 k, one contiguous 2 KiB run.
 #include "kernels.hpp"
 #include "device_utils.hpp"
 
 namespace gptrs {
 namespace k {
 
-bool mfma_gemm_supported(int, int64_t, int64_t, int64_t) { return false; }
-void mfma_gemm(hipStream_t, int, const void*, const void*, const void*, const void*, void*, int64_t, int64_t, int64_t, int) {}
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+constexpr int kBN = 128, kBK = 64;  // kBN: column padding unit of the derived weights
+constexpr int kKb = kBK / 8;                       // groups of 8 k per tile
+
+int64_t mfma_padded_n(int64_t n) { return cdiv(n, kBN) * kBN; }
+size_t mfma_weight_bytes(int dtype, int64_t k, int64_t n) {
+    (void)dtype;
+    return (size_t)cdiv(k, 8) * (size_t)mfma_padded_n(n) * 8 * sizeof(bf16_t);
+}
+
+// Wk8[kb][n][i] = W[kb*8+i][n]; one thread per (kb, n); reads coalesced along n, one 16-byte store.
+__global__ __launch_bounds__(256) void k8_weights_kernel(const bf16_t* __restrict__ w, bf16_t* __restrict__ out, int64_t K,
+                                                         int64_t N, int64_t Npad) {
+    const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t kb = blockIdx.y;
+    if (n >= Npad) return;
+    uint32_t r[4] = {0, 0, 0, 0};
+    if (n < N) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int64_t kx = kb * 8 + i;
+            const uint32_t v = kx < K ? (uint32_t)w[kx * N + n] : 0u;
+            r[i >> 1] |= v << ((i & 1) * 16);
+        }
+    }
+    *reinterpret_cast<uint4*>(out + (kb * Npad + n) * 8) = make_uint4(r[0], r[1], r[2], r[3]);
+}
+
+void mfma_pack_weights(hipStream_t s, int dtype, const void* w, void* out, int64_t k, int64_t n) {
+    (void)dtype;
+    const int64_t npad = mfma_padded_n(n);
+    dim3 grid((unsigned)cdiv(npad, 256), (unsigned)cdiv(k, 8));
+    k8_weights_kernel<<<grid, 256, 0, s>>>((const bf16_t*)w, (bf16_t*)out, k, n, npad);
+}
+
+__device__ __forceinline__ float mfma_finish(float v, float v2, bool dual, int act, float bias, bool has_res, float res) {
+    if (dual) v = (v / (1.0f + expf(v * -1.0f))) * v2;        // activation.rs:141-162
+    v += bias;                                                // tensor_ops.rs:42-56
+    if (act == 1) v = (v * 0.5f) * (erff(v / 1.41421354f) + 1.0f);  // activation.rs:96-113
+    if (has_res) v += res;
+    return v;
+}
+
+// Block tile BM x BN (128x128 as launched), BK = 64, four waves in a 2x2 grid; each wave owns
+// (BM/2) x (BN/2) outputs as TM x TN MFMA tiles of 32x32.  LDS holds two stages of fragments,
+// k-group-major ([kb][row or column][8 k], one spare row per k-group as CK does on gfx950), so a
+// fragment read is a contiguous 512 bytes per half-wave.  Per k tile: one barrier; the tile after
+// next is fetched global -> registers while the current one is multiplied, and the registers are
+// stored into the idle LDS stage in the middle of the multiply.  Fragment reads run one k-step
+// (16 k) ahead of the MFMAs that consume them.
+//
+// The staging registers are native vectors and every load is unconditional (the index is clamped
+// instead): with HIP's uint4 struct and a guarded load the compiler keeps the staging array in
+// scratch memory and waits for every load at once, which cost a factor of four.
+//
+// Requires K % 64 == 0; M and N are guarded (rows clamp on load, stores are masked; the derived
+// weights are padded to whole 128-column tiles).
+// DUAL: SwiGLU pair silu(x.W) * (x.W2).  The block covers BN/2 real columns; the B tile holds, per
+// wave column, TN/2 fragments of W followed by the same columns of W2, so gate and up of one
+// output meet in the same lane.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+template <int BM, int BN, bool DUAL>
+__global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wk,
+                                                             const bf16_t* __restrict__ wk2, const bf16_t* __restrict__ bias,
+                                                             const bf16_t* __restrict__ residual, bf16_t* __restrict__ y,
+                                                             int M, int K, int N, int Npad, int act) {
+    constexpr int SA = (BM + 1) * 16, SB = (BN + 1) * 16;     // bytes between k-groups
+    constexpr int STAGE = kKb * (SA + SB);
+    constexpr int TM = BM / 64, TN = BN / 64;
+    constexpr int CA = BM * kKb / 256, CB = BN * kKb / 256;   // 16-byte chunks per thread per tile
+    constexpr int WN = BN / 2;                                // B-tile columns per wave column
+    constexpr int NREAL = DUAL ? BN / 2 : BN;                 // output columns per block
+    static_assert(!DUAL || TN % 2 == 0, "dual tiles need an even number of column fragments");
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * NREAL;
+
+    // global -> LDS chunk assignment (16 bytes each)
+    // A: chunk c -> kb = c % 8, row = c / 8: eight lanes read 128 contiguous bytes of one row
+    // B: chunk c -> tile column = c % BN, kb = c / BN: contiguous runs of the k-grouped weights
+    const bf16_t* a_src[CA];
+    const bf16_t* b_src[CB];
+    int a_dst[CA], b_dst[CB];
+#pragma unroll
+    for (int j = 0; j < CA; ++j) {
+        const int c = tid + 256 * j;
+        const int kb = c & 7, row = c >> 3;
+        int m = m0 + row;
+        if (m > M - 1) m = M - 1;
+        a_src[j] = x + (int64_t)m * K + kb * 8;
+        a_dst[j] = kb * SA + row * 16;
+    }
+#pragma unroll
+    for (int j = 0; j < CB; ++j) {
+        const int c = tid + 256 * j;
+        const int bc = c % BN, bkb = c / BN;
+        int col = n0 + bc;
+        const bf16_t* src = wk;
+        if (DUAL) {
+            // tile column -> (wave column, gate|up, column inside the half)
+            const int wcol = bc / WN, in_w = bc % WN, half = in_w / (WN / 2), cc = in_w % (WN / 2);
+            col = n0 + wcol * (WN / 2) + cc;
+            src = half ? wk2 : wk;
+        }
+        b_src[j] = src + ((int64_t)bkb * Npad + col) * 8;
+        b_dst[j] = kKb * SA + bkb * SB + bc * 16;
+    }
+
+    f32x16_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    u32x4_t ra[CA], rb[CB];
+    const int nt = K / kBK;
+    const int64_t b_tile_step = (int64_t)kKb * Npad * 8;  // elements between consecutive k tiles of Wk8
+    auto gload = [&](int t) {
+#pragma unroll
+        for (int j = 0; j < CA; ++j) ra[j] = *reinterpret_cast<const u32x4_t*>(a_src[j] + (int64_t)t * kBK);
+#pragma unroll
+        for (int j = 0; j < CB; ++j) rb[j] = *reinterpret_cast<const u32x4_t*>(b_src[j] + (int64_t)t * b_tile_step);
+    };
+    auto lwrite = [&](int buf) {
+        unsigned char* base = lds + buf * STAGE;
+#pragma unroll
+        for (int j = 0; j < CA; ++j) *reinterpret_cast<u32x4_t*>(base + a_dst[j]) = ra[j];
+#pragma unroll
+        for (int j = 0; j < CB; ++j) *reinterpret_cast<u32x4_t*>(base + b_dst[j]) = rb[j];
+    };
+    const int a_rd = (wm * (BM / 2) + (lane & 31)) * 16 + (lane >> 5) * SA;
+    const int b_rd = kKb * SA + (wn * WN + (lane & 31)) * 16 + (lane >> 5) * SB;
+    bf16x8_t af[2][TM], bfr[2][TN];
+    auto fread = [&](int buf, int kk, int slot) {
+        const unsigned char* base = lds + buf * STAGE;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) af[slot][i] = *reinterpret_cast<const bf16x8_t*>(base + a_rd + kk * 2 * SA + i * 32 * 16);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bfr[slot][j] = *reinterpret_cast<const bf16x8_t*>(base + b_rd + kk * 2 * SB + j * 32 * 16);
+    };
+
+    gload(0);
+    lwrite(0);
+    gload(nt > 1 ? 1 : 0);
+    __syncthreads();
+    for (int t = 0; t < nt; ++t) {
+        const int cur = t & 1;
+        fread(cur, 0, 0);
+#pragma unroll
+        for (int kk = 0; kk < kBK / 16; ++kk) {
+            if (kk + 1 < kBK / 16) fread(cur, kk + 1, (kk + 1) & 1);
+            if (kk == 1) {
+                lwrite(cur ^ 1);  // tile t+1; past the last tile this stores a copy nobody reads
+                gload(t + 2 < nt ? t + 2 : nt - 1);
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], bfr[kk & 1][j], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+    // epilogue: lane holds column (lane % 32), rows 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 tile
+    constexpr int TNO = DUAL ? TN / 2 : TN;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TNO; ++j) {
+            const int n = n0 + wn * (NREAL / 2) + j * 32 + (lane & 31);
+            if (n >= N) continue;
+            const float bv = bias ? bf16_to_f32(bias[n]) : 0.f;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int m = m0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                if (m >= M) continue;
+                const float r = residual ? bf16_to_f32(residual[(int64_t)m * N + n]) : 0.f;
+                const float g = acc[i][j][v];
+                const float u = DUAL ? acc[i][DUAL ? j + TN / 2 : j][v] : 0.f;
+                y[(int64_t)m * N + n] = f32_to_bf16(mfma_finish(g, u, DUAL, act, bv, residual != nullptr, r));
+            }
+        }
+}
+
+bool mfma_gemm_supported(int dtype, int64_t m, int64_t k, int64_t n) {
+    return dtype == 2 && m > 16 && k >= kBK && k % kBK == 0 && n >= 1 && m < (1ll << 31) && n < (1ll << 31) - kBN &&
+           k < (1ll << 31);
+}
+
+template <int BM, int BN, bool DUAL>
+static void launch_mfma(hipStream_t s, const MfmaLinearArgs& a) {
+    constexpr int lds_bytes = 2 * kKb * ((BM + 1) * 16 + (BN + 1) * 16);
+    auto kern = gemm_bf16_mfma_kernel<BM, BN, DUAL>;
+    static bool configured = false;  // the attribute is per function, not per stream or device state
+    if (!configured) {
+        (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        configured = true;
+    }
+    const int64_t npad = mfma_padded_n(a.n);
+    constexpr int nreal = DUAL ? BN / 2 : BN;
+    dim3 grid((unsigned)cdiv(npad, nreal), (unsigned)cdiv(a.m, BM));
+    kern<<<grid, 256, lds_bytes, s>>>((const bf16_t*)a.x, (const bf16_t*)a.wk, (const bf16_t*)a.wk2, (const bf16_t*)a.bias,
+                                      (const bf16_t*)a.residual, (bf16_t*)a.y, (int)a.m, (int)a.k, (int)a.n, (int)npad, a.act);
+}
+
+void mfma_gemm(hipStream_t s, const MfmaLinearArgs& a) {
+    if (a.wk2) launch_mfma<128, 128, true>(s, a);
+    else launch_mfma<128, 128, false>(s, a);
+}
 
 }  // namespace k
 }  // namespace gptrs

@@ -487,7 +487,7 @@ void Builder::describe(Step& st) {
         case OpKind::FLinear: {
             const Spec& x = spec_of(in, 0);
             const Spec& w = spec_of(in, 1);
-            if (in.tiled) {
+            if (in.tiled || in.mfma) {
                 auto pos = [&](size_t op) {
                     const int v = in.operands[op].value;
                     const int p = v >= 0 && v < (int)param_pos.size() ? param_pos[v] : -1;
@@ -819,17 +819,50 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
         case OpKind::FLinear: {
             const Spec& x = in_spec(0);
             const Spec& w = in_spec(1);
+            if (in.mfma) {
+                k::MfmaLinearArgs ma{};
+                ma.x = src_ptr(st, cx, 0);
+                ma.m = x.dims[0]; ma.k = x.dims[1]; ma.n = w.dims[1];
+                BufferP wk = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], 1, x.dtype, ma.k, ma.n);
+                BufferP wk2;
+                ma.wk = wk->ptr;
+                size_t oi = 2;
+                if (in.act == 2) {
+                    wk2 = cx.be->derived_weights(cx.input_bufs[st.tiled_w2_input], 1, x.dtype, ma.k, ma.n);
+                    ma.wk2 = wk2->ptr;
+                    ++oi;
+                }
+                if (in.has_bias) ma.bias = src_ptr(st, cx, oi++);
+                if (in.has_residual) ma.residual = src_ptr(st, cx, oi++);
+                ma.y = dst;
+                ma.act = in.act == 1 ? 1 : 0;
+                hipEvent_t e0 = nullptr, e1 = nullptr;
+                if (cx.profile) {
+                    GPTRS_HIP_CHECK(hipEventCreate(&e0));
+                    GPTRS_HIP_CHECK(hipEventCreate(&e1));
+                    GPTRS_HIP_CHECK(hipEventRecord(e0, s));
+                }
+                k::mfma_gemm(s, ma);
+                if (cx.profile) {
+                    GPTRS_HIP_CHECK(hipEventRecord(e1, s));
+                    cx.be->prof_events.emplace_back(e0, e1);
+                    ++cx.be->prof_linear_calls;
+                    cx.be->prof_linear_bytes += (int64_t)dtype_size(x.dtype) * (ma.m * ma.k + ma.k * ma.n * (ma.wk2 ? 2 : 1) + ma.m * ma.n);
+                }
+                ++cx.launches;
+                break;
+            }
             if (in.tiled) {
                 k::TiledLinearArgs ta{};
                 ta.dtype = (int)x.dtype;
                 ta.x = src_ptr(st, cx, 0);
                 ta.m = x.dims[0]; ta.k = x.dims[1]; ta.n = w.dims[1];
-                BufferP wt = cx.be->tiled_weights(cx.input_bufs[st.tiled_w_input], x.dtype, ta.k, ta.n);
+                BufferP wt = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], 0, x.dtype, ta.k, ta.n);
                 BufferP wt2;
                 ta.wt = wt->ptr;
                 size_t oi = 2;
                 if (in.act == 2) {
-                    wt2 = cx.be->tiled_weights(cx.input_bufs[st.tiled_w2_input], x.dtype, ta.k, ta.n);
+                    wt2 = cx.be->derived_weights(cx.input_bufs[st.tiled_w2_input], 0, x.dtype, ta.k, ta.n);
                     ta.wt2 = wt2->ptr;
                     ++oi;
                 }

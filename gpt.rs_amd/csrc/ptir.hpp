@@ -111,6 +111,7 @@ struct Instr {
     int act = 0;                      // FLinear epilogue: 0 none, 1 gelu, 2 swiglu (dual weights)
     bool has_bias = false, has_residual = false;
     float fparam[4] = {0.f, 0.f, 0.f, 0.f};  // FGelu: half, divisor, one
+    bool mfma = false;                       // FLinear: prefill GEMM over the k-grouped weight copy
     bool tiled = false;                      // FLinear: decode GEMV over the column-tiled weight copy
     bool norm = false;                       // FLinear: RMSNorm of x fused in (last operand = gamma; eps, scale)
     bool scalar_rhs = false;                 // Binary whose rhs is a broadcast scalar literal

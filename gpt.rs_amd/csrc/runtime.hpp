@@ -158,9 +158,10 @@ class Backend {
     void check_device_errors();
 
     BufferP new_buffer(size_t bytes);
-    // Column-tiled copy of a weight tensor (kernels_gemv_tiled.hip), built on first use and kept while
-    // the source buffer lives: the backend-side memo of derived weight formats.
-    BufferP tiled_weights(const BufferP& src, DType dtype, int64_t k, int64_t n);
+    // Derived layouts of a weight tensor, built on first use and kept while the source buffer lives
+    // (the backend-side memo of derived weight formats).  kind 0: column-tiled copy for the decode
+    // GEMV (kernels_gemv_tiled.hip); kind 1: k-grouped copy for the MFMA GEMM (kernels_mfma.hip).
+    BufferP derived_weights(const BufferP& src, int kind, DType dtype, int64_t k, int64_t n);
     int64_t n_tiled_built = 0;
     void release_block(void* p, size_t cap) { pool_.release(p, cap); }
 

@@ -147,6 +147,25 @@ def test_matmul(hip, m, k, n, dtype):
     check_program(hip, prog(lambda fb, x, y: x.matmul(y), [(dtype, [m, k]), (dtype, [k, n])]), [a, b], **tol)
 
 
+@pytest.mark.parametrize("m,k,n", [(17, 64, 8), (100, 128, 72), (128, 192, 256), (300, 64, 200), (257, 320, 129)])
+def test_prefill_linear_on_matrix_cores(hip, m, k, n):
+    """bf16 linears with more than 16 rows and K % 64 == 0 run on the MFMA kernel over the k-grouped
+    weight copy: plain matmul, bias + exact GELU + residual epilogue, and the SwiGLU pair.  Ragged M
+    and N exercise the row clamp, the column padding and the store masks.  The oracle rounds every
+    op to bf16, the fused kernel once at the end, hence the bf16-sized tolerance."""
+    x = rng_uniform(40, (m, k))
+    w, w2 = rng_uniform(41, (k, n)) / np.sqrt(k) * 2, rng_uniform(42, (k, n)) / np.sqrt(k) * 2
+    b, r = rng_uniform(43, (n,)), rng_uniform(44, (m, n))
+    tol = dict(atol=3e-2, rtol=3e-2)
+    before = hip.counter("derived_weights_built")
+    check_program(hip, prog(lambda fb, a, c: a.matmul(c), [("Bf16", [m, k]), ("Bf16", [k, n])]), [x, w], **tol)
+    check_program(hip, prog(lambda fb, a, c, d, e: F.gelu(F.linear(a, c, d)) + e,
+                            [("Bf16", [m, k]), ("Bf16", [k, n]), ("Bf16", [n]), ("Bf16", [m, n])]), [x, w, b, r], **tol)
+    check_program(hip, prog(lambda fb, a, c, d: F.swiglu(a.matmul(c), a.matmul(d)),
+                            [("Bf16", [m, k]), ("Bf16", [k, n]), ("Bf16", [k, n])]), [x, w, w2], **tol)
+    assert hip.counter("derived_weights_built") - before >= 4  # the fused legs took the derived-weight path
+
+
 @pytest.mark.parametrize("b,m,k,n", [(1, 4, 5, 2), (2, 7, 13, 9), (8, 4, 8, 4), (3, 33, 65, 31)])
 def test_matmul_batched(hip, b, m, k, n):
     a, c = rng_uniform(9, (b, m, k)), rng_uniform(10, (b, k, n))
