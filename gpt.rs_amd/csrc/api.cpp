@@ -1,5 +1,6 @@
 // Backend implementation and the extern "C" surface declared in include/gptrs_hip.h.
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 
 #include "../../include/gptrs_hip.h"
@@ -54,6 +55,15 @@ Backend::Backend(int dev) : device(dev) {
         fail_exec("no HIP device is visible: the hip backend has no CPU fallback");
     if (dev < 0 || dev >= count) fail_exec("device index out of range");
     GPTRS_HIP_CHECK(hipSetDevice(dev));
+    // Graph replay is off when GPTRS_HIP_GRAPHS=0, and under a rocprofiler-sdk tool (rocprofv3): a
+    // replayed graph of this size under its kernel tracing was answered with "AQL packet is
+    // malformed" and a stalled queue, while the same steps launched one by one trace fine.
+    {
+        const char* g = getenv("GPTRS_HIP_GRAPHS");
+        const char* tool = getenv("ROCP_TOOL_LIBRARIES");
+        const char* pre = getenv("LD_PRELOAD");
+        if ((g && g[0] == '0') || (tool && tool[0]) || (pre && strstr(pre, "rocprofiler-sdk"))) opt_graphs = false;
+    }
     GPTRS_HIP_CHECK(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
     GPTRS_HIP_CHECK(hipMalloc((void**)&d_err_flag_, 256));
     GPTRS_HIP_CHECK(hipMalloc((void**)&d_counters_, k::kLinearCounters * sizeof(int)));
@@ -61,6 +71,12 @@ Backend::Backend(int dev) : device(dev) {
     GPTRS_HIP_CHECK(hipMalloc((void**)&d_argmax_idx_, 1024 * sizeof(int32_t)));
     GPTRS_HIP_CHECK(hipMalloc((void**)&d_token_, 256));
     GPTRS_HIP_CHECK(hipHostMalloc(&h_pinned_, 256, hipHostMallocDefault));
+    GPTRS_HIP_CHECK(hipMalloc((void**)&d_chain_bar_, k::kChainBarrierBytes));
+    k::fill_zero(stream, d_chain_bar_, k::kChainBarrierBytes);
+    {
+        const char* c = getenv("GPTRS_HIP_CHAIN");
+        if (c && c[0] == '0') opt_chain = false;
+    }
     k::fill_zero(stream, d_err_flag_, 256);
     k::fill_zero(stream, d_counters_, k::kLinearCounters * sizeof(int));
     GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
@@ -77,7 +93,9 @@ Backend::~Backend() {
     plan_index_.clear();
     plan_lru_.clear();
     tiled_cache_.clear();
+    chain_tables_.clear();
     pool_.trim();
+    (void)hipFree(d_chain_bar_);
     (void)hipFree(d_err_flag_);
     (void)hipFree(d_counters_);
     (void)hipFree(d_argmax_val_);
@@ -113,29 +131,58 @@ BufferP Backend::new_buffer(size_t bytes) {
     return b;
 }
 
-BufferP Backend::derived_weights(const BufferP& src, int kind, DType dtype, int64_t k, int64_t n) {
-    const uint64_t ckey = src->id * 2 + (uint64_t)kind;
+BufferP Backend::derived_weights(const BufferP& src, int kind, DType dtype, int64_t k, int64_t n, const BufferP& src2) {
+    const std::array<uint64_t, 3> ckey{src->id, src2 ? src2->id : 0, (uint64_t)kind};
     auto it = tiled_cache_.find(ckey);
     if (it != tiled_cache_.end()) {
-        if (it->second.src.lock() == src) return it->second.tiled;
+        if (it->second.src.lock() == src && it->second.src2.lock() == src2) return it->second.tiled;
         tiled_cache_.erase(it);
     }
     if (capturing) fail_exec("derived weight copy missing while recording a graph");
     if (tiled_cache_.size() >= 64 && (tiled_cache_.size() & 63) == 0) {  // drop entries whose source died
         for (auto e = tiled_cache_.begin(); e != tiled_cache_.end();)
-            e = e->second.src.expired() ? tiled_cache_.erase(e) : std::next(e);
+            e = (e->second.src.expired() || (e->first[1] && e->second.src2.expired())) ? tiled_cache_.erase(e) : std::next(e);
     }
     BufferP t;
     if (kind == 0) {
         t = new_buffer(k::tiled_weight_bytes((int)dtype, k, n));
         k::tile_weights(stream, (int)dtype, src->ptr, t->ptr, k, n);
-    } else {
+    } else if (kind == 1) {
         t = new_buffer(k::mfma_weight_bytes((int)dtype, k, n));
         k::mfma_pack_weights(stream, (int)dtype, src->ptr, t->ptr, k, n);
+    } else {
+        t = new_buffer(k::chain_weight_bytes(k, n, src2 != nullptr));
+        k::chain_pack_weights(stream, src->ptr, src2 ? src2->ptr : nullptr, t->ptr, k, n);
     }
-    tiled_cache_[ckey] = Derived{src, t};
+    Derived d;
+    d.src = src;
+    if (src2) d.src2 = src2;
+    d.tiled = t;
+    tiled_cache_[ckey] = std::move(d);
     ++n_tiled_built;
     return t;
+}
+
+const k::ChainPhase* Backend::chain_table(const std::vector<k::ChainPhase>& phases) {
+    const size_t bytes = phases.size() * sizeof(k::ChainPhase);
+    for (auto& t : chain_tables_)
+        if (t.host.size() == phases.size() && !memcmp(t.host.data(), phases.data(), bytes)) {
+            t.last_use = ++chain_clock_;
+            return (const k::ChainPhase*)t.dev->ptr;
+        }
+    if (capturing) fail_exec("chain table missing while recording a graph");
+    // Recorded graphs keep table addresses, so a table is never freed while the backend lives;
+    // past the cap the caller runs the linears one by one instead.
+    if (chain_tables_.size() >= 4096) return nullptr;
+    ChainTable t;
+    t.host = phases;
+    t.dev = new_buffer(bytes);
+    t.last_use = ++chain_clock_;
+    // pageable source: wait, so the vector may go away (tables are built once per address set)
+    GPTRS_HIP_CHECK(hipMemcpyAsync(t.dev->ptr, phases.data(), bytes, hipMemcpyHostToDevice, stream));
+    GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
+    chain_tables_.push_back(std::move(t));
+    return (const k::ChainPhase*)chain_tables_.back().dev->ptr;
 }
 
 gptrs_hip_tensor* Backend::materialize(const Spec& spec, const void* host, size_t nbytes) {
@@ -169,9 +216,15 @@ gptrs_hip_tensor* Backend::materialize(const Spec& spec, const void* host, size_
 void Backend::check_device_errors() {
     // called after a stream synchronisation
     int* flag = (int*)h_pinned_ + 32;
-    GPTRS_HIP_CHECK(hipMemcpyAsync(flag, d_err_flag_, sizeof(int), hipMemcpyDeviceToHost, stream));
+    GPTRS_HIP_CHECK(hipMemcpyAsync(flag, d_err_flag_, 2 * sizeof(int), hipMemcpyDeviceToHost, stream));
     GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
-    if (*flag) {
+    if (flag[1]) {
+        // a grid barrier of the persistent decode chain gave up: its counters are mid-phase
+        k::fill_zero(stream, d_err_flag_, 256);
+        k::fill_zero(stream, d_chain_bar_, k::kChainBarrierBytes);
+        fail_exec("decode chain: grid barrier timed out (workgroups of one launch were not all resident)");
+    }
+    if (flag[0]) {
         k::fill_zero(stream, d_err_flag_, 256);
         fail_exec("take index out of bounds");  // cpu.rs:1632-1634
     }
@@ -300,6 +353,7 @@ bool Backend::run_graphed(Plan& plan, ExecCtx& cx, const std::vector<BufferP>& o
     key.reserve(cx.input_bufs.size() + out_bufs.size() + 8);
     for (const auto& b : cx.input_bufs) key.push_back((uint64_t)(uintptr_t)b->ptr);
     for (const auto& b : out_bufs) key.push_back((uint64_t)(uintptr_t)b->ptr);
+    key.push_back(opt_chain ? 1 : 0);
     for (const Step& st : plan.steps) {
         if (st.tiled_w_input >= 0) key.push_back(cx.input_bufs[st.tiled_w_input]->id);
         if (st.tiled_w2_input >= 0) key.push_back(cx.input_bufs[st.tiled_w2_input]->id);
@@ -403,6 +457,7 @@ void Backend::execute(Plan& plan, gptrs_hip_tensor* const* inputs, const uint8_t
     cx.err_flag = d_err_flag_;
     cx.counters = d_counters_;
     cx.profile = opt_profile;
+    cx.chain = opt_chain && k::chain_grid() > 0;
     cx.input_bufs.resize(n_in);
     for (size_t i = 0; i < n_in; ++i) cx.input_bufs[i] = inputs[i]->buf;
     cx.ptr.assign(plan.values.size(), nullptr);
@@ -672,6 +727,7 @@ int gptrs_hip_set_option(gptrs_hip_backend* b, const char* name, int64_t value) 
         std::lock_guard<std::mutex> g(b->impl.mu);
         if (!strcmp(name, "fusion")) b->impl.opt_fusion = value != 0;
         else if (!strcmp(name, "graphs")) b->impl.opt_graphs = value != 0;
+        else if (!strcmp(name, "chain")) b->impl.opt_chain = value != 0;
         else if (!strcmp(name, "profile")) { b->impl.profile_reset(); b->impl.opt_profile = value != 0; }
         else gptrs::fail_spec(std::string("unknown option `") + name + "`");
     });
@@ -699,6 +755,8 @@ int64_t gptrs_hip_counter(const gptrs_hip_backend* b, const char* name) {
     if (!strcmp(name, "last_program_launches")) return i.last_launches;
     if (!strcmp(name, "graph_launches")) return i.n_graph_launches;
     if (!strcmp(name, "graphs_built")) return i.n_graphs_built;
+    if (!strcmp(name, "chain_launches")) return i.n_chain_launches;
+    if (!strcmp(name, "chain_phases")) return i.n_chain_phases;
     return -1;
 }
 

@@ -109,6 +109,35 @@ void tile_weights(hipStream_t s, int dtype, const void* w, void* wt, int64_t k, 
 bool gemv_tiled_supported(int dtype, int64_t m, int64_t k, int64_t n);
 void gemv_tiled(hipStream_t s, const TiledLinearArgs& a);
 
+// Persistent decode chain (kernels_chain.hip): a run of consecutive M = 1 bf16 linear layers in
+// ONE launch of one workgroup per CU, phases separated by a grid barrier, weights read from a
+// 4-column / k-pair tiled copy, Wc[tile][k/2][4][2].  `flags` of a phase: RMSNorm prologue
+// (gamma, inv_n, eps), SwiGLU pair (weights of gate and up interleaved column by column in one
+// copy), bias, exact-erf GELU, residual.  x, residual and y may be produced by earlier phases of
+// the same launch.
+constexpr int kChainCounters = 16;        // striped arrival counters of the grid barrier
+constexpr int kChainMaxPhases = 64;
+constexpr int kChainMaxXsWords = 16384;   // staged activation pairs: K <= 32768
+constexpr size_t kChainBarrierBytes = (kChainCounters * 64 + 64) * sizeof(unsigned);  // zero-initialised once
+enum : int { kChainNorm = 1, kChainDual = 2, kChainGelu = 4, kChainResidual = 8, kChainBias = 16 };
+struct ChainPhase {
+    const void* w; const void* x; const void* gamma; const void* bias; const void* residual;
+    void* y;
+    int K, N, Kw, ntiles, wpt, units, upb, flags;
+    float inv_n, eps;
+};
+int chain_grid();  // workgroups per launch (one per CU), 0 when no device is current
+bool chain_supported(int dtype, int64_t m, int64_t k, int64_t n, bool dual, bool norm);
+size_t chain_weight_bytes(int64_t k, int64_t n, bool dual);
+// w2 != nullptr: SwiGLU pair, columns of w (gate) and w2 (up) interleaved
+void chain_pack_weights(hipStream_t s, const void* w, const void* w2, void* out, int64_t k, int64_t n);
+// fills K, N, Kw, ntiles, wpt, units, upb (and the dual flag); false when one workgroup would own
+// more bias/residual columns than the kernel stages
+bool chain_fill_phase(ChainPhase& p, int64_t k, int64_t n, bool dual);
+// bar: kChainBarrierBytes of device memory zeroed once; abort_flag: raised when a barrier wait
+// gives up (every wave then leaves the kernel).  false: launch not possible (caller falls back).
+bool chain_launch(hipStream_t s, const ChainPhase* dev_table, int nphases, int max_kw, unsigned* bar, int* abort_flag);
+
 // Prefill GEMM (M > 16, bf16) on the matrix cores over a k-grouped copy of the weights,
 // Wk8[K/8][Npad][8] (kernels_mfma.hip).  wk2 != nullptr: SwiGLU pair.
 struct MfmaLinearArgs {

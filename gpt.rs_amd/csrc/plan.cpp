@@ -683,6 +683,27 @@ void Builder::build() {
         for (int v : dying[s]) ws_free(plan.storage[v].offset, plan.storage[v].bytes);
     }
     plan.workspace_bytes = high;
+
+    // runs of consecutive decode linears -> one persistent launch each
+    auto chainable = [&](const Step& st) {
+        const Instr& in = st.in;
+        if (in.op != OpKind::FLinear || !in.tiled || st.tiled_w_input < 0) return false;
+        const Spec& x = plan.values[st.src[0]].spec;
+        const Spec& w = plan.values[st.src[1]].spec;
+        if (x.rank() != 2 || w.rank() != 2) return false;
+        const bool dual = in.act == 2;
+        if (!k::chain_supported((int)x.dtype, x.dims[0], x.dims[1], w.dims[1], dual, in.norm)) return false;
+        k::ChainPhase p{};
+        return k::chain_fill_phase(p, x.dims[1], w.dims[1], dual);
+    };
+    for (int s = 0; s < n_steps;) {
+        if (!chainable(plan.steps[s])) { ++s; continue; }
+        int e = s + 1;
+        while (e < n_steps && e - s < k::kChainMaxPhases && chainable(plan.steps[e])) ++e;
+        plan.steps[s].chain_len = e - s;
+        for (int i = s + 1; i < e; ++i) plan.steps[i].chain_member = true;
+        s = e;
+    }
 }
 
 void build_plan(Plan& plan, const std::vector<bool>& donated) {
@@ -693,6 +714,62 @@ void build_plan(Plan& plan, const std::vector<bool>& donated) {
 // ------------------------------------------------------------------------------ execution
 static inline const void* src_ptr(const Step& st, const ExecCtx& cx, size_t i) {
     return st.src[i] >= 0 ? cx.ptr[st.src[i]] : (const void*)(cx.consts + st.src_const[i]);
+}
+
+// One persistent launch for the steps [st, st + chain_len): builds the phase table from the resolved
+// pointers, fetches its cached device copy and launches.  false: the caller runs the steps one by one
+// (cx.chain is cleared so the members run too).
+static bool run_chain(const Plan& plan, const Step& head, ExecCtx& cx) {
+    std::vector<k::ChainPhase> phases((size_t)head.chain_len);
+    int max_kw = 0;
+    int64_t bytes = 0;
+    for (int i = 0; i < head.chain_len; ++i) {
+        const Step& st = (&head)[i];
+        const Instr& in = st.in;
+        const Spec& x = plan.values[st.src[0]].spec;
+        const Spec& w = plan.values[st.src[1]].spec;
+        const bool dual = in.act == 2;
+        k::ChainPhase& p = phases[(size_t)i];
+        p = k::ChainPhase{};
+        if (!k::chain_fill_phase(p, x.dims[1], w.dims[1], dual)) { cx.chain = false; return false; }
+        BufferP wc = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], 2, x.dtype, x.dims[1], w.dims[1],
+                                            dual ? cx.input_bufs[st.tiled_w2_input] : nullptr);
+        p.w = wc->ptr;
+        p.x = src_ptr(st, cx, 0);
+        size_t oi = dual ? 3 : 2;
+        if (in.has_bias) { p.bias = src_ptr(st, cx, oi++); p.flags |= k::kChainBias; }
+        if (in.has_residual) { p.residual = src_ptr(st, cx, oi++); p.flags |= k::kChainResidual; }
+        if (in.norm) { p.gamma = src_ptr(st, cx, oi++); p.inv_n = in.scale; p.eps = in.eps; p.flags |= k::kChainNorm; }
+        if (in.act == 1) p.flags |= k::kChainGelu;
+        p.y = cx.ptr[st.dst[0]];
+        if (((uintptr_t)p.x | (uintptr_t)p.y | (uintptr_t)p.residual | (uintptr_t)p.bias | (uintptr_t)p.gamma) & 7)
+            fail_exec("decode chain: operand buffers must be 8-byte aligned");
+        max_kw = std::max(max_kw, p.Kw);
+        bytes += (int64_t)dtype_size(x.dtype) * (x.dims[1] + x.dims[1] * w.dims[1] * (dual ? 2 : 1) + w.dims[1]);
+    }
+    const k::ChainPhase* table = cx.be->chain_table(phases);
+    if (!table) { cx.chain = false; return false; }
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (cx.profile) {
+        GPTRS_HIP_CHECK(hipEventCreate(&e0));
+        GPTRS_HIP_CHECK(hipEventCreate(&e1));
+        GPTRS_HIP_CHECK(hipEventRecord(e0, cx.stream));
+    }
+    if (!k::chain_launch(cx.stream, table, head.chain_len, max_kw, cx.be->chain_barrier(), cx.be->chain_abort_flag())) {
+        if (e0) { (void)hipEventDestroy(e0); (void)hipEventDestroy(e1); }
+        cx.chain = false;
+        return false;
+    }
+    if (cx.profile) {
+        GPTRS_HIP_CHECK(hipEventRecord(e1, cx.stream));
+        cx.be->prof_events.emplace_back(e0, e1);
+        ++cx.be->prof_linear_calls;
+        cx.be->prof_linear_bytes += bytes;
+    }
+    ++cx.be->n_chain_launches;
+    cx.be->n_chain_phases += head.chain_len;
+    ++cx.launches;
+    return true;
 }
 
 void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
@@ -817,6 +894,8 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
             ++cx.launches;
             break;
         case OpKind::FLinear: {
+            if (cx.chain && st.chain_member) break;  // executed by the launch of the run's first step
+            if (cx.chain && st.chain_len > 0 && run_chain(plan, st, cx)) break;
             const Spec& x = in_spec(0);
             const Spec& w = in_spec(1);
             if (in.mfma) {

@@ -98,6 +98,10 @@ struct Step {
     bool copy_base = false;        // DynamicUpdateSlice / FAttnDecode: copy base -> out first
     bool lhs_pack = false, rhs_pack = false;    // Dot: operands repacked into scratch first
     int tiled_w_input = -1, tiled_w2_input = -1;  // FLinear over column-tiled weights: input positions of W, W2
+    // Run of consecutive decode linears executed by ONE persistent launch (kernels_chain.hip): the
+    // first step of the run carries its length, the others are marked as members.
+    int chain_len = 0;
+    bool chain_member = false;
     k::CopyDesc pack_l{}, pack_r{};
     size_t pack_l_off = 0, pack_r_off = 0;
 };
@@ -161,7 +165,15 @@ class Backend {
     // Derived layouts of a weight tensor, built on first use and kept while the source buffer lives
     // (the backend-side memo of derived weight formats).  kind 0: column-tiled copy for the decode
     // GEMV (kernels_gemv_tiled.hip); kind 1: k-grouped copy for the MFMA GEMM (kernels_mfma.hip).
-    BufferP derived_weights(const BufferP& src, int kind, DType dtype, int64_t k, int64_t n);
+    // kind 2: 4-column / k-pair tiled copy for the persistent decode chain (kernels_chain.hip); with
+    // src2 the SwiGLU pair (gate = src, up = src2) interleaved column by column in one copy.
+    BufferP derived_weights(const BufferP& src, int kind, DType dtype, int64_t k, int64_t n, const BufferP& src2 = nullptr);
+    // Device copy of a chain's phase table, cached by content (steady-state decode repeats a few tables).
+    const k::ChainPhase* chain_table(const std::vector<k::ChainPhase>& phases);
+    unsigned* chain_barrier() const { return d_chain_bar_; }
+    int* chain_abort_flag() const { return d_err_flag_ + 1; }
+    bool opt_chain = true;
+    int64_t n_chain_launches = 0, n_chain_phases = 0;
     int64_t n_tiled_built = 0;
     void release_block(void* p, size_t cap) { pool_.release(p, cap); }
 
@@ -200,8 +212,12 @@ class Backend {
     int32_t* d_argmax_idx_ = nullptr;
     int64_t* d_token_ = nullptr;
     void* h_pinned_ = nullptr;  // 64 bytes of pinned host memory for readbacks
-    struct Derived { std::weak_ptr<Buffer> src; BufferP tiled; };
-    std::unordered_map<uint64_t, Derived> tiled_cache_;
+    struct Derived { std::weak_ptr<Buffer> src, src2; BufferP tiled; };
+    std::map<std::array<uint64_t, 3>, Derived> tiled_cache_;
+    unsigned* d_chain_bar_ = nullptr;
+    struct ChainTable { std::vector<k::ChainPhase> host; BufferP dev; uint64_t last_use = 0; };
+    std::vector<ChainTable> chain_tables_;
+    uint64_t chain_clock_ = 0;
     uint64_t next_buffer_id_ = 1;
 };
 
@@ -220,6 +236,7 @@ struct ExecCtx {
     int* counters;
     int64_t launches = 0;
     bool profile = false;
+    bool chain = false;               // run decode linears as persistent chain launches
     std::vector<BufferP> input_bufs;  // per input position
 };
 void run_step(const Plan& plan, const Step& st, ExecCtx& cx);
