@@ -1,5 +1,6 @@
 // Backend implementation and the extern "C" surface declared in include/gptrs_hip.h.
 #include <algorithm>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 
@@ -322,6 +323,12 @@ std::shared_ptr<Plan> Backend::get_plan(const char* json, size_t len, uint64_t k
     }
     ++n_compiled;
     n_fused += plan->fused_ops;
+    if (getenv("GPTRS_HIP_DUMP_PLAN")) {
+        fprintf(stderr, "[gptrs_hip] plan key=%llx: %zu steps\n", (unsigned long long)key, plan->steps.size());
+        for (const Step& st : plan->steps)
+            fprintf(stderr, "  %-22s -> %s%s%s\n", st.in.op_name.c_str(), st.in.out_specs[0].str().c_str(),
+                    st.chain_len ? (" [chain of " + std::to_string(st.chain_len) + "]").c_str() : "", st.chain_member ? " [chain member]" : "");
+    }
     if (key) {
         plan_lru_.emplace_front(k2, plan);
         plan_index_[k2] = plan_lru_.begin();

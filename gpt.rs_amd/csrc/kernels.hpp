@@ -116,15 +116,30 @@ void gemv_tiled(hipStream_t s, const TiledLinearArgs& a);
 // copy), bias, exact-erf GELU, residual.  x, residual and y may be produced by earlier phases of
 // the same launch.
 constexpr int kChainCounters = 16;        // striped arrival counters of the grid barrier
-constexpr int kChainMaxPhases = 64;
+constexpr int kChainMaxPhases = 192;
 constexpr int kChainMaxXsWords = 16384;   // staged activation pairs: K <= 32768
 constexpr size_t kChainBarrierBytes = (kChainCounters * 64 + 64) * sizeof(unsigned);  // zero-initialised once
 enum : int { kChainNorm = 1, kChainDual = 2, kChainGelu = 4, kChainResidual = 8, kChainBias = 16 };
+enum : int { kChainLinear = 0, kChainAttnPartial = 1, kChainAttnCombine = 2 };
+// One phase of a chain.  Linear: y = act(norm?(x) . W + bias) (+ residual).  Decode attention
+// (attention.rs:657-779, T = 1) takes two phases: "partial" appends this step's K/V row and leaves
+// one online-softmax record (max, sum, weighted V) per query head and position chunk in `part`;
+// "combine" merges the records of a head into the context row y.
 struct ChainPhase {
+    int kind, flags;
     const void* w; const void* x; const void* gamma; const void* bias; const void* residual;
     void* y;
-    int K, N, Kw, ntiles, wpt, units, upb, flags;
+    int K, N, Kw, ntiles, wpt, units, upb, lds_bytes;
     float inv_n, eps;
+    // attention: x = packed qkv row [(n_q + 2 n_kv) * head_dim], y = context row [n_q * head_dim]
+    void* k_cache; void* v_cache;              // [n_kv, capacity, head_dim], updated in place
+    const int32_t* update_starts;              // si32[3]
+    const int32_t* query_start;                // si32[1]
+    const void* cos; const void* sin;          // RoPE rows of this position, or null (qkv already rotated)
+    float* part;                               // [n_q][nch][head_dim + 2] f32
+    int n_q, n_kv, head_dim, capacity, rot_half, nch;
+    float scale;
+    int pad;
 };
 int chain_grid();  // workgroups per launch (one per CU), 0 when no device is current
 bool chain_supported(int dtype, int64_t m, int64_t k, int64_t n, bool dual, bool norm);
@@ -134,9 +149,15 @@ void chain_pack_weights(hipStream_t s, const void* w, const void* w2, void* out,
 // fills K, N, Kw, ntiles, wpt, units, upb (and the dual flag); false when one workgroup would own
 // more bias/residual columns than the kernel stages
 bool chain_fill_phase(ChainPhase& p, int64_t k, int64_t n, bool dual);
+// Decode attention inside a chain: supported shapes, scratch for the per-chunk records, and the
+// two phases (shape fields filled; the caller sets the pointers of both).
+bool chain_attn_supported(int dtype, int64_t t, int64_t n_q, int64_t n_kv, int64_t head_dim, int64_t rot_half);
+size_t chain_attn_part_bytes(int64_t n_q, int64_t n_kv, int64_t head_dim);
+void chain_fill_attn(ChainPhase& partial, ChainPhase& combine, int64_t n_q, int64_t n_kv, int64_t head_dim, int64_t capacity,
+                     int64_t rot_half, float scale);
 // bar: kChainBarrierBytes of device memory zeroed once; abort_flag: raised when a barrier wait
 // gives up (every wave then leaves the kernel).  false: launch not possible (caller falls back).
-bool chain_launch(hipStream_t s, const ChainPhase* dev_table, int nphases, int max_kw, unsigned* bar, int* abort_flag);
+bool chain_launch(hipStream_t s, const ChainPhase* dev_table, int nphases, int lds_bytes, unsigned* bar, int* abort_flag);
 
 // Prefill GEMM (M > 16, bf16) on the matrix cores over a k-grouped copy of the weights,
 // Wk8[K/8][Npad][8] (kernels_mfma.hip).  wk2 != nullptr: SwiGLU pair.

@@ -18,9 +18,15 @@
 //     L2 write-back / invalidate is needed between phases; a phase's input vector is staged into
 //     LDS by all 9 waves together right after the barrier (RMSNorm statistics included).
 //
+// Decode attention (T = 1 over the KV cache) runs inside the same launch as two more phase kinds,
+// executed by all 9 waves of a workgroup together: "partial" (one workgroup per kv head and
+// position chunk: append this step's K/V row, online softmax over the chunk for the query heads
+// of the group) and "combine" (one workgroup per query head merges the chunk records).
+//
 // Every wait is bounded: a barrier that does not complete raises the abort flag, every wave
 // leaves the kernel, and the host reports an execution error.
 #include <algorithm>
+#include <cstdlib>
 
 #include "kernels.hpp"
 #include "device_utils.hpp"
@@ -48,22 +54,38 @@ template <typename T> __device__ __forceinline__ T* uni_ptr(T* p) {
     const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(v >> 32));
     return (T*)(((unsigned long long)hi << 32) | lo);
 }
+// Pointers read out of the phase table are generic to the compiler; every access goes through an
+// explicit global-address-space pointer so it becomes a global_* instruction.  (A flat access counts
+// on the LDS counter too, and a wait for an LDS read would then also wait for every weight load in
+// flight.)
+#define GPTRS_GLOBAL __attribute__((address_space(1)))
+#define GPTRS_LDS __attribute__((address_space(3)))
+template <typename T> __device__ __forceinline__ const GPTRS_GLOBAL T* as_global(const T* p) { return (const GPTRS_GLOBAL T*)p; }
+template <typename T> __device__ __forceinline__ GPTRS_GLOBAL T* as_global(T* p) { return (GPTRS_GLOBAL T*)p; }
+template <typename T> __device__ __forceinline__ T gload(const T* p) { return *as_global(p); }   // scalar T
+template <typename T> __device__ __forceinline__ void gstore(T* p, const T& v) { *as_global(p) = v; }
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint2 gload2(const void* p) { const u32x2 v = *(const GPTRS_GLOBAL u32x2*)p; return make_uint2(v.x, v.y); }
+__device__ __forceinline__ uint4 gload4(const void* p) { const u32x4 v = *(const GPTRS_GLOBAL u32x4*)p; return make_uint4(v.x, v.y, v.z, v.w); }
+__device__ __forceinline__ void gstore4(void* p, const uint4& v) { u32x4 w; w.x = v.x; w.y = v.y; w.z = v.z; w.w = v.w; *(GPTRS_GLOBAL u32x4*)p = w; }
 // agent-scope accesses: coherent across the XCDs' L2s without cache maintenance
 __device__ __forceinline__ unsigned long long cload8(const void* p) {
-    return __hip_atomic_load((const unsigned long long*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return __hip_atomic_load(as_global((const unsigned long long*)p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ unsigned cload4(const void* p) {
-    return __hip_atomic_load((const unsigned*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return __hip_atomic_load(as_global((const unsigned*)p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ void cstore8(void* p, unsigned long long v) {
-    __hip_atomic_store((unsigned long long*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(as_global((unsigned long long*)p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ void cstore4(void* p, unsigned v) {
-    __hip_atomic_store((unsigned*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(as_global((unsigned*)p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ float rbf(float v) { return bf16_to_f32(f32_to_bf16(v)); }
-__device__ __forceinline__ int lds_ld(const int* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
-__device__ __forceinline__ void lds_st(int* p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
+template <typename P> __device__ __forceinline__ int lds_ld(P p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
+template <typename P> __device__ __forceinline__ void lds_st(P p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
 #define GPTRS_LDS_RELEASE() __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local")
 #define GPTRS_LDS_ACQUIRE() __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local")
 // workgroup barrier that waits for LDS traffic only: outstanding weight loads stay in flight
@@ -71,6 +93,17 @@ __device__ __forceinline__ void lds_barrier() {
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
 }
+
+#ifdef GPTRS_CHAIN_STAMPS
+__device__ unsigned long long* g_chain_stamps = nullptr;   // lab builds: [phase][8] wall-clock stamps of workgroup 0
+#define GPTRS_STAMP(i) do { if (g_chain_stamps && blockIdx.x == 0 && (threadIdx.x & 63) == 0) g_chain_stamps[ph * 16 + (i)] = wall_clock64(); } while (0)
+#define GPTRS_STAMP_W0(i) do { if (g_chain_stamps && blockIdx.x == 0 && threadIdx.x == 0) g_chain_stamps[phase * 16 + (i)] = wall_clock64(); } while (0)
+#define GPTRS_STAMP_C(i) do { if (g_chain_stamps && blockIdx.x == 0 && threadIdx.x == NS) g_chain_stamps[phase * 16 + (i)] = wall_clock64(); } while (0)
+#else
+#define GPTRS_STAMP(i) do { } while (0)
+#define GPTRS_STAMP_W0(i) do { } while (0)
+#define GPTRS_STAMP_C(i) do { } while (0)
+#endif
 
 struct Shared {
     float red[NSLOT][NWS][16];
@@ -99,7 +132,7 @@ __device__ void stage_block(const ChainPhase& P, unsigned* xs, float* ssq) {
         for (int u = 0; u < MAXI; ++u) {
             const int i = u * NT + t;
             v[u] = i < n ? cload8(x + 8 * (size_t)i) : 0ull;
-            gg[u] = i < n ? g[i] : make_uint2(0u, 0u);
+            gg[u] = i < n ? gload2(g + i) : make_uint2(0u, 0u);
         }
         float q = 0.f;
 #pragma unroll
@@ -143,6 +176,358 @@ __device__ void stage_block(const ChainPhase& P, unsigned* xs, float* ssq) {
     lds_barrier();
 }
 
+
+// ---------------------------------------------------------------------------- decode attention
+constexpr int NW = NT / 64;
+
+__device__ __forceinline__ void unpack8(unsigned long long a, unsigned long long b, float (&o)[8]) {
+    const unsigned a0 = (unsigned)a, a1 = (unsigned)(a >> 32), b0 = (unsigned)b, b1 = (unsigned)(b >> 32);
+    o[0] = bf16lo(a0); o[1] = bf16hi(a0); o[2] = bf16lo(a1); o[3] = bf16hi(a1);
+    o[4] = bf16lo(b0); o[5] = bf16hi(b0); o[6] = bf16lo(b1); o[7] = bf16hi(b1);
+}
+// 8 consecutive bf16: coherent (written earlier in this launch) / plain (older than the launch)
+__device__ __forceinline__ void cload_bf16x8(const bf16_t* p, float (&o)[8]) { unpack8(cload8(p), cload8(p + 4), o); }
+__device__ __forceinline__ void load_bf16x8(const bf16_t* p, float (&o)[8]) {
+    const uint4 v = gload4(p);
+    o[0] = bf16lo(v.x); o[1] = bf16hi(v.x); o[2] = bf16lo(v.y); o[3] = bf16hi(v.y);
+    o[4] = bf16lo(v.z); o[5] = bf16hi(v.z); o[6] = bf16lo(v.w); o[7] = bf16hi(v.w);
+}
+// Rotate-half RoPE (ops/functional/rotary.rs:430-536) while loading dims [c0, c0+8) of one head of
+// the packed projection: dims below `half` pair with dim+half, the next `half` dims with dim-half,
+// the rest pass through; the result is rounded to bf16 like a stored post-RoPE row.
+__device__ __forceinline__ void cload_roped(const bf16_t* head, int c0, int half, const bf16_t* cs, const bf16_t* sn, float (&out)[8]) {
+    float own[8];
+    cload_bf16x8(head + c0, own);
+    if (cs == nullptr || c0 >= 2 * half) {
+#pragma unroll
+        for (int v = 0; v < 8; ++v) out[v] = own[v];
+        return;
+    }
+    const bool first = c0 < half;
+    float other[8], c[8], sv[8];
+    cload_bf16x8(head + (first ? c0 + half : c0 - half), other);
+    const int j0 = first ? c0 : c0 - half;
+    load_bf16x8(cs + j0, c);
+    load_bf16x8(sn + j0, sv);
+#pragma unroll
+    for (int v = 0; v < 8; ++v) out[v] = rbf(first ? own[v] * c[v] - other[v] * sv[v] : own[v] * c[v] + other[v] * sv[v]);
+}
+__device__ __forceinline__ long clampl(long v, long lo, long hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+__device__ __forceinline__ void unpack_u4(const uint4& v, float (&o)[8]) {
+    o[0] = bf16lo(v.x); o[1] = bf16hi(v.x); o[2] = bf16lo(v.y); o[3] = bf16hi(v.y);
+    o[4] = bf16lo(v.z); o[5] = bf16hi(v.z); o[6] = bf16lo(v.w); o[7] = bf16hi(v.w);
+}
+// streaming waves wait here until the control wave has seen the grid barrier of `phase`
+template <typename IP>
+__device__ __forceinline__ bool wait_go(IP go, IP abort, int phase) {
+    unsigned spins = 0;
+    while (uni(lds_ld(go)) < phase) {
+        __builtin_amdgcn_s_sleep(1);
+        if (uni(lds_ld(abort)) || ++spins > (1u << 24)) return false;
+    }
+    return true;
+}
+
+// exp through v_exp_f32 (2^x): softmax weights only, about one ulp, exp(-inf) = 0
+__device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896f); }
+// sum over the lpr (8, 16 or 32) consecutive lanes of a lane group, result in each of them
+__device__ __forceinline__ float group_sum(float v, int lpr) {
+    int x = __float_as_int(v);
+#define GPTRS_DPP_ADD(ctrl) x = __float_as_int(__int_as_float(x) + __int_as_float(__builtin_amdgcn_update_dpp(0, x, (ctrl), 0xf, 0xf, false)))
+    GPTRS_DPP_ADD(0xB1);    // quad_perm [1,0,3,2]
+    GPTRS_DPP_ADD(0x4E);    // quad_perm [2,3,0,1]
+    GPTRS_DPP_ADD(0x141);   // row_half_mirror: 8 lanes
+    if (lpr >= 16) GPTRS_DPP_ADD(0x140);  // row_mirror: 16 lanes
+#undef GPTRS_DPP_ADD
+    float r = __int_as_float(x);
+    if (lpr == 32) {
+        const u32x2 sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(r), __float_as_uint(r), false, false);
+        r = __uint_as_float(sw.x) + __uint_as_float(sw.y);
+    }
+    return r;
+}
+// the values of v held by this lane and by its partner lane ^ off (off = 8, 16 or 32), in an order
+// that is the same for both partners of a pair up to a swap: for symmetric merges only
+__device__ __forceinline__ void lane_pair(float v, int off, float& a, float& b) {
+    if (off == 8) {
+        a = v;
+        b = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xf, 0xf, false));  // row_ror:8
+    } else if (off == 16) {
+        const u32x2 sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        a = __uint_as_float(sw.x); b = __uint_as_float(sw.y);
+    } else {
+        const u32x2 sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+        a = __uint_as_float(sw.x); b = __uint_as_float(sw.y);
+    }
+}
+
+// unit = kv head * nch + chunk.  Each of the 8 streaming waves serves ONE query head of the kv
+// head's group (wave w: head w % G, position subset w / G of 8 / G), so a lane carries a single
+// online-softmax state; a cache row (head_dim bf16) is read by head_dim/8 lanes, 16 bytes each, and
+// the waves of different heads re-read the same rows out of the caches.  Cache rows older than
+// this launch are requested BEFORE the grid barrier is awaited (they do not depend on the
+// previous phase); only the query row and this step's K/V row are read after it.
+__device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const ChainPhase& P, GPTRS_LDS float* lds, int unit, int phase) {
+    constexpr int PP = 3;   // positions per lane group requested ahead of the barrier
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const bool control = wave == NWS;
+    const int dh = P.head_dim, n_q = P.n_q, n_kv = P.n_kv, nch = P.nch, half = P.rot_half;
+    const int G = n_q / n_kv, nparts = NWS / G;
+    const long cap = P.capacity;
+    const int lpr = dh >> 3, rpw = 64 / lpr, sub = lane / lpr, li = lane % lpr;
+    const int g = wave % G, part = wave / G;
+    const int stride = nparts * rpw, sid = part * rpw + sub;   // position slots of this head's waves
+    const int kvh = unit / nch, c = unit - kvh * nch;
+    const bf16_t* qkv = (const bf16_t*)P.x;
+    bf16_t* kc = (bf16_t*)P.k_cache;
+    bf16_t* vc = (bf16_t*)P.v_cache;
+    const bf16_t* cs = (const bf16_t*)P.cos;
+    const bf16_t* sn = (const bf16_t*)P.sin;
+    const long qpos = clampl(uni(gload(P.query_start)), 0, cap - 1);       // DynamicSlice clamp (cpu.rs:804-820)
+    const long upd = clampl(uni(gload(P.update_starts + 1)), 0, cap - 1);  // DynamicUpdateSlice clamp
+    const float scale = P.scale;
+    const long L = qpos + 1, CL = (L + nch - 1) / nch;
+    const long p0 = c * CL, p1 = min(L, p0 + CL);
+    const int owner = (int)min(upd / CL, (long)nch - 1);
+    const bf16_t* knew = qkv + (long)n_q * dh + (long)kvh * dh;
+    const bf16_t* vnew = qkv + (long)(n_q + n_kv) * dh + (long)kvh * dh;
+    const int c0 = li * 8;
+
+    GPTRS_STAMP_W0(8);
+    uint4 kraw[PP], vraw[PP];
+#pragma unroll
+    for (int j = 0; j < PP; ++j) {
+        const long p = p0 + sid + (long)j * stride;
+        if (!control && p < p1 && p != upd) {
+            const long row = ((long)kvh * cap + p) * dh + c0;
+            kraw[j] = gload4(kc + row);
+            vraw[j] = gload4(vc + row);
+        } else {
+            kraw[j] = make_uint4(0, 0, 0, 0);
+            vraw[j] = make_uint4(0, 0, 0, 0);
+        }
+    }
+    GPTRS_STAMP_W0(9);
+    if (!control && !wait_go(go, abort, phase)) return false;
+    GPTRS_STAMP_W0(10);
+
+    float m = -INFINITY, l = 0.f, o[8];
+#pragma unroll
+    for (int v = 0; v < 8; ++v) o[v] = 0.f;
+    if (!control) {
+        // the wave's query head (RoPE applied on the fly) and, in the first lane group of each head's
+        // first wave of the workgroup that owns position `upd`, this step's K/V row: all requested
+        // before any is consumed
+        const bool rot = cs != nullptr && c0 < 2 * half;
+        const bool first = c0 < half;
+        const int j0 = first ? c0 : c0 - half, co = first ? c0 + half : c0 - half;
+        float cosv[8], sinv[8];
+        if (rot) { load_bf16x8(cs + j0, cosv); load_bf16x8(sn + j0, sinv); }
+        const bf16_t* head = qkv + (long)(kvh * G + g) * dh;
+        unsigned long long qa[2], qb[2] = {0ull, 0ull};
+        qa[0] = cload8(head + c0); qa[1] = cload8(head + c0 + 4);
+        if (rot) { qb[0] = cload8(head + co); qb[1] = cload8(head + co + 4); }
+        const bool fresh = c == owner && sid == 0;           // this lane group handles the new row
+        unsigned long long ka[2] = {0ull, 0ull}, kb[2] = {0ull, 0ull}, va[2] = {0ull, 0ull};
+        if (fresh) {
+            ka[0] = cload8(knew + c0); ka[1] = cload8(knew + c0 + 4);
+            if (rot) { kb[0] = cload8(knew + co); kb[1] = cload8(knew + co + 4); }
+            va[0] = cload8(vnew + c0); va[1] = cload8(vnew + c0 + 4);
+        }
+        auto rope = [&](const unsigned long long (&own2)[2], const unsigned long long (&oth2)[2], float (&out)[8]) {
+            float own[8], other[8];
+            unpack8(own2[0], own2[1], own);
+            if (!rot) {
+#pragma unroll
+                for (int v = 0; v < 8; ++v) out[v] = own[v];
+                return;
+            }
+            unpack8(oth2[0], oth2[1], other);
+#pragma unroll
+            for (int v = 0; v < 8; ++v)
+                out[v] = rbf(first ? own[v] * cosv[v] - other[v] * sinv[v] : own[v] * cosv[v] + other[v] * sinv[v]);
+        };
+        float qf[8];
+        rope(qa, qb, qf);
+        GPTRS_STAMP_W0(11);
+
+        auto visit = [&](const float (&kf)[8], const float (&vf)[8]) {
+            float sc = 0.f;
+#pragma unroll
+            for (int v = 0; v < 8; ++v) sc += qf[v] * kf[v];
+            sc = group_sum(sc, lpr) * scale;
+            const float mn = fmaxf(m, sc);
+            const float corr = fast_exp(m - mn);
+            const float pe = fast_exp(sc - mn);
+            l = l * corr + pe;
+#pragma unroll
+            for (int v = 0; v < 8; ++v) o[v] = o[v] * corr + pe * vf[v];
+            m = mn;
+        };
+#pragma unroll
+        for (int j = 0; j < PP; ++j) {
+            const long p = p0 + sid + (long)j * stride;
+            if (p < p1 && p != upd) {
+                float kf[8], vf[8];
+                unpack_u4(kraw[j], kf);
+                unpack_u4(vraw[j], vf);
+                visit(kf, vf);
+            }
+        }
+        for (long p = p0 + sid + (long)PP * stride; p < p1; p += stride) {
+            if (p == upd) continue;
+            float kf[8], vf[8];
+            const long row = ((long)kvh * cap + p) * dh + c0;
+            load_bf16x8(kc + row, kf);
+            load_bf16x8(vc + row, vf);
+            visit(kf, vf);
+        }
+        if (fresh) {   // this step's row: attended to when in range; appended once (by head 0's wave)
+            float kf[8], vf[8];
+            rope(ka, kb, kf);
+            unpack8(va[0], va[1], vf);
+            if (g == 0) {
+                const long row = ((long)kvh * cap + upd) * dh + c0;
+                gstore4(kc + row, make_uint4(pack_bf16x2(kf[0], kf[1]), pack_bf16x2(kf[2], kf[3]), pack_bf16x2(kf[4], kf[5]), pack_bf16x2(kf[6], kf[7])));
+                gstore4(vc + row, make_uint4((unsigned)va[0], (unsigned)(va[0] >> 32), (unsigned)va[1], (unsigned)(va[1] >> 32)));
+            }
+            if (upd >= p0 && upd < p1) visit(kf, vf);
+        }
+        GPTRS_STAMP_W0(12);
+        // merge the lane groups of this wave
+        for (int off = lpr; off < 64; off <<= 1) {
+            float ma, mb, la, lb;
+            lane_pair(m, off, ma, mb);
+            lane_pair(l, off, la, lb);
+            const float mn = fmaxf(ma, mb);
+            const float ca = mn == -INFINITY ? 0.f : fast_exp(ma - mn);
+            const float cb = mn == -INFINITY ? 0.f : fast_exp(mb - mn);
+            l = la * ca + lb * cb;
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                float oa, ob;
+                lane_pair(o[v], off, oa, ob);
+                o[v] = oa * ca + ob * cb;
+            }
+            m = mn;
+        }
+    }
+    // merge the waves of each head through LDS and leave one record per query head
+    GPTRS_LDS float* sm = lds;
+    GPTRS_LDS float* sl = lds + NWS;
+    GPTRS_LDS float* so = lds + 2 * NWS;
+    if (!control && sub == 0) {
+        if (li == 0) { sm[wave] = m; sl[wave] = l; }
+#pragma unroll
+        for (int v = 0; v < 8; ++v) so[wave * dh + c0 + v] = o[v];
+    }
+    GPTRS_STAMP_W0(13);
+    lds_barrier();
+    GPTRS_STAMP_W0(14);
+    GPTRS_STAMP_C(6);
+    float* partp = P.part;
+    for (int idx = t; idx < G * dh; idx += NT) {
+        const int gg = idx / dh, d = idx - gg * dh;
+        float mn = -INFINITY;
+        for (int w = gg; w < NWS; w += G) mn = fmaxf(mn, sm[w]);
+        float Ls = 0.f, O = 0.f;
+        if (mn != -INFINITY) {
+            for (int w = gg; w < NWS; w += G) {
+                const float cw = fast_exp(sm[w] - mn);
+                Ls += sl[w] * cw;
+                O += so[w * dh + d] * cw;
+            }
+        }
+        float* rec = partp + ((long)(kvh * G + gg) * nch + c) * (dh + 2);
+        if (d == 0) { cstore4(rec, __float_as_uint(mn)); cstore4(rec + 1, __float_as_uint(Ls)); }
+        cstore4(rec + 2 + d, __float_as_uint(O));
+    }
+    GPTRS_STAMP_W0(15);
+    lds_barrier();
+    GPTRS_STAMP_C(7);
+    return true;
+}
+
+// unit = query head: softmax-merge of its nch chunk records into the context row.  Thread
+// (sg, d2) reads the records of the chunks s = sg, sg + NW, ... for the dims (2 d2, 2 d2 + 1) in
+// one round of loads and merges them locally; the NW subsets meet in LDS.
+__device__ bool attn_combine(GPTRS_LDS int* go, GPTRS_LDS int* abort, const ChainPhase& P, GPTRS_LDS float* lds, int hq, int phase) {
+    constexpr int MAXC = 8;   // chunks per thread: nch <= MAXC * NW
+    const int t = threadIdx.x, wave = t >> 6;
+    const int dh = P.head_dim, nch = P.nch;
+    if (wave != NWS && !wait_go(go, abort, phase)) return false;
+    const float* base = P.part + (long)hq * nch * (dh + 2);
+    bf16_t* ctx = (bf16_t*)P.y;
+    const int h2 = dh / 2;
+    for (int d0 = 0; d0 < h2; d0 += 64) {
+        const int d2 = d0 + (t & 63);
+        const bool act = d2 < h2;
+        unsigned long long ml[MAXC], ov[MAXC];
+#pragma unroll
+        for (int u = 0; u < MAXC; ++u) {
+            const int s = wave + u * NW;
+            const bool ok = act && s < nch;
+            ml[u] = ok ? cload8(base + (long)s * (dh + 2)) : 0ull;
+            ov[u] = ok ? cload8(base + (long)s * (dh + 2) + 2 + 2 * d2) : 0ull;
+        }
+        float mn = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < MAXC; ++u)
+            if (wave + u * NW < nch) mn = fmaxf(mn, __uint_as_float((unsigned)ml[u]));
+        float Ls = 0.f, o0 = 0.f, o1 = 0.f;
+#pragma unroll
+        for (int u = 0; u < MAXC; ++u) {
+            if (wave + u * NW < nch) {
+                const float ms = __uint_as_float((unsigned)ml[u]);
+                const float cw = ms == -INFINITY ? 0.f : fast_exp(ms - mn);
+                Ls += __uint_as_float((unsigned)(ml[u] >> 32)) * cw;
+                o0 += __uint_as_float((unsigned)ov[u]) * cw;
+                o1 += __uint_as_float((unsigned)(ov[u] >> 32)) * cw;
+            }
+        }
+        GPTRS_LDS f32x4* rec = (GPTRS_LDS f32x4*)lds;
+        { f32x4 r4; r4.x = mn; r4.y = Ls; r4.z = o0; r4.w = o1; rec[wave * 64 + (t & 63)] = r4; }
+        lds_barrier();
+        if (wave == 0 && act) {
+            float M = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) M = fmaxf(M, rec[w * 64 + t].x);
+            float Lt = 0.f, a0 = 0.f, a1 = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) {
+                const f32x4 r = rec[w * 64 + t];
+                const float cw = r.x == -INFINITY ? 0.f : fast_exp(r.x - M);
+                Lt += r.y * cw; a0 += r.z * cw; a1 += r.w * cw;
+            }
+            cstore4(ctx + (long)hq * dh + 2 * d2, pack_bf16x2(a0 / Lt, a1 / Lt));
+        }
+        lds_barrier();
+    }
+    return true;
+}
+
+// All waves of the workgroup: the units blk, blk + grid, ... of an attention phase.  Kept out of
+// line (its register needs must not leak into the streaming loop); the LDS operands travel as
+// explicit local-address-space pointers so their accesses stay ds_* instructions.
+__device__ __forceinline__ bool run_attn_phase(GPTRS_LDS const ChainPhase* php, GPTRS_LDS float* lds, GPTRS_LDS int* go, GPTRS_LDS int* abort, int phase) {
+    ChainPhase P;
+    {
+        int* dst = reinterpret_cast<int*>(&P);
+        GPTRS_LDS const int* src = (GPTRS_LDS const int*)php;
+#pragma unroll
+        for (int i = 0; i < (int)(sizeof(ChainPhase) / 4); ++i) dst[i] = uni(src[i]);
+    }
+    const int kind = P.kind, units = P.units;
+    for (int u = blockIdx.x; u < units; u += gridDim.x) {
+        bool ok;
+        if (kind == kChainAttnCombine) ok = attn_combine(go, abort, P, lds, u, phase);
+        else ok = attn_partial(go, abort, P, lds, u, phase);
+        if (!ok) return false;
+    }
+    return true;
+}
+
 // ---------------------------------------------------------------------------- control wave
 __device__ __forceinline__ float finish(float v, int flags, float bias, float res) {
     if (flags & kChainBias) v += bias;                                           // tensor_ops.rs:42-56
@@ -154,31 +539,40 @@ __device__ __forceinline__ float finish(float v, int flags, float bias, float re
 __device__ void control_wave(Shared& sh, unsigned* xs, int nphases, unsigned* bar, int* abort_flag) {
     const int lane = threadIdx.x & 63;
     const int blk = blockIdx.x, per = gridDim.x / NC;
-    const unsigned epoch = bar[NC * 64];   // written by the previous launch, stable during this one
+    const unsigned epoch = gload(bar + NC * 64);   // written by the previous launch, stable during this one
     int ucount = 0;
     for (int ph = 0; ph < nphases; ++ph) {
         const ChainPhase& P = sh.ph[ph];
+        const int kind = uni(P.kind);
         const int upb = uni(P.upb), units = uni(P.units);
-        const int u0 = blk * upb, u1 = min(u0 + upb, units);
+        const int u0 = kind == kChainLinear ? blk * upb : 0;
+        const int u1 = kind == kChainLinear ? min(u0 + upb, units) : 0;
+        GPTRS_STAMP(0);
         if (ph > 0) {
             const unsigned target = epoch + (unsigned)ph * per;
             unsigned spins = 0;
             bool ok = true;
             for (;;) {
-                const unsigned v = lane < NC ? __hip_atomic_load(bar + lane * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : target;
+                const unsigned v = lane < NC ? __hip_atomic_load(as_global(bar) + lane * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : target;
                 if (__builtin_amdgcn_ballot_w64((int)(v - target) < 0) == 0) break;
                 __builtin_amdgcn_s_sleep(1);
                 if ((++spins & 63u) == 0) {
-                    if (__hip_atomic_load(abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) || spins > (1u << 19)) { ok = false; break; }
+                    if (__hip_atomic_load(as_global(abort_flag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) || spins > (1u << 19)) { ok = false; break; }
                 }
             }
             if (!ok) {
-                __hip_atomic_store(abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(as_global(abort_flag), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 lds_st(&sh.abort, 1);
                 return;
             }
         }
-        if (u0 < u1) {
+        GPTRS_STAMP(1);
+        if (kind != kChainLinear) {
+            if (blk < units) {
+                if (lane == 0) lds_st(&sh.go, ph);
+                run_attn_phase((GPTRS_LDS const ChainPhase*)&sh.ph[ph], (GPTRS_LDS float*)xs, (GPTRS_LDS int*)&sh.go, (GPTRS_LDS int*)&sh.abort, ph);
+            }
+        } else if (u0 < u1) {
             const int flags = uni(P.flags), ntiles = uni(P.ntiles), N = uni(P.N);
             const bool dual = flags & kChainDual;
             const int cpt = dual ? 2 : 4;              // output columns per tile
@@ -192,13 +586,14 @@ __device__ void control_wave(Shared& sh, unsigned* xs, int nphases, unsigned* ba
             if (bias || resid) {
                 for (int i = lane * 2; i < ncols; i += 128) {
                     const int col = col0 + i;
-                    const unsigned bw = (bias && col < N) ? bias[col >> 1] : 0u;
+                    const unsigned bw = (bias && col < N) ? gload(bias + (col >> 1)) : 0u;
                     const unsigned rw = (resid && col < N) ? cload4(resid + 2 * (size_t)col) : 0u;
                     *reinterpret_cast<float2*>(&sh.epi_bias[i]) = make_float2(bf16lo(bw), bf16hi(bw));
                     *reinterpret_cast<float2*>(&sh.epi_res[i]) = make_float2(bf16lo(rw), bf16hi(rw));
                 }
             }
             stage_block(P, xs, sh.ssq);
+            GPTRS_STAMP(2);
             char* out = (char*)uni_ptr(P.y);
             for (int u = u0; u < u1; ++u, ++ucount) {
                 const int slot = ucount % NSLOT;
@@ -207,7 +602,7 @@ __device__ void control_wave(Shared& sh, unsigned* xs, int nphases, unsigned* ba
                     __builtin_amdgcn_s_sleep(1);
                     if (++spins > (1u << 24)) {
                         lds_st(&sh.abort, 1);
-                        __hip_atomic_store(abort_flag, 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        __hip_atomic_store(as_global(abort_flag), 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                         return;
                     }
                 }
@@ -239,13 +634,15 @@ __device__ void control_wave(Shared& sh, unsigned* xs, int nphases, unsigned* ba
                 }
             }
         }
+        GPTRS_STAMP(4);
         // this workgroup's outputs have left the CU before it arrives at the barrier
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         asm volatile("" ::: "memory");
-        if (lane == 0) __hip_atomic_fetch_add(bar + (blk % NC) * 64, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        GPTRS_STAMP(5);
+        if (lane == 0) __hip_atomic_fetch_add(as_global(bar) + (blk % NC) * 64, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     // every launch advances each counter by nphases * per: the next launch starts from there
-    if (blk == 0 && lane == 0) bar[NC * 64] = epoch + (unsigned)nphases * per;
+    if (blk == 0 && lane == 0) gstore(bar + NC * 64, epoch + (unsigned)nphases * per);
 }
 
 // ---------------------------------------------------------------------------- streaming waves
@@ -258,14 +655,14 @@ __device__ void stream_waves(Shared& sh, const unsigned* xs, int nphases) {
     long l_Kw = 0;
     const uint4* l_w = nullptr;
     bool l_active = true;
-    const uint4* l_base[TP];
+    const GPTRS_GLOBAL u32x4* l_base[TP];
 #pragma unroll
     for (int p = 0; p < TP; ++p) l_base[p] = nullptr;
     auto l_setbase = [&]() {
 #pragma unroll
         for (int p = 0; p < TP; ++p) {
             const int tile = min(l_unit * TP + p, l_ntiles - 1);   // a group's last tiles may not exist: re-read, never stored
-            l_base[p] = l_w + (long)tile * l_Kw + t;
+            l_base[p] = (const GPTRS_GLOBAL u32x4*)l_w + (long)tile * l_Kw + t;
         }
         l_j = 0;
     };
@@ -274,6 +671,7 @@ __device__ void stream_waves(Shared& sh, const unsigned* xs, int nphases) {
             ++l_phase;
             if (l_phase >= nphases) { l_active = false; break; }
             const ChainPhase& ph = sh.ph[l_phase];
+            if (uni(ph.kind) != kChainLinear) continue;   // no weights to stream
             const int upb = uni(ph.upb), units = uni(ph.units);
             l_unit = blk * upb;
             l_unit_end = min(l_unit + upb, units);
@@ -284,7 +682,7 @@ __device__ void stream_waves(Shared& sh, const unsigned* xs, int nphases) {
         }
         if (l_active) l_setbase();
     };
-    auto l_fetch = [&](uint4 (&dst)[TP]) {   // requires l_active
+    auto l_fetch = [&](u32x4 (&dst)[TP]) {   // requires l_active
 #pragma unroll
         for (int p = 0; p < TP; ++p) dst[p] = l_base[p][(long)l_j * NS];
         if (++l_j == l_wpt) {
@@ -295,29 +693,31 @@ __device__ void stream_waves(Shared& sh, const unsigned* xs, int nphases) {
 
     // compute iterator
     int c_phase = -1, c_unit = 0, c_unit_end = 0, c_j = 0, c_wpt = 1, ucount = 0;
+    // advance to this workgroup's next linear unit, taking part in attention phases on the way
     auto c_seek = [&]() -> bool {
-        while (c_unit >= c_unit_end) {
+        for (;;) {
             ++c_phase;
             if (c_phase >= nphases) return false;
             const ChainPhase& ph = sh.ph[c_phase];
-            const int upb = uni(ph.upb), units = uni(ph.units);
+            const int units = uni(ph.units);
+            if (uni(ph.kind) != kChainLinear) {
+                if (blk >= units) continue;
+                if (!run_attn_phase((GPTRS_LDS const ChainPhase*)&sh.ph[c_phase], (GPTRS_LDS float*)xs, (GPTRS_LDS int*)&sh.go, (GPTRS_LDS int*)&sh.abort, c_phase)) return false;
+                continue;
+            }
+            const int upb = uni(ph.upb);
             c_unit = blk * upb;
             c_unit_end = min(c_unit + upb, units);
-            if (c_unit < c_unit_end) {
-                c_wpt = uni(ph.wpt);
-                unsigned spins = 0;
-                while (uni(lds_ld(&sh.go)) < c_phase) {
-                    __builtin_amdgcn_s_sleep(1);
-                    if (uni(lds_ld(&sh.abort)) || ++spins > (1u << 24)) return false;
-                }
-                stage_block(sh.ph[c_phase], const_cast<unsigned*>(xs), sh.ssq);
-            }
+            if (c_unit >= c_unit_end) continue;
+            c_wpt = uni(ph.wpt);
+            if (!wait_go(&sh.go, &sh.abort, c_phase)) return false;
+            stage_block(ph, const_cast<unsigned*>(xs), sh.ssq);
+            c_j = 0;
+            return true;
         }
-        c_j = 0;
-        return true;
     };
 
-    uint4 cur[TP], nxt[TP];
+    u32x4 cur[TP], nxt[TP];
     bool have_nxt = false;
     l_seek();
     if (l_active) { l_fetch(nxt); have_nxt = true; }
@@ -335,11 +735,13 @@ __device__ void stream_waves(Shared& sh, const unsigned* xs, int nphases) {
         const bf16x2 xv = __builtin_bit_cast(bf16x2, xs[c_j * NS + t]);
 #pragma unroll
         for (int p = 0; p < TP; ++p) {
-            const uint4 q = cur[p];
-            acc[p][0] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q.x), xv, acc[p][0], false);
-            acc[p][1] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q.y), xv, acc[p][1], false);
-            acc[p][2] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q.z), xv, acc[p][2], false);
-            acc[p][3] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q.w), xv, acc[p][3], false);
+            // element reads go through scalars: __builtin_bit_cast applied directly to `vec.y` of an
+            // ext-vector reads element 0 with this compiler
+            const unsigned q0 = cur[p].x, q1 = cur[p].y, q2 = cur[p].z, q3 = cur[p].w;
+            acc[p][0] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q0), xv, acc[p][0], false);
+            acc[p][1] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q1), xv, acc[p][1], false);
+            acc[p][2] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q2), xv, acc[p][2], false);
+            acc[p][3] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q3), xv, acc[p][3], false);
         }
         if (++c_j == c_wpt) {
             const int slot = ucount % NSLOT;
@@ -456,14 +858,48 @@ bool chain_fill_phase(ChainPhase& p, int64_t k, int64_t n, bool dual) {
     p.wpt = p.Kw / NS;
     p.units = (p.ntiles + TP - 1) / TP;
     p.upb = grid > 0 ? (p.units + grid - 1) / grid : p.units;
+    p.kind = kChainLinear;
+    p.lds_bytes = p.Kw * 4;
     if (dual) p.flags |= kChainDual;
     return (int64_t)p.upb * TP * (dual ? 2 : 4) <= EPI_MAX && p.Kw <= kChainMaxXsWords;
 }
 
-bool chain_launch(hipStream_t s, const ChainPhase* dev_table, int nphases, int max_kw, unsigned* bar, int* abort_flag) {
+bool chain_attn_supported(int dtype, int64_t t, int64_t n_q, int64_t n_kv, int64_t head_dim, int64_t rot_half) {
+    static const bool enabled = [] { const char* e = getenv("GPTRS_HIP_CHAIN_ATTN"); return !(e && e[0] == '0'); }();
+    if (!enabled) return false;   // GPTRS_HIP_CHAIN_ATTN=0: decode attention keeps its stand-alone kernels
+    if (dtype != 2 || t != 1 || n_kv <= 0 || n_q % n_kv != 0) return false;
+    const int64_t g = n_q / n_kv;
+    if (g != 1 && g != 2 && g != 4 && g != 8) return false;
+    if (head_dim != 64 && head_dim != 128 && head_dim != 256) return false;
+    if (rot_half != 0 && (rot_half % 8 != 0 || 2 * rot_half > head_dim)) return false;
+    return chain_grid() > 0;
+}
+static int chain_attn_nch(int64_t n_kv) {
+    const int64_t n = chain_grid() / n_kv;
+    return (int)(n < 1 ? 1 : (n > 64 ? 64 : n));
+}
+size_t chain_attn_part_bytes(int64_t n_q, int64_t n_kv, int64_t head_dim) {
+    return (size_t)n_q * (size_t)chain_attn_nch(n_kv) * (size_t)(head_dim + 2) * sizeof(float);
+}
+void chain_fill_attn(ChainPhase& partial, ChainPhase& combine, int64_t n_q, int64_t n_kv, int64_t head_dim, int64_t capacity,
+                     int64_t rot_half, float scale) {
+    const int nch = chain_attn_nch(n_kv);
+    for (ChainPhase* p : {&partial, &combine}) {
+        p->n_q = (int)n_q; p->n_kv = (int)n_kv; p->head_dim = (int)head_dim; p->capacity = (int)capacity;
+        p->rot_half = (int)rot_half; p->nch = nch; p->scale = scale;
+    }
+    partial.kind = kChainAttnPartial;
+    partial.units = (int)n_kv * nch;
+    partial.lds_bytes = (int)((2 * NWS + NWS * head_dim) * sizeof(float));
+    combine.kind = kChainAttnCombine;
+    combine.units = (int)n_q;
+    combine.lds_bytes = (int)(NW * 64 * sizeof(float4));
+}
+
+bool chain_launch(hipStream_t s, const ChainPhase* dev_table, int nphases, int lds_bytes, unsigned* bar, int* abort_flag) {
     const int grid = chain_grid();
-    if (grid <= 0 || nphases <= 0 || nphases > kChainMaxPhases || max_kw > kChainMaxXsWords) return false;
-    const size_t smem = sizeof(Shared) + (size_t)max_kw * 4;
+    if (grid <= 0 || nphases <= 0 || nphases > kChainMaxPhases || lds_bytes > kChainMaxXsWords * 4) return false;
+    const size_t smem = sizeof(Shared) + (size_t)((lds_bytes + 15) / 16 * 16);
     if (smem > g_smem_set) {
         const size_t want = sizeof(Shared) + (size_t)kChainMaxXsWords * 4;
         if (hipFuncSetAttribute((const void*)chain_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)want) != hipSuccess) return false;

@@ -503,7 +503,8 @@ void Builder::describe(Step& st) {
         }
         case OpKind::FAttnDecode: {
             const Spec& ck = spec_of(in, 1);
-            st.scratch_bytes = k::attn_decode_workspace_bytes(in.n_q, in.head_dim, ck.dims[1]);
+            st.scratch_bytes = std::max(k::attn_decode_workspace_bytes(in.n_q, in.head_dim, ck.dims[1]),
+                                        k::chain_attn_part_bytes(in.n_q, in.n_kv, in.head_dim));
             break;
         }
         default:
@@ -684,24 +685,38 @@ void Builder::build() {
     }
     plan.workspace_bytes = high;
 
-    // runs of consecutive decode linears -> one persistent launch each
-    auto chainable = [&](const Step& st) {
+    // runs of consecutive decode linears / decode attentions -> one persistent launch each
+    auto chain_phases = [&](const Step& st) -> int {   // phases the step takes in a chain, 0: not chainable
         const Instr& in = st.in;
-        if (in.op != OpKind::FLinear || !in.tiled || st.tiled_w_input < 0) return false;
+        if (in.op == OpKind::FAttnDecode) {
+            const Spec& x = plan.values[st.src[0]].spec;
+            return k::chain_attn_supported((int)x.dtype, x.dims[0], in.n_q, in.n_kv, in.head_dim, in.rot_half) ? 2 : 0;
+        }
+        if (in.op != OpKind::FLinear || !in.tiled || st.tiled_w_input < 0) return 0;
         const Spec& x = plan.values[st.src[0]].spec;
         const Spec& w = plan.values[st.src[1]].spec;
-        if (x.rank() != 2 || w.rank() != 2) return false;
+        if (x.rank() != 2 || w.rank() != 2) return 0;
         const bool dual = in.act == 2;
-        if (!k::chain_supported((int)x.dtype, x.dims[0], x.dims[1], w.dims[1], dual, in.norm)) return false;
+        if (!k::chain_supported((int)x.dtype, x.dims[0], x.dims[1], w.dims[1], dual, in.norm)) return 0;
         k::ChainPhase p{};
-        return k::chain_fill_phase(p, x.dims[1], w.dims[1], dual);
+        return k::chain_fill_phase(p, x.dims[1], w.dims[1], dual) ? 1 : 0;
     };
     for (int s = 0; s < n_steps;) {
-        if (!chainable(plan.steps[s])) { ++s; continue; }
+        int np = chain_phases(plan.steps[s]);
+        if (!np) { ++s; continue; }
         int e = s + 1;
-        while (e < n_steps && e - s < k::kChainMaxPhases && chainable(plan.steps[e])) ++e;
-        plan.steps[s].chain_len = e - s;
-        for (int i = s + 1; i < e; ++i) plan.steps[i].chain_member = true;
+        bool has_linear = plan.steps[s].in.op == OpKind::FLinear;
+        while (e < n_steps) {
+            const int q = chain_phases(plan.steps[e]);
+            if (!q || np + q > k::kChainMaxPhases) break;
+            np += q;
+            has_linear = has_linear || plan.steps[e].in.op == OpKind::FLinear;
+            ++e;
+        }
+        if (has_linear) {   // an attention on its own keeps its stand-alone kernels
+            plan.steps[s].chain_len = e - s;
+            for (int i = s + 1; i < e; ++i) plan.steps[i].chain_member = true;
+        }
         s = e;
     }
 }
@@ -720,17 +735,47 @@ static inline const void* src_ptr(const Step& st, const ExecCtx& cx, size_t i) {
 // pointers, fetches its cached device copy and launches.  false: the caller runs the steps one by one
 // (cx.chain is cleared so the members run too).
 static bool run_chain(const Plan& plan, const Step& head, ExecCtx& cx) {
-    std::vector<k::ChainPhase> phases((size_t)head.chain_len);
-    int max_kw = 0;
+    std::vector<k::ChainPhase> phases;
+    phases.reserve((size_t)head.chain_len * 2);
+    int lds_bytes = 0;
     int64_t bytes = 0;
+    auto aligned8 = [](std::initializer_list<const void*> ps) {
+        for (const void* q : ps) if ((uintptr_t)q & 7) fail_exec("decode chain: operand buffers must be 8-byte aligned");
+    };
     for (int i = 0; i < head.chain_len; ++i) {
         const Step& st = (&head)[i];
         const Instr& in = st.in;
+        if (in.op == OpKind::FAttnDecode) {
+            const Spec& ck = plan.values[st.src[1]].spec;
+            void* kout = cx.ptr[st.dst[1]];
+            void* vout = cx.ptr[st.dst[2]];
+            const void* kin = src_ptr(st, cx, 1);
+            const void* vin = src_ptr(st, cx, 2);
+            // caches that were not donated are copied ahead of the launch (they are inputs of the run)
+            if (kout != kin) { GPTRS_HIP_CHECK(hipMemcpyAsync(kout, kin, ck.bytes(), hipMemcpyDeviceToDevice, cx.stream)); ++cx.launches; }
+            if (vout != vin) { GPTRS_HIP_CHECK(hipMemcpyAsync(vout, vin, ck.bytes(), hipMemcpyDeviceToDevice, cx.stream)); ++cx.launches; }
+            k::ChainPhase pa{}, pc{};
+            k::chain_fill_attn(pa, pc, in.n_q, in.n_kv, in.head_dim, ck.dims[1], in.rot_half, in.scale);
+            pa.x = src_ptr(st, cx, 0);
+            pa.k_cache = kout; pa.v_cache = vout;
+            pa.update_starts = (const int32_t*)src_ptr(st, cx, 3);
+            pa.query_start = (const int32_t*)src_ptr(st, cx, 4);
+            if (in.rot_half > 0) { pa.cos = src_ptr(st, cx, 5); pa.sin = src_ptr(st, cx, 6); }
+            pa.part = (float*)(cx.ws + st.scratch_off);
+            pc.part = pa.part;
+            pc.y = cx.ptr[st.dst[0]];
+            aligned8({pa.x, pa.part, pc.y});
+            if (((uintptr_t)kout | (uintptr_t)vout | (uintptr_t)pa.cos | (uintptr_t)pa.sin) & 15)
+                fail_exec("decode chain: cache and RoPE buffers must be 16-byte aligned");
+            lds_bytes = std::max(lds_bytes, std::max(pa.lds_bytes, pc.lds_bytes));
+            phases.push_back(pa);
+            phases.push_back(pc);
+            continue;
+        }
         const Spec& x = plan.values[st.src[0]].spec;
         const Spec& w = plan.values[st.src[1]].spec;
         const bool dual = in.act == 2;
-        k::ChainPhase& p = phases[(size_t)i];
-        p = k::ChainPhase{};
+        k::ChainPhase p{};
         if (!k::chain_fill_phase(p, x.dims[1], w.dims[1], dual)) { cx.chain = false; return false; }
         BufferP wc = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], 2, x.dtype, x.dims[1], w.dims[1],
                                             dual ? cx.input_bufs[st.tiled_w2_input] : nullptr);
@@ -742,10 +787,10 @@ static bool run_chain(const Plan& plan, const Step& head, ExecCtx& cx) {
         if (in.norm) { p.gamma = src_ptr(st, cx, oi++); p.inv_n = in.scale; p.eps = in.eps; p.flags |= k::kChainNorm; }
         if (in.act == 1) p.flags |= k::kChainGelu;
         p.y = cx.ptr[st.dst[0]];
-        if (((uintptr_t)p.x | (uintptr_t)p.y | (uintptr_t)p.residual | (uintptr_t)p.bias | (uintptr_t)p.gamma) & 7)
-            fail_exec("decode chain: operand buffers must be 8-byte aligned");
-        max_kw = std::max(max_kw, p.Kw);
+        aligned8({p.x, p.y, p.residual, p.bias, p.gamma});
+        lds_bytes = std::max(lds_bytes, p.lds_bytes);
         bytes += (int64_t)dtype_size(x.dtype) * (x.dims[1] + x.dims[1] * w.dims[1] * (dual ? 2 : 1) + w.dims[1]);
+        phases.push_back(p);
     }
     const k::ChainPhase* table = cx.be->chain_table(phases);
     if (!table) { cx.chain = false; return false; }
@@ -755,7 +800,7 @@ static bool run_chain(const Plan& plan, const Step& head, ExecCtx& cx) {
         GPTRS_HIP_CHECK(hipEventCreate(&e1));
         GPTRS_HIP_CHECK(hipEventRecord(e0, cx.stream));
     }
-    if (!k::chain_launch(cx.stream, table, head.chain_len, max_kw, cx.be->chain_barrier(), cx.be->chain_abort_flag())) {
+    if (!k::chain_launch(cx.stream, table, (int)phases.size(), lds_bytes, cx.be->chain_barrier(), cx.be->chain_abort_flag())) {
         if (e0) { (void)hipEventDestroy(e0); (void)hipEventDestroy(e1); }
         cx.chain = false;
         return false;
@@ -767,7 +812,7 @@ static bool run_chain(const Plan& plan, const Step& head, ExecCtx& cx) {
         cx.be->prof_linear_bytes += bytes;
     }
     ++cx.be->n_chain_launches;
-    cx.be->n_chain_phases += head.chain_len;
+    cx.be->n_chain_phases += (int64_t)phases.size();
     ++cx.launches;
     return true;
 }
@@ -1005,6 +1050,8 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
             break;
         }
         case OpKind::FAttnDecode: {
+            if (cx.chain && st.chain_member) break;  // executed by the launch of the run's first step
+            if (cx.chain && st.chain_len > 0 && run_chain(plan, st, cx)) break;
             const Spec& ck = in_spec(1);
             void* kout = cx.ptr[st.dst[1]];
             void* vout = cx.ptr[st.dst[2]];

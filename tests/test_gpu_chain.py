@@ -1,0 +1,148 @@
+"""GPU parity of the persistent decode chain (one launch for a run of M = 1 bf16 linears and decode
+attentions) against the CPU oracle, at the widths of the Ministral-3B-shaped decoder: several
+words per lane and tile (K 3072..9216), several units per workgroup, RMSNorm prologue, SwiGLU pair,
+bias + exact GELU, residual, and chains of dependent phases.
+
+Reference: the oracle run in F32 on the same bf16-representable inputs (the reference's CPU backends
+execute f32 only).  The chain keeps f32 inside a linear and rounds its output to bf16 once, so it
+sits within a few bf16 quanta of that reference; the per-op-rounded bf16 oracle is further away from
+it than the chain is (its RMSNorm scale alone is rounded to 8 bits), so it is not the yardstick
+here.  The chain must also agree with the one-kernel-per-linear path of the same backend."""
+import numpy as np
+import pytest
+
+from parity import FunctionBuilder, Program, assert_close, hip_run, oracle_run
+from gptrs_amd import functional as F
+from gptrs_amd.ptir import f32_to_bf16_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def rnd(seed, shape, scale=1.0):
+    return (np.random.default_rng(seed).uniform(-1.0, 1.0, size=shape) * scale).astype(np.float32)
+
+
+def prog(build, param_specs):
+    fb = FunctionBuilder("main")
+    params = [fb.param(dt, dims) for dt, dims in param_specs]
+    res = build(fb, *params)
+    fb.set_results(list(res) if isinstance(res, (list, tuple)) else [res])
+    return Program(fb)
+
+
+def bf16_round(a):
+    return (f32_to_bf16_bits(np.asarray(a, np.float32)).astype(np.uint32) << 16).view(np.float32)
+
+
+def run_both(hip, build, specs, arrays, atol, rtol):
+    """chain on vs the f32 oracle, and chain on vs chain off (same backend, one kernel per linear)."""
+    p = prog(build, [("Bf16", d) for d in specs])
+    before = hip.counter("chain_launches")
+    got = hip_run(hip, p, arrays)
+    assert hip.counter("chain_launches") > before, "the program did not take the chain path"
+    want = oracle_run(prog(build, [("F32", d) for d in specs]), [bf16_round(a) for a in arrays])
+    hip.set_option("chain", 0)
+    try:
+        plain = hip_run(hip, p, arrays)
+    finally:
+        hip.set_option("chain", 1)
+    for i, (g, w, q) in enumerate(zip(got, want, plain)):
+        assert_close(g, w, atol=atol, rtol=rtol, what=f"result {i} vs oracle")
+        assert_close(g, q, atol=atol, rtol=rtol, what=f"result {i} vs per-linear kernels")
+
+
+@pytest.mark.parametrize("k,n", [(3072, 6144), (4096, 3072), (9216, 3072), (3072, 1000), (512, 40), (64, 12)])
+def test_single_linear(hip, k, n):
+    x, w = rnd(1, (1, k)), rnd(2, (k, n), 2.0 / np.sqrt(k))
+    run_both(hip, lambda fb, a, b: a.matmul(b), [[1, k], [k, n]], [x, w], 2e-2, 2e-2)
+
+
+@pytest.mark.parametrize("k,n", [(3072, 6144), (1024, 256)])
+def test_norm_linear(hip, k, n):
+    x, g, w = rnd(3, (1, k), 3.0), rnd(4, (k,)) + 1.5, rnd(5, (k, n), 2.0 / np.sqrt(k))
+    run_both(hip, lambda fb, a, gm, b: F.rms_norm(a, gm, 1e-5)[0].matmul(b), [[1, k], [k], [k, n]], [x, g, w], 4e-2, 2e-2)
+
+
+@pytest.mark.parametrize("k,n", [(3072, 9216), (256, 96)])
+def test_swiglu_pair(hip, k, n):
+    x, g = rnd(6, (1, k), 3.0), rnd(7, (k,)) + 1.5
+    wg, wu = rnd(8, (k, n), 2.0 / np.sqrt(k)), rnd(9, (k, n), 2.0 / np.sqrt(k))
+
+    def build(fb, a, gm, b, c):
+        h = F.rms_norm(a, gm, 1e-5)[0]
+        return F.swiglu(h.matmul(b), h.matmul(c))
+
+    run_both(hip, build, [[1, k], [k], [k, n], [k, n]], [x, g, wg, wu], 6e-2, 3e-2)
+
+
+@pytest.mark.parametrize("k,n", [(9216, 3072), (768, 3072), (128, 64)])
+def test_bias_gelu_residual(hip, k, n):
+    x, w, b, r = rnd(10, (1, k)), rnd(11, (k, n), 2.0 / np.sqrt(k)), rnd(12, (n,)), rnd(13, (1, n))
+    run_both(hip, lambda fb, a, c, d, e: F.gelu(F.linear(a, c, d)) + e, [[1, k], [k, n], [n], [1, n]], [x, w, b, r], 3e-2, 2e-2)
+
+
+@pytest.mark.parametrize("d,f", [(3072, 9216), (256, 640)])
+def test_block_tail_chain(hip, d, f):
+    """out-proj (+residual) -> RMSNorm -> gate/up SwiGLU -> down (+residual) -> RMSNorm -> next
+    projection: five dependent phases in one launch (model/ministral.rs:166-201)."""
+    qp = d + d // 3 // 4 * 4
+    ctx, x = rnd(20, (1, qp)), rnd(21, (1, d))
+    wo, wg, wu = rnd(22, (qp, d), 2.0 / np.sqrt(qp)), rnd(23, (d, f), 2.0 / np.sqrt(d)), rnd(24, (d, f), 2.0 / np.sqrt(d))
+    wd, wq = rnd(25, (f, d), 2.0 / np.sqrt(f)), rnd(26, (d, 2 * d), 2.0 / np.sqrt(d))
+    g1, g2 = rnd(27, (d,)) + 1.5, rnd(28, (d,)) + 1.5
+
+    def build(fb, c, xx, a_wo, a_wg, a_wu, a_wd, a_wq, a_g1, a_g2):
+        h = c.matmul(a_wo) + xx
+        n1 = F.rms_norm(h, a_g1, 1e-5)[0]
+        ff = F.swiglu(n1.matmul(a_wg), n1.matmul(a_wu)).matmul(a_wd) + h
+        return [F.rms_norm(ff, a_g2, 1e-5)[0].matmul(a_wq), ff]
+
+    specs = [[1, qp], [1, d], [qp, d], [d, f], [d, f], [f, d], [d, 2 * d], [d], [d]]
+    before = hip.counter("chain_phases")
+    run_both(hip, build, specs, [ctx, x, wo, wg, wu, wd, wq, g1, g2], 1e-1, 5e-2)
+    assert hip.counter("chain_phases") - before >= 4
+
+
+@pytest.mark.parametrize("hq,hkv,dh,rope", [(8, 2, 128, True), (4, 4, 64, False), (8, 1, 128, True), (4, 2, 256, False)])
+def test_decode_attention_in_chain(hip, hq, hkv, dh, rope):
+    """projection -> (RoPE) -> attention_decode_cache -> out-projection as ONE launch: the attention takes
+    two phases of the chain (per-chunk online softmax, then the merge).  Positions cover an empty cache,
+    fewer positions than chunks, chunk boundaries, more positions per lane group than are requested
+    ahead of the barrier, and the last slot; the updated caches must match as well (bit-exact when no
+    RoPE touches the appended row)."""
+    d, cap = 256, 2048
+    cfg = F.AttentionConfig(embed_dim=d, num_query_heads=hq, num_key_value_heads=hkv, head_dim=dh)
+    tp, qp = cfg.total_projection_dim, cfg.query_projection_dim
+    rcfg = F.RopeConfig(rotary_dim=dh, theta=10000.0) if rope else None
+    x = rnd(30, (1, d))
+    wqkv, wo = rnd(31, (d, tp), 2.0 / np.sqrt(d)), rnd(32, (qp, d), 2.0 / np.sqrt(qp))
+    kc, vc = rnd(33, (hkv, cap, dh)), rnd(34, (hkv, cap, dh))
+
+    def build(fb, a, w1, w2, k, v, us, qs, *cs):
+        qkv = a.matmul(w1)
+        if cs:
+            qkv = F.apply_rope_qkv_packed(cfg, qkv, cs[0], cs[1])
+        c, k2, v2 = F.attention_decode_cache(cfg, qkv, k, v, us, qs)
+        return [c.matmul(w2), k2, v2]
+
+    fspecs = [[1, d], [d, tp], [qp, d], [hkv, cap, dh], [hkv, cap, dh]]
+    for pos in (0, 5, 31, 32, 100, 1500, cap - 1):
+        us, qs = np.array([0, pos, 0], np.int32), np.array([pos], np.int32)
+        arrays, ispecs = [x, wqkv, wo, kc, vc], [("Si32", [3]), ("Si32", [1])]
+        extra, especs = [], []
+        if rope:
+            cos, sin = F.rotary_cos_sin_cache_slice(pos, 1, rcfg)
+            extra, especs = [cos, sin], [list(cos.shape), list(sin.shape)]
+        pb = prog(build, [("Bf16", s) for s in fspecs] + ispecs + [("Bf16", s) for s in especs])
+        pf = prog(build, [("F32", s) for s in fspecs] + ispecs + [("F32", s) for s in especs])
+        before = hip.counter("chain_phases")
+        got = hip_run(hip, pb, arrays + [us, qs] + extra)
+        assert hip.counter("chain_phases") - before == 4, "projection, attention (2 phases) and out-projection must share one launch"
+        want = oracle_run(pf, [bf16_round(a) for a in arrays] + [us, qs] + [bf16_round(a) for a in extra])
+        assert_close(got[0], want[0], atol=3e-2, rtol=2e-2, what=f"context projection at pos {pos}")
+        for i in (1, 2):
+            g, w = np.asarray(got[i], np.float32), np.asarray(want[i], np.float32)
+            mask = np.ones(cap, bool)
+            mask[pos] = False
+            assert np.array_equal(g[:, mask], w[:, mask]), "cache rows other than the appended one must be untouched"
+            assert_close(g[:, pos], w[:, pos], atol=2e-2, rtol=2e-2, what=f"appended row of cache {i} at pos {pos}")
