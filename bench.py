@@ -8,8 +8,9 @@ fixed-capacity KV cache.  One "step" = one decode token: upload of the per-step 
 reference's decode-steady protocol (crates/gpt-rs-cli/src/main.rs:976-1051).
 
 Prints ONE JSON line; `value` = tokens/s with all weights and the KV cache resident in HBM.
-`roofline` covers the dominant kernel family (the linear-layer GEMV launches): algorithmic bytes
-(every weight element once + activations in/out) over the HIP-event time of those launches on
+`roofline` covers the dominant kernel, the persistent decode chain (one launch per step: every
+linear layer and the decode attention): the step's algorithmic bytes (every weight element once,
+the valid KV rows once, activations and logits once) over the HIP-event time of those launches on
 the backend's stream.  `cpu_baseline` times the reference C backend's own GEMV kernels
 (oracle/_ref, built from the reference checkout) on one host core over a bounded sample.
 """
@@ -29,6 +30,10 @@ sys.path.insert(0, ROOT)
 import __graft_entry__ as entry  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes moved by one chain_kernel launch of the default workload (26 layers, prompt 1024, cache
+# length ~1040), from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a copy kernel of known size; the
+# commands and raw figures are in profiles/chain_kernel_ministral3b_bf16_b1_decode.md
+MEASURED_CHAIN_TRAFFIC_BYTES = 7.010e9 + 0.0216e9
 
 
 def algorithmic_bytes_per_step(cfg, dtype_bytes: int, cache_len: int) -> int:
@@ -106,6 +111,9 @@ def main():
     ap.add_argument("--prompt", type=int, default=1024)
     ap.add_argument("--layers", type=int, default=26, help="debug only: fewer layers is NOT the benchmark config")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run only a plain elementwise kernel of known traffic (x + 0 over 2^28 f32: 1 GiB read, 1 GiB written, "
+                         "kernel binary_scalar_kernel) so FETCH_SIZE / WRITE_SIZE can be scaled to bytes")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (no collectives, no sharding); --gpus must be 1", file=sys.stderr)
@@ -116,6 +124,19 @@ def main():
     from gptrs_amd.backend import HipBackend
 
     be = HipBackend(0)
+    if args.copy_calibration:
+        from gptrs_amd.ptir import FunctionBuilder, Program, TensorSpec
+        n = 1 << 28
+        fb = FunctionBuilder("main")
+        x = fb.param("F32", [n])
+        fb.set_results([x + 0.0])
+        prog = Program(fb)
+        h = be.materialize(TensorSpec("F32", [n]), None)
+        for _ in range(10):
+            be.run_program(prog, [h])
+        be.synchronize()
+        print(json.dumps({"copy_calibration": "10 launches of x + 0.0 over %d f32" % n, "bytes_read_per_launch": 4 * n, "bytes_written_per_launch": 4 * n}))
+        return
     cfg = models.MinistralConfig(num_layers=args.layers)
     total_len = args.prompt + args.warmup + args.steps + 1
     capacity = max(1280, (total_len + 255) // 256 * 256)
@@ -145,10 +166,14 @@ def main():
     elapsed = time.perf_counter() - t0
     launches = be.counter("last_program_launches")
 
-    # second pass over fresh steps with every linear launch bracketed by HIP events
+    # second pass over fresh steps with the dominant launches bracketed by HIP events on the backend's
+    # stream: the persistent decode chain (one launch per step carrying every linear layer and the
+    # decode attention), or the per-linear GEMV kernels when the chain is switched off
     prof_steps = min(32, capacity - gen.processed_len - 1)
     roof = None
     if prof_steps > 0:
+        prof_start = gen.processed_len
+        chains0 = be.counter("chain_launches")
         be.set_option("profile", 1)
         for _ in range(prof_steps):
             gen.step()
@@ -156,11 +181,22 @@ def main():
         calls = be.counter("linear_calls")
         nbytes = be.counter("linear_bytes")
         be.set_option("profile", 0)
+        chains = be.counter("chain_launches") - chains0
         if t_ns > 0:
+            if chains == calls:
+                # the timed launches are whole decode steps minus embedding and argmax: price them with
+                # the step's algorithmic bytes (weights once, valid KV once, logits once)
+                nbytes = sum(algorithmic_bytes_per_step(cfg, 2, prof_start + i) for i in range(prof_steps))
+                kernel = "chain_kernel: persistent decode chain, %d phases per launch (all linear layers + decode attention of a step)" % (
+                    be.counter("chain_phases") // max(be.counter("chain_launches"), 1))
+            else:
+                kernel = "gemv_tiled_kernel<bf16>: all linear layers of a decode step"
             achieved = nbytes / (t_ns * 1e-9) / 1e9
+            default_workload = chains == calls and args.layers == 26 and args.prompt == 1024
             roof = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                    "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
-                    "kernel": "gemv_kernel<bf16> (+gemv_reduce_kernel): all linear layers of a decode step",
+                    "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                    "traffic": MEASURED_CHAIN_TRAFFIC_BYTES if default_workload else None,
+                    "kernel": kernel,
                     "launches": calls, "avg_launch_us": round(t_ns / max(calls, 1) / 1e3, 2),
                     "bytes_per_launch": round(nbytes / max(calls, 1))}
 
