@@ -36,15 +36,25 @@ HBM_PEAK_GBPS = 8000.0
 MEASURED_CHAIN_TRAFFIC_BYTES = 7.010e9 + 0.0216e9
 
 
-def algorithmic_bytes_per_step(cfg, dtype_bytes: int, cache_len: int) -> int:
+def algorithmic_bytes_per_step(cfg, dtype_bytes: int, cache_len: int, quant: str = "none") -> int:
     """Minimum HBM traffic of one decode token: every weight once, the valid KV once, the new KV
-    row and the logits written once."""
+    row and the logits written once.  Quantised linear weights count their codes (1 or 1/2 byte per
+    element) plus their scales (one per column, or one per column and 128 rows)."""
     a = cfg.attention_config()
-    per_layer = (cfg.embed_dim * a.total_projection_dim + a.query_projection_dim * cfg.embed_dim
-                 + 3 * cfg.embed_dim * cfg.ffn_dim + 2 * cfg.embed_dim)
-    weights = cfg.num_layers * per_layer + cfg.embed_dim + cfg.embed_dim * cfg.vocab_size
+    mats = cfg.num_layers * [(cfg.embed_dim, a.total_projection_dim), (a.query_projection_dim, cfg.embed_dim),
+                             (cfg.embed_dim, cfg.ffn_dim), (cfg.embed_dim, cfg.ffn_dim), (cfg.ffn_dim, cfg.embed_dim)]
+    mats.append((cfg.embed_dim, cfg.vocab_size))
+
+    def mat_bytes(k, n):
+        if quant == "w8":
+            return k * n + n * dtype_bytes
+        if quant == "w4g128":
+            return k * n // 2 + (k // 128) * n * dtype_bytes
+        return k * n * dtype_bytes
+
+    weights = sum(mat_bytes(k, n) for k, n in mats) + dtype_bytes * (cfg.num_layers * 2 * cfg.embed_dim + cfg.embed_dim)
     kv_row = cfg.num_layers * 2 * cfg.num_kv_heads * cfg.head_dim
-    return dtype_bytes * (weights + kv_row * (cache_len + 1) + cfg.vocab_size + cfg.embed_dim)
+    return weights + dtype_bytes * (kv_row * (cache_len + 1) + cfg.vocab_size + cfg.embed_dim)
 
 
 def cpu_baseline(cfg, seconds_budget: float = 25.0):
@@ -110,6 +120,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--prompt", type=int, default=1024)
     ap.add_argument("--layers", type=int, default=26, help="debug only: fewer layers is NOT the benchmark config")
+    ap.add_argument("--quant", choices=["none", "w8", "w4g128"], default="none",
+                    help="weight-only quantisation of every linear weight (BASELINE configs[4]: w8 = int8 per output channel, "
+                         "w4g128 = int4 in groups of 128); activations, KV cache and embeddings stay bf16")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain elementwise kernel of known traffic (x + 0 over 2^28 f32: 1 GiB read, 1 GiB written, "
@@ -143,7 +156,7 @@ def main():
     if capacity > cfg.context_length:
         raise SystemExit(f"prompt + warmup + steps = {total_len} exceeds the context length {cfg.context_length}")
     t0 = time.perf_counter()
-    model = models.Ministral.random(cfg, be, seed=5, dtype="Bf16")
+    model = models.Ministral.random(cfg, be, seed=5, dtype="Bf16", quant=None if args.quant == "none" else args.quant)
     t_init = time.perf_counter() - t0
     prompt = np.random.default_rng(6).integers(0, cfg.vocab_size, args.prompt).tolist()
 
@@ -186,13 +199,13 @@ def main():
             if chains == calls:
                 # the timed launches are whole decode steps minus embedding and argmax: price them with
                 # the step's algorithmic bytes (weights once, valid KV once, logits once)
-                nbytes = sum(algorithmic_bytes_per_step(cfg, 2, prof_start + i) for i in range(prof_steps))
+                nbytes = sum(algorithmic_bytes_per_step(cfg, 2, prof_start + i, args.quant) for i in range(prof_steps))
                 kernel = "chain_kernel: persistent decode chain, %d phases per launch (all linear layers + decode attention of a step)" % (
                     be.counter("chain_phases") // max(be.counter("chain_launches"), 1))
             else:
                 kernel = "gemv_tiled_kernel<bf16>: all linear layers of a decode step"
             achieved = nbytes / (t_ns * 1e-9) / 1e9
-            default_workload = chains == calls and args.layers == 26 and args.prompt == 1024
+            default_workload = chains == calls and args.layers == 26 and args.prompt == 1024 and args.quant == "none"
             roof = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
                     "traffic": MEASURED_CHAIN_TRAFFIC_BYTES if default_workload else None,
@@ -201,14 +214,15 @@ def main():
                     "bytes_per_launch": round(nbytes / max(calls, 1))}
 
     mid_len = start_len + args.steps // 2
-    step_bytes = algorithmic_bytes_per_step(cfg, 2, mid_len)
+    step_bytes = algorithmic_bytes_per_step(cfg, 2, mid_len, args.quant)
+    wname = {"none": "bf16", "w8": "int8-weight-only (per output channel) bf16", "w4g128": "int4-weight-only (groups of 128) bf16"}[args.quant]
     ms_per_step = elapsed / args.steps * 1e3
     out = {
-        "metric": "decode tokens/s, Ministral-3B-shape bf16 batch 1 (HBM GB/s as % of 8 TB/s in hbm_frac)",
+        "metric": "decode tokens/s, Ministral-3B-shape %s batch 1 (HBM GB/s as %% of 8 TB/s in hbm_frac)" % wname,
         "value": round(args.steps / elapsed, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "ministral-3b-shape bf16 decode, batch 1, prompt 1024, greedy, KV capacity %d" % capacity,
+        "config": {"workload": "ministral-3b-shape %s decode, batch 1, prompt %d, greedy, KV capacity %d" % (wname, args.prompt, capacity),
                    "layers": cfg.num_layers, "d_model": cfg.embed_dim, "heads": cfg.num_heads, "kv_heads": cfg.num_kv_heads,
                    "head_dim": cfg.head_dim, "ffn": cfg.ffn_dim, "vocab": cfg.vocab_size, "cache_len_mid": mid_len},
         "hbm_gbps": round(step_bytes / (elapsed / args.steps) / 1e9, 1),

@@ -151,9 +151,21 @@ BufferP Backend::derived_weights(const BufferP& src, int kind, DType dtype, int6
     } else if (kind == 1) {
         t = new_buffer(k::mfma_weight_bytes((int)dtype, k, n));
         k::mfma_pack_weights(stream, (int)dtype, src->ptr, t->ptr, k, n);
-    } else {
-        t = new_buffer(k::chain_weight_bytes(k, n, src2 != nullptr));
-        k::chain_pack_weights(stream, src->ptr, src2 ? src2->ptr : nullptr, t->ptr, k, n);
+    } else if (kind == 2 || kind == 3 || kind == 4) {   // decode chain: bf16 / int8 codes / int4 codes (src2: SwiGLU partner)
+        const int wfmt = kind - 2;
+        t = new_buffer(k::chain_weight_bytes(k, n, src2 != nullptr, wfmt));
+        k::chain_pack_weights(stream, src->ptr, src2 ? src2->ptr : nullptr, t->ptr, k, n, wfmt);
+    } else if (kind == 5) {                             // decode chain: int4 group scales (src2: the partner's)
+        t = new_buffer(k::chain_scale_bytes(k, n, src2 != nullptr));
+        k::chain_pack_scales_w4(stream, (int)dtype, src->ptr, src2 ? src2->ptr : nullptr, t->ptr, k, n);
+    } else {                                            // 6 / 7: MFMA copy of dequantised int8 / int4 (src2: scales)
+        if (!src2) fail_exec("quantised weight copy needs its scales");
+        BufferP full = new_buffer((size_t)k * n * dtype_size(dtype));
+        if (kind == 6) k::dequant_w8(stream, (int)dtype, (const int8_t*)src->ptr, src2->ptr, full->ptr, k, n);
+        else k::dequant_w4g128(stream, (int)dtype, (const uint8_t*)src->ptr, src2->ptr, full->ptr, k, n);
+        t = new_buffer(k::mfma_weight_bytes((int)dtype, k, n));
+        k::mfma_pack_weights(stream, (int)dtype, full->ptr, t->ptr, k, n);
+        // `full` returns to the pool here; later users are ordered behind the pack on the one stream
     }
     Derived d;
     d.src = src;
@@ -364,6 +376,8 @@ bool Backend::run_graphed(Plan& plan, ExecCtx& cx, const std::vector<BufferP>& o
     for (const Step& st : plan.steps) {
         if (st.tiled_w_input >= 0) key.push_back(cx.input_bufs[st.tiled_w_input]->id);
         if (st.tiled_w2_input >= 0) key.push_back(cx.input_bufs[st.tiled_w2_input]->id);
+        if (st.tiled_s_input >= 0) key.push_back(cx.input_bufs[st.tiled_s_input]->id);
+        if (st.tiled_s2_input >= 0) key.push_back(cx.input_bufs[st.tiled_s2_input]->id);
     }
     for (auto& g : plan.graphs)
         if (g.key == key) {

@@ -613,6 +613,19 @@ struct Fuser {
             in.act = 0;
             ++fused;
         }
+        // quantised dots (already validated as written) take the same epilogues
+        for (auto& in : fn.body) {
+            if (in.dead || in.op != OpKind::CustomCall) continue;
+            const int q = quant_dot_target(in.target);
+            if (!q || in.operands.size() != 3) continue;
+            bool vals = true;
+            for (auto& o : in.operands) vals = vals && o.value >= 0;
+            if (!vals) continue;
+            in.op = OpKind::FLinear;
+            in.op_name = q == 1 ? "fused.linear_w8" : "fused.linear_w4g128";
+            in.quant = q;
+            in.act = 0;
+        }
         reindex();
         // 2. epilogues, each absorbed only when the linear's value has no other reader
         bool changed = true;
@@ -683,12 +696,14 @@ struct Fuser {
                     Instr* lg = linear_of(in.operands[0].value);
                     Instr* lu = linear_of(in.operands[1].value);
                     if (lg && lu && lg != lu && lg->act == 0 && lu->act == 0 && !lg->has_bias && !lu->has_bias &&
-                        !lg->has_residual && !lu->has_residual && lg->operands[0].value == lu->operands[0].value) {
+                        !lg->has_residual && !lu->has_residual && lg->operands[0].value == lu->operands[0].value &&
+                        lg->quant == lu->quant) {
                         const Spec* wg = spec_of(lg->operands[1].value);
                         const Spec* wu = spec_of(lu->operands[1].value);
                         if (wg && wu && *wg == *wu) {
                             Instr ni = *lg;
                             ni.operands.push_back(lu->operands[1]);
+                            if (lg->quant) ni.operands.push_back(lu->operands[2]);
                             ni.act = 2;
                             ni.out_ids = {v};
                             lg->dead = true;
@@ -715,9 +730,14 @@ struct Fuser {
             if (!xs || !ws) continue;
             const int64_t M = xs->dims[0];
             if (!is_param(in.operands[1].value)) continue;
-            if (in.act == 2 && !is_param(in.operands[2].value)) continue;
+            if (in.act == 2 && !is_param(in.operands[linear_w2_pos(in)].value)) continue;
+            if (in.quant && (!is_param(in.operands[2].value) || (in.act == 2 && !is_param(in.operands[4].value)))) continue;
             if (k::mfma_gemm_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1])) {
                 in.mfma = true;
+                continue;
+            }
+            if (in.quant) {   // decode: only the persistent chain reads the codes directly
+                in.tiled = k::chain_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1], in.act == 2, false, in.quant);
                 continue;
             }
             if (!k::gemv_tiled_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1])) continue;

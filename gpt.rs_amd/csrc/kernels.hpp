@@ -109,6 +109,22 @@ void tile_weights(hipStream_t s, int dtype, const void* w, void* wt, int64_t k, 
 bool gemv_tiled_supported(int dtype, int64_t m, int64_t k, int64_t n);
 void gemv_tiled(hipStream_t s, const TiledLinearArgs& a);
 
+// ---- weight-only quantisation (kernels_quant.hip) ------------------------------------------
+// Build-defined extension (the reference has no quantisation scheme, docs/backend.md:620-632):
+//   int8: symmetric, one scale per output column of W[K,N]: s_n = bf16(max_k |W[k,n]| / 127) (1 when 0),
+//         q = clamp(rint(W / s_n), -127, 127)
+//   int4: symmetric, groups of 128 along K per column: s[g,n] = bf16(max |w| / 7) (1 when 0), q in [-7,7],
+//         two per byte along K: byte[k/2, n] = (q[k] & 0xF) | ((q[k+1] & 0xF) << 4)
+// All arithmetic in f32 with IEEE division and round-half-even, so the results are bit-identical to
+// the numpy closed form.  dtype tags: 0 f32, 2 bf16 (of w / scales / dequantised output).
+void quant_w8_scales(hipStream_t s, int dtype, const void* w, void* scales, int64_t k, int64_t n);
+void quant_w8(hipStream_t s, int dtype, const void* w, const void* scales, int8_t* q, int64_t k, int64_t n);
+void quant_w4g128_scales(hipStream_t s, int dtype, const void* w, void* scales, int64_t k, int64_t n);
+void quant_w4g128(hipStream_t s, int dtype, const void* w, const void* scales, uint8_t* packed, int64_t k, int64_t n);
+// out[k,n] = dtype(f32(q) * f32(scale))
+void dequant_w8(hipStream_t s, int dtype, const int8_t* q, const void* scales, void* out, int64_t k, int64_t n);
+void dequant_w4g128(hipStream_t s, int dtype, const uint8_t* packed, const void* scales, void* out, int64_t k, int64_t n);
+
 // Persistent decode chain (kernels_chain.hip): a run of consecutive M = 1 bf16 linear layers in
 // ONE launch of one workgroup per CU, phases separated by a grid barrier, weights read from a
 // 4-column / k-pair tiled copy, Wc[tile][k/2][4][2].  `flags` of a phase: RMSNorm prologue
@@ -120,6 +136,7 @@ constexpr int kChainMaxPhases = 192;
 constexpr int kChainMaxXsWords = 16384;   // staged activation pairs: K <= 32768
 constexpr size_t kChainBarrierBytes = (kChainCounters * 64 + 64) * sizeof(unsigned);  // zero-initialised once
 enum : int { kChainNorm = 1, kChainDual = 2, kChainGelu = 4, kChainResidual = 8, kChainBias = 16 };
+enum : int { kChainW16 = 0, kChainW8 = 1, kChainW4 = 2 };   // weight format of a linear phase
 enum : int { kChainLinear = 0, kChainAttnPartial = 1, kChainAttnCombine = 2 };
 // One phase of a chain.  Linear: y = act(norm?(x) . W + bias) (+ residual).  Decode attention
 // (attention.rs:657-779, T = 1) takes two phases: "partial" appends this step's K/V row and leaves
@@ -131,6 +148,11 @@ struct ChainPhase {
     void* y;
     int K, N, Kw, ntiles, wpt, units, upb, lds_bytes;
     float inv_n, eps;
+    // quantised weights: wfmt 1 = int8 (16-byte word = 4 columns x 4 k, biased by 128; `scale`/`scale2` = the
+    // per-column scale tensors of W and of the SwiGLU partner, as wscale/wscale2), wfmt 2 = int4 groups of 128 (word = 4 columns x 8 k,
+    // biased by 8; `wscale` = derived copy sc[tile][group][4] bf16, staged into LDS behind the activations)
+    int wfmt, lds_total;   // lds_total: lds_bytes plus what the phase stages behind the activations
+    const void* wscale; const void* wscale2;
     // attention: x = packed qkv row [(n_q + 2 n_kv) * head_dim], y = context row [n_q * head_dim]
     void* k_cache; void* v_cache;              // [n_kv, capacity, head_dim], updated in place
     const int32_t* update_starts;              // si32[3]
@@ -142,13 +164,17 @@ struct ChainPhase {
     int pad;
 };
 int chain_grid();  // workgroups per launch (one per CU), 0 when no device is current
-bool chain_supported(int dtype, int64_t m, int64_t k, int64_t n, bool dual, bool norm);
-size_t chain_weight_bytes(int64_t k, int64_t n, bool dual);
-// w2 != nullptr: SwiGLU pair, columns of w (gate) and w2 (up) interleaved
-void chain_pack_weights(hipStream_t s, const void* w, const void* w2, void* out, int64_t k, int64_t n);
-// fills K, N, Kw, ntiles, wpt, units, upb (and the dual flag); false when one workgroup would own
-// more bias/residual columns than the kernel stages
-bool chain_fill_phase(ChainPhase& p, int64_t k, int64_t n, bool dual);
+bool chain_supported(int dtype, int64_t m, int64_t k, int64_t n, bool dual, bool norm, int wfmt = kChainW16);
+size_t chain_weight_bytes(int64_t k, int64_t n, bool dual, int wfmt = kChainW16);
+// w2 != nullptr: SwiGLU pair, columns of w (gate) and w2 (up) interleaved.  wfmt 0: w is bf16 [k,n];
+// 1: si8 [k,n]; 2: packed int4, ui8 [k/2,n]
+void chain_pack_weights(hipStream_t s, const void* w, const void* w2, void* out, int64_t k, int64_t n, int wfmt = kChainW16);
+// int4 only: derived scale copy sc[tile][group][4] (bf16) from s [k/128, n] (and the partner's s2)
+size_t chain_scale_bytes(int64_t k, int64_t n, bool dual);
+void chain_pack_scales_w4(hipStream_t s, int dtype, const void* sc, const void* sc2, void* out, int64_t k, int64_t n);
+// fills K, N, Kw, ntiles, wpt, units, upb, lds_bytes, wfmt (and the dual flag); false when one workgroup would
+// own more bias/residual columns than the kernel stages
+bool chain_fill_phase(ChainPhase& p, int64_t k, int64_t n, bool dual, int wfmt = kChainW16);
 // Decode attention inside a chain: supported shapes, scratch for the per-chunk records, and the
 // two phases (shape fields filled; the caller sets the pointers of both).
 bool chain_attn_supported(int dtype, int64_t t, int64_t n_q, int64_t n_kv, int64_t head_dim, int64_t rot_half);
@@ -157,7 +183,8 @@ void chain_fill_attn(ChainPhase& partial, ChainPhase& combine, int64_t n_q, int6
                      int64_t rot_half, float scale);
 // bar: kChainBarrierBytes of device memory zeroed once; abort_flag: raised when a barrier wait
 // gives up (every wave then leaves the kernel).  false: launch not possible (caller falls back).
-bool chain_launch(hipStream_t s, const ChainPhase* dev_table, int nphases, int lds_bytes, unsigned* bar, int* abort_flag);
+bool chain_launch(hipStream_t s, const ChainPhase* dev_table, int nphases, int lds_bytes, unsigned* bar, int* abort_flag,
+                  int wfmt = kChainW16);   // wfmt: the weight format of EVERY linear phase of the table
 
 // Prefill GEMM (M > 16, bf16) on the matrix cores over a k-grouped copy of the weights,
 // Wk8[K/8][Npad][8] (kernels_mfma.hip).  wk2 != nullptr: SwiGLU pair.

@@ -23,9 +23,17 @@
 // position chunk: append this step's K/V row, online softmax over the chunk for the query heads
 // of the group) and "combine" (one workgroup per query head merges the chunk records).
 //
+// Weight-only quantised linears stream the same 16-byte words with more k per word: int8 codes
+// (4 columns x 4 k, stored biased by 128) and int4 codes (4 columns x 8 k, biased by 8, with one bf16
+// scale per column and group of 128 k fetched beside the word).  Codes are converted with the
+// unsigned-byte converts and accumulated in f32 against the bf16 activations (every product is
+// exact); the bias is taken out per word (-128 or -8 times the sum of the word's activations), the
+// per-column int8 scale is applied by the control wave.
+//
 // Every wait is bounded: a barrier that does not complete raises the abort flag, every wave
 // leaves the kernel, and the host reports an execution error.
 #include <algorithm>
+#include <climits>
 #include <cstdlib>
 
 #include "kernels.hpp"
@@ -109,6 +117,9 @@ struct Shared {
     float red[NSLOT][NWS][16];
     float epi_bias[EPI_MAX];
     float epi_res[EPI_MAX];
+    // int8: [0, EPI_MAX) scale of each owned output column (gate of a SwiGLU pair), [EPI_MAX, 2 EPI_MAX) the pair's
+    // up column.  (int4 group scales are staged behind the activations, see stage_block.)
+    float epi_s[2 * EPI_MAX];
     float ssq[16];
     int red_cnt[NSLOT];
     int go, consumed, abort, pad;
@@ -120,10 +131,29 @@ struct Shared {
 // RMSNorm kernel stores, ((x * inv_rms) -> bf16) * gamma -> bf16 (normalization.rs:183-217).
 __device__ void stage_block(const ChainPhase& P, unsigned* xs, float* ssq) {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int K = uni(P.K), Kw = uni(P.Kw);
-    const int n = K / 4;        // 8-byte items holding data (K % 4 == 0)
-    const int npad = Kw / 2;    // items to write
+    const int K = uni(P.K);
+    const int n = K / 4;                     // 8-byte items holding data (K % 4 == 0)
+    const int npad = uni(P.lds_bytes) >> 3;  // items to write: the words of every lane read zeros beyond K
     const char* x = (const char*)uni_ptr(P.x);
+    // int4: the group scales of this workgroup's tiles, one contiguous range of the tile-ordered copy
+    // sc[tile][group][4] (bf16, 8 bytes per entry), go behind the activations; the first round of
+    // loads is in flight while the activations are staged
+    constexpr int SB = 8;
+    int sc_n = 0;
+    const uint2* sc_src = nullptr;
+    uint2* sc_dst = reinterpret_cast<uint2*>(xs + 2 * npad);
+    uint2 sv[SB];
+    if (uni(P.wfmt) == kChainW4) {
+        const int G = uni(P.Kw) >> 4, upb = uni(P.upb);
+        const int t0 = (int)blockIdx.x * upb * TP, t1 = min(min(t0 + upb * TP, uni(P.units) * TP), uni(P.ntiles));
+        sc_n = max(t1 - t0, 0) * G;
+        sc_src = (const uint2*)uni_ptr(P.wscale) + (long)t0 * G;
+#pragma unroll
+        for (int u = 0; u < SB; ++u) {
+            const int i = u * NT + t;
+            sv[u] = i < sc_n ? gload2(sc_src + i) : make_uint2(0u, 0u);
+        }
+    }
     if (uni(P.flags) & kChainNorm) {
         const uint2* g = (const uint2*)uni_ptr(P.gamma);
         unsigned long long v[MAXI];
@@ -170,6 +200,25 @@ __device__ void stage_block(const ChainPhase& P, unsigned* xs, float* ssq) {
             for (int u = 0; u < MAXI; ++u) {
                 const int i = i0 + u * NT + t;
                 if (i < npad) *reinterpret_cast<uint2*>(&xs[2 * i]) = make_uint2((unsigned)v[u], (unsigned)(v[u] >> 32));
+            }
+        }
+    }
+    if (sc_n > 0) {
+#pragma unroll
+        for (int u = 0; u < SB; ++u) {
+            const int i = u * NT + t;
+            if (i < sc_n) sc_dst[i] = sv[u];
+        }
+        for (int i0 = SB * NT; i0 < sc_n; i0 += SB * NT) {
+#pragma unroll
+            for (int u = 0; u < SB; ++u) {
+                const int i = i0 + u * NT + t;
+                sv[u] = i < sc_n ? gload2(sc_src + i) : make_uint2(0u, 0u);
+            }
+#pragma unroll
+            for (int u = 0; u < SB; ++u) {
+                const int i = i0 + u * NT + t;
+                if (i < sc_n) sc_dst[i] = sv[u];
             }
         }
     }
@@ -536,6 +585,7 @@ __device__ __forceinline__ float finish(float v, int flags, float bias, float re
     return v;
 }
 
+template <int FMT>
 __device__ void control_wave(Shared& sh, unsigned* xs, int nphases, unsigned* bar, int* abort_flag) {
     const int lane = threadIdx.x & 63;
     const int blk = blockIdx.x, per = gridDim.x / NC;
@@ -592,6 +642,18 @@ __device__ void control_wave(Shared& sh, unsigned* xs, int nphases, unsigned* ba
                     *reinterpret_cast<float2*>(&sh.epi_res[i]) = make_float2(bf16lo(rw), bf16hi(rw));
                 }
             }
+            constexpr int wfmt = FMT;   // every linear phase of a launch has the kernel's weight format
+            if (wfmt == kChainW8) {
+                const unsigned* sg = (const unsigned*)uni_ptr(P.wscale);
+                const unsigned* su = (const unsigned*)uni_ptr(P.wscale2);
+                for (int i = lane * 2; i < ncols; i += 128) {
+                    const int col = col0 + i;
+                    const unsigned a = col < N ? gload(sg + (col >> 1)) : 0u;
+                    const unsigned b = (su && col < N) ? gload(su + (col >> 1)) : 0u;
+                    *reinterpret_cast<float2*>(&sh.epi_s[i]) = make_float2(bf16lo(a), bf16hi(a));
+                    *reinterpret_cast<float2*>(&sh.epi_s[EPI_MAX + i]) = make_float2(bf16lo(b), bf16hi(b));
+                }
+            }
             stage_block(P, xs, sh.ssq);
             GPTRS_STAMP(2);
             char* out = (char*)uni_ptr(P.y);
@@ -620,6 +682,10 @@ __device__ void control_wave(Shared& sh, unsigned* xs, int nphases, unsigned* ba
                 const int tile = u * TP + lane;
                 if (lane < TP && tile < ntiles) {
                     const int e = min(((u - u0) * TP + lane) * cpt, EPI_MAX - 4);
+                    if (wfmt == kChainW8) {
+                        if (dual) { s[0] *= sh.epi_s[e]; s[1] *= sh.epi_s[EPI_MAX + e]; s[2] *= sh.epi_s[e + 1]; s[3] *= sh.epi_s[EPI_MAX + e + 1]; }
+                        else { s[0] *= sh.epi_s[e]; s[1] *= sh.epi_s[e + 1]; s[2] *= sh.epi_s[e + 2]; s[3] *= sh.epi_s[e + 3]; }
+                    }
                     if (dual) {   // columns interleaved (gate, up, gate, up): activation.rs:141-162
                         const float a0 = finish((s[0] / (1.0f + expf(s[0] * -1.0f))) * s[1], flags, sh.epi_bias[e], sh.epi_res[e]);
                         const float a1 = finish((s[2] / (1.0f + expf(s[2] * -1.0f))) * s[3], flags, sh.epi_bias[e + 1], sh.epi_res[e + 1]);
@@ -646,6 +712,7 @@ __device__ void control_wave(Shared& sh, unsigned* xs, int nphases, unsigned* ba
 }
 
 // ---------------------------------------------------------------------------- streaming waves
+template <int FMT>
 __device__ void stream_waves(Shared& sh, const unsigned* xs, int nphases) {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int blk = blockIdx.x;
@@ -692,7 +759,8 @@ __device__ void stream_waves(Shared& sh, const unsigned* xs, int nphases) {
     };
 
     // compute iterator
-    int c_phase = -1, c_unit = 0, c_unit_end = 0, c_j = 0, c_wpt = 1, ucount = 0;
+    int c_phase = -1, c_unit = 0, c_unit_end = 0, c_j = 0, c_wpt = 1, c_sidx = 0, c_G = 0, c_soff = 0, ucount = 0;
+    constexpr int c_fmt = FMT;
     // advance to this workgroup's next linear unit, taking part in attention phases on the way
     auto c_seek = [&]() -> bool {
         for (;;) {
@@ -710,6 +778,9 @@ __device__ void stream_waves(Shared& sh, const unsigned* xs, int nphases) {
             c_unit_end = min(c_unit + upb, units);
             if (c_unit >= c_unit_end) continue;
             c_wpt = uni(ph.wpt);
+            c_G = uni(ph.Kw) >> 4;
+            c_sidx = 0;   // int4: entry of the unit's first tile and group in the staged scales ...
+            c_soff = uni(ph.lds_bytes) >> 2;   // ... which sit behind the activations
             if (!wait_go(&sh.go, &sh.abort, c_phase)) return false;
             stage_block(ph, const_cast<unsigned*>(xs), sh.ssq);
             c_j = 0;
@@ -732,16 +803,64 @@ __device__ void stream_waves(Shared& sh, const unsigned* xs, int nphases) {
 #pragma unroll
         for (int p = 0; p < TP; ++p) cur[p] = nxt[p];
         if (l_active) l_fetch(nxt); else have_nxt = false;
-        const bf16x2 xv = __builtin_bit_cast(bf16x2, xs[c_j * NS + t]);
+        // element reads go through scalars: __builtin_bit_cast applied directly to `vec.y` of an
+        // ext-vector reads element 0 with this compiler
+        if (c_fmt == kChainW16) {
+            const bf16x2 xv = __builtin_bit_cast(bf16x2, xs[c_j * NS + t]);
 #pragma unroll
-        for (int p = 0; p < TP; ++p) {
-            // element reads go through scalars: __builtin_bit_cast applied directly to `vec.y` of an
-            // ext-vector reads element 0 with this compiler
-            const unsigned q0 = cur[p].x, q1 = cur[p].y, q2 = cur[p].z, q3 = cur[p].w;
-            acc[p][0] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q0), xv, acc[p][0], false);
-            acc[p][1] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q1), xv, acc[p][1], false);
-            acc[p][2] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q2), xv, acc[p][2], false);
-            acc[p][3] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q3), xv, acc[p][3], false);
+            for (int p = 0; p < TP; ++p) {
+                const unsigned q0 = cur[p].x, q1 = cur[p].y, q2 = cur[p].z, q3 = cur[p].w;
+                acc[p][0] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q0), xv, acc[p][0], false);
+                acc[p][1] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q1), xv, acc[p][1], false);
+                acc[p][2] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q2), xv, acc[p][2], false);
+                acc[p][3] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q3), xv, acc[p][3], false);
+            }
+        } else if (c_fmt == kChainW8) {
+            const u32x2 xw = *reinterpret_cast<const u32x2*>(&xs[2 * (c_j * NS + t)]);
+            const unsigned xa = xw.x, xb = xw.y;
+            const float x0 = bf16lo(xa), x1 = bf16hi(xa), x2 = bf16lo(xb), x3 = bf16hi(xb);
+            const float corr = -128.0f * ((x0 + x1) + (x2 + x3));
+#pragma unroll
+            for (int p = 0; p < TP; ++p) {
+                const unsigned q[4] = {cur[p].x, cur[p].y, cur[p].z, cur[p].w};
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    float a = acc[p][c] + corr;
+                    a = __builtin_fmaf((float)(q[c] & 0xFFu), x0, a);
+                    a = __builtin_fmaf((float)((q[c] >> 8) & 0xFFu), x1, a);
+                    a = __builtin_fmaf((float)((q[c] >> 16) & 0xFFu), x2, a);
+                    a = __builtin_fmaf((float)(q[c] >> 24), x3, a);
+                    acc[p][c] = a;
+                }
+            }
+        } else {
+            const u32x4 xw = *reinterpret_cast<const u32x4*>(&xs[4 * (c_j * NS + t)]);
+            const unsigned xa = xw.x, xb = xw.y, xc = xw.z, xd = xw.w;
+            const float x0 = bf16lo(xa), x1 = bf16hi(xa), x2 = bf16lo(xb), x3 = bf16hi(xb);
+            const float x4 = bf16lo(xc), x5 = bf16hi(xc), x6 = bf16lo(xd), x7 = bf16hi(xd);
+            const float corr = -8.0f * (((x0 + x1) + (x2 + x3)) + ((x4 + x5) + (x6 + x7)));
+#pragma unroll
+            for (int p = 0; p < TP; ++p) {
+                const unsigned q[4] = {cur[p].x, cur[p].y, cur[p].z, cur[p].w};
+                const u32x2 sw = *reinterpret_cast<const u32x2*>(&xs[c_soff + 2 * (c_sidx + p * c_G + c_j * (NS / 16) + (t >> 4))]);
+                const unsigned sa = sw.x, sb = sw.y;
+                const float sc[4] = {bf16lo(sa), bf16hi(sa), bf16lo(sb), bf16hi(sb)};
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    // byte i of a column's dword: k = 2i in the low nibble, k = 2i + 1 in the high one
+                    const unsigned lo = q[c] & 0x0F0F0F0Fu, hi = (q[c] >> 4) & 0x0F0F0F0Fu;
+                    float a = corr;
+                    a = __builtin_fmaf((float)(lo & 0xFFu), x0, a);
+                    a = __builtin_fmaf((float)(hi & 0xFFu), x1, a);
+                    a = __builtin_fmaf((float)((lo >> 8) & 0xFFu), x2, a);
+                    a = __builtin_fmaf((float)((hi >> 8) & 0xFFu), x3, a);
+                    a = __builtin_fmaf((float)((lo >> 16) & 0xFFu), x4, a);
+                    a = __builtin_fmaf((float)((hi >> 16) & 0xFFu), x5, a);
+                    a = __builtin_fmaf((float)(lo >> 24), x6, a);
+                    a = __builtin_fmaf((float)(hi >> 24), x7, a);
+                    acc[p][c] = __builtin_fmaf(sc[c], a, acc[p][c]);
+                }
+            }
         }
         if (++c_j == c_wpt) {
             const int slot = ucount % NSLOT;
@@ -764,11 +883,12 @@ __device__ void stream_waves(Shared& sh, const unsigned* xs, int nphases) {
             if (lane == 0) __hip_atomic_fetch_add(&sh.red_cnt[slot], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             ++ucount;
             ++c_unit;
-            if (c_unit >= c_unit_end) alive = c_seek(); else c_j = 0;
+            if (c_unit >= c_unit_end) alive = c_seek(); else { c_j = 0; c_sidx += TP * c_G; }
         }
     }
 }
 
+template <int FMT>
 __global__ __launch_bounds__(NT, 1) void chain_kernel(const ChainPhase* __restrict__ phases, int nphases, unsigned* bar, int* abort_flag) {
     extern __shared__ __align__(16) unsigned char smem[];
     Shared& sh = *reinterpret_cast<Shared*>(smem);
@@ -782,8 +902,8 @@ __global__ __launch_bounds__(NT, 1) void chain_kernel(const ChainPhase* __restri
         if (threadIdx.x == 0) { sh.go = -1; sh.consumed = 0; sh.abort = 0; }
         __syncthreads();
     }
-    if (threadIdx.x >= NS) control_wave(sh, xs, nphases, bar, abort_flag);
-    else stream_waves(sh, xs, nphases);
+    if (threadIdx.x >= NS) control_wave<FMT>(sh, xs, nphases, bar, abort_flag);
+    else stream_waves<FMT>(sh, xs, nphases);
 }
 
 // ---------------------------------------------------------------------------- weight layout
@@ -809,8 +929,46 @@ __global__ void chain_pack_kernel(const bf16_t* __restrict__ w, const bf16_t* __
     }
 }
 
+// Quantised codes: the same tile order with one byte per (column, code row): word j of a tile holds code rows
+// 4j .. 4j+3 of its 4 columns.  int8: a code row is one k, bytes stored as q + 128 (flip = 0x80).  int4: a code
+// row is a packed byte (k = 2r low nibble, 2r + 1 high nibble), both nibbles stored as q + 8 (flip = 0x88).
+// Bytes outside the matrix hold the biased zero.
+__global__ void chain_pack_codes_kernel(const uint8_t* __restrict__ w, const uint8_t* __restrict__ w2, uint32_t* __restrict__ out,
+                                        int64_t rows, int64_t N, int64_t Kw, int64_t ntiles, uint32_t flip) {
+    const int64_t total = ntiles * Kw * 4;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int c = (int)(idx & 3);
+        const int64_t j = (idx >> 2) % Kw, tile = (idx >> 2) / Kw;
+        const uint8_t* src = w;
+        int64_t col;
+        if (w2) { col = tile * 2 + (c >> 1); if (c & 1) src = w2; }
+        else col = tile * 4 + c;
+        uint32_t v = 0;
+        for (int h = 0; h < 4; ++h) {
+            const int64_t r = 4 * j + h;
+            const uint32_t b = (col < N && r < rows) ? ((uint32_t)src[r * N + col] ^ flip) : flip;
+            v |= b << (8 * h);
+        }
+        out[idx] = v;
+    }
+}
+// int4 group scales in tile order: sc[tile][g][c] (bf16) for g < Kw / 16, zero outside the matrix
+__global__ void chain_pack_scales_kernel(const bf16_t* __restrict__ sc, const bf16_t* __restrict__ sc2, bf16_t* __restrict__ out,
+                                         int64_t groups, int64_t N, int64_t G, int64_t ntiles) {
+    const int64_t total = ntiles * G * 4;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int c = (int)(idx & 3);
+        const int64_t g = (idx >> 2) % G, tile = (idx >> 2) / G;
+        const bf16_t* src = sc;
+        int64_t col;
+        if (sc2) { col = tile * 2 + (c >> 1); if (c & 1) src = sc2; }
+        else col = tile * 4 + c;
+        out[idx] = (col < N && g < groups) ? src[g * N + col] : (bf16_t)0;
+    }
+}
+
 static int g_grid = 0;
-static size_t g_smem_set = 0;
+static size_t g_smem_set[3] = {0, 0, 0};
 
 }  // namespace
 
@@ -825,43 +983,67 @@ int chain_grid() {
     return g_grid > 0 ? g_grid : 0;
 }
 
-bool chain_supported(int dtype, int64_t m, int64_t k, int64_t n, bool dual, bool norm) {
+static inline int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+static inline int chain_kpw(int wfmt) { return wfmt == kChainW16 ? 2 : (wfmt == kChainW8 ? 4 : 8); }   // k per column of a word
+static inline int64_t chain_kw(int64_t k, int wfmt) { return cdiv64(cdiv64(k, chain_kpw(wfmt)), NS) * NS; }
+
+bool chain_supported(int dtype, int64_t m, int64_t k, int64_t n, bool dual, bool norm, int wfmt) {
     if (dtype != 2 || m != 1 || k < 4 || n < 4) return false;
+    if (wfmt < kChainW16 || wfmt > kChainW4) return false;
     if (k % 4 != 0 || n % (dual ? 2 : 4) != 0) return false;
+    if (wfmt == kChainW4 && k % 128 != 0) return false;
     if (norm && k > 4 * MAXI * NT) return false;
-    if (k > 2 * kChainMaxXsWords) return false;
+    if (chain_kw(k, wfmt) * (chain_kpw(wfmt) / 2) > kChainMaxXsWords) return false;
     return true;
 }
 
-static inline int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
-static inline int64_t chain_kw(int64_t k) { return cdiv64(cdiv64(k, 2), NS) * NS; }
-
-size_t chain_weight_bytes(int64_t k, int64_t n, bool dual) {
+size_t chain_weight_bytes(int64_t k, int64_t n, bool dual, int wfmt) {
     const int64_t ncols = dual ? 2 * n : n;
-    return (size_t)(cdiv64(ncols, 4) * chain_kw(k) * 16);
+    return (size_t)(cdiv64(ncols, 4) * chain_kw(k, wfmt) * 16);
 }
 
-void chain_pack_weights(hipStream_t s, const void* w, const void* w2, void* out, int64_t k, int64_t n) {
-    const int64_t ncols = w2 ? 2 * n : n, ntiles = cdiv64(ncols, 4), kw = chain_kw(k);
+void chain_pack_weights(hipStream_t s, const void* w, const void* w2, void* out, int64_t k, int64_t n, int wfmt) {
+    const int64_t ncols = w2 ? 2 * n : n, ntiles = cdiv64(ncols, 4), kw = chain_kw(k, wfmt);
     const int64_t total = ntiles * kw * 4;
     if (total <= 0) return;
     const unsigned g = (unsigned)std::min<int64_t>(cdiv64(total, 256), 65536);
-    chain_pack_kernel<<<g, 256, 0, s>>>((const bf16_t*)w, (const bf16_t*)w2, (uint32_t*)out, k, n, kw, ntiles);
+    if (wfmt == kChainW16)
+        chain_pack_kernel<<<g, 256, 0, s>>>((const bf16_t*)w, (const bf16_t*)w2, (uint32_t*)out, k, n, kw, ntiles);
+    else
+        chain_pack_codes_kernel<<<g, 256, 0, s>>>((const uint8_t*)w, (const uint8_t*)w2, (uint32_t*)out, wfmt == kChainW8 ? k : k / 2, n, kw,
+                                                  ntiles, wfmt == kChainW8 ? 0x80u : 0x88u);
 }
 
-bool chain_fill_phase(ChainPhase& p, int64_t k, int64_t n, bool dual) {
+size_t chain_scale_bytes(int64_t k, int64_t n, bool dual) {
+    return (size_t)(cdiv64(dual ? 2 * n : n, 4) * (chain_kw(k, kChainW4) / 16) * 4 * sizeof(bf16_t));
+}
+
+void chain_pack_scales_w4(hipStream_t s, int dtype, const void* sc, const void* sc2, void* out, int64_t k, int64_t n) {
+    if (dtype != 2) return;   // the chain only takes bf16 activations and scales
+    const int64_t ntiles = cdiv64(sc2 ? 2 * n : n, 4), G = chain_kw(k, kChainW4) / 16;
+    const int64_t total = ntiles * G * 4;
+    if (total <= 0) return;
+    const unsigned g = (unsigned)std::min<int64_t>(cdiv64(total, 256), 65536);
+    chain_pack_scales_kernel<<<g, 256, 0, s>>>((const bf16_t*)sc, (const bf16_t*)sc2, (bf16_t*)out, k / 128, n, G, ntiles);
+}
+
+bool chain_fill_phase(ChainPhase& p, int64_t k, int64_t n, bool dual, int wfmt) {
     const int grid = chain_grid();
     p.K = (int)k;
     p.N = (int)n;
-    p.Kw = (int)chain_kw(k);
+    p.Kw = (int)chain_kw(k, wfmt);
     p.ntiles = (int)cdiv64(dual ? 2 * n : n, 4);
     p.wpt = p.Kw / NS;
     p.units = (p.ntiles + TP - 1) / TP;
     p.upb = grid > 0 ? (p.units + grid - 1) / grid : p.units;
     p.kind = kChainLinear;
-    p.lds_bytes = p.Kw * 4;
+    p.wfmt = wfmt;
+    p.lds_bytes = p.Kw * (chain_kpw(wfmt) / 2) * 4;
+    // int4: the workgroup's group scales (8 bytes per tile and group) are staged behind the activations
+    const int64_t total = p.lds_bytes + (wfmt == kChainW4 ? (int64_t)p.upb * TP * (p.Kw / 16) * 8 : 0);
+    p.lds_total = (int)std::min<int64_t>(total, INT32_MAX);
     if (dual) p.flags |= kChainDual;
-    return (int64_t)p.upb * TP * (dual ? 2 : 4) <= EPI_MAX && p.Kw <= kChainMaxXsWords;
+    return (int64_t)p.upb * TP * (dual ? 2 : 4) <= EPI_MAX && total <= (int64_t)kChainMaxXsWords * 4;
 }
 
 bool chain_attn_supported(int dtype, int64_t t, int64_t n_q, int64_t n_kv, int64_t head_dim, int64_t rot_half) {
@@ -890,22 +1072,27 @@ void chain_fill_attn(ChainPhase& partial, ChainPhase& combine, int64_t n_q, int6
     }
     partial.kind = kChainAttnPartial;
     partial.units = (int)n_kv * nch;
-    partial.lds_bytes = (int)((2 * NWS + NWS * head_dim) * sizeof(float));
+    partial.lds_bytes = partial.lds_total = (int)((2 * NWS + NWS * head_dim) * sizeof(float));
     combine.kind = kChainAttnCombine;
     combine.units = (int)n_q;
-    combine.lds_bytes = (int)(NW * 64 * sizeof(float4));
+    combine.lds_bytes = combine.lds_total = (int)(NW * 64 * sizeof(float4));
 }
 
-bool chain_launch(hipStream_t s, const ChainPhase* dev_table, int nphases, int lds_bytes, unsigned* bar, int* abort_flag) {
+bool chain_launch(hipStream_t s, const ChainPhase* dev_table, int nphases, int lds_bytes, unsigned* bar, int* abort_flag, int wfmt) {
     const int grid = chain_grid();
     if (grid <= 0 || nphases <= 0 || nphases > kChainMaxPhases || lds_bytes > kChainMaxXsWords * 4) return false;
+    if (wfmt < kChainW16 || wfmt > kChainW4) return false;
+    const void* fn = wfmt == kChainW16 ? (const void*)chain_kernel<kChainW16>
+                   : wfmt == kChainW8  ? (const void*)chain_kernel<kChainW8> : (const void*)chain_kernel<kChainW4>;
     const size_t smem = sizeof(Shared) + (size_t)((lds_bytes + 15) / 16 * 16);
-    if (smem > g_smem_set) {
+    if (smem > g_smem_set[wfmt]) {
         const size_t want = sizeof(Shared) + (size_t)kChainMaxXsWords * 4;
-        if (hipFuncSetAttribute((const void*)chain_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)want) != hipSuccess) return false;
-        g_smem_set = want;
+        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)want) != hipSuccess) return false;
+        g_smem_set[wfmt] = want;
     }
-    chain_kernel<<<grid, NT, smem, s>>>(dev_table, nphases, bar, abort_flag);
+    if (wfmt == kChainW16) chain_kernel<kChainW16><<<grid, NT, smem, s>>>(dev_table, nphases, bar, abort_flag);
+    else if (wfmt == kChainW8) chain_kernel<kChainW8><<<grid, NT, smem, s>>>(dev_table, nphases, bar, abort_flag);
+    else chain_kernel<kChainW4><<<grid, NT, smem, s>>>(dev_table, nphases, bar, abort_flag);
     return true;
 }
 

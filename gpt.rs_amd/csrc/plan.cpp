@@ -311,9 +311,60 @@ void Builder::validate(Instr& in) {
             expect(out.dtype == l.dtype && out.dims == want, "dot_general output shape mismatch");
             break;
         }
-        case OpKind::CustomCall:
-            // docs/backend.md:581-582: unknown targets MUST answer Unimplemented
-            fail_unimpl("custom_call", "unknown target `" + in.target + "`");
+        case OpKind::CustomCall: {
+            // Weight-only quantisation extension of this backend; its targets are validated here and become
+            // FLinear(quant) / FQuant.  docs/backend.md:581-582: unknown targets MUST answer Unimplemented.
+            const int qd = quant_dot_target(in.target), qo = quant_op_target(in.target);
+            if (!qd && !qo) fail_unimpl("custom_call", "unknown target `" + in.target + "`");
+            auto is_f = [](const Spec& sp) { return sp.dtype == DType::F32 || sp.dtype == DType::BF16; };
+            // (codes, scales) of a [K,N] weight matrix in scheme q (1 int8 per column, 2 int4 groups of 128)
+            auto check_pair = [&](int q, const Spec& codes, const Spec& scales, int64_t K, int64_t N, DType fdt) {
+                if (q == 1) {
+                    expect(codes.dtype == DType::SI8 && codes.dims == std::vector<int64_t>{K, N}, in.target + ": codes must be si8[K,N]");
+                    expect(scales.dtype == fdt && scales.dims == std::vector<int64_t>{N}, in.target + ": scales must be [N] of the float dtype");
+                } else {
+                    expect(K % 128 == 0, in.target + ": K must be a multiple of the group size 128");
+                    expect(codes.dtype == DType::UI8 && codes.dims == std::vector<int64_t>{K / 2, N}, in.target + ": codes must be ui8[K/2,N]");
+                    expect(scales.dtype == fdt && scales.dims == std::vector<int64_t>{K / 128, N}, in.target + ": scales must be [K/128,N] of the float dtype");
+                }
+            };
+            if (qd) {
+                expect(in.operands.size() == 3, in.target + ": expects (x, codes, scales)");
+                const Spec& x = spec_of(in, 0);
+                expect(is_f(x) && x.rank() == 2, in.target + ": x must be a float matrix [M,K]");
+                const Spec& c = spec_of(in, 1);
+                expect(c.rank() == 2, in.target + ": codes must be a matrix");
+                check_pair(qd, c, spec_of(in, 2), x.dims[1], c.dims[1], x.dtype);
+                expect(out.dtype == x.dtype && out.dims == std::vector<int64_t>{x.dims[0], c.dims[1]}, in.target + ": output must be [M,N] of x's dtype");
+                in.op = OpKind::FLinear;
+                in.op_name = qd == 1 ? "fused.linear_w8" : "fused.linear_w4g128";
+                in.quant = qd;
+                in.act = 0;
+                break;
+            }
+            const int scheme = (qo == 1 || qo == 2 || qo == 5) ? 1 : 2;
+            if (qo == 1 || qo == 3) {          // scales(w)
+                expect(in.operands.size() == 1, in.target + ": expects (w)");
+                const Spec& w = spec_of(in, 0);
+                expect(is_f(w) && w.rank() == 2, in.target + ": w must be a float matrix [K,N]");
+                if (scheme == 2) expect(w.dims[0] % 128 == 0, in.target + ": K must be a multiple of the group size 128");
+                const std::vector<int64_t> want = scheme == 1 ? std::vector<int64_t>{w.dims[1]} : std::vector<int64_t>{w.dims[0] / 128, w.dims[1]};
+                expect(out.dtype == w.dtype && out.dims == want, in.target + ": output shape mismatch");
+            } else if (qo == 2 || qo == 4) {   // codes(w, scales)
+                expect(in.operands.size() == 2, in.target + ": expects (w, scales)");
+                const Spec& w = spec_of(in, 0);
+                expect(is_f(w) && w.rank() == 2, in.target + ": w must be a float matrix [K,N]");
+                check_pair(scheme, out, spec_of(in, 1), w.dims[0], w.dims[1], w.dtype);
+            } else {                           // dequantise(codes, scales)
+                expect(in.operands.size() == 2, in.target + ": expects (codes, scales)");
+                expect(is_f(out) && out.rank() == 2, in.target + ": output must be a float matrix [K,N]");
+                check_pair(scheme, spec_of(in, 0), spec_of(in, 1), out.dims[0], out.dims[1], out.dtype);
+            }
+            in.op = OpKind::FQuant;
+            in.op_name = "quant." + in.target;
+            in.quant = qo;
+            break;
+        }
         case OpKind::Unsupported:
             fail_unimpl(in.op_name, "operation not supported in the hip backend");
         default:
@@ -495,8 +546,19 @@ void Builder::describe(Step& st) {
                     return p;
                 };
                 st.tiled_w_input = pos(1);
-                if (in.act == 2) st.tiled_w2_input = pos(2);
-            } else {
+                if (in.act == 2) st.tiled_w2_input = pos(linear_w2_pos(in));
+                if (in.quant) {
+                    st.tiled_s_input = pos(2);
+                    if (in.act == 2) st.tiled_s2_input = pos(4);
+                }
+            }
+            if (in.quant && !in.mfma) {
+                // stand-alone path of a quantised linear: (RMSNorm of x,) dequantised weights, then the generic kernel
+                const size_t es = dtype_size(x.dtype);
+                st.scratch_bytes = align_up(in.norm ? (size_t)x.count() * es : 0) +
+                                   align_up((size_t)x.dims[1] * w.dims[1] * es) * (in.act == 2 ? 2 : 1) +
+                                   k::linear_workspace_bytes((int)x.dtype, x.dims[0], x.dims[1], w.dims[1], in.act == 2);
+            } else if (!in.tiled && !in.mfma) {
                 st.scratch_bytes = k::linear_workspace_bytes((int)x.dtype, x.dims[0], x.dims[1], w.dims[1], in.act == 2);
             }
             break;
@@ -697,20 +759,26 @@ void Builder::build() {
         const Spec& w = plan.values[st.src[1]].spec;
         if (x.rank() != 2 || w.rank() != 2) return 0;
         const bool dual = in.act == 2;
-        if (!k::chain_supported((int)x.dtype, x.dims[0], x.dims[1], w.dims[1], dual, in.norm)) return 0;
+        if (!k::chain_supported((int)x.dtype, x.dims[0], x.dims[1], w.dims[1], dual, in.norm, in.quant)) return 0;
         k::ChainPhase p{};
-        return k::chain_fill_phase(p, x.dims[1], w.dims[1], dual) ? 1 : 0;
+        return k::chain_fill_phase(p, x.dims[1], w.dims[1], dual, in.quant) ? 1 : 0;
     };
     for (int s = 0; s < n_steps;) {
         int np = chain_phases(plan.steps[s]);
         if (!np) { ++s; continue; }
         int e = s + 1;
         bool has_linear = plan.steps[s].in.op == OpKind::FLinear;
+        int fmt = has_linear ? plan.steps[s].in.quant : -1;   // one weight format per launch
         while (e < n_steps) {
-            const int q = chain_phases(plan.steps[e]);
+            const Step& nx = plan.steps[e];
+            const int q = chain_phases(nx);
             if (!q || np + q > k::kChainMaxPhases) break;
+            if (nx.in.op == OpKind::FLinear) {
+                if (fmt >= 0 && nx.in.quant != fmt) break;
+                fmt = nx.in.quant;
+                has_linear = true;
+            }
             np += q;
-            has_linear = has_linear || plan.steps[e].in.op == OpKind::FLinear;
             ++e;
         }
         if (has_linear) {   // an attention on its own keeps its stand-alone kernels
@@ -731,13 +799,20 @@ static inline const void* src_ptr(const Step& st, const ExecCtx& cx, size_t i) {
     return st.src[i] >= 0 ? cx.ptr[st.src[i]] : (const void*)(cx.consts + st.src_const[i]);
 }
 
+// algorithmic bytes of the weights an FLinear reads once: codes and scales when quantised
+static int64_t linear_weight_bytes(const Instr& in, const Spec& x, const Spec& w) {
+    const int64_t K = x.dims[1], N = w.dims[1], es = (int64_t)dtype_size(x.dtype);
+    int64_t b = in.quant == 0 ? K * N * es : (in.quant == 1 ? K * N + N * es : K * N / 2 + (K / 128) * N * es);
+    return b * (in.act == 2 ? 2 : 1);
+}
+
 // One persistent launch for the steps [st, st + chain_len): builds the phase table from the resolved
 // pointers, fetches its cached device copy and launches.  false: the caller runs the steps one by one
 // (cx.chain is cleared so the members run too).
 static bool run_chain(const Plan& plan, const Step& head, ExecCtx& cx) {
     std::vector<k::ChainPhase> phases;
     phases.reserve((size_t)head.chain_len * 2);
-    int lds_bytes = 0;
+    int lds_bytes = 0, wfmt = k::kChainW16;
     int64_t bytes = 0;
     auto aligned8 = [](std::initializer_list<const void*> ps) {
         for (const void* q : ps) if ((uintptr_t)q & 7) fail_exec("decode chain: operand buffers must be 8-byte aligned");
@@ -767,7 +842,7 @@ static bool run_chain(const Plan& plan, const Step& head, ExecCtx& cx) {
             aligned8({pa.x, pa.part, pc.y});
             if (((uintptr_t)kout | (uintptr_t)vout | (uintptr_t)pa.cos | (uintptr_t)pa.sin) & 15)
                 fail_exec("decode chain: cache and RoPE buffers must be 16-byte aligned");
-            lds_bytes = std::max(lds_bytes, std::max(pa.lds_bytes, pc.lds_bytes));
+            lds_bytes = std::max(lds_bytes, std::max(pa.lds_total, pc.lds_total));
             phases.push_back(pa);
             phases.push_back(pc);
             continue;
@@ -776,20 +851,30 @@ static bool run_chain(const Plan& plan, const Step& head, ExecCtx& cx) {
         const Spec& w = plan.values[st.src[1]].spec;
         const bool dual = in.act == 2;
         k::ChainPhase p{};
-        if (!k::chain_fill_phase(p, x.dims[1], w.dims[1], dual)) { cx.chain = false; return false; }
-        BufferP wc = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], 2, x.dtype, x.dims[1], w.dims[1],
-                                            dual ? cx.input_bufs[st.tiled_w2_input] : nullptr);
+        if (!k::chain_fill_phase(p, x.dims[1], w.dims[1], dual, in.quant)) { cx.chain = false; return false; }
+        wfmt = in.quant;
+        BufferP wc = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], in.quant == 0 ? 2 : (in.quant == 1 ? 3 : 4), x.dtype,
+                                            x.dims[1], w.dims[1], dual ? cx.input_bufs[st.tiled_w2_input] : nullptr);
         p.w = wc->ptr;
         p.x = src_ptr(st, cx, 0);
-        size_t oi = dual ? 3 : 2;
+        if (in.quant == 1) {         // per-column scales are read as they are
+            p.wscale = src_ptr(st, cx, 2);
+            if (dual) p.wscale2 = src_ptr(st, cx, 4);
+            if (((uintptr_t)p.wscale | (uintptr_t)p.wscale2) & 3) fail_exec("decode chain: scale buffers must be 4-byte aligned");
+        } else if (in.quant == 2) {  // group scales follow the tile order of the weights
+            BufferP sc = cx.be->derived_weights(cx.input_bufs[st.tiled_s_input], 5, x.dtype, x.dims[1], w.dims[1],
+                                                dual ? cx.input_bufs[st.tiled_s2_input] : nullptr);
+            p.wscale = sc->ptr;
+        }
+        size_t oi = linear_extra_pos(in);
         if (in.has_bias) { p.bias = src_ptr(st, cx, oi++); p.flags |= k::kChainBias; }
         if (in.has_residual) { p.residual = src_ptr(st, cx, oi++); p.flags |= k::kChainResidual; }
         if (in.norm) { p.gamma = src_ptr(st, cx, oi++); p.inv_n = in.scale; p.eps = in.eps; p.flags |= k::kChainNorm; }
         if (in.act == 1) p.flags |= k::kChainGelu;
         p.y = cx.ptr[st.dst[0]];
         aligned8({p.x, p.y, p.residual, p.bias, p.gamma});
-        lds_bytes = std::max(lds_bytes, p.lds_bytes);
-        bytes += (int64_t)dtype_size(x.dtype) * (x.dims[1] + x.dims[1] * w.dims[1] * (dual ? 2 : 1) + w.dims[1]);
+        lds_bytes = std::max(lds_bytes, p.lds_total);
+        bytes += (int64_t)dtype_size(x.dtype) * (x.dims[1] + w.dims[1]) + linear_weight_bytes(in, x, w);
         phases.push_back(p);
     }
     const k::ChainPhase* table = cx.be->chain_table(phases);
@@ -800,7 +885,7 @@ static bool run_chain(const Plan& plan, const Step& head, ExecCtx& cx) {
         GPTRS_HIP_CHECK(hipEventCreate(&e1));
         GPTRS_HIP_CHECK(hipEventRecord(e0, cx.stream));
     }
-    if (!k::chain_launch(cx.stream, table, (int)phases.size(), lds_bytes, cx.be->chain_barrier(), cx.be->chain_abort_flag())) {
+    if (!k::chain_launch(cx.stream, table, (int)phases.size(), lds_bytes, cx.be->chain_barrier(), cx.be->chain_abort_flag(), wfmt)) {
         if (e0) { (void)hipEventDestroy(e0); (void)hipEventDestroy(e1); }
         cx.chain = false;
         return false;
@@ -947,14 +1032,17 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
                 k::MfmaLinearArgs ma{};
                 ma.x = src_ptr(st, cx, 0);
                 ma.m = x.dims[0]; ma.k = x.dims[1]; ma.n = w.dims[1];
-                BufferP wk = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], 1, x.dtype, ma.k, ma.n);
+                // quantised weights: the k-grouped copy is built once from the dequantised matrix
+                const int kind = in.quant == 0 ? 1 : (in.quant == 1 ? 6 : 7);
+                BufferP wk = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], kind, x.dtype, ma.k, ma.n,
+                                                    in.quant ? cx.input_bufs[st.tiled_s_input] : nullptr);
                 BufferP wk2;
                 ma.wk = wk->ptr;
-                size_t oi = 2;
+                size_t oi = linear_extra_pos(in);
                 if (in.act == 2) {
-                    wk2 = cx.be->derived_weights(cx.input_bufs[st.tiled_w2_input], 1, x.dtype, ma.k, ma.n);
+                    wk2 = cx.be->derived_weights(cx.input_bufs[st.tiled_w2_input], kind, x.dtype, ma.k, ma.n,
+                                                 in.quant ? cx.input_bufs[st.tiled_s2_input] : nullptr);
                     ma.wk2 = wk2->ptr;
-                    ++oi;
                 }
                 if (in.has_bias) ma.bias = src_ptr(st, cx, oi++);
                 if (in.has_residual) ma.residual = src_ptr(st, cx, oi++);
@@ -971,12 +1059,12 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
                     GPTRS_HIP_CHECK(hipEventRecord(e1, s));
                     cx.be->prof_events.emplace_back(e0, e1);
                     ++cx.be->prof_linear_calls;
-                    cx.be->prof_linear_bytes += (int64_t)dtype_size(x.dtype) * (ma.m * ma.k + ma.k * ma.n * (ma.wk2 ? 2 : 1) + ma.m * ma.n);
+                    cx.be->prof_linear_bytes += (int64_t)dtype_size(x.dtype) * (ma.m * ma.k + ma.m * ma.n) + linear_weight_bytes(in, x, w);
                 }
                 ++cx.launches;
                 break;
             }
-            if (in.tiled) {
+            if (in.tiled && !in.quant) {
                 k::TiledLinearArgs ta{};
                 ta.dtype = (int)x.dtype;
                 ta.x = src_ptr(st, cx, 0);
@@ -1015,15 +1103,41 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
             a.dtype = (int)x.dtype;
             a.x = src_ptr(st, cx, 0);
             a.w = src_ptr(st, cx, 1);
-            size_t i = 2;
-            if (in.act == 2) a.w2 = src_ptr(st, cx, i++);
+            a.m = x.dims[0]; a.k = x.dims[1]; a.n = w.dims[1];
+            a.ws = cx.ws + st.scratch_off;
+            a.ws_bytes = st.scratch_bytes;
+            size_t i = linear_extra_pos(in);
+            if (in.quant) {
+                // stand-alone path of a quantised linear: the weights are dequantised into scratch and the generic
+                // kernel runs over them (the decode chain and the cached MFMA copy are the fast paths)
+                const size_t es = dtype_size(x.dtype);
+                char* wsp = cx.ws + st.scratch_off;
+                const size_t wbytes = align_up((size_t)a.k * a.n * es);
+                auto deq = [&](size_t codes, size_t scales, void* to) {
+                    if (in.quant == 1) k::dequant_w8(s, (int)x.dtype, (const int8_t*)src_ptr(st, cx, codes), src_ptr(st, cx, scales), to, a.k, a.n);
+                    else k::dequant_w4g128(s, (int)x.dtype, (const uint8_t*)src_ptr(st, cx, codes), src_ptr(st, cx, scales), to, a.k, a.n);
+                    ++cx.launches;
+                };
+                if (in.norm) {
+                    const size_t gi = i + (in.has_bias ? 1 : 0) + (in.has_residual ? 1 : 0);
+                    k::rms_norm(s, (int)x.dtype, a.x, src_ptr(st, cx, gi), wsp, a.m, a.k, in.scale, in.eps);
+                    ++cx.launches;
+                    a.x = wsp;
+                    wsp += align_up((size_t)x.count() * es);
+                }
+                deq(1, 2, wsp);
+                a.w = wsp;
+                wsp += wbytes;
+                if (in.act == 2) { deq(3, 4, wsp); a.w2 = wsp; wsp += wbytes; }
+                a.ws = wsp;
+                a.ws_bytes = st.scratch_bytes - (size_t)(wsp - (cx.ws + st.scratch_off));
+            } else if (in.act == 2) {
+                a.w2 = src_ptr(st, cx, 2);
+            }
             if (in.has_bias) a.bias = src_ptr(st, cx, i++);
             if (in.has_residual) a.residual = src_ptr(st, cx, i++);
             a.y = dst;
-            a.m = x.dims[0]; a.k = x.dims[1]; a.n = w.dims[1];
             a.act = in.act == 1 ? 1 : 0;
-            a.ws = cx.ws + st.scratch_off;
-            a.ws_bytes = st.scratch_bytes;
             a.counters = cx.counters;
             hipEvent_t e0 = nullptr, e1 = nullptr;
             if (cx.profile) {
@@ -1037,9 +1151,28 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
                 cx.be->prof_events.emplace_back(e0, e1);
                 ++cx.be->prof_linear_calls;
                 // algorithmic bytes: activations in, every weight once, result out
-                cx.be->prof_linear_bytes += (int64_t)dtype_size(x.dtype) * (a.m * a.k + a.k * a.n * (a.w2 ? 2 : 1) + a.m * a.n);
+                cx.be->prof_linear_bytes += (int64_t)dtype_size(x.dtype) * (a.m * a.k + a.m * a.n) + linear_weight_bytes(in, x, w);
             }
             cx.launches += (in.act == 2 && a.m > 16) ? 3 : 1;
+            break;
+        }
+        case OpKind::FQuant: {
+            const int qo = in.quant;
+            if (qo == 1 || qo == 3) {
+                const Spec& w = in_spec(0);
+                (qo == 1 ? k::quant_w8_scales : k::quant_w4g128_scales)(s, (int)w.dtype, src_ptr(st, cx, 0), dst, w.dims[0], w.dims[1]);
+            } else if (qo == 2) {
+                const Spec& w = in_spec(0);
+                k::quant_w8(s, (int)w.dtype, src_ptr(st, cx, 0), src_ptr(st, cx, 1), (int8_t*)dst, w.dims[0], w.dims[1]);
+            } else if (qo == 4) {
+                const Spec& w = in_spec(0);
+                k::quant_w4g128(s, (int)w.dtype, src_ptr(st, cx, 0), src_ptr(st, cx, 1), (uint8_t*)dst, w.dims[0], w.dims[1]);
+            } else if (qo == 5) {
+                k::dequant_w8(s, (int)out.dtype, (const int8_t*)src_ptr(st, cx, 0), src_ptr(st, cx, 1), dst, out.dims[0], out.dims[1]);
+            } else {
+                k::dequant_w4g128(s, (int)out.dtype, (const uint8_t*)src_ptr(st, cx, 0), src_ptr(st, cx, 1), dst, out.dims[0], out.dims[1]);
+            }
+            ++cx.launches;
             break;
         }
         case OpKind::FRope: {

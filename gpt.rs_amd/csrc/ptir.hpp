@@ -71,7 +71,7 @@ enum class OpKind {
     BroadcastTo, Slice, Concat, Iota, Take, DynamicSlice, DynamicUpdateSlice, CustomCall,
     // fused forms produced by the executor's pattern pass (never present on the wire)
     FLayerNorm, FRmsNorm, FSoftmax, FGelu, FSilu, FSwiglu, FLinear, FRope, FAttnDecode, FAttnPrefill,
-    FEmbed,
+    FEmbed, FQuant,
     Unsupported
 };
 enum class UnaryOp { Neg, Abs, Exp, Log, Tanh, Erf, Rsqrt, Reciprocal };
@@ -114,9 +114,32 @@ struct Instr {
     bool mfma = false;                       // FLinear: prefill GEMM over the k-grouped weight copy
     bool tiled = false;                      // FLinear: decode GEMV over the column-tiled weight copy
     bool norm = false;                       // FLinear: RMSNorm of x fused in (last operand = gamma; eps, scale)
+    // FLinear over weight-only quantised weights (0: none; 1: int8 per column, 2: int4 groups of 128): every
+    // weight operand is then a (codes, scales) pair: (x, q, s, [q2, s2], [bias], [residual], [gamma]).
+    // FQuant: 1 int8 scales, 2 int8 codes, 3 int4 scales, 4 int4 codes, 5 int8 dequantise, 6 int4 dequantise
+    int quant = 0;
     bool scalar_rhs = false;                 // Binary whose rhs is a broadcast scalar literal
     float scalar_val = 0.f;
 };
+
+// operand position of the SwiGLU partner's weights / of the first epilogue operand of an FLinear
+inline size_t linear_w2_pos(const Instr& in) { return in.quant ? 3 : 2; }
+inline size_t linear_extra_pos(const Instr& in) { return 1 + (size_t)(in.quant ? 2 : 1) * (in.act == 2 ? 2 : 1); }
+// CustomCall targets of the weight-only quantisation extension (build-defined; the reference has none)
+inline int quant_dot_target(const std::string& t) {
+    if (t == "gpt_rs.hip.dot_w8.v1") return 1;
+    if (t == "gpt_rs.hip.dot_w4g128.v1") return 2;
+    return 0;
+}
+inline int quant_op_target(const std::string& t) {
+    if (t == "gpt_rs.hip.quantize_w8_scales.v1") return 1;
+    if (t == "gpt_rs.hip.quantize_w8.v1") return 2;
+    if (t == "gpt_rs.hip.quantize_w4g128_scales.v1") return 3;
+    if (t == "gpt_rs.hip.quantize_w4g128.v1") return 4;
+    if (t == "gpt_rs.hip.dequantize_w8.v1") return 5;
+    if (t == "gpt_rs.hip.dequantize_w4g128.v1") return 6;
+    return 0;
+}
 
 struct Function {
     std::string name;

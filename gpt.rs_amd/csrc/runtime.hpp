@@ -98,6 +98,7 @@ struct Step {
     bool copy_base = false;        // DynamicUpdateSlice / FAttnDecode: copy base -> out first
     bool lhs_pack = false, rhs_pack = false;    // Dot: operands repacked into scratch first
     int tiled_w_input = -1, tiled_w2_input = -1;  // FLinear over column-tiled weights: input positions of W, W2
+    int tiled_s_input = -1, tiled_s2_input = -1;  // ... and of their scale tensors when the weights are quantised
     // Run of consecutive decode linears executed by ONE persistent launch (kernels_chain.hip): the
     // first step of the run carries its length, the others are marked as members.
     int chain_len = 0;
@@ -167,6 +168,9 @@ class Backend {
     // GEMV (kernels_gemv_tiled.hip); kind 1: k-grouped copy for the MFMA GEMM (kernels_mfma.hip).
     // kind 2: 4-column / k-pair tiled copy for the persistent decode chain (kernels_chain.hip); with
     // src2 the SwiGLU pair (gate = src, up = src2) interleaved column by column in one copy.
+    // Quantised weights: kind 3 / 4: chain copies of int8 / int4 codes (src2: the partner's codes); kind 5:
+    // chain copy of int4 group scales (src2: the partner's); kind 6 / 7: MFMA copy of the dequantised int8 /
+    // int4 matrix (src = codes, src2 = scales).
     BufferP derived_weights(const BufferP& src, int kind, DType dtype, int64_t k, int64_t n, const BufferP& src2 = nullptr);
     // Device copy of a chain's phase table, cached by content (steady-state decode repeats a few tables).
     const k::ChainPhase* chain_table(const std::vector<k::ChainPhase>& phases);

@@ -14,7 +14,7 @@ from typing import Optional, Tuple
 
 import numpy as np
 
-from .ptir import Tensor
+from .ptir import Tensor, TensorSpec
 
 
 # --------------------------------------------------------------------------- basics
@@ -35,6 +35,66 @@ def linear(x: Tensor, weight: Tensor, bias: Optional[Tensor] = None) -> Tensor:
     if x.dims[1] != weight.dims[0]:
         raise ValueError(f"input features ({x.dims[1]}) must match weight rows ({weight.dims[0]})")
     out = matmul(x, weight)
+    if bias is not None:
+        out = add_bias(out, bias)
+    return out
+
+
+# --------------------------------------------------------------------------- weight-only quantisation
+# Build-defined extension (the reference has no quantisation scheme: docs/backend.md:620-632 leaves
+# Quantize/Dequantize backend-defined and ref-cpu answers Unimplemented).  Two symmetric schemes:
+#   "w8":     int8, one scale per output column:  s_n = bf16(max_k |W[k,n]| / 127), q = clamp(rint(W / s_n), +-127)
+#   "w4g128": int4, groups of 128 along K:        s[g,n] = bf16(max |w| / 7), q in [-7, 7], two codes per byte
+#             along K: byte[k/2, n] = (q[k] & 0xF) | ((q[k+1] & 0xF) << 4)
+# Scales carry the float dtype of the weights they came from.
+QUANT_SCHEMES = ("w8", "w4g128")
+
+
+def _scheme(scheme: str) -> str:
+    if scheme not in QUANT_SCHEMES:
+        raise ValueError(f"unknown quantisation scheme {scheme!r}; expected one of {QUANT_SCHEMES}")
+    return scheme
+
+
+def quantize_weight(w: Tensor, scheme: str) -> Tuple[Tensor, Tensor]:
+    """(codes, scales) of W[K,N] in `scheme`, computed on the device."""
+    _scheme(scheme)
+    if w.spec.rank != 2:
+        raise ValueError(f"quantize_weight expects a matrix, got shape {w.dims}")
+    K, N = w.dims
+    if scheme == "w8":
+        s = w.fb.custom_call("gpt_rs.hip.quantize_w8_scales.v1", [w], TensorSpec(w.dtype, [N]))
+        q = w.fb.custom_call("gpt_rs.hip.quantize_w8.v1", [w, s], TensorSpec("Si8", [K, N]))
+    else:
+        if K % 128:
+            raise ValueError(f"w4g128 needs K to be a multiple of 128, got {K}")
+        s = w.fb.custom_call("gpt_rs.hip.quantize_w4g128_scales.v1", [w], TensorSpec(w.dtype, [K // 128, N]))
+        q = w.fb.custom_call("gpt_rs.hip.quantize_w4g128.v1", [w, s], TensorSpec("Ui8", [K // 2, N]))
+    return q, s
+
+
+def dequantize_weight(q: Tensor, s: Tensor) -> Tensor:
+    """W[K,N] = codes * scales in the scales' dtype; the scheme follows from the code dtype."""
+    if q.dtype == "Si8":
+        return q.fb.custom_call("gpt_rs.hip.dequantize_w8.v1", [q, s], TensorSpec(s.dtype, q.dims))
+    if q.dtype == "Ui8":
+        return q.fb.custom_call("gpt_rs.hip.dequantize_w4g128.v1", [q, s], TensorSpec(s.dtype, [q.dims[0] * 2, q.dims[1]]))
+    raise ValueError(f"codes must be Si8 (w8) or Ui8 (w4g128), got {q.dtype}")
+
+
+def linear_quantized(x: Tensor, q: Tensor, s: Tensor, bias: Optional[Tensor] = None) -> Tensor:
+    """x[T,K] . dequantise(q, s)[K,N] (+ b) without materialising the matrix: f32 accumulation, result in x's dtype."""
+    if x.spec.rank != 2:
+        raise ValueError(f"linear expects 2D input, got shape {x.dims}")
+    if q.dtype == "Si8":
+        target, k = "gpt_rs.hip.dot_w8.v1", q.dims[0]
+    elif q.dtype == "Ui8":
+        target, k = "gpt_rs.hip.dot_w4g128.v1", q.dims[0] * 2
+    else:
+        raise ValueError(f"codes must be Si8 (w8) or Ui8 (w4g128), got {q.dtype}")
+    if x.dims[1] != k:
+        raise ValueError(f"input features ({x.dims[1]}) must match weight rows ({k})")
+    out = x.fb.custom_call(target, [x, q, s], TensorSpec(x.dtype, [x.dims[0], q.dims[1]]))
     if bias is not None:
         out = add_bias(out, bias)
     return out

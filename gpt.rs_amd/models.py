@@ -98,6 +98,42 @@ class _ModelBase:
         self.param_specs[name] = spec
         self._param_handles = None
 
+    def set_param_handle(self, name: str, handle):
+        """Register a tensor that already lives on the device."""
+        self.backend.param_resolver().set(param_id(self.namespace, name), handle)
+        if name not in self.param_specs:
+            self.param_names.append(name)
+        self.param_specs[name] = handle.spec
+        self._param_handles = None
+        self._programs.clear()
+
+    def drop_param(self, name: str):
+        """Forget a parameter and release its device memory (the memo keeps a 1-element stand-in)."""
+        spec = self.param_specs.pop(name)
+        self.param_names.remove(name)
+        stub = self.backend.materialize(TensorSpec(spec.dtype, [1]), None)
+        self.backend.param_resolver().set(param_id(self.namespace, name), stub)
+        self._param_handles = None
+        self._programs.clear()
+
+    _quant_programs: Dict[tuple, Program] = {}
+
+    def quantize_param(self, name: str, scheme: str):
+        """Replace the matrix `name` by `name.q` (codes) and `name.s` (scales), quantised on the device
+        (functional.quantize_weight); layers that find `name.q` read the codes directly."""
+        spec = self.param_specs[name]
+        key = (scheme, spec.dtype, tuple(spec.dims))
+        prog = _ModelBase._quant_programs.get(key)
+        if prog is None:
+            fb = FunctionBuilder("main", spec.dtype)
+            q, s = F.quantize_weight(fb.param(spec.dtype, spec.dims), scheme)
+            fb.set_results([q, s])
+            prog = _ModelBase._quant_programs[key] = Program(fb)
+        q, s = self.backend.run_program(prog, [self.param_handle(name)])
+        self.drop_param(name)
+        self.set_param_handle(name + ".q", q)
+        self.set_param_handle(name + ".s", s)
+
     def param_handle(self, name: str):
         h = self.backend.param_resolver().get(param_id(self.namespace, name))
         if h is None:
@@ -379,12 +415,13 @@ class Ministral(_ModelBase):
 
     @classmethod
     def random(cls, config: MinistralConfig, backend, seed: int = 0, dtype: str = "Bf16", std: float = 0.02,
-               bf16_values: bool = False):
+               bf16_values: bool = False, quant: Optional[str] = None):
         """Shapes and constant inits of Ministral::random (model/ministral.rs:262-330).  Every
         tensor draws from its own numpy stream SeedSequence([seed, index]), so the weights do not
         depend on the order or the number of worker threads that generate them.  `bf16_values`
         rounds the draws to bf16-representable values whatever the storage dtype, so an f32
-        model can be given exactly the weights of a bf16 one."""
+        model can be given exactly the weights of a bf16 one.  `quant` ("w8" / "w4g128") quantises
+        every linear weight (projections, feed-forward, lm_head) as it arrives on the device."""
         from concurrent.futures import ThreadPoolExecutor
         m = cls(config, backend, dtype)
         d, a = config.embed_dim, config.attention_config()
@@ -421,7 +458,19 @@ class Ministral(_ModelBase):
                     nxt += 1
                 name, shape, data = pending.pop(0).result()
                 m.set_param_bytes(name, TensorSpec(dtype, shape), data)
+                if quant and len(shape) == 2 and name != "tok_embeddings.weight":
+                    m.quantize_param(name, quant)
         return m
+
+    QUANTIZABLE = ("attention.w_qkv", "attention.w_out", "feed_forward.w_gate", "feed_forward.w_up",
+                   "feed_forward.w_down", "lm_head")
+
+    def quantize(self, scheme: str):
+        """Weight-only quantisation of every linear weight of a loaded model, in place."""
+        for name in list(self.param_names):
+            if name.endswith(self.QUANTIZABLE) and len(self.param_specs[name].dims) == 2:
+                self.quantize_param(name, scheme)
+        return self
 
     @property
     def num_layers(self): return self.config.num_layers
@@ -429,7 +478,9 @@ class Ministral(_ModelBase):
     def context_length(self): return self.config.context_length
 
     def _linear(self, P, name: str, x: Tensor) -> Tensor:
-        """nn/layers/linear.rs:50-71 without bias.  Subclasses swap in quantized weights."""
+        """nn/layers/linear.rs:50-71 without bias; quantised weights are read as codes and scales."""
+        if name + ".q" in P:
+            return F.linear_quantized(x, P[name + ".q"], P[name + ".s"])
         return F.linear(x, P[name])
 
     def _build(self, seq: int, capacity: int, decode: bool, batch: int = 1) -> Tuple[Program, dict]:
@@ -487,7 +538,7 @@ class Ministral(_ModelBase):
             ff = self._linear(P, p + "feed_forward.w_down", act)
             hidden = ff + residual
         normalized, *_ = F.rms_norm(hidden, P["final_norm.gamma"], cfg.eps)
-        logits = normalized.matmul(P["lm_head"])
+        logits = self._linear(P, "lm_head", normalized)
         results = []
         for b in range(batch):
             for i in range(L):

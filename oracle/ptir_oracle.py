@@ -421,6 +421,18 @@ def _custom_call(target: str, attrs, ins: List[OTensor], out_dtype: str, out_dim
     elif target == "gpt_rs.hip.dot_w4g128.v1":
         x, q, s = ins
         w = dequantize_int4_g128(q.a, s.a)
+    elif target in ("gpt_rs.hip.quantize_w8_scales.v1", "gpt_rs.hip.quantize_w4g128_scales.v1"):
+        (w,) = ins
+        s = (quantize_int8_per_channel if "w8" in target else quantize_int4_g128)(w.a)[1]
+        return _finish(out_dtype, s)           # bf16-representable either way: the store is exact
+    elif target in ("gpt_rs.hip.quantize_w8.v1", "gpt_rs.hip.quantize_w4g128.v1"):
+        w = ins[0]                              # the scales operand is by definition the scheme's own
+        q = (quantize_int8_per_channel if "w8" in target else quantize_int4_g128)(w.a)[0]
+        return OTensor(out_dtype, q)
+    elif target == "gpt_rs.hip.dequantize_w8.v1":
+        return _finish(out_dtype, dequantize_int8(ins[0].a, ins[1].a))
+    elif target == "gpt_rs.hip.dequantize_w4g128.v1":
+        return _finish(out_dtype, dequantize_int4_g128(ins[0].a, ins[1].a))
     else:
         raise OracleError("unimplemented", f"custom_call target {target}")
     # reference semantics for "dequantize + dot_general": f32 accumulate, output rounded
