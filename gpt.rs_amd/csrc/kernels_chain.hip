@@ -711,6 +711,45 @@ __device__ void control_wave(Shared& sh, unsigned* xs, int nphases, unsigned* ba
     if (blk == 0 && lane == 0) gstore(bar + NC * 64, epoch + (unsigned)nphases * per);
 }
 
+// Sums each of a wave's 12 per-lane accumulators (3 tiles x 4 columns) over its 64 lanes as a
+// reduce-scatter: exchanging half of the values with lane ^ 32 and then lane ^ 16 leaves every 16-lane row
+// with 3 values already summed over 4 lanes, which 4 row-wide DPP steps finish: 30 cross-lane operations where
+// 12 separate wave sums take 120.  Returns in lanes 16r + s (s < 3) the total of accumulator 3r + s, i.e.
+// element 3r + s of acc[p][c] taken as acc[0][0..3], acc[1][0..3], acc[2][0..3].
+__device__ __forceinline__ float reduce_unit(const float (&acc)[TP][4], int lane) {
+    static_assert(TP == 3, "12 accumulators per lane");
+    float v[12];
+#pragma unroll
+    for (int p = 0; p < TP; ++p)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) v[p * 4 + c] = acc[p][c];
+    float h[6];
+#pragma unroll
+    for (int k = 0; k < 6; ++k) {   // lanes < 32 keep values 0..5, lanes >= 32 values 6..11
+        const u32x2 sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[k]), __float_as_uint(v[k + 6]), false, false);
+        h[k] = __uint_as_float(sw.x) + __uint_as_float(sw.y);
+    }
+    float q[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {   // even rows keep values k, odd rows values k + 3 of their half
+        const u32x2 sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(h[k]), __float_as_uint(h[k + 3]), false, false);
+        q[k] = __uint_as_float(sw.x) + __uint_as_float(sw.y);
+    }
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        int x = __float_as_int(q[k]);
+#define GPTRS_DPP_ADD(ctrl) x = __float_as_int(__int_as_float(x) + __int_as_float(__builtin_amdgcn_update_dpp(0, x, (ctrl), 0xf, 0xf, false)))
+        GPTRS_DPP_ADD(0xB1);    // quad_perm [1,0,3,2]
+        GPTRS_DPP_ADD(0x4E);    // quad_perm [2,3,0,1]
+        GPTRS_DPP_ADD(0x141);   // row_half_mirror
+        GPTRS_DPP_ADD(0x140);   // row_mirror
+#undef GPTRS_DPP_ADD
+        q[k] = __int_as_float(x);
+    }
+    const int sidx = lane & 15;
+    return sidx == 0 ? q[0] : (sidx == 1 ? q[1] : q[2]);
+}
+
 // ---------------------------------------------------------------------------- streaming waves
 template <int FMT>
 __device__ void stream_waves(Shared& sh, const unsigned* xs, int nphases) {
@@ -864,21 +903,17 @@ __device__ void stream_waves(Shared& sh, const unsigned* xs, int nphases) {
         }
         if (++c_j == c_wpt) {
             const int slot = ucount % NSLOT;
-            float v = 0.f;
+            const float v = reduce_unit(acc, lane);
 #pragma unroll
             for (int p = 0; p < TP; ++p)
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const float a = wave_sum(acc[p][c]);
-                    if (lane == p * 4 + c) v = a;
-                    acc[p][c] = 0.f;
-                }
+                for (int c = 0; c < 4; ++c) acc[p][c] = 0.f;
             unsigned spins = 0;
             while (uni(lds_ld(&sh.consumed)) < ucount - NSLOT + 1) {
                 __builtin_amdgcn_s_sleep(1);
                 if (uni(lds_ld(&sh.abort)) || ++spins > (1u << 24)) return;
             }
-            if (lane < TP * 4) sh.red[slot][wave][lane] = v;
+            if ((lane & 15) < 3) sh.red[slot][wave][3 * (lane >> 4) + (lane & 15)] = v;
             GPTRS_LDS_RELEASE();
             if (lane == 0) __hip_atomic_fetch_add(&sh.red_cnt[slot], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             ++ucount;
