@@ -4,6 +4,8 @@
 // Both compute softmax((q.k) * scale + mask) . v with the additive -1e9 mask replaced by its
 // exact f32 effect: masked positions contribute exactly 0 (exp underflows), so only positions
 // <= the query position are visited.  GQA: query head h reads kv head h / group.
+#include <cstdlib>
+
 #include "kernels.hpp"
 #include "device_utils.hpp"
 
@@ -364,8 +366,183 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const T* __restrict__
         if (d < dh) stf(ctx, i * (int64_t)n_q * dh + (int64_t)h * dh + d, o[c] / l);
     }
 }
+// bf16 prefill attention on the matrix cores (flash-attention style, causal, grouped-query).
+//
+// A workgroup (4 waves) serves one kv head and up to 4 query heads of its group over 32 query rows each, so a key /
+// value tile staged in LDS is used by every query head that shares it and all waves see the same causal range.  Per
+// tile of 32 keys a wave computes with v_mfma_f32_32x32x16_bf16
+//   S^T[key, q] = K[key, :] . Q[q, :]      (A = K rows from LDS, B = Q fragments kept in registers)
+//   O^T[d, q]  += V^T[d, key] . P^T[key, q] (A = V^T from LDS, B = the probabilities just computed, from registers)
+// Both products are taken transposed so that a lane always owns ONE query (column lane % 32): the 16 scores a lane
+// holds belong to its query, the online-softmax state (running maximum and sum, in the log2 domain) is a per-lane
+// scalar, the rescaling of O^T is a per-lane multiply, and P^T needs no cross-lane movement to become the B operand:
+// the k-slots of the second product are simply numbered in the order the lane holds its keys, and V^T is written to
+// LDS in that order (key bits 2 and 3 swapped).
+typedef __bf16 bf16x8_v __attribute__((ext_vector_type(8)));
+typedef float f32x16_v __attribute__((ext_vector_type(16)));
+
+template <int DH>
+__global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ctx, int T,
+                                                                int n_q, int n_kv, float scale_log2e) {
+    constexpr int KT = 32;            // keys per tile
+    constexpr int KS = DH + 8;        // K tile row stride in elements (16 bytes of padding)
+    constexpr int VS = KT + 8;        // V^T row stride in elements
+    constexpr int ND = DH / 32;       // 32-row blocks of d in O^T
+    constexpr int NK = DH / 16;       // k-steps of the score product
+    constexpr int CH = KT * DH / 8;   // 16-byte chunks of a K (or V) tile
+    constexpr int CPT = (CH + 255) / 256;
+    __shared__ __align__(16) bf16_t ksm[2][KT * KS];
+    __shared__ __align__(16) bf16_t vsm[2][DH * VS];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, half = lane >> 5;
+    const int G = n_q / n_kv;
+    const int gw = G >= 4 ? 4 : G;                 // query heads of the group in this workgroup
+    const int rtpb = 4 / gw;                       // 32-row tiles per workgroup
+    const int kvh = blockIdx.y;
+    const int head = kvh * G + blockIdx.z * gw + wave % gw;
+    const int q0 = (blockIdx.x * rtpb + wave / gw) * 32;
+    const int64_t P = (int64_t)(n_q + 2 * n_kv) * DH;
+    const int64_t koff = (int64_t)n_q * DH + (int64_t)kvh * DH;
+    const int64_t voff = (int64_t)(n_q + n_kv) * DH + (int64_t)kvh * DH;
+    const int kend = min(T, (blockIdx.x * rtpb + rtpb) * 32);   // keys any row of the workgroup may see
+    const int ntiles = (kend + KT - 1) / KT;
+    const bool active = q0 < T;
+    const int my_tiles = active ? min(ntiles, (q0 + 31) / KT + 1) : 0;   // tiles holding a key <= this wave's last row
+
+    // Q fragments (B operand: column = query, 8 consecutive d per lane and k-step)
+    bf16x8_v qf[NK];
+    {
+        const int row = min(q0 + col, T - 1);
+        const bf16_t* qp = qkv + (int64_t)row * P + (int64_t)head * DH + 8 * half;
+#pragma unroll
+        for (int kk = 0; kk < NK; ++kk) qf[kk] = *reinterpret_cast<const bf16x8_v*>(qp + 16 * kk);
+    }
+    f32x16_v acc_o[ND];
+#pragma unroll
+    for (int db = 0; db < ND; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc_o[db][v] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+
+    uint4 kreg[CPT], vreg[CPT];
+    auto gload = [&](int t) {
+#pragma unroll
+        for (int j = 0; j < CPT; ++j) {
+            const int c = tid + 256 * j;
+            if (CH % 256 == 0 || c < CH) {
+                const int r = c / (DH / 8), ch = c % (DH / 8);
+                const int64_t key = min(t * KT + r, T - 1);
+                kreg[j] = *reinterpret_cast<const uint4*>(qkv + key * P + koff + ch * 8);
+                vreg[j] = *reinterpret_cast<const uint4*>(qkv + key * P + voff + ch * 8);
+            }
+        }
+    };
+    auto lwrite = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < CPT; ++j) {
+            const int c = tid + 256 * j;
+            if (CH % 256 == 0 || c < CH) {
+                const int r = c / (DH / 8), ch = c % (DH / 8);
+                *reinterpret_cast<uint4*>(&ksm[buf][r * KS + ch * 8]) = kreg[j];
+                // key r goes to k-slot position p: bits 2 and 3 of r swapped
+                const int pos = (r & 0x13) | ((r & 4) << 1) | ((r & 8) >> 1);
+                const uint32_t w[4] = {vreg[j].x, vreg[j].y, vreg[j].z, vreg[j].w};
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    vsm[buf][(ch * 8 + e) * VS + pos] = (bf16_t)((w[e >> 1] >> ((e & 1) * 16)) & 0xFFFFu);
+            }
+        }
+    };
+
+    gload(0);
+    lwrite(0);
+    __syncthreads();
+    for (int t = 0; t < ntiles; ++t) {
+        const int buf = t & 1;
+        if (t + 1 < ntiles) gload(t + 1);
+        if (t < my_tiles) {
+            // scores, transposed: rows = keys of the tile, column = this lane's query
+            f32x16_v sc;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) sc[v] = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < NK; ++kk) {
+                const bf16x8_v kf = *reinterpret_cast<const bf16x8_v*>(&ksm[buf][col * KS + 16 * kk + 8 * half]);
+                sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], sc, 0, 0, 0);
+            }
+            const int qrow = q0 + col;
+            const int kbase = t * KT + 4 * half;
+            float mx = -INFINITY;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int key = kbase + 8 * (v >> 2) + (v & 3);
+                const float x = key <= qrow ? sc[v] * scale_log2e : -INFINITY;
+                sc[v] = x;
+                mx = fmaxf(mx, x);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m_run, mx);   // finite from the first tile on: key 0 is visible to every query
+            const float corr = exp2f(m_run - m_new);
+            float ls = 0.f;
+            bf16x8_v pb[2];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const float pv = exp2f(sc[v] - m_new);
+                ls += pv;
+                pb[v >> 3][v & 7] = (__bf16)pv;
+            }
+            ls += __shfl_xor(ls, 32, 64);
+            l_run = l_run * corr + ls;
+            m_run = m_new;
+#pragma unroll
+            for (int db = 0; db < ND; ++db) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc_o[db][v] *= corr;
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    const bf16x8_v vf = *reinterpret_cast<const bf16x8_v*>(&vsm[buf][(db * 32 + col) * VS + 16 * i + 8 * half]);
+                    acc_o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[i], acc_o[db], 0, 0, 0);
+                }
+            }
+        }
+        if (t + 1 < ntiles) lwrite(buf ^ 1);
+        __syncthreads();
+    }
+    if (active && q0 + col < T) {
+        const float inv = 1.0f / l_run;
+        bf16_t* op = ctx + (int64_t)(q0 + col) * n_q * DH + (int64_t)head * DH;
+#pragma unroll
+        for (int db = 0; db < ND; ++db)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const int d = db * 32 + 8 * g4 + 4 * half;
+                const uint32_t lo = pack_bf16x2(acc_o[db][4 * g4 + 0] * inv, acc_o[db][4 * g4 + 1] * inv);
+                const uint32_t hi = pack_bf16x2(acc_o[db][4 * g4 + 2] * inv, acc_o[db][4 * g4 + 3] * inv);
+                *reinterpret_cast<uint2*>(op + d) = make_uint2(lo, hi);
+            }
+    }
+}
+
+static bool attn_prefill_mfma_ok(const AttnPrefillArgs& a) {
+    if (a.dtype != 2 || a.n_kv <= 0 || a.n_q % a.n_kv != 0 || a.t >= (1ll << 30)) return false;
+    if (a.head_dim != 32 && a.head_dim != 64 && a.head_dim != 128) return false;
+    const int64_t g = a.n_q / a.n_kv;
+    return g == 1 || g == 2 || g % 4 == 0;
+}
+
 void attn_prefill(hipStream_t s, const AttnPrefillArgs& a) {
     if (a.t <= 0) return;
+    static const bool use_mfma = [] { const char* e = getenv("GPTRS_HIP_MFMA_ATTN"); return !(e && e[0] == '0'); }();
+    if (use_mfma && attn_prefill_mfma_ok(a)) {
+        const int g = (int)(a.n_q / a.n_kv), gw = g >= 4 ? 4 : g;
+        dim3 grid((unsigned)cdiv(cdiv(a.t, 32), 4 / gw), (unsigned)a.n_kv, (unsigned)(g >= 4 ? g / 4 : 1));
+        const float sl = a.scale * 1.44269504088896f;
+        if (a.head_dim == 32) attn_prefill_mfma_kernel<32><<<grid, 256, 0, s>>>((const bf16_t*)a.qkv, (bf16_t*)a.ctx, (int)a.t, (int)a.n_q, (int)a.n_kv, sl);
+        else if (a.head_dim == 64) attn_prefill_mfma_kernel<64><<<grid, 256, 0, s>>>((const bf16_t*)a.qkv, (bf16_t*)a.ctx, (int)a.t, (int)a.n_q, (int)a.n_kv, sl);
+        else attn_prefill_mfma_kernel<128><<<grid, 256, 0, s>>>((const bf16_t*)a.qkv, (bf16_t*)a.ctx, (int)a.t, (int)a.n_q, (int)a.n_kv, sl);
+        return;
+    }
     dim3 grid((unsigned)cdiv(a.t, 4), (unsigned)a.n_q);
     if (a.dtype == 0)
         attn_prefill_kernel<float><<<grid, 256, 0, s>>>((const float*)a.qkv, (float*)a.ctx, a.t, (int)a.n_q, (int)a.n_kv, (int)a.head_dim, a.scale);

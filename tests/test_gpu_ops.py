@@ -275,6 +275,24 @@ def test_attention_prefill(hip, hq, hkv, dh, seq):
     check_program(hip, p, [qkv])
 
 
+@pytest.mark.parametrize("hq,hkv,dh,seq", [(4, 4, 32, 1), (4, 2, 32, 31), (8, 2, 32, 33), (4, 1, 64, 64), (12, 12, 64, 100),
+                                           (8, 2, 128, 257), (32, 8, 128, 96), (8, 1, 64, 130)])
+def test_attention_prefill_bf16_matrix_cores(hip, hq, hkv, dh, seq):
+    """bf16 prefill attention on the MFMA kernel (head_dim 32/64/128; group sizes 1, 2, 4, 8; sequence lengths
+    around the 32-row / 32-key tile edges) against the f32 oracle on the same bf16-representable input.  The kernel
+    keeps f32 scores and sums and rounds the probabilities to bf16 for the P.V product; the result is stored as bf16."""
+    from gptrs_amd.ptir import f32_to_bf16_bits
+    cfg = F.AttentionConfig(hq * dh, hq, hkv, dh)
+    P = cfg.total_projection_dim
+    qkv = rng_uniform(33, (seq, P))
+    qkv = (f32_to_bf16_bits(qkv).astype(np.uint32) << 16).view(np.float32)
+    got = hip_run(hip, prog(lambda fb, a: list(F.attention(cfg, a, None)), [("Bf16", [seq, P])]), [qkv])
+    want = oracle_run(prog(lambda fb, a: list(F.attention(cfg, a, None)), [("F32", [seq, P])]), [qkv])
+    assert_close(got[0], want[0], atol=1e-2, rtol=1e-2, what="context")
+    for i in (1, 2):   # K and V in cache layout: pure copies
+        assert np.array_equal(np.asarray(got[i], np.float32), want[i])
+
+
 def test_attention_with_concat_cache(hip):
     cfg = F.AttentionConfig(16, 4, 2, 4)
     qkv = rng_uniform(27, (3, cfg.total_projection_dim))
