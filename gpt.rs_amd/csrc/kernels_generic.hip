@@ -2,6 +2,8 @@
 // every instruction no fused kernel claims.  Semantics follow the reference interpreter
 // (crates/gpt-rs-backend-ref-cpu/src/cpu.rs) and docs/backend.md; integer / index ops are
 // bit-exact, float ops compute in f32 and round once to the output dtype.
+#include <cstring>
+
 #include "kernels.hpp"
 #include "device_utils.hpp"
 
@@ -416,65 +418,55 @@ void argmax_last_row(hipStream_t s, int dtype, const void* logits, int64_t rows,
 
 // Temperature sampling, single block: softmax(logits/T) then inverse CDF at u.  The running
 // sum is taken in index order by one wave so the chosen token does not depend on launch shape.
+// Temperature sampling as the reference's device path does it
+// (crates/gpt-rs-backend-triton/src/kernels/sample_temperature_last_axis_f32.triton:24-72): Gumbel-max with a
+// stateless per-index hash of (index ^ seed); the score of index i is logit_i / temperature - log(-log(u_i)), the
+// token is the index of the largest score, the smallest index on ties.  seed = bits(random_u) * 747796405 +
+// 2891336453 (runtime/sampling.rs:98-101).
+__device__ __forceinline__ float gumbel_of(uint32_t idx, uint32_t seed) {
+    uint32_t x = idx ^ seed;
+    x ^= x >> 16;
+    x *= 0x7FEB352Du;
+    x ^= x >> 15;
+    x *= 0x846CA68Bu;
+    x ^= x >> 16;
+    float u = ((float)x + 1.0f) * 2.3283064365386963e-10f;   // f32(1 / 4294967297) = 2^-32
+    u = fmaxf(u, 1e-7f);
+    u = fminf(u, 1.0f - 1e-7f);
+    return -logf(-logf(u));
+}
 template <typename T>
-__global__ void sample_temperature_kernel(const T* __restrict__ row, int64_t n, float inv_t, float u, int64_t* out) {
-    __shared__ float sred[16];
-    __shared__ float s_max, s_sum;
-    float mx = -INFINITY;
-    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) mx = fmaxf(mx, ldf(row, i) * inv_t);
-    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_down(mx, off, 64));
-    if ((threadIdx.x & 63) == 0) sred[threadIdx.x >> 6] = mx;
+__global__ void sample_temperature_kernel(const T* __restrict__ row, int64_t n, float inv_t, uint32_t seed, int64_t* out) {
+    __shared__ float s_score[16];
+    __shared__ int64_t s_idx[16];
+    float best = -INFINITY;
+    int64_t best_i = 0;
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+        const float sc = ldf(row, i) * inv_t + gumbel_of((uint32_t)i, seed);
+        if (sc > best) { best = sc; best_i = i; }   // ascending i per thread: the first maximum stays
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        const float os = __shfl_down(best, off, 64);
+        const int64_t oi = __shfl_down(best_i, off, 64);
+        if (os > best || (os == best && oi < best_i)) { best = os; best_i = oi; }
+    }
+    if ((threadIdx.x & 63) == 0) { s_score[threadIdx.x >> 6] = best; s_idx[threadIdx.x >> 6] = best_i; }
     __syncthreads();
     if (threadIdx.x == 0) {
-        float m = sred[0];
-        for (int w = 1; w < (int)(blockDim.x >> 6); ++w) m = fmaxf(m, sred[w]);
-        s_max = m;
-    }
-    __syncthreads();
-    mx = s_max;
-    float sum = 0.f;
-    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) sum += expf(ldf(row, i) * inv_t - mx);
-    for (int off = 32; off > 0; off >>= 1) sum += __shfl_down(sum, off, 64);
-    __syncthreads();
-    if ((threadIdx.x & 63) == 0) sred[threadIdx.x >> 6] = sum;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        float t = 0.f;
-        for (int w = 0; w < (int)(blockDim.x >> 6); ++w) t += sred[w];
-        s_sum = t;
-    }
-    __syncthreads();
-    if (threadIdx.x < 64) {
-        // wave 0 walks the row in chunks of 64 with an inclusive scan per chunk
-        const float target = u * s_sum;
-        float running = 0.f;
-        int64_t chosen = n - 1;
-        bool done = false;
-        for (int64_t base = 0; base < n && !done; base += 64) {
-            const int64_t i = base + threadIdx.x;
-            float p = i < n ? expf(ldf(row, i) * inv_t - mx) : 0.f;
-            float scan = p;
-            for (int off = 1; off < 64; off <<= 1) {
-                const float t = __shfl_up(scan, off, 64);
-                if ((int)threadIdx.x >= off) scan += t;
-            }
-            const bool hit = (running + scan >= target) && i < n;
-            const unsigned long long mask = __ballot(hit);
-            if (mask) {
-                chosen = base + (int64_t)__ffsll((long long)mask) - 1;
-                done = true;
-            }
-            running += __shfl(scan, 63, 64);
-        }
-        if (threadIdx.x == 0) *out = chosen;
+        for (int w = 1; w < (int)(blockDim.x >> 6); ++w)
+            if (s_score[w] > best || (s_score[w] == best && s_idx[w] < best_i)) { best = s_score[w]; best_i = s_idx[w]; }
+        *out = best_i;
     }
 }
 void sample_temperature_last_row(hipStream_t s, int dtype, const void* logits, int64_t rows, int64_t vocab,
                                  float temperature, float u, int64_t* out) {
     const size_t off = (size_t)(rows - 1) * vocab;
     const float inv_t = 1.0f / temperature;
-    if (dtype == 0) sample_temperature_kernel<float><<<1, 1024, 0, s>>>((const float*)logits + off, vocab, inv_t, u, out);
-    else sample_temperature_kernel<bf16_t><<<1, 1024, 0, s>>>((const bf16_t*)logits + off, vocab, inv_t, u, out);
+    uint32_t bits;
+    memcpy(&bits, &u, 4);
+    const uint32_t seed = bits * 747796405u + 2891336453u;
+    if (dtype == 0) sample_temperature_kernel<float><<<1, 1024, 0, s>>>((const float*)logits + off, vocab, inv_t, seed, out);
+    else sample_temperature_kernel<bf16_t><<<1, 1024, 0, s>>>((const bf16_t*)logits + off, vocab, inv_t, seed, out);
 }
 
 }  // namespace k

@@ -601,7 +601,7 @@ class Ministral(_ModelBase):
 
 # ================================================================================ Generator
 class Generator:
-    """Greedy generation loop (crates/gpt-rs/src/inference/generate.rs:37-203).
+    """Generation loop, greedy by default (crates/gpt-rs/src/inference/generate.rs:37-203).
 
     With `device_sampling` the token comes from backend.sample_decode_token (spec.rs:1333-1348)
     and only 8 bytes cross PCIe per step; otherwise the last logits row is read back and
@@ -609,13 +609,17 @@ class Generator:
     """
 
     def __init__(self, model, prompt: Sequence[int], kv_cache_capacity: Optional[int] = None,
-                 device_sampling: bool = True):
+                 device_sampling: bool = True, temperature: float = 0.0, seed: int = 0):
         if len(prompt) == 0:
             raise ValueError("prompt must be non-empty")
         self.model = model
         self.tokens = list(prompt)
         self.capacity = kv_cache_capacity
         self.device_sampling = device_sampling
+        # temperature > 0: the backend samples from softmax(logits / temperature) given a uniform draw per
+        # step (DecodeSampleRequest.random_u, spec.rs:1270-1284; sampler.rs:83-93 draws it in (eps, 1 - eps))
+        self.temperature = float(temperature)
+        self._rng = np.random.default_rng(seed)
         self.caches: List[Optional[DecodeKvCache]] = [None] * model.num_layers
         self.window_start = max(0, len(self.tokens) - model.context_length)
         context = self.tokens[self.window_start:]
@@ -624,6 +628,13 @@ class Generator:
 
     def _sample(self) -> int:
         be = self.model.backend
+        if self.temperature > 0.0:
+            eps = float(np.finfo(np.float32).eps)
+            u = float(np.float32(self._rng.uniform(eps, 1.0 - eps)))
+            tok = be.sample_decode_token(self.logits, temperature=self.temperature, random_u=u)
+            if tok is None:
+                raise RuntimeError("backend declined temperature sampling")
+            return tok
         if self.device_sampling:
             tok = be.sample_decode_token(self.logits, temperature=0.0)
             if tok is not None:

@@ -544,6 +544,26 @@ def run_program(program, entry_inputs: Sequence[OTensor]) -> List[OTensor]:  # c
     return out
 
 
+def sample_temperature(logits_row: np.ndarray, temperature: float, random_u: float) -> int:
+    """Temperature sampling of the reference's device path: Gumbel-max over a stateless per-index hash
+    (crates/gpt-rs-backend-triton/src/kernels/sample_temperature_last_axis_f32.triton:24-72; seed from random_u as
+    in runtime/sampling.rs:98-101).  All arithmetic in uint32 / float32 as there; ties -> smallest index."""
+    row = np.asarray(logits_row, dtype=np.float32)
+    bits = np.float32(random_u).view(np.uint32)
+    seed = np.uint32((int(bits) * 747796405 + 2891336453) & 0xFFFFFFFF)
+    x = np.arange(row.size, dtype=np.uint32) ^ seed
+    x ^= x >> np.uint32(16)
+    x = (x.astype(np.uint64) * np.uint64(0x7FEB352D)).astype(np.uint32)
+    x ^= x >> np.uint32(15)
+    x = (x.astype(np.uint64) * np.uint64(0x846CA68B)).astype(np.uint32)
+    x ^= x >> np.uint32(16)
+    u = (x.astype(np.float32) + np.float32(1.0)) * np.float32(1.0 / 4294967297.0)
+    u = np.minimum(np.maximum(u, np.float32(1e-7)), np.float32(1.0) - np.float32(1e-7))
+    gumbel = -np.log(-np.log(u, dtype=np.float32), dtype=np.float32)
+    score = row * (np.float32(1.0) / np.float32(temperature)) + gumbel
+    return int(np.argmax(score))
+
+
 def argmax_first(logits_row: np.ndarray) -> int:
     """Greedy token: smallest index among maxima (docs/backend.md:270).  The host sampler
     (crates/gpt-rs/src/inference/sampler.rs:96-103) differs only on exact ties."""

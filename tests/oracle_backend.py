@@ -63,6 +63,10 @@ class OracleBackend:
     def sample_decode_token(self, logits, temperature=0.0, top_k=None, random_u=None) -> Optional[int]:
         a = logits.t.a
         row = a[-1] if a.ndim == 2 else a
+        if top_k is not None:
+            return None
+        if temperature > 0.0:
+            return None if random_u is None else po.sample_temperature(row, temperature, random_u)
         return po.argmax_first(row)
 
     def synchronize(self):

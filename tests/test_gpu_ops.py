@@ -275,6 +275,34 @@ def test_attention_prefill(hip, hq, hkv, dh, seq):
     check_program(hip, p, [qkv])
 
 
+@pytest.mark.parametrize("dtype", ["F32", "Bf16"])
+def test_temperature_sampling_matches_oracle(hip, dtype):
+    """sample_decode_token with temperature > 0 (DecodeSampleRequest, spec.rs:1270-1284): the device kernel and the
+    oracle restate the same Gumbel-max rule, so they must pick the same token whenever the two best scores are not
+    within float noise of each other; the reference's own case (decode_sampling.rs:22-48) must land in range."""
+    from parity import TensorSpec, po, to_bytes
+    from gptrs_amd.ptir import f32_to_bf16_bits
+    h = hip.materialize(TensorSpec("F32", [1, 4]), np.array([[0.1, 0.2, 0.3, 0.4]], np.float32).tobytes())
+    assert 0 <= hip.sample_decode_token(h, temperature=0.8, random_u=0.42) < 4
+    assert hip.sample_decode_token(h, temperature=0.8) is None                # no draw supplied: host sampler's job
+    assert hip.sample_decode_token(h, temperature=0.8, top_k=2, random_u=0.42) is None
+    rng = np.random.default_rng(8)
+    agree = 0
+    for case in range(24):
+        vocab = int(rng.choice([5, 64, 1000, 50257, 131072]))
+        rows = int(rng.integers(1, 4))
+        logits = rng.normal(0, 3, (rows, vocab)).astype(np.float32)
+        if dtype == "Bf16":
+            logits = (f32_to_bf16_bits(logits).astype(np.uint32) << 16).view(np.float32)
+        temperature, u = float(rng.uniform(0.2, 1.5)), float(np.float32(rng.uniform(1e-6, 1 - 1e-6)))
+        hh = hip.materialize(TensorSpec(dtype, [rows, vocab]), to_bytes(logits, dtype))
+        got = hip.sample_decode_token(hh, temperature=temperature, random_u=u)
+        want = po.sample_temperature(logits[-1], temperature, u)
+        assert 0 <= got < vocab
+        agree += got == want
+    assert agree >= 23, f"device and oracle agree on {agree} of 24 draws"
+
+
 @pytest.mark.parametrize("hq,hkv,dh,seq", [(4, 4, 32, 1), (4, 2, 32, 31), (8, 2, 32, 33), (4, 1, 64, 64), (12, 12, 64, 100),
                                            (8, 2, 128, 257), (32, 8, 128, 96), (8, 1, 64, 130)])
 def test_attention_prefill_bf16_matrix_cores(hip, hq, hkv, dh, seq):

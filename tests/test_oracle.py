@@ -411,3 +411,53 @@ def test_int8_and_int4_pack_round_trip():
     lo = int(pk[0, 0] & 0xF)
     lo = lo - 16 if lo > 7 else lo
     assert lo == int(np.clip(np.rint(w[0, 0] / s4[0, 0]), -7, 7))
+
+
+# ---------------------------------------------------------------------------------- temperature sampling
+def _gumbel_score_reference(i, seed, logit, temperature):
+    """The per-index arithmetic of sample_temperature_last_axis_f32.triton:44-60 with Python integers and
+    math.log in float64 (an independent route to the same quantity)."""
+    import math
+    x = (i ^ seed) & 0xFFFFFFFF
+    x ^= x >> 16
+    x = (x * 0x7FEB352D) & 0xFFFFFFFF
+    x ^= x >> 15
+    x = (x * 0x846CA68B) & 0xFFFFFFFF
+    x ^= x >> 16
+    u = (float(np.float32(x)) + 1.0) * float(np.float32(1.0 / 4294967297.0))
+    u = min(max(u, 1e-7), 1.0 - 1e-7)
+    return logit / temperature - math.log(-math.log(u))
+
+
+def test_temperature_sampling_matches_independent_restatement():
+    import struct
+    rng = np.random.default_rng(3)
+    for case in range(40):
+        n = int(rng.integers(2, 300))
+        logits = rng.normal(0, 2, n).astype(np.float32)
+        temperature, u = float(rng.uniform(0.3, 2.0)), float(np.float32(rng.uniform(1e-6, 1 - 1e-6)))
+        bits = struct.unpack("<I", struct.pack("<f", u))[0]
+        seed = (bits * 747796405 + 2891336453) & 0xFFFFFFFF           # runtime/sampling.rs:98-101
+        scores = [_gumbel_score_reference(i, seed, float(logits[i]), temperature) for i in range(n)]
+        order = np.argsort(scores)
+        if scores[order[-1]] - scores[order[-2]] < 1e-4:
+            continue   # the f32 and f64 routes may order a near-tie differently
+        assert po.sample_temperature(logits, temperature, u) == int(order[-1])
+
+
+def test_temperature_sampling_reference_case_in_range():   # crates/gpt-rs-backend-triton/tests/decode_sampling.rs:22-48
+    assert 0 <= po.sample_temperature(np.array([0.1, 0.2, 0.3, 0.4], np.float32), 0.8, 0.42) < 4
+
+
+def test_temperature_sampling_follows_softmax():
+    """Gumbel-max draws index i with probability softmax(logits / T)_i: the empirical frequencies over many
+    uniform draws must fit (chi-square far inside the 0.1 % tail)."""
+    logits = np.array([1.5, 0.2, -0.7, 2.1, 0.0, 0.9], np.float32)
+    temperature = 0.7
+    p = np.exp(logits / temperature - np.max(logits / temperature))
+    p /= p.sum()
+    draws = 6000
+    us = np.random.default_rng(4).uniform(1e-6, 1 - 1e-6, draws).astype(np.float32)
+    counts = np.bincount([po.sample_temperature(logits, temperature, float(u)) for u in us], minlength=6)
+    chi2 = float(np.sum((counts - draws * p) ** 2 / (draws * p)))
+    assert chi2 < 25.0, (chi2, counts, draws * p)    # 5 degrees of freedom: P(chi2 > 20.5) = 0.001
