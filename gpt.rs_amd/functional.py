@@ -186,12 +186,74 @@ def swiglu(gate: Tensor, up: Tensor) -> Tensor:
 
 # --------------------------------------------------------------------------- RoPE
 @dataclass
+class YarnScaling:
+    """RopeScaling::Yarn (ops/functional/rotary.rs:29-43); unset fields take the reference's defaults."""
+
+    factor: float
+    original_max_position_embeddings: int
+    mscale: Optional[float] = None
+    mscale_all_dim: Optional[float] = None
+    beta_fast: Optional[float] = None
+    beta_slow: Optional[float] = None
+    truncate: bool = True
+
+
+@dataclass
 class RopeConfig:
-    """ops/functional/rotary.rs:49-67 (scaling: None | ("linear", factor))."""
+    """ops/functional/rotary.rs:49-67 (scaling: None | ("linear", factor) | YarnScaling)."""
 
     rotary_dim: int = 128
     theta: float = 10_000.0
-    scaling: Optional[tuple] = None
+    scaling: Optional[object] = None
+
+
+def _yarn_inv_freqs(cfg: RopeConfig, y: YarnScaling) -> Tuple[np.ndarray, np.float32]:
+    """ops/functional/rotary.rs:102-190, every step in f32: blend of the extrapolated (base) and interpolated
+    (base / factor) inverse frequencies over a linear ramp between the correction dims of beta_fast and
+    beta_slow, and the attention magnitude 0.1 * mscale * ln(factor) + 1."""
+    f32 = np.float32
+    factor = f32(y.factor)
+    if not (np.isfinite(factor) and factor > 0):
+        raise ValueError(f"rope yarn factor must be finite and positive (got {y.factor})")
+    if y.original_max_position_embeddings is None or y.original_max_position_embeddings <= 0:
+        raise ValueError("rope yarn original_max_position_embeddings must be > 0")
+    beta_fast = f32(32.0 if y.beta_fast is None else y.beta_fast)
+    beta_slow = f32(1.0 if y.beta_slow is None else y.beta_slow)
+    if not (np.isfinite(beta_fast) and np.isfinite(beta_slow) and beta_fast >= beta_slow):
+        raise ValueError(f"rope yarn beta range is invalid: beta_fast={beta_fast} beta_slow={beta_slow}")
+
+    def get_mscale(scale, mscale):
+        return f32(1.0) if scale <= 1.0 else f32(f32(f32(0.1) * f32(mscale)) * np.log(scale, dtype=np.float32)) + f32(1.0)
+
+    if y.mscale is not None and y.mscale_all_dim is not None and y.mscale != 0.0 and y.mscale_all_dim != 0.0:
+        magnitude = f32(get_mscale(factor, y.mscale) / get_mscale(factor, y.mscale_all_dim))
+    else:
+        magnitude = f32(get_mscale(factor, 1.0))
+    if not (np.isfinite(magnitude) and magnitude > 0):
+        raise ValueError(f"rope yarn magnitude must be finite and positive (got {magnitude})")
+    rot, theta = f32(cfg.rotary_dim), f32(cfg.theta)
+    orig = f32(y.original_max_position_embeddings)
+
+    def correction_dim(num_rotations):
+        return f32(f32(rot * np.log(f32(orig / f32(f32(num_rotations * f32(2.0)) * f32(np.pi))), dtype=np.float32))
+                   / f32(f32(2.0) * np.log(theta, dtype=np.float32)))
+
+    low, high = correction_dim(beta_fast), correction_dim(beta_slow)
+    if y.truncate:
+        low, high = f32(np.floor(low)), f32(np.ceil(high))
+    low = f32(max(low, f32(0.0)))
+    high = f32(min(high, f32(max(cfg.rotary_dim - 1, 0))))
+    ramp_max = high
+    if abs(f32(low - ramp_max)) < np.finfo(np.float32).eps:
+        ramp_max = f32(ramp_max + f32(0.001))
+    i = np.arange(cfg.rotary_dim // 2, dtype=np.float32)
+    base = np.power(theta, (f32(2.0) * i) / rot, dtype=np.float32)
+    extrapolation = (f32(1.0) / base).astype(np.float32)
+    interpolation = (f32(1.0) / (factor * base).astype(np.float32)).astype(np.float32)
+    ramp = np.clip(((i - low) / f32(ramp_max - low)).astype(np.float32), f32(0.0), f32(1.0))
+    extrapolation_factor = (f32(1.0) - ramp).astype(np.float32)
+    inv = (interpolation * (f32(1.0) - extrapolation_factor) + extrapolation * extrapolation_factor).astype(np.float32)
+    return inv, magnitude
 
 
 def rotary_cos_sin_cache_slice(start: int, length: int, cfg: RopeConfig) -> Tuple[np.ndarray, np.ndarray]:
@@ -208,14 +270,19 @@ def rotary_cos_sin_cache_slice(start: int, length: int, cfg: RopeConfig) -> Tupl
     i = np.arange(half, dtype=np.float32)
     exponent = (np.float32(2.0) * i) / np.float32(cfg.rotary_dim)
     inv = np.power(np.float32(cfg.theta), -exponent, dtype=np.float32)
-    if cfg.scaling is not None:
+    magnitude = np.float32(1.0)
+    if isinstance(cfg.scaling, YarnScaling):
+        inv, magnitude = _yarn_inv_freqs(cfg, cfg.scaling)
+    elif cfg.scaling is not None:
         kind, factor = cfg.scaling
         if kind != "linear":
             raise NotImplementedError(f"rope scaling {kind}")
+        if not (math.isfinite(factor) and factor > 0):
+            raise ValueError(f"rope scaling factor must be finite and positive (got {factor})")
         inv = (inv / np.float32(factor)).astype(np.float32)
     pos = np.arange(start, start + length, dtype=np.float32)[:, None]
     angle = (pos * inv[None, :]).astype(np.float32)
-    return np.cos(angle).astype(np.float32), np.sin(angle).astype(np.float32)
+    return (np.cos(angle).astype(np.float32) * magnitude).astype(np.float32), (np.sin(angle).astype(np.float32) * magnitude).astype(np.float32)
 
 
 @dataclass

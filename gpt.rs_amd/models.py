@@ -396,6 +396,7 @@ class MinistralConfig:
     rotary_dim: int = 128
     rope_theta: float = 1e6
     eps: float = 1e-5
+    rope_scaling: Optional[object] = None   # None | ("linear", factor) | functional.YarnScaling (rotary.rs:20-43)
 
     def attention_config(self) -> F.AttentionConfig:
         return F.AttentionConfig(self.embed_dim, self.num_heads, self.num_kv_heads, self.head_dim)
@@ -411,7 +412,7 @@ class Ministral(_ModelBase):
         super().__init__(backend, dtype)
         self.config = config
         self.attn = config.attention_config()
-        self.rope = F.RopeConfig(config.rotary_dim, config.rope_theta, None)
+        self.rope = F.RopeConfig(config.rotary_dim, config.rope_theta, config.rope_scaling)
 
     @classmethod
     def random(cls, config: MinistralConfig, backend, seed: int = 0, dtype: str = "Bf16", std: float = 0.02,
