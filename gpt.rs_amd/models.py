@@ -134,6 +134,40 @@ class _ModelBase:
         self.set_param_handle(name + ".q", q)
         self.set_param_handle(name + ".s", s)
 
+    # -- checkpoints -----------------------------------------------------------------
+    def _load_tensors(self, ck, expected: Dict[str, tuple]):
+        """Upload every expected tensor from an open checkpoint (checkpoint/loader.rs: by name, shape checked),
+        one at a time out of the file mapping."""
+        from .checkpoint import CheckpointError
+        for name, dims in expected.items():
+            e = ck.entry(name)
+            if tuple(e.dims) != tuple(dims):
+                raise CheckpointError(f"tensor `{name}` has shape {list(e.dims)}, the model expects {list(dims)}")
+            arr = ck.array(name)
+            if e.dtype == "F32":
+                host = np.asarray(arr, np.float32)
+            elif e.dtype == "Bf16":
+                host = bf16_bits_to_f32(np.asarray(arr))
+            else:
+                raise CheckpointError(f"tensor `{name}`: dtype {e.dtype} cannot feed a model parameter")
+            self.set_param(name, host)
+
+    def save_checkpoint(self, path: str, kind: str, config: Dict[str, object]):
+        """Write the parameters back as a GPTRSCHK v2 file (checkpoint/saver.rs), in their storage dtype."""
+        from .checkpoint import write_checkpoint
+        tensors, dtypes = {}, {}
+        for name in self.param_names:
+            spec = self.param_specs[name]
+            if spec.dtype not in ("F32", "Bf16"):
+                raise ValueError(f"parameter {name} of dtype {spec.dtype} has no checkpoint representation")
+            raw = self.backend.to_literal(self.param_handle(name))
+            if spec.dtype == "F32":
+                tensors[name] = np.frombuffer(raw, "<f4").reshape(spec.dims)
+            else:
+                tensors[name] = np.frombuffer(raw, "<u2").reshape(spec.dims)
+                dtypes[name] = "Bf16"
+        write_checkpoint(path, kind, config, tensors, dtypes)
+
     def param_handle(self, name: str):
         h = self.backend.param_resolver().get(param_id(self.namespace, name))
         if h is None:
@@ -218,6 +252,39 @@ class Gpt(_ModelBase):
         m.set_param("final_ln.beta", np.zeros(d, np.float32))
         m.set_param("lm_head", rn(d, config.vocab_size))
         return m
+
+    def expected_params(self) -> Dict[str, tuple]:
+        """Names and shapes as Gpt::build_from_params reads them (model/gpt.rs:300-370)."""
+        c = self.config
+        d, hid = c.embed_dim, c.embed_dim * c.mlp_ratio
+        out = {"tok_embeddings.weight": (c.vocab_size, d), "pos_embeddings": (c.context_length, d)}
+        for i in range(c.num_layers):
+            p = f"blocks.{i}."
+            out.update({p + "ln_1.gamma": (d,), p + "ln_1.beta": (d,), p + "attention.w_qkv": (d, 3 * d),
+                        p + "attention.b_qkv": (3 * d,), p + "attention.w_out": (d, d), p + "attention.b_out": (d,),
+                        p + "ln_2.gamma": (d,), p + "ln_2.beta": (d,), p + "feed_forward.w_in": (d, hid),
+                        p + "feed_forward.b_in": (hid,), p + "feed_forward.w_out": (hid, d), p + "feed_forward.b_out": (d,)})
+        out.update({"final_ln.gamma": (d,), "final_ln.beta": (d,), "lm_head": (d, c.vocab_size)})
+        return out
+
+    @classmethod
+    def from_checkpoint(cls, path: str, backend, dtype: str = "F32") -> "Gpt":
+        """runtime/loader.rs:19-241 for kind "gpt": config from the file, tensors streamed by name."""
+        from .checkpoint import Checkpoint, CheckpointError
+        with Checkpoint(path) as ck:
+            if ck.kind != "gpt":
+                raise CheckpointError(f"checkpoint holds a `{ck.kind}` model, not `gpt`")
+            c = ck.config
+            cfg = GptConfig(vocab_size=int(c["vocab_size"]), context_length=int(c["context_length"]), embed_dim=int(c["embed_dim"]),
+                            num_layers=int(c["num_layers"]), num_heads=int(c["num_heads"]), mlp_ratio=int(c.get("mlp_ratio", 4)))
+            m = cls(cfg, backend, dtype)
+            m._load_tensors(ck, m.expected_params())
+        return m
+
+    def checkpoint_config(self) -> Dict[str, object]:
+        c = self.config
+        return {"vocab_size": c.vocab_size, "context_length": c.context_length, "embed_dim": c.embed_dim,
+                "num_layers": c.num_layers, "num_heads": c.num_heads, "mlp_ratio": c.mlp_ratio, "dropout": 0.0}
 
     @property
     def num_layers(self): return self.config.num_layers
@@ -462,6 +529,73 @@ class Ministral(_ModelBase):
                 if quant and len(shape) == 2 and name != "tok_embeddings.weight":
                     m.quantize_param(name, quant)
         return m
+
+    def expected_params(self) -> Dict[str, tuple]:
+        """Names and shapes as Ministral::build_from_params reads them (model/ministral.rs:360-425)."""
+        c, a = self.config, self.attn
+        d = c.embed_dim
+        out = {"tok_embeddings.weight": (c.vocab_size, d)}
+        for i in range(c.num_layers):
+            p = f"blocks.{i}."
+            out.update({p + "norm_1.gamma": (d,), p + "attention.w_qkv": (d, a.total_projection_dim),
+                        p + "attention.w_out": (a.query_projection_dim, d), p + "norm_2.gamma": (d,),
+                        p + "feed_forward.w_gate": (d, c.ffn_dim), p + "feed_forward.w_up": (d, c.ffn_dim),
+                        p + "feed_forward.w_down": (c.ffn_dim, d)})
+        out.update({"final_norm.gamma": (d,), "lm_head": (d, c.vocab_size)})
+        return out
+
+    @staticmethod
+    def _scaling_from_json(js) -> Optional[object]:
+        """RopeScaling's serde form: {"kind": "none" | "linear" | "yarn", ...} (ops/functional/rotary.rs:20-43)."""
+        if not js or js.get("kind", "none") == "none":
+            return None
+        if js["kind"] == "linear":
+            return ("linear", float(js["factor"]))
+        if js["kind"] == "yarn":
+            return F.YarnScaling(factor=float(js["factor"]), original_max_position_embeddings=js.get("original_max_position_embeddings"),
+                                 mscale=js.get("mscale"), mscale_all_dim=js.get("mscale_all_dim"), beta_fast=js.get("beta_fast"),
+                                 beta_slow=js.get("beta_slow"), truncate=bool(js.get("truncate", True)))
+        raise ValueError(f"unknown rope scaling kind {js['kind']!r}")
+
+    @classmethod
+    def from_checkpoint(cls, path: str, backend, dtype: str = "Bf16", quant: Optional[str] = None) -> "Ministral":
+        """runtime/loader.rs:19-241 for kind "ministral" (MinistralConfig, model/ministral.rs:13-30)."""
+        from .checkpoint import Checkpoint, CheckpointError
+        with Checkpoint(path) as ck:
+            if ck.kind != "ministral":
+                raise CheckpointError(f"checkpoint holds a `{ck.kind}` model, not `ministral`")
+            c = ck.config
+            head_dim = int(c["head_dim"]) if c.get("head_dim") else int(c["embed_dim"]) // int(c["num_heads"])
+            if c.get("kv_head_dim") and int(c["kv_head_dim"]) != head_dim:
+                raise CheckpointError("kv_head_dim different from head_dim is not supported")
+            cfg = MinistralConfig(vocab_size=int(c["vocab_size"]), context_length=int(c["context_length"]), embed_dim=int(c["embed_dim"]),
+                                  num_layers=int(c["num_layers"]), num_heads=int(c["num_heads"]), num_kv_heads=int(c["num_kv_heads"]),
+                                  head_dim=head_dim, ffn_dim=int(c["mlp_hidden_dim"]), rotary_dim=int(c["rotary_dim"]),
+                                  rope_theta=float(c["rope_theta"]), eps=float(c["rms_norm_eps"]),
+                                  rope_scaling=cls._scaling_from_json(c.get("rope_scaling")))
+            m = cls(cfg, backend, dtype)
+            for name, dims in m.expected_params().items():
+                m._load_tensors(ck, {name: dims})
+                if quant and len(dims) == 2 and name != "tok_embeddings.weight":
+                    m.quantize_param(name, quant)
+        return m
+
+    def checkpoint_config(self) -> Dict[str, object]:
+        c = self.config
+        out = {"vocab_size": c.vocab_size, "context_length": c.context_length, "embed_dim": c.embed_dim, "num_layers": c.num_layers,
+               "num_heads": c.num_heads, "num_kv_heads": c.num_kv_heads, "head_dim": c.head_dim, "mlp_hidden_dim": c.ffn_dim,
+               "rms_norm_eps": c.eps, "rope_theta": c.rope_theta, "rotary_dim": c.rotary_dim}
+        sc = c.rope_scaling
+        if sc is None:
+            out["rope_scaling"] = {"kind": "none"}
+        elif isinstance(sc, F.YarnScaling):
+            out["rope_scaling"] = {k: v for k, v in dict(kind="yarn", factor=sc.factor, mscale=sc.mscale, mscale_all_dim=sc.mscale_all_dim,
+                                                         beta_fast=sc.beta_fast, beta_slow=sc.beta_slow,
+                                                         original_max_position_embeddings=sc.original_max_position_embeddings,
+                                                         truncate=sc.truncate).items() if v is not None}
+        else:
+            out["rope_scaling"] = {"kind": "linear", "factor": sc[1]}
+        return out
 
     QUANTIZABLE = ("attention.w_qkv", "attention.w_out", "feed_forward.w_gate", "feed_forward.w_up",
                    "feed_forward.w_down", "lm_head")

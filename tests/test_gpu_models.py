@@ -60,6 +60,22 @@ def test_tiny_gpt_temperature_sampling_matches_oracle(hip):
     assert len(set(t_hip)) > 3   # a sampled sequence, not one token repeated
 
 
+def test_model_from_checkpoint_on_device(hip, tmp_path):
+    """A GPTRSCHK v2 file written from one backend feeds the other (checkpoint/loader.rs, runtime/loader.rs:19-241):
+    same greedy tokens, logits within the f32 bar; bf16 storage and on-load quantisation go through as well."""
+    ref = OracleBackend()
+    m_ref = models.Ministral.random(MID_MINISTRAL, ref, seed=3, dtype="F32", std=0.05)
+    path = str(tmp_path / "mid.gptrs")
+    m_ref.save_checkpoint(path, "ministral", m_ref.checkpoint_config())
+    m_hip = models.Ministral.from_checkpoint(path, hip, dtype="F32")
+    g_ref, g_hip = models.Generator(m_ref, PROMPT, kv_cache_capacity=32), models.Generator(m_hip, PROMPT, kv_cache_capacity=32)
+    assert g_hip.generate(6) == g_ref.generate(6)
+    assert rel_err(hip.to_numpy(g_hip.logits)[-1], ref.to_numpy(g_ref.logits)[-1]) < 1e-4
+    m_q = models.Ministral.from_checkpoint(path, hip, dtype="Bf16", quant="w8")
+    assert "lm_head.q" in m_q.param_specs and m_q.param_specs["tok_embeddings.weight"].dtype == "Bf16"
+    assert len(models.Generator(m_q, PROMPT, kv_cache_capacity=32).generate(4)) == 4
+
+
 def test_tiny_gpt_kv_cache_equals_full_context(hip):
     # smoke.rs:43-82: KV-cache greedy decode == full-context greedy decode for 16 steps
     m = models.Gpt.random(TINY_GPT, hip, seed=11, std=0.2)
