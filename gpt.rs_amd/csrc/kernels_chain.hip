@@ -91,7 +91,16 @@ __device__ __forceinline__ void cstore8(void* p, unsigned long long v) {
 __device__ __forceinline__ void cstore4(void* p, unsigned v) {
     __hip_atomic_store(as_global((unsigned*)p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ float rbf(float v) { return bf16_to_f32(f32_to_bf16(v)); }
+// bf16 rounding with the hardware converter (v_cvt_pk_bf16_f32, round to nearest even): the staging of a
+// normalised row runs these on every wave of the workgroup at once, where each instruction counts three times
+// on the SIMD that holds three waves
+__device__ __forceinline__ unsigned pack_hw(float lo, float hi) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    f32x2_t f;
+    f.x = lo; f.y = hi;
+    return __builtin_bit_cast(unsigned, __builtin_convertvector(f, bf16x2));
+}
+__device__ __forceinline__ float rbf(float v) { return bf16lo(pack_hw(v, 0.f)); }
 template <typename P> __device__ __forceinline__ int lds_ld(P p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
 template <typename P> __device__ __forceinline__ void lds_st(P p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
 #define GPTRS_LDS_RELEASE() __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local")
@@ -107,10 +116,13 @@ __device__ unsigned long long* g_chain_stamps = nullptr;   // lab builds: [phase
 #define GPTRS_STAMP(i) do { if (g_chain_stamps && blockIdx.x == 0 && (threadIdx.x & 63) == 0) g_chain_stamps[ph * 16 + (i)] = wall_clock64(); } while (0)
 #define GPTRS_STAMP_W0(i) do { if (g_chain_stamps && blockIdx.x == 0 && threadIdx.x == 0) g_chain_stamps[phase * 16 + (i)] = wall_clock64(); } while (0)
 #define GPTRS_STAMP_C(i) do { if (g_chain_stamps && blockIdx.x == 0 && threadIdx.x == NS) g_chain_stamps[phase * 16 + (i)] = wall_clock64(); } while (0)
+__device__ int g_chain_stage_phase = 0;
+#define GPTRS_STAMP_S(i) do { if (g_chain_stamps && blockIdx.x == 0 && threadIdx.x == NS) g_chain_stamps[g_chain_stage_phase * 16 + (i)] = wall_clock64(); } while (0)
 #else
 #define GPTRS_STAMP(i) do { } while (0)
 #define GPTRS_STAMP_W0(i) do { } while (0)
 #define GPTRS_STAMP_C(i) do { } while (0)
+#define GPTRS_STAMP_S(i) do { } while (0)
 #endif
 
 struct Shared {
@@ -161,30 +173,42 @@ __device__ void stage_block(const ChainPhase& P, unsigned* xs, float* ssq) {
 #pragma unroll
         for (int u = 0; u < MAXI; ++u) {
             const int i = u * NT + t;
-            v[u] = i < n ? cload8(x + 8 * (size_t)i) : 0ull;
-            gg[u] = i < n ? gload2(g + i) : make_uint2(0u, 0u);
+            v[u] = 0ull;
+            gg[u] = make_uint2(0u, 0u);
+            if (u * NT < n && i < n) {
+                v[u] = cload8(x + 8 * (size_t)i);
+                gg[u] = gload2(g + i);
+            }
         }
+        // rounds beyond the row (wave-uniform test) are skipped: a short row must not pay for MAXI of them
         float q = 0.f;
 #pragma unroll
         for (int u = 0; u < MAXI; ++u) {
-            const unsigned lo = (unsigned)v[u], hi = (unsigned)(v[u] >> 32);
-            const float a = bf16lo(lo), b = bf16hi(lo), c = bf16lo(hi), d = bf16hi(hi);
-            q += a * a; q += b * b; q += c * c; q += d * d;
+            if (u * NT < n) {
+                const unsigned lo = (unsigned)v[u], hi = (unsigned)(v[u] >> 32);
+                const float a = bf16lo(lo), b = bf16hi(lo), c = bf16lo(hi), d = bf16hi(hi);
+                q += a * a; q += b * b; q += c * c; q += d * d;
+            }
         }
+        GPTRS_STAMP_S(6);
         const float ws = wave_sum(q);
         if (lane == 0) ssq[wave] = ws;
         lds_barrier();
+        GPTRS_STAMP_S(7);
         float tot = 0.f;
 #pragma unroll
         for (int w = 0; w < NT / 64; ++w) tot += ssq[w];
         const float inv = 1.0f / sqrtf(tot * P.inv_n + P.eps);
+        GPTRS_STAMP_S(15);
 #pragma unroll
         for (int u = 0; u < MAXI; ++u) {
             const int i = u * NT + t;
-            if (i < npad) {
+            if (u * NT < npad && i < npad) {
                 const unsigned lo = (unsigned)v[u], hi = (unsigned)(v[u] >> 32);
-                const unsigned o0 = pack_bf16x2(rbf(bf16lo(lo) * inv) * bf16lo(gg[u].x), rbf(bf16hi(lo) * inv) * bf16hi(gg[u].x));
-                const unsigned o1 = pack_bf16x2(rbf(bf16lo(hi) * inv) * bf16lo(gg[u].y), rbf(bf16hi(hi) * inv) * bf16hi(gg[u].y));
+                // ((x * inv) -> bf16) * gamma -> bf16, two values per conversion
+                const unsigned n0 = pack_hw(bf16lo(lo) * inv, bf16hi(lo) * inv), n1 = pack_hw(bf16lo(hi) * inv, bf16hi(hi) * inv);
+                const unsigned o0 = pack_hw(bf16lo(n0) * bf16lo(gg[u].x), bf16hi(n0) * bf16hi(gg[u].x));
+                const unsigned o1 = pack_hw(bf16lo(n1) * bf16lo(gg[u].y), bf16hi(n1) * bf16hi(gg[u].y));
                 *reinterpret_cast<uint2*>(&xs[2 * i]) = make_uint2(o0, o1);
             }
         }
@@ -203,6 +227,7 @@ __device__ void stage_block(const ChainPhase& P, unsigned* xs, float* ssq) {
             }
         }
     }
+    GPTRS_STAMP_S(14);
     if (sc_n > 0) {
 #pragma unroll
         for (int u = 0; u < SB; ++u) {
@@ -628,34 +653,50 @@ __device__ void control_wave(Shared& sh, unsigned* xs, int nphases, unsigned* ba
             const int cpt = dual ? 2 : 4;              // output columns per tile
             const int col0 = u0 * TP * cpt;
             const int ncols = min((u1 - u0) * TP * cpt, EPI_MAX);
-            // bias / residual of this workgroup's columns: requested before the staging loads so
-            // their latency hides behind the staging
+            // bias / residual / int8 scales of this workgroup's columns: the first round is requested before the
+            // staging loads and written to LDS after the staging, so that its latency hides behind the staging
+            // instead of holding up the workgroup's barrier inside it
             const unsigned* bias = (const unsigned*)uni_ptr(P.bias);
             const char* resid = (const char*)uni_ptr(P.residual);
+            constexpr int wfmt = FMT;   // every linear phase of a launch has the kernel's weight format
+            const unsigned* sg = wfmt == kChainW8 ? (const unsigned*)uni_ptr(P.wscale) : nullptr;
+            const unsigned* su = wfmt == kChainW8 ? (const unsigned*)uni_ptr(P.wscale2) : nullptr;
             if (lane == 0) lds_st(&sh.go, ph);
-            if (bias || resid) {
-                for (int i = lane * 2; i < ncols; i += 128) {
-                    const int col = col0 + i;
-                    const unsigned bw = (bias && col < N) ? gload(bias + (col >> 1)) : 0u;
-                    const unsigned rw = (resid && col < N) ? cload4(resid + 2 * (size_t)col) : 0u;
+            auto epi_load = [&](int i, unsigned& bw, unsigned& rw, unsigned& ga, unsigned& gb) {
+                const int col = col0 + i;
+                const bool in = i < ncols && col < N;
+                bw = (bias && in) ? gload(bias + (col >> 1)) : 0u;
+                rw = (resid && in) ? cload4(resid + 2 * (size_t)col) : 0u;
+                ga = (sg && in) ? gload(sg + (col >> 1)) : 0u;
+                gb = (su && in) ? gload(su + (col >> 1)) : 0u;
+            };
+            auto epi_store = [&](int i, unsigned bw, unsigned rw, unsigned ga, unsigned gb) {
+                if (i >= ncols) return;
+                if (bias || resid) {
                     *reinterpret_cast<float2*>(&sh.epi_bias[i]) = make_float2(bf16lo(bw), bf16hi(bw));
                     *reinterpret_cast<float2*>(&sh.epi_res[i]) = make_float2(bf16lo(rw), bf16hi(rw));
                 }
-            }
-            constexpr int wfmt = FMT;   // every linear phase of a launch has the kernel's weight format
-            if (wfmt == kChainW8) {
-                const unsigned* sg = (const unsigned*)uni_ptr(P.wscale);
-                const unsigned* su = (const unsigned*)uni_ptr(P.wscale2);
-                for (int i = lane * 2; i < ncols; i += 128) {
-                    const int col = col0 + i;
-                    const unsigned a = col < N ? gload(sg + (col >> 1)) : 0u;
-                    const unsigned b = (su && col < N) ? gload(su + (col >> 1)) : 0u;
-                    *reinterpret_cast<float2*>(&sh.epi_s[i]) = make_float2(bf16lo(a), bf16hi(a));
-                    *reinterpret_cast<float2*>(&sh.epi_s[EPI_MAX + i]) = make_float2(bf16lo(b), bf16hi(b));
+                if (sg) {
+                    *reinterpret_cast<float2*>(&sh.epi_s[i]) = make_float2(bf16lo(ga), bf16hi(ga));
+                    *reinterpret_cast<float2*>(&sh.epi_s[EPI_MAX + i]) = make_float2(bf16lo(gb), bf16hi(gb));
                 }
-            }
+            };
+            const bool has_epi = bias || resid || sg;
+            unsigned e_bw = 0u, e_rw = 0u, e_ga = 0u, e_gb = 0u;
+            if (has_epi) epi_load(lane * 2, e_bw, e_rw, e_ga, e_gb);
+#ifdef GPTRS_CHAIN_STAMPS
+            if (blockIdx.x == 0 && lane == 0) g_chain_stage_phase = ph;
+            GPTRS_STAMP(3);
+#endif
             stage_block(P, xs, sh.ssq);
             GPTRS_STAMP(2);
+            if (has_epi) {
+                epi_store(lane * 2, e_bw, e_rw, e_ga, e_gb);
+                for (int i = lane * 2 + 128; i < ncols; i += 128) {
+                    epi_load(i, e_bw, e_rw, e_ga, e_gb);
+                    epi_store(i, e_bw, e_rw, e_ga, e_gb);
+                }
+            }
             char* out = (char*)uni_ptr(P.y);
             for (int u = u0; u < u1; ++u, ++ucount) {
                 const int slot = ucount % NSLOT;
