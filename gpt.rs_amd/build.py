@@ -14,7 +14,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libgptrs_hip.so")
 
 SOURCES = ["ptir.cpp", "fuse.cpp", "plan.cpp", "api.cpp", "kernels_generic.hip", "kernels_fused.hip",
-           "kernels_linear.hip", "kernels_gemv_tiled.hip", "kernels_attn.hip", "kernels_mfma.hip", "kernels_chain.hip", "kernels_quant.hip"]
+           "kernels_linear.hip", "kernels_gemv_tiled.hip", "kernels_attn.hip", "kernels_mfma.hip", "kernels_chain.hip", "kernels_quant.hip", "kernels_skinny.hip"]
 
 # -packed-fp32-ops is switched off: the compiler must not form v_pk_*_f32 from float code.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-fast-math", "-ffp-contract=off",

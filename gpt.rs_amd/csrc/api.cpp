@@ -158,6 +158,9 @@ BufferP Backend::derived_weights(const BufferP& src, int kind, DType dtype, int6
     } else if (kind == 5) {                             // decode chain: int4 group scales (src2: the partner's)
         t = new_buffer(k::chain_scale_bytes(k, n, src2 != nullptr));
         k::chain_pack_scales_w4(stream, (int)dtype, src->ptr, src2 ? src2->ptr : nullptr, t->ptr, k, n);
+    } else if (kind == 8) {                             // batched decode: 16-column tiles, k-grouped (kernels_skinny.hip)
+        t = new_buffer(k::skinny_weight_bytes(k, n));
+        k::skinny_pack_weights(stream, src->ptr, t->ptr, k, n);
     } else {                                            // 6 / 7: MFMA copy of dequantised int8 / int4 (src2: scales)
         if (!src2) fail_exec("quantised weight copy needs its scales");
         BufferP full = new_buffer((size_t)k * n * dtype_size(dtype));

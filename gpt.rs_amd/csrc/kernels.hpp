@@ -109,6 +109,19 @@ void tile_weights(hipStream_t s, int dtype, const void* w, void* wt, int64_t k, 
 bool gemv_tiled_supported(int dtype, int64_t m, int64_t k, int64_t n);
 void gemv_tiled(hipStream_t s, const TiledLinearArgs& a);
 
+// Batched-decode linear layers (2 <= M <= 16, bf16) on the matrix cores over a 16-column tiled, k-grouped copy
+// of the weights, Ws[tile][K/8][16][8] (kernels_skinny.hip).  ws2 != nullptr: SwiGLU pair.  act: 0 none, 1 gelu.
+struct SkinnyLinearArgs {
+    const void* x; const void* ws; const void* ws2; const void* bias; const void* residual;
+    void* y;
+    int64_t m, k, n;
+    int act;
+};
+bool skinny_gemm_supported(int dtype, int64_t m, int64_t k, int64_t n);
+size_t skinny_weight_bytes(int64_t k, int64_t n);
+void skinny_pack_weights(hipStream_t s, const void* w, void* out, int64_t k, int64_t n);
+void skinny_gemm(hipStream_t s, const SkinnyLinearArgs& a);
+
 // ---- weight-only quantisation (kernels_quant.hip) ------------------------------------------
 // Build-defined extension (the reference has no quantisation scheme, docs/backend.md:620-632):
 //   int8: symmetric, one scale per output column of W[K,N]: s_n = bf16(max_k |W[k,n]| / 127) (1 when 0),

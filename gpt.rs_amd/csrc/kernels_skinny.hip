@@ -1,0 +1,140 @@
+// Batched-decode linear layers (2 <= M <= 16 rows, bf16) on the matrix cores.
+//
+// With a handful of rows a linear layer is still one pass over the weights, i.e. bound by HBM, but the
+// per-element work of a vector GEMV grows with M (M multiply-adds per weight element plus the activation reads)
+// until the vector ALUs, not memory, set the pace.  One v_mfma_f32_16x16x32_bf16 multiplies 16 rows by a
+// 32 x 16 block of W at a cost that does not depend on M, so the kernel below only has to stream W.
+//
+// Weights are read from a derived copy Ws[tile][K/8][16 columns][8 k] (tile = 16 output columns): the 64 lanes of
+// a wave fetch 32 consecutive k of the tile's 16 columns as ONE contiguous KiB in exactly the B-operand layout
+// (lane = 16 * k-group + column holds 8 consecutive k of its column).  A workgroup owns one tile; its 4 waves take
+// the 32-k steps round-robin (so the workgroup reads 4 consecutive KiB per round) and add their partial products
+// through LDS.  The A operand (lane = 16 * k-group + row) comes straight from x, which is small and stays in L2.
+// DUAL computes silu(x.W) * (x.W2) (ops/functional/activation.rs:141-162) from two weight copies.
+#include "kernels.hpp"
+#include "device_utils.hpp"
+
+namespace gptrs {
+namespace k {
+
+namespace {
+
+typedef __bf16 bf16x8_s __attribute__((ext_vector_type(8)));
+typedef float f32x4_s __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_s __attribute__((ext_vector_type(4)));
+
+inline int64_t cdiv_s(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Ws[tile][kb][c][i] = W[8 kb + i][16 tile + c], zero outside [K) x [N); one thread per 16-byte group
+__global__ __launch_bounds__(256) void skinny_pack_kernel(const bf16_t* __restrict__ w, bf16_t* __restrict__ out, int64_t K, int64_t N,
+                                                          int64_t KB, int64_t ntiles) {
+    const int64_t total = ntiles * KB * 16;
+    for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < total; g += (int64_t)gridDim.x * blockDim.x) {
+        const int c = (int)(g & 15);
+        const int64_t kb = (g >> 4) % KB, tile = (g >> 4) / KB;
+        const int64_t col = tile * 16 + c;
+        uint32_t r[4] = {0, 0, 0, 0};
+        if (col < N) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int64_t kx = kb * 8 + i;
+                const uint32_t v = kx < K ? (uint32_t)w[kx * N + col] : 0u;
+                r[i >> 1] |= v << ((i & 1) * 16);
+            }
+        }
+        *reinterpret_cast<uint4*>(out + g * 8) = make_uint4(r[0], r[1], r[2], r[3]);
+    }
+}
+
+__device__ __forceinline__ float skinny_finish(float v, float v2, bool dual, int act, float bias, bool has_res, float res) {
+    if (dual) v = (v / (1.0f + expf(v * -1.0f))) * v2;              // activation.rs:141-162
+    v += bias;                                                      // tensor_ops.rs:42-56
+    if (act == 1) v = (v * 0.5f) * (erff(v / 1.41421354f) + 1.0f);  // activation.rs:96-113
+    if (has_res) v += res;
+    return v;
+}
+
+template <bool DUAL>
+__global__ __launch_bounds__(256) void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ ws,
+                                                          const bf16_t* __restrict__ ws2, const bf16_t* __restrict__ bias,
+                                                          const bf16_t* __restrict__ residual, bf16_t* __restrict__ y, int M, int K,
+                                                          int N, int act) {
+    constexpr int U = 4;                         // 32-k steps per wave and round, all requested before the first is used
+    __shared__ float red[4][DUAL ? 2 : 1][64][4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = lane & 15, kg = lane >> 4;     // B: column c, k-group kg; A: row c, k-group kg
+    const int tile = blockIdx.x;
+    const int nsteps = K / 32;
+    const u32x4_s* bsrc = reinterpret_cast<const u32x4_s*>(ws) + (int64_t)tile * (K / 8) * 16 + lane;
+    const u32x4_s* bsrc2 = DUAL ? reinterpret_cast<const u32x4_s*>(ws2) + (int64_t)tile * (K / 8) * 16 + lane : nullptr;
+    const int arow = c < M ? c : M - 1;          // rows beyond M re-read the last one; their products are never stored
+    const u32x4_s* asrc = reinterpret_cast<const u32x4_s*>(x + (int64_t)arow * K + 8 * kg);
+
+    f32x4_s acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = wave; s0 < nsteps; s0 += 4 * U) {
+        u32x4_s b[U], b2[DUAL ? U : 1], a[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int s = s0 + 4 * u < nsteps ? s0 + 4 * u : s0;   // a step past the end repeats the first, weight zero below
+            b[u] = bsrc[(int64_t)s * 64];
+            if (DUAL) b2[u] = bsrc2[(int64_t)s * 64];
+            a[u] = asrc[s * 4];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (s0 + 4 * u < nsteps) {
+                const bf16x8_s av = __builtin_bit_cast(bf16x8_s, a[u]);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, __builtin_bit_cast(bf16x8_s, b[u]), acc, 0, 0, 0);
+                if (DUAL) acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, __builtin_bit_cast(bf16x8_s, b2[u]), acc2, 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        red[wave][0][lane][i] = acc[i];
+        if (DUAL) red[wave][DUAL ? 1 : 0][lane][i] = acc2[i];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    const int n = tile * 16 + c;
+    if (n >= N) return;
+    const float bv = bias ? bf16_to_f32(bias[n]) : 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = 4 * kg + i;                // D: lane holds rows 4 kg .. 4 kg + 3 of column c
+        if (m >= M) continue;
+        float g = 0.f, up = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            g += red[w][0][lane][i];
+            if (DUAL) up += red[w][DUAL ? 1 : 0][lane][i];
+        }
+        const float r = residual ? bf16_to_f32(residual[(int64_t)m * N + n]) : 0.f;
+        y[(int64_t)m * N + n] = f32_to_bf16(skinny_finish(g, up, DUAL, act, bv, residual != nullptr, r));
+    }
+}
+
+}  // namespace
+
+bool skinny_gemm_supported(int dtype, int64_t m, int64_t k, int64_t n) {
+    return dtype == 2 && m >= 2 && m <= 16 && k >= 32 && k % 32 == 0 && n >= 1 && k < (1ll << 31) && n < (1ll << 31) - 16;
+}
+size_t skinny_weight_bytes(int64_t k, int64_t n) { return (size_t)(cdiv_s(n, 16) * cdiv_s(k, 8) * 16 * 8) * sizeof(bf16_t); }
+void skinny_pack_weights(hipStream_t s, const void* w, void* out, int64_t k, int64_t n) {
+    const int64_t ntiles = cdiv_s(n, 16), kb = cdiv_s(k, 8), total = ntiles * kb * 16;
+    if (total <= 0) return;
+    const unsigned g = (unsigned)(cdiv_s(total, 256) > 65536 ? 65536 : cdiv_s(total, 256));
+    skinny_pack_kernel<<<g, 256, 0, s>>>((const bf16_t*)w, (bf16_t*)out, k, n, kb, ntiles);
+}
+void skinny_gemm(hipStream_t s, const SkinnyLinearArgs& a) {
+    const unsigned grid = (unsigned)cdiv_s(a.n, 16);
+    if (a.ws2)
+        skinny_gemm_kernel<true><<<grid, 256, 0, s>>>((const bf16_t*)a.x, (const bf16_t*)a.ws, (const bf16_t*)a.ws2, (const bf16_t*)a.bias,
+                                                      (const bf16_t*)a.residual, (bf16_t*)a.y, (int)a.m, (int)a.k, (int)a.n, a.act);
+    else
+        skinny_gemm_kernel<false><<<grid, 256, 0, s>>>((const bf16_t*)a.x, (const bf16_t*)a.ws, nullptr, (const bf16_t*)a.bias,
+                                                       (const bf16_t*)a.residual, (bf16_t*)a.y, (int)a.m, (int)a.k, (int)a.n, a.act);
+}
+
+}  // namespace k
+}  // namespace gptrs

@@ -552,6 +552,10 @@ void Builder::describe(Step& st) {
                     if (in.act == 2) st.tiled_s2_input = pos(4);
                 }
             }
+            if (in.tiled && !in.quant && in.norm && x.dims[0] >= 2) {
+                // batched decode normalises into scratch first (the matrix-core kernel reads plain rows)
+                st.scratch_bytes = align_up((size_t)x.count() * dtype_size(x.dtype));
+            }
             if (in.quant && !in.mfma) {
                 // stand-alone path of a quantised linear: (RMSNorm of x,) dequantised weights, then the generic kernel
                 const size_t es = dtype_size(x.dtype);
@@ -1060,6 +1064,46 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
                     cx.be->prof_events.emplace_back(e0, e1);
                     ++cx.be->prof_linear_calls;
                     cx.be->prof_linear_bytes += (int64_t)dtype_size(x.dtype) * (ma.m * ma.k + ma.m * ma.n) + linear_weight_bytes(in, x, w);
+                }
+                ++cx.launches;
+                break;
+            }
+            if (in.tiled && !in.quant && k::skinny_gemm_supported((int)x.dtype, x.dims[0], x.dims[1], w.dims[1]) &&
+                (!in.norm || st.scratch_bytes >= (size_t)x.count() * dtype_size(x.dtype))) {
+                k::SkinnyLinearArgs sa{};
+                sa.x = src_ptr(st, cx, 0);
+                sa.m = x.dims[0]; sa.k = x.dims[1]; sa.n = w.dims[1];
+                BufferP wsk = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], 8, x.dtype, sa.k, sa.n);
+                BufferP wsk2;
+                sa.ws = wsk->ptr;
+                size_t oi = 2;
+                if (in.act == 2) {
+                    wsk2 = cx.be->derived_weights(cx.input_bufs[st.tiled_w2_input], 8, x.dtype, sa.k, sa.n);
+                    sa.ws2 = wsk2->ptr;
+                    ++oi;
+                }
+                if (in.has_bias) sa.bias = src_ptr(st, cx, oi++);
+                if (in.has_residual) sa.residual = src_ptr(st, cx, oi++);
+                if (in.norm) {
+                    void* xn = cx.ws + st.scratch_off;
+                    k::rms_norm(s, (int)x.dtype, sa.x, src_ptr(st, cx, oi++), xn, sa.m, sa.k, in.scale, in.eps);
+                    ++cx.launches;
+                    sa.x = xn;
+                }
+                sa.y = dst;
+                sa.act = in.act == 1 ? 1 : 0;
+                hipEvent_t e0 = nullptr, e1 = nullptr;
+                if (cx.profile) {
+                    GPTRS_HIP_CHECK(hipEventCreate(&e0));
+                    GPTRS_HIP_CHECK(hipEventCreate(&e1));
+                    GPTRS_HIP_CHECK(hipEventRecord(e0, s));
+                }
+                k::skinny_gemm(s, sa);
+                if (cx.profile) {
+                    GPTRS_HIP_CHECK(hipEventRecord(e1, s));
+                    cx.be->prof_events.emplace_back(e0, e1);
+                    ++cx.be->prof_linear_calls;
+                    cx.be->prof_linear_bytes += (int64_t)dtype_size(x.dtype) * (sa.m * sa.k + sa.m * sa.n) + linear_weight_bytes(in, x, w);
                 }
                 ++cx.launches;
                 break;

@@ -275,6 +275,41 @@ def test_attention_prefill(hip, hq, hkv, dh, seq):
     check_program(hip, p, [qkv])
 
 
+@pytest.mark.parametrize("m,k,n", [(2, 3072, 6144), (8, 4096, 3072), (8, 9216, 3072), (16, 3072, 1000), (5, 512, 40), (3, 64, 24),
+                                   (8, 3072, 32768)])
+def test_batched_decode_linear_on_matrix_cores(hip, m, k, n):
+    """2..16 bf16 rows (batched decode): the 16x16x32 MFMA kernel over the 16-column tiled weight copy, plain and
+    under bias + exact GELU + residual; reference = the f32 oracle on the same bf16-representable inputs."""
+    from gptrs_amd.ptir import f32_to_bf16_bits
+    r16 = lambda a: (f32_to_bf16_bits(np.asarray(a, np.float32)).astype(np.uint32) << 16).view(np.float32)  # noqa: E731
+    x, w = r16(rng_uniform(50, (m, k))), r16(rng_uniform(51, (k, n)) * (2.0 / np.sqrt(k)))
+    b, r = r16(rng_uniform(52, (n,))), r16(rng_uniform(53, (m, n)))
+    for build, arrays, dims in [
+        (lambda fb, a, c: a.matmul(c), [x, w], [[m, k], [k, n]]),
+        (lambda fb, a, c, d, e: F.gelu(F.linear(a, c, d)) + e, [x, w, b, r], [[m, k], [k, n], [n], [m, n]]),
+    ]:
+        got = hip_run(hip, prog(build, [("Bf16", d) for d in dims]), arrays)[0]
+        want = oracle_run(prog(build, [("F32", d) for d in dims]), arrays)[0]
+        assert_close(got, want, atol=3e-2, rtol=2e-2, what=f"m={m} k={k} n={n}")
+
+
+@pytest.mark.parametrize("m,k,n", [(8, 3072, 9216), (4, 256, 96)])
+def test_batched_decode_norm_swiglu_on_matrix_cores(hip, m, k, n):
+    from gptrs_amd.ptir import f32_to_bf16_bits
+    r16 = lambda a: (f32_to_bf16_bits(np.asarray(a, np.float32)).astype(np.uint32) << 16).view(np.float32)  # noqa: E731
+    x, g = r16(rng_uniform(54, (m, k)) * 3.0), r16(rng_uniform(55, (k,)) + 1.5)
+    wg, wu = r16(rng_uniform(56, (k, n)) * (2.0 / np.sqrt(k))), r16(rng_uniform(57, (k, n)) * (2.0 / np.sqrt(k)))
+
+    def build(fb, a, gm, c, d):
+        h = F.rms_norm(a, gm, 1e-5)[0]
+        return F.swiglu(h.matmul(c), h.matmul(d))
+
+    dims = [[m, k], [k], [k, n], [k, n]]
+    got = hip_run(hip, prog(build, [("Bf16", d) for d in dims]), [x, g, wg, wu])[0]
+    want = oracle_run(prog(build, [("F32", d) for d in dims]), [x, g, wg, wu])[0]
+    assert_close(got, want, atol=8e-2, rtol=4e-2, what=f"m={m} k={k} n={n}")
+
+
 @pytest.mark.parametrize("dtype", ["F32", "Bf16"])
 def test_temperature_sampling_matches_oracle(hip, dtype):
     """sample_decode_token with temperature > 0 (DecodeSampleRequest, spec.rs:1270-1284): the device kernel and the
