@@ -588,6 +588,71 @@ struct Fuser {
         reindex();
     }
 
+    // Batched decode (the reference has no batch dimension: a batch is B independent sequences whose rows share the
+    // linear layers): Concat_0(ctx_0 .. ctx_{B-1}) of B decode attentions over the rows Slice([b,0],[1,P]) of one
+    // stacked projection, with the same position operands, becomes ONE attention over all sequences.
+    void pass_attention_batch() {
+        const std::vector<int> uses = count_uses();
+        for (size_t ci = 0; ci < fn.body.size(); ++ci) {
+            Instr& cc = fn.body[ci];
+            if (cc.dead || cc.op != OpKind::Concat || cc.axis != 0) continue;
+            const int64_t B = (int64_t)cc.operands.size();
+            if (B < 2 || B > 16) continue;
+            std::vector<Instr*> ats, sls;
+            int src = -1;
+            bool ok = true;
+            for (int64_t b = 0; b < B && ok; ++b) {
+                const int cv = cc.operands[b].value;
+                ok = cv >= 0 && def[cv] >= 0 && uses[cv] == 1;
+                if (!ok) break;
+                Instr* at = &fn.body[def[cv]];
+                ok = at->op == OpKind::FAttnDecode && !at->dead && at->batch <= 1 && at->out_ids[0] == cv;
+                if (!ok) break;
+                const int qv = at->operands[0].value;
+                ok = qv >= 0 && def[qv] >= 0 && uses[qv] == 1;
+                if (!ok) break;
+                Instr* sl = &fn.body[def[qv]];
+                const Spec* ss = sl->op == OpKind::Slice && !sl->dead ? spec_of(sl->operands[0].value) : nullptr;
+                ok = ss && ss->rank() == 2 && ss->dims[0] == B && sl->a == std::vector<int64_t>{b, 0} &&
+                     sl->b == std::vector<int64_t>{1, ss->dims[1]};
+                if (!ok) break;
+                if (b == 0) src = sl->operands[0].value;
+                ok = sl->operands[0].value == src;
+                if (ok && b > 0) {
+                    const Instr* a0 = ats[0];
+                    ok = at->n_q == a0->n_q && at->n_kv == a0->n_kv && at->head_dim == a0->head_dim && at->rot_half == a0->rot_half &&
+                         at->scale == a0->scale && at->operands.size() == a0->operands.size() && at->out_specs == a0->out_specs;
+                    for (size_t o = 3; o < at->operands.size() && ok; ++o) ok = at->operands[o].value >= 0 && at->operands[o].value == a0->operands[o].value;
+                    const Spec* k0 = spec_of(a0->operands[1].value);
+                    const Spec* kb = spec_of(at->operands[1].value);
+                    ok = ok && k0 && kb && *k0 == *kb;
+                }
+                ats.push_back(at);
+                sls.push_back(sl);
+            }
+            if (!ok || (int64_t)ats.size() != B) continue;
+            Instr ni = *ats[0];
+            ni.batch = B;
+            ni.operands[0] = sls[0]->operands[0];
+            for (int64_t b = 1; b < B; ++b) {
+                ni.operands.push_back(ats[b]->operands[1]);
+                ni.operands.push_back(ats[b]->operands[2]);
+            }
+            ni.out_ids = {cc.out_ids[0]};
+            ni.out_specs = {cc.out_specs[0]};
+            for (int64_t b = 0; b < B; ++b) {
+                ni.out_ids.push_back(ats[b]->out_ids[1]); ni.out_specs.push_back(ats[b]->out_specs[1]);
+                ni.out_ids.push_back(ats[b]->out_ids[2]); ni.out_specs.push_back(ats[b]->out_specs[2]);
+            }
+            ni.op_name = "fused.attention_decode_batch";
+            for (Instr* a : ats) a->dead = true;
+            for (Instr* sl : sls) sl->dead = true;
+            fn.body[ci] = ni;
+            ++fused;
+            reindex();
+        }
+    }
+
     // ---------------------------------------------------------------- linear layers
     std::vector<int> count_uses() const {
         std::vector<int> uses(fn.max_value_id + 1, 0);
@@ -849,6 +914,8 @@ int fuse_function(Function& fn) {
     f.pass_attention();
     f.dce();
     f.pass_rope_into_attention();
+    f.dce();
+    f.pass_attention_batch();
     f.dce();
     f.pass_linear();
     f.dce();

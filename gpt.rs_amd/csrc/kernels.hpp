@@ -233,6 +233,10 @@ struct AttnDecodeArgs {
     // optional fused RoPE of Q and of the appended K row (qkv is then the pre-RoPE projection):
     // cos/sin rows [rot_half] of this position; requires rot_half % (16 / element size) == 0
     const void* cos; const void* sin; int64_t rot_half;
+    // batch > 1: `batch` independent sequences in one launch: qkv is [batch, P], ctx [batch, n_q * head_dim], the caches
+    // of sequence b are k_caches[b] / v_caches[b] (k_cache / v_cache are ignored), ws holds batch x the single size
+    int batch;
+    void* k_caches[16]; void* v_caches[16];
 };
 size_t attn_decode_workspace_bytes(int64_t n_q, int64_t head_dim, int64_t capacity);
 void attn_decode(hipStream_t s, const AttnDecodeArgs& a);

@@ -91,13 +91,24 @@ __device__ __forceinline__ T roped_elem(const T* __restrict__ head, int d, int h
 // its own online-softmax state for the G query heads of this kv head.  States are merged by
 // shuffles inside the wave, through LDS across the four waves, and across splits by
 // attn_decode_combine_kernel.
+struct DecodeCaches { void* k[16]; void* v[16]; };   // per-sequence cache pointers of a batched launch (blockIdx.z)
+
 template <typename T, int G>
 __global__ __launch_bounds__(256) void attn_decode_kernel(const T* __restrict__ qkv, T* __restrict__ kc,
                                                           T* __restrict__ vc, const int32_t* __restrict__ us,
                                                           const int32_t* __restrict__ qs, T* __restrict__ ctx,
                                                           float* __restrict__ ws, int n_q, int n_kv, int dh,
                                                           int64_t cap, float scale, int64_t chunk, int nsplit,
-                                                          const T* __restrict__ cs, const T* __restrict__ sn, int half) {
+                                                          const T* __restrict__ cs, const T* __restrict__ sn, int half,
+                                                          int batched, DecodeCaches caches) {
+    if (batched) {   // sequence blockIdx.z: its row of the stacked projection and of the context, its caches, its records
+        const int b = blockIdx.z;
+        kc = (T*)caches.k[b];
+        vc = (T*)caches.v[b];
+        qkv += (int64_t)b * (n_q + 2 * n_kv) * dh;
+        ctx += (int64_t)b * n_q * dh;
+        ws += (int64_t)b * n_q * nsplit * (dh + 2);
+    }
     constexpr int VEC = Vec16<T>::N;
     const int lpr = dh / VEC;          // lanes per cache row (power of two, <= 64)
     const int rpw = 64 / lpr;          // rows per wave-iteration
@@ -235,6 +246,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const T* __restrict__ 
 
 template <typename T>
 __global__ void attn_decode_combine_kernel(const float* __restrict__ ws, T* __restrict__ ctx, int dh, int nsplit) {
+    // grid (n_q, batch): sequence blockIdx.y owns gridDim.x heads of records and of the context
+    ws += (int64_t)blockIdx.y * gridDim.x * nsplit * (dh + 2);
+    ctx += (int64_t)blockIdx.y * gridDim.x * dh;
     // per-split weights exp(m_s - max) are computed once into LDS; the slice loads of the output
     // loop are then independent of each other
     __shared__ float wgt[kMaxDecodeSplits];
@@ -289,12 +303,23 @@ static void attn_decode_t(hipStream_t s, const AttnDecodeArgs& a) {
     int nsplit;
     int64_t chunk;
     decode_geometry(a.dtype, a.head_dim, a.capacity, &nsplit, &chunk);
-    dim3 grid((unsigned)a.n_kv, (unsigned)nsplit);
+    const int nb = a.batch > 1 ? a.batch : 1;
+    // a batch multiplies the workgroups: longer chunks keep the launch near six workgroups per CU, so the fixed cost
+    // of a workgroup (query load, state merges, record) is spread over more positions (fewer splits than the
+    // workspace was sized for is always safe)
+    const int64_t step = chunk;
+    while (nsplit > 1 && (int64_t)a.n_kv * nb * nsplit > 1536) {
+        chunk += step;
+        nsplit = (int)cdiv(a.capacity, chunk);
+    }
+    dim3 grid((unsigned)a.n_kv, (unsigned)nsplit, (unsigned)nb);
     const int g = (int)(a.n_q / a.n_kv);
+    DecodeCaches caches{};
+    for (int b = 0; b < nb && b < 16; ++b) { caches.k[b] = a.k_caches[b]; caches.v[b] = a.v_caches[b]; }
 #define GPTRS_LAUNCH(G)                                                                                          \
     attn_decode_kernel<T, G><<<grid, 256, 0, s>>>((const T*)a.qkv, (T*)a.k_cache, (T*)a.v_cache, a.update_starts,    \
         a.query_start, (T*)a.ctx, (float*)a.ws, (int)a.n_q, (int)a.n_kv, (int)a.head_dim, a.capacity, a.scale, chunk, nsplit, \
-        (const T*)a.cos, (const T*)a.sin, (int)a.rot_half)
+        (const T*)a.cos, (const T*)a.sin, (int)a.rot_half, a.batch > 1 ? 1 : 0, caches)
     switch (g) {
         case 1: GPTRS_LAUNCH(1); break;
         case 2: GPTRS_LAUNCH(2); break;
@@ -304,7 +329,7 @@ static void attn_decode_t(hipStream_t s, const AttnDecodeArgs& a) {
 #undef GPTRS_LAUNCH
     if (nsplit > 1) {
         const int block = a.head_dim <= 64 ? 64 : (a.head_dim <= 128 ? 128 : 256);
-        attn_decode_combine_kernel<T><<<(unsigned)a.n_q, block, 0, s>>>((const float*)a.ws, (T*)a.ctx, (int)a.head_dim, nsplit);
+        attn_decode_combine_kernel<T><<<dim3((unsigned)a.n_q, (unsigned)nb), block, 0, s>>>((const float*)a.ws, (T*)a.ctx, (int)a.head_dim, nsplit);
     }
 }
 void attn_decode(hipStream_t s, const AttnDecodeArgs& a) {

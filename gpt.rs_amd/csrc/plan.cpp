@@ -570,7 +570,7 @@ void Builder::describe(Step& st) {
         case OpKind::FAttnDecode: {
             const Spec& ck = spec_of(in, 1);
             st.scratch_bytes = std::max(k::attn_decode_workspace_bytes(in.n_q, in.head_dim, ck.dims[1]),
-                                        k::chain_attn_part_bytes(in.n_q, in.n_kv, in.head_dim));
+                                        k::chain_attn_part_bytes(in.n_q, in.n_kv, in.head_dim)) * (size_t)std::max<int64_t>(in.batch, 1);
             break;
         }
         default:
@@ -677,7 +677,11 @@ void Builder::build() {
     for (auto& st : plan.steps) {
         std::vector<std::pair<int, int>> pairs;  // (base operand slot, output slot)
         if (st.in.op == OpKind::DynamicUpdateSlice) pairs = {{0, 0}};
-        if (st.in.op == OpKind::FAttnDecode) pairs = {{1, 1}, {2, 2}};
+        if (st.in.op == OpKind::FAttnDecode)
+            for (int64_t b = 0; b < std::max<int64_t>(st.in.batch, 1); ++b) {
+                pairs.push_back({(int)attn_cache_operand(st.in, b), (int)attn_cache_output(b)});
+                pairs.push_back({(int)attn_cache_operand(st.in, b) + 1, (int)attn_cache_output(b) + 1});
+            }
         bool all_inplace = !pairs.empty();
         for (auto& pr : pairs) {
             const int bv = st.src[pr.first];
@@ -755,6 +759,7 @@ void Builder::build() {
     auto chain_phases = [&](const Step& st) -> int {   // phases the step takes in a chain, 0: not chainable
         const Instr& in = st.in;
         if (in.op == OpKind::FAttnDecode) {
+            if (in.batch > 1) return 0;
             const Spec& x = plan.values[st.src[0]].spec;
             return k::chain_attn_supported((int)x.dtype, x.dims[0], in.n_q, in.n_kv, in.head_dim, in.rot_half) ? 2 : 0;
         }
@@ -1230,16 +1235,22 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
             if (cx.chain && st.chain_member) break;  // executed by the launch of the run's first step
             if (cx.chain && st.chain_len > 0 && run_chain(plan, st, cx)) break;
             const Spec& ck = in_spec(1);
-            void* kout = cx.ptr[st.dst[1]];
-            void* vout = cx.ptr[st.dst[2]];
-            const void* kin = src_ptr(st, cx, 1);
-            const void* vin = src_ptr(st, cx, 2);
-            if (kout != kin) { GPTRS_HIP_CHECK(hipMemcpyAsync(kout, kin, ck.bytes(), hipMemcpyDeviceToDevice, s)); ++cx.launches; }
-            if (vout != vin) { GPTRS_HIP_CHECK(hipMemcpyAsync(vout, vin, ck.bytes(), hipMemcpyDeviceToDevice, s)); ++cx.launches; }
             k::AttnDecodeArgs a{};
+            const int64_t nb = std::max<int64_t>(in.batch, 1);
+            for (int64_t b = 0; b < nb; ++b) {   // caches that were not donated are copied first
+                const size_t ci = attn_cache_operand(in, b), oi = attn_cache_output(b);
+                void* kout = cx.ptr[st.dst[oi]];
+                void* vout = cx.ptr[st.dst[oi + 1]];
+                const void* kin = src_ptr(st, cx, ci);
+                const void* vin = src_ptr(st, cx, ci + 1);
+                if (kout != kin) { GPTRS_HIP_CHECK(hipMemcpyAsync(kout, kin, ck.bytes(), hipMemcpyDeviceToDevice, s)); ++cx.launches; }
+                if (vout != vin) { GPTRS_HIP_CHECK(hipMemcpyAsync(vout, vin, ck.bytes(), hipMemcpyDeviceToDevice, s)); ++cx.launches; }
+                if (b == 0) { a.k_cache = kout; a.v_cache = vout; }
+                a.k_caches[b] = kout; a.v_caches[b] = vout;
+            }
+            a.batch = (int)in.batch;
             a.dtype = (int)out.dtype;
             a.qkv = src_ptr(st, cx, 0);
-            a.k_cache = kout; a.v_cache = vout;
             a.update_starts = (const int32_t*)src_ptr(st, cx, 3);
             a.query_start = (const int32_t*)src_ptr(st, cx, 4);
             a.ctx = dst;

@@ -108,6 +108,10 @@ struct Instr {
     // fused-op parameters
     float eps = 0.f, scale = 0.f;
     int64_t n_q = 0, n_kv = 0, head_dim = 0, rot_half = 0;
+    // FAttnDecode over `batch` independent sequences in one launch (0 / 1: a single sequence): operand 0 is the
+    // stacked [batch, P] projection, the caches of sequence b >= 1 follow the single-sequence operands in pairs,
+    // outputs are (ctx[batch, q_proj], k_0, v_0, k_1, v_1, ...)
+    int64_t batch = 0;
     int act = 0;                      // FLinear epilogue: 0 none, 1 gelu, 2 swiglu (dual weights)
     bool has_bias = false, has_residual = false;
     float fparam[4] = {0.f, 0.f, 0.f, 0.f};  // FGelu: half, divisor, one
@@ -121,6 +125,10 @@ struct Instr {
     bool scalar_rhs = false;                 // Binary whose rhs is a broadcast scalar literal
     float scalar_val = 0.f;
 };
+
+// FAttnDecode: operand slots of the K / V cache of sequence b, output slot of its updated K cache (V follows)
+inline size_t attn_cache_operand(const Instr& in, int64_t b) { return b == 0 ? 1 : (size_t)(5 + (in.rot_half > 0 ? 2 : 0) + 2 * (b - 1)); }
+inline size_t attn_cache_output(int64_t b) { return (size_t)(1 + 2 * b); }
 
 // operand position of the SwiGLU partner's weights / of the first epilogue operand of an FLinear
 inline size_t linear_w2_pos(const Instr& in) { return in.quant ? 3 : 2; }

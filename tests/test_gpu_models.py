@@ -216,6 +216,42 @@ def test_batched_decode_matches_single_sequences(hip):
     assert toks == singles
 
 
+@pytest.mark.parametrize("dtype", ["F32", "Bf16"])
+def test_batched_ministral_decode_one_attention_launch_per_layer(hip, dtype):
+    """Batched decode runs ONE attention over all sequences per layer (their rows of the stacked projection, their
+    own caches) instead of slice -> attention -> concat per sequence: same logits as the sequences run alone, and
+    the launch count of a step no longer grows with the batch."""
+    cfg = MID_MINISTRAL
+    m = models.Ministral.random(cfg, hip, seed=23, dtype=dtype, std=0.05)
+    prompts = [[1, 2, 3, 4, 5], [9, 8, 7, 6, 5], [5, 5, 5, 5, 5], [11, 400, 30, 2, 77], [6, 1, 6, 1, 6]]
+    B, seq = len(prompts), len(prompts[0])
+    single_logits = []
+    for p in prompts:
+        gen = models.Generator(m, p, kv_cache_capacity=32, device_sampling=False)
+        rows = []
+        for _ in range(4):
+            gen.step()
+            rows.append(hip.to_numpy(gen.logits)[-1].astype(np.float32).copy())
+        single_logits.append(rows)
+    caches = [[None] * cfg.num_layers for _ in prompts]
+    lg = hip.to_numpy(m.forward_batch(prompts, 0, caches, 32)).astype(np.float32)
+    toks = [int(np.argmax(lg[b * seq + seq - 1])) for b in range(B)]
+    for step in range(4):
+        lg = hip.to_numpy(m.forward_batch([[t] for t in toks], seq + step, caches, 32)).astype(np.float32)
+        launches = hip.counter("last_program_launches")
+        for b in range(B):
+            if dtype == "F32":
+                assert rel_err(lg[b], single_logits[b][step]) < 1e-4, (step, b)
+            else:
+                assert float(np.max(np.abs(lg[b] - single_logits[b][step]))) < 2e-2, (step, b)
+        toks = [int(np.argmax(single_logits[b][step])) for b in range(B)]
+    # one attention (+ its combine) per layer whatever the batch: a batch of two launches as many kernels as five
+    caches2 = [[None] * cfg.num_layers for _ in range(2)]
+    m.forward_batch(prompts[:2], 0, caches2, 32)
+    m.forward_batch([[1], [2]], seq, caches2, 32)
+    assert hip.counter("last_program_launches") == launches
+
+
 # ------------------------------------------------------------------ full-size shapes
 def test_gpt2_small_f32_greedy_64_tokens_vs_oracle(hip):
     """BASELINE config 0: GPT-2 small f32, weights N(0,0.02) seed 0, prompt 16 ids seed 1, greedy 64
