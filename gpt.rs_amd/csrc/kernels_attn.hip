@@ -40,6 +40,9 @@ template <> struct Vec16<bf16_t> {
 
 constexpr int kMaxDecodeSplits = 512;
 
+typedef __bf16 bf16x8_v __attribute__((ext_vector_type(8)));
+typedef float f32x16_v __attribute__((ext_vector_type(16)));
+
 __device__ __forceinline__ int64_t clamp_i64(int64_t v, int64_t lo, int64_t hi) { return v < lo ? lo : (v > hi ? hi : v); }
 
 // Rotate-half RoPE (ops/functional/rotary.rs:430-536) applied while loading VEC consecutive dims
@@ -244,6 +247,204 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const T* __restrict__ 
     }
 }
 
+// bf16 decode attention with the scores on the matrix cores.  grid (n_kv, nsplit, batch), 256 threads; wave w of a
+// workgroup takes the 32-key tiles w, w+4, ... of the workgroup's chunk.  Per tile
+//   S^T[key, q] = K[key, :] . Q[q, :]   v_mfma_f32_32x32x16_bf16, A = cache rows straight from memory (lane = key row),
+//                                       B = the group's G query heads in columns 0..G-1 (other columns repeat them)
+// so a lane owns ONE query: its 16 scores, the running maximum and sum (log2 domain) are per-lane values and the
+// softmax costs a few instructions per key instead of a cross-lane reduction per key and head.  The probabilities go
+// through LDS to the layout of the second product, which stays on the vector ALUs in f32: lane-group `sub` (DH/8
+// lanes, 16 bytes of a V row each) accumulates O[g, :] over its keys of the tile.  States are merged across
+// lane-groups by shuffles, across waves through LDS, across splits by attn_decode_combine_kernel (same records as
+// attn_decode_kernel, maxima in natural-log units).
+template <int DH, int G>
+__global__ __launch_bounds__(256) void attn_decode_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ kc,
+                                                               bf16_t* __restrict__ vc, const int32_t* __restrict__ us,
+                                                               const int32_t* __restrict__ qs, bf16_t* __restrict__ ctx,
+                                                               float* __restrict__ ws, int n_q, int n_kv, int64_t cap,
+                                                               float scale_log2e, int64_t chunk, int nsplit,
+                                                               const bf16_t* __restrict__ cs, const bf16_t* __restrict__ sn,
+                                                               int half_rot, int batched, DecodeCaches caches) {
+    constexpr int NK = DH / 16;        // k-steps of the score product
+    constexpr int LPR = DH / 8;        // lanes per V row
+    constexpr int NSUB = 64 / LPR;     // lane-groups per wave
+    constexpr int NV = 32 / NSUB;      // keys of a tile per lane-group
+    __shared__ __align__(16) float p_lds[2][4][G][32];
+    __shared__ float corr_lds[2][4][G];
+    __shared__ float sm[4][G], sl[4][G];
+    __shared__ float so[4][G][DH];
+    __shared__ __align__(16) bf16_t q_lds[G][DH];
+    if (batched) {
+        const int b = blockIdx.z;
+        kc = (bf16_t*)caches.k[b];
+        vc = (bf16_t*)caches.v[b];
+        qkv += (int64_t)b * (n_q + 2 * n_kv) * DH;
+        ctx += (int64_t)b * n_q * DH;
+        ws += (int64_t)b * n_q * nsplit * (DH + 2);
+    }
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, half = lane >> 5;
+    const int sub = lane / LPR, li = lane % LPR;
+    const int kvh = blockIdx.x, split = blockIdx.y;
+    const int64_t qpos = clamp_i64(qs[0], 0, cap - 1);
+    const int64_t upd = clamp_i64(us[1], 0, cap - 1);
+    const bf16_t* knew = qkv + (int64_t)n_q * DH + (int64_t)kvh * DH;
+    const bf16_t* vnew = qkv + (int64_t)(n_q + n_kv) * DH + (int64_t)kvh * DH;
+    bf16_t* kbase = kc + (int64_t)kvh * cap * DH;
+    bf16_t* vbase = vc + (int64_t)kvh * cap * DH;
+
+    // append this step's row (one workgroup per kv head owns position `upd`); the rows are read back below, by this
+    // workgroup only, after the barrier
+    if (upd / chunk == split) {
+        for (int d = tid; d < DH; d += 256) {
+            kbase[upd * DH + d] = cs ? roped_elem<bf16_t>(knew, d, half_rot, cs, sn) : knew[d];
+            vbase[upd * DH + d] = vnew[d];
+        }
+        __threadfence_block();
+    }
+    // the group's query heads, rotated once per workgroup (16 bytes per thread)
+    for (int c = tid; c < G * LPR; c += 256) {
+        const int g = c / LPR, c0 = (c % LPR) * 8;
+        const bf16_t* qh = qkv + (int64_t)(kvh * G + g) * DH;
+        if (cs) {
+            float f[8];
+            load_roped<bf16_t>(qh, c0, half_rot, cs, sn, f);
+            bf16x8_v r;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) r[e] = (__bf16)f[e];   // exact: f holds bf16 values
+            *reinterpret_cast<bf16x8_v*>(&q_lds[g][c0]) = r;
+        } else {
+            *reinterpret_cast<uint4*>(&q_lds[g][c0]) = *reinterpret_cast<const uint4*>(qh + c0);
+        }
+    }
+    __syncthreads();
+
+    const int64_t p0 = (int64_t)split * chunk;
+    int64_t p1 = p0 + chunk;
+    if (p1 > qpos + 1) p1 = qpos + 1;
+
+    // query fragments: column = query head col % G, 8 consecutive d per lane and k-step
+    bf16x8_v qf[NK];
+#pragma unroll
+    for (int kk = 0; kk < NK; ++kk) qf[kk] = *reinterpret_cast<const bf16x8_v*>(&q_lds[col % G][16 * kk + 8 * half]);
+    float o[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[g][e] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+
+    const int ntiles = p1 > p0 ? (int)((p1 - p0 + 31) / 32) : 0;
+    const int iters = (ntiles + 3) / 4;   // uniform over the workgroup
+    for (int it = 0; it < iters; ++it) {
+        const int buf = it & 1;
+        const int64_t kb = p0 + (int64_t)(it * 4 + wave) * 32;
+        const bool active = kb < p1;
+        uint4 vreg[NV];
+        if (active) {
+            // rows past the last attended position re-read that position and get probability zero
+            const bf16_t* krow = kbase + (kb + col < p1 ? kb + col : p1 - 1) * DH + 8 * half;
+            bf16x8_v kf[NK];
+#pragma unroll
+            for (int kk = 0; kk < NK; ++kk) kf[kk] = *reinterpret_cast<const bf16x8_v*>(krow + 16 * kk);
+#pragma unroll
+            for (int j = 0; j < NV; ++j) {
+                const int64_t key = kb + NV * sub + j;
+                vreg[j] = *reinterpret_cast<const uint4*>(vbase + (key < p1 ? key : p1 - 1) * DH + li * 8);
+            }
+            f32x16_v sc;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) sc[v] = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < NK; ++kk) sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[kk], qf[kk], sc, 0, 0, 0);
+            float mx = -INFINITY;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int64_t key = kb + 8 * (v >> 2) + (v & 3) + 4 * half;
+                const float x = key < p1 ? sc[v] * scale_log2e : -INFINITY;
+                sc[v] = x;
+                mx = fmaxf(mx, x);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m_run, mx);   // finite: the tile holds at least one attended key
+            const float corr = exp2f(m_run - m_new);
+            float ls = 0.f;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                sc[v] = exp2f(sc[v] - m_new);
+                ls += sc[v];
+            }
+            ls += __shfl_xor(ls, 32, 64);
+            l_run = l_run * corr + ls;
+            m_run = m_new;
+            if (col < G) {
+#pragma unroll
+                for (int q4 = 0; q4 < 4; ++q4)
+                    *reinterpret_cast<float4*>(&p_lds[buf][wave][col][8 * q4 + 4 * half]) =
+                        make_float4(sc[4 * q4], sc[4 * q4 + 1], sc[4 * q4 + 2], sc[4 * q4 + 3]);
+                if (half == 0) corr_lds[buf][wave][col] = corr;
+            }
+        }
+        __syncthreads();
+        if (active) {
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const float c = corr_lds[buf][wave][g];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[g][e] *= c;
+            }
+#pragma unroll
+            for (int j = 0; j < NV; ++j) {
+                const float vf[8] = {bf16lo(vreg[j].x), bf16hi(vreg[j].x), bf16lo(vreg[j].y), bf16hi(vreg[j].y),
+                                     bf16lo(vreg[j].z), bf16hi(vreg[j].z), bf16lo(vreg[j].w), bf16hi(vreg[j].w)};
+#pragma unroll
+                for (int g = 0; g < G; ++g) {
+                    const float pj = p_lds[buf][wave][g][NV * sub + j];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) o[g][e] += pj * vf[e];
+                }
+            }
+        }
+    }
+
+    // merge the lane-groups of this wave (they share the wave's maximum), then the four waves through LDS
+#pragma unroll
+    for (int off = LPR; off < 64; off <<= 1)
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[g][e] += __shfl_xor(o[g][e], off, 64);
+    if (sub == 0) {
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) so[wave][g][li * 8 + e] = o[g][e];
+    }
+    if (lane < G) { sm[wave][lane] = m_run; sl[wave][lane] = l_run; }
+    __syncthreads();
+    for (int idx = tid; idx < G * DH; idx += 256) {
+        const int g = idx / DH, d = idx % DH;
+        const float mn = fmaxf(fmaxf(sm[0][g], sm[1][g]), fmaxf(sm[2][g], sm[3][g]));
+        float L = 0.f, O = 0.f;
+        if (mn != -INFINITY) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const float c = exp2f(sm[w][g] - mn);
+                L += sl[w][g] * c;
+                O += so[w][g][d] * c;
+            }
+        }
+        const int h = kvh * G + g;
+        if (nsplit == 1) {
+            stf(ctx, (int64_t)h * DH + d, O / L);
+        } else {
+            float* rec = ws + ((int64_t)h * nsplit + split) * (DH + 2);
+            if (d == 0) { rec[0] = mn * 0.6931471805599453f; rec[1] = L; }
+            rec[2 + d] = O;
+        }
+    }
+}
+
 template <typename T>
 __global__ void attn_decode_combine_kernel(const float* __restrict__ ws, T* __restrict__ ctx, int dh, int nsplit) {
     // grid (n_q, batch): sequence blockIdx.y owns gridDim.x heads of records and of the context
@@ -298,6 +499,55 @@ size_t attn_decode_workspace_bytes(int64_t n_q, int64_t head_dim, int64_t capaci
     return (size_t)n_q * (size_t)ns * (size_t)(head_dim + 2) * sizeof(float);
 }
 
+// Matrix-core decode path: bf16, head_dim 64 / 128, group sizes 1, 2, 4, 8 (GPTRS_HIP_MFMA_ATTN=0 turns it off).
+static bool attn_decode_mfma_ok(const AttnDecodeArgs& a) {
+    static const bool use = [] { const char* e = getenv("GPTRS_HIP_MFMA_ATTN"); return !(e && e[0] == '0'); }();
+    if (!use || a.dtype != 2 || a.n_kv <= 0 || a.n_q % a.n_kv != 0) return false;
+    if (a.head_dim != 64 && a.head_dim != 128) return false;
+    if (a.cos && a.rot_half % 8 != 0) return false;
+    const int64_t g = a.n_q / a.n_kv;
+    return g == 1 || g == 2 || g == 4 || g == 8;
+}
+
+static void attn_decode_mfma(hipStream_t s, const AttnDecodeArgs& a) {
+    int nsplit;
+    int64_t chunk;
+    decode_geometry(a.dtype, a.head_dim, a.capacity, &nsplit, &chunk);   // the workspace holds this many splits
+    const int nb = a.batch > 1 ? a.batch : 1;
+    // chunks of whole 32-key tiles, never shorter than the workspace geometry's; lengthened until the launch is
+    // near four workgroups per CU (each wave then walks several tiles)
+    const int64_t step = chunk > 32 ? chunk : 32;
+    chunk = step;
+    nsplit = (int)cdiv(a.capacity, chunk);
+    while (nsplit > 1 && (int64_t)a.n_kv * nb * nsplit > 1024) {
+        chunk += step;
+        nsplit = (int)cdiv(a.capacity, chunk);
+    }
+    dim3 grid((unsigned)a.n_kv, (unsigned)nsplit, (unsigned)nb);
+    DecodeCaches caches{};
+    for (int b = 0; b < nb && b < 16; ++b) { caches.k[b] = a.k_caches[b]; caches.v[b] = a.v_caches[b]; }
+    const float sl = a.scale * 1.44269504088896f;
+    const int g = (int)(a.n_q / a.n_kv);
+#define GPTRS_LAUNCH(DH, G)                                                                                          \
+    attn_decode_mfma_kernel<DH, G><<<grid, 256, 0, s>>>((const bf16_t*)a.qkv, (bf16_t*)a.k_cache, (bf16_t*)a.v_cache, \
+        a.update_starts, a.query_start, (bf16_t*)a.ctx, (float*)a.ws, (int)a.n_q, (int)a.n_kv, a.capacity, sl, chunk, \
+        nsplit, (const bf16_t*)a.cos, (const bf16_t*)a.sin, (int)a.rot_half, a.batch > 1 ? 1 : 0, caches)
+#define GPTRS_LAUNCH_G(DH)                                                                                           \
+    switch (g) {                                                                                                     \
+        case 1: GPTRS_LAUNCH(DH, 1); break;                                                                          \
+        case 2: GPTRS_LAUNCH(DH, 2); break;                                                                          \
+        case 4: GPTRS_LAUNCH(DH, 4); break;                                                                          \
+        default: GPTRS_LAUNCH(DH, 8); break;                                                                         \
+    }
+    if (a.head_dim == 64) { GPTRS_LAUNCH_G(64) } else { GPTRS_LAUNCH_G(128) }
+#undef GPTRS_LAUNCH_G
+#undef GPTRS_LAUNCH
+    if (nsplit > 1) {
+        const int block = a.head_dim <= 64 ? 64 : 128;
+        attn_decode_combine_kernel<bf16_t><<<dim3((unsigned)a.n_q, (unsigned)nb), block, 0, s>>>((const float*)a.ws, (bf16_t*)a.ctx, (int)a.head_dim, nsplit);
+    }
+}
+
 template <typename T>
 static void attn_decode_t(hipStream_t s, const AttnDecodeArgs& a) {
     int nsplit;
@@ -333,7 +583,8 @@ static void attn_decode_t(hipStream_t s, const AttnDecodeArgs& a) {
     }
 }
 void attn_decode(hipStream_t s, const AttnDecodeArgs& a) {
-    if (a.dtype == 0) attn_decode_t<float>(s, a);
+    if (attn_decode_mfma_ok(a)) attn_decode_mfma(s, a);
+    else if (a.dtype == 0) attn_decode_t<float>(s, a);
     else attn_decode_t<bf16_t>(s, a);
 }
 
@@ -403,9 +654,6 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const T* __restrict__
 // scalar, the rescaling of O^T is a per-lane multiply, and P^T needs no cross-lane movement to become the B operand:
 // the k-slots of the second product are simply numbered in the order the lane holds its keys, and V^T is written to
 // LDS in that order (key bits 2 and 3 swapped).
-typedef __bf16 bf16x8_v __attribute__((ext_vector_type(8)));
-typedef float f32x16_v __attribute__((ext_vector_type(16)));
-
 template <int DH>
 __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ctx, int T,
                                                                 int n_q, int n_kv, float scale_log2e) {

@@ -216,12 +216,17 @@ def test_batched_decode_matches_single_sequences(hip):
     assert toks == singles
 
 
+WIDE_HEAD_MINISTRAL = models.MinistralConfig(vocab_size=512, context_length=128, embed_dim=256, num_layers=2, num_heads=8,
+                                             num_kv_heads=2, head_dim=64, ffn_dim=512, rotary_dim=64, rope_theta=1e6)
+
+
+@pytest.mark.parametrize("cfg", [MID_MINISTRAL, WIDE_HEAD_MINISTRAL], ids=["head32", "head64"])
 @pytest.mark.parametrize("dtype", ["F32", "Bf16"])
-def test_batched_ministral_decode_one_attention_launch_per_layer(hip, dtype):
+def test_batched_ministral_decode_one_attention_launch_per_layer(hip, dtype, cfg):
     """Batched decode runs ONE attention over all sequences per layer (their rows of the stacked projection, their
     own caches) instead of slice -> attention -> concat per sequence: same logits as the sequences run alone, and
-    the launch count of a step no longer grows with the batch."""
-    cfg = MID_MINISTRAL
+    the launch count of a step no longer grows with the batch.  (head32: the vector-ALU kernel; head64 in bf16: the
+    matrix-core kernel.)"""
     m = models.Ministral.random(cfg, hip, seed=23, dtype=dtype, std=0.05)
     prompts = [[1, 2, 3, 4, 5], [9, 8, 7, 6, 5], [5, 5, 5, 5, 5], [11, 400, 30, 2, 77], [6, 1, 6, 1, 6]]
     B, seq = len(prompts), len(prompts[0])

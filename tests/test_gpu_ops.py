@@ -366,7 +366,8 @@ def test_attention_with_concat_cache(hip):
 
 
 @pytest.mark.parametrize("dtype", ["F32", "Bf16"])
-@pytest.mark.parametrize("hq,hkv,dh,cap", [(4, 4, 8, 16), (4, 2, 8, 32), (8, 2, 16, 128), (12, 12, 64, 128), (32, 8, 128, 256), (4, 4, 1, 8), (6, 2, 4, 16)])
+@pytest.mark.parametrize("hq,hkv,dh,cap", [(4, 4, 8, 16), (4, 2, 8, 32), (8, 2, 16, 128), (12, 12, 64, 128), (32, 8, 128, 256), (4, 4, 1, 8), (6, 2, 4, 16),
+                                           (8, 2, 128, 2048), (16, 2, 64, 1024), (4, 2, 64, 640), (24, 2, 64, 64)])
 def test_attention_decode_cache(hip, dtype, hq, hkv, dh, cap):
     cfg = F.AttentionConfig(hq * dh, hq, hkv, dh)
     P = cfg.total_projection_dim
