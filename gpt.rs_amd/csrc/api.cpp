@@ -72,8 +72,8 @@ Backend::Backend(int dev) : device(dev) {
     GPTRS_HIP_CHECK(hipMalloc((void**)&d_argmax_idx_, 1024 * sizeof(int32_t)));
     GPTRS_HIP_CHECK(hipMalloc((void**)&d_token_, 256));
     GPTRS_HIP_CHECK(hipHostMalloc(&h_pinned_, 256, hipHostMallocDefault));
-    GPTRS_HIP_CHECK(hipMalloc((void**)&d_chain_bar_, k::kChainBarrierBytes));
-    k::fill_zero(stream, d_chain_bar_, k::kChainBarrierBytes);
+    GPTRS_HIP_CHECK(hipMalloc((void**)&d_chain_bar_, k::kChainBarrierBytes + k::kSkinnyTickets * sizeof(unsigned)));
+    k::fill_zero(stream, d_chain_bar_, k::kChainBarrierBytes + k::kSkinnyTickets * sizeof(unsigned));
     {
         const char* c = getenv("GPTRS_HIP_CHAIN");
         if (c && c[0] == '0') opt_chain = false;

@@ -806,7 +806,8 @@ struct Fuser {
                 continue;
             }
             if (!k::gemv_tiled_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1])) continue;
-            if (in.act == 2 && M > 8) continue;
+            // SwiGLU pairs: the vector kernel holds up to 8 rows, the matrix-core kernel of batched decode up to 16
+            if (in.act == 2 && M > 8 && !k::skinny_gemm_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1])) continue;
             in.tiled = true;
         }
         const std::vector<int> uses = count_uses();

@@ -116,7 +116,13 @@ struct SkinnyLinearArgs {
     void* y;
     int64_t m, k, n;
     int act;
+    // split-K over workgroups (layers with few tiles): part = skinny_workspace_bytes() of scratch, tickets =
+    // kSkinnyTickets counters zeroed once (every launch leaves them zero); without them the layer runs unsplit
+    void* part; size_t part_bytes; unsigned* tickets;
 };
+constexpr size_t kSkinnyTickets = 1024;
+int skinny_ksplit(int64_t k, int64_t n);
+size_t skinny_workspace_bytes(int64_t k, int64_t n, bool dual);
 bool skinny_gemm_supported(int dtype, int64_t m, int64_t k, int64_t n);
 size_t skinny_weight_bytes(int64_t k, int64_t n);
 void skinny_pack_weights(hipStream_t s, const void* w, void* out, int64_t k, int64_t n);

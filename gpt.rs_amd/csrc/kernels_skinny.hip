@@ -11,6 +11,11 @@
 // the 32-k steps round-robin (so the workgroup reads 4 consecutive KiB per round) and add their partial products
 // through LDS.  The A operand (lane = 16 * k-group + row) comes straight from x, which is small and stays in L2.
 // DUAL computes silu(x.W) * (x.W2) (ops/functional/activation.rs:141-162) from two weight copies.
+//
+// A layer with few tiles (N = 3072 has 192, fewer than there are CUs) is split along K over gridDim.y workgroups per
+// tile so the whole chip streams: each writes its 16 x 16 partial sums to a workspace and takes a ticket; the
+// workgroup that draws the last ticket of a tile adds the partials in split order (so the result does not depend on
+// which one that is), applies the epilogue and resets the ticket for the next launch.
 #include "kernels.hpp"
 #include "device_utils.hpp"
 
@@ -58,20 +63,21 @@ template <bool DUAL>
 __global__ __launch_bounds__(256) void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ ws,
                                                           const bf16_t* __restrict__ ws2, const bf16_t* __restrict__ bias,
                                                           const bf16_t* __restrict__ residual, bf16_t* __restrict__ y, int M, int K,
-                                                          int N, int act) {
+                                                          int N, int act, float* __restrict__ part, unsigned* __restrict__ tickets) {
     constexpr int U = 4;                         // 32-k steps per wave and round, all requested before the first is used
     __shared__ float red[4][DUAL ? 2 : 1][64][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int c = lane & 15, kg = lane >> 4;     // B: column c, k-group kg; A: row c, k-group kg
     const int tile = blockIdx.x;
-    const int nsteps = K / 32;
+    const int ksplit = gridDim.y, ks = blockIdx.y;
+    const int s_begin = (int)((int64_t)(K / 32) * ks / ksplit), nsteps = (int)((int64_t)(K / 32) * (ks + 1) / ksplit);
     const u32x4_s* bsrc = reinterpret_cast<const u32x4_s*>(ws) + (int64_t)tile * (K / 8) * 16 + lane;
     const u32x4_s* bsrc2 = DUAL ? reinterpret_cast<const u32x4_s*>(ws2) + (int64_t)tile * (K / 8) * 16 + lane : nullptr;
     const int arow = c < M ? c : M - 1;          // rows beyond M re-read the last one; their products are never stored
     const u32x4_s* asrc = reinterpret_cast<const u32x4_s*>(x + (int64_t)arow * K + 8 * kg);
 
     f32x4_s acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
-    for (int s0 = wave; s0 < nsteps; s0 += 4 * U) {
+    for (int s0 = s_begin + wave; s0 < nsteps; s0 += 4 * U) {
         u32x4_s b[U], b2[DUAL ? U : 1], a[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -96,6 +102,46 @@ __global__ __launch_bounds__(256) void skinny_gemm_kernel(const bf16_t* __restri
     }
     __syncthreads();
     if (wave != 0) return;
+    constexpr int NP = DUAL ? 2 : 1;
+    float g[4], up[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        g[i] = up[i] = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            g[i] += red[w][0][lane][i];
+            if (DUAL) up[i] += red[w][DUAL ? 1 : 0][lane][i];
+        }
+    }
+    if (ksplit > 1) {
+        // partials and tickets cross workgroups through device-scope accesses only (coherent across the L2s of the
+        // XCDs without cache maintenance): stores acknowledged, then the ticket
+        float* mine = part + ((int64_t)tile * ksplit + ks) * NP * 256 + lane * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            __hip_atomic_store(mine + i, g[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (DUAL) __hip_atomic_store(mine + 256 + i, up[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);                         // vmcnt(0)
+        asm volatile("" ::: "memory");
+        unsigned t = 0;
+        if (lane == 0) t = __hip_atomic_fetch_add(&tickets[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        t = __shfl(t, 0, 64);
+        if (t != (unsigned)(ksplit - 1)) return;
+        asm volatile("" ::: "memory");                              // the partials are read after the ticket is known
+        // every ticket of this launch has been drawn: leave the counter at zero for the next one
+        if (lane == 0) __hip_atomic_store(&tickets[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) g[i] = up[i] = 0.f;
+        for (int q = 0; q < ksplit; ++q) {
+            const float* src = part + ((int64_t)tile * ksplit + q) * NP * 256 + lane * 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {                           // device-scope loads: the partials come from other CUs
+                g[i] += __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (DUAL) up[i] += __hip_atomic_load(src + 256 + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    }
     const int n = tile * 16 + c;
     if (n >= N) return;
     const float bv = bias ? bf16_to_f32(bias[n]) : 0.f;
@@ -103,14 +149,8 @@ __global__ __launch_bounds__(256) void skinny_gemm_kernel(const bf16_t* __restri
     for (int i = 0; i < 4; ++i) {
         const int m = 4 * kg + i;                // D: lane holds rows 4 kg .. 4 kg + 3 of column c
         if (m >= M) continue;
-        float g = 0.f, up = 0.f;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            g += red[w][0][lane][i];
-            if (DUAL) up += red[w][DUAL ? 1 : 0][lane][i];
-        }
         const float r = residual ? bf16_to_f32(residual[(int64_t)m * N + n]) : 0.f;
-        y[(int64_t)m * N + n] = f32_to_bf16(skinny_finish(g, up, DUAL, act, bv, residual != nullptr, r));
+        y[(int64_t)m * N + n] = f32_to_bf16(skinny_finish(g[i], up[i], DUAL, act, bv, residual != nullptr, r));
     }
 }
 
@@ -126,14 +166,32 @@ void skinny_pack_weights(hipStream_t s, const void* w, void* out, int64_t k, int
     const unsigned g = (unsigned)(cdiv_s(total, 256) > 65536 ? 65536 : cdiv_s(total, 256));
     skinny_pack_kernel<<<g, 256, 0, s>>>((const bf16_t*)w, (bf16_t*)out, k, n, kb, ntiles);
 }
+// Workgroups per tile: doubled while the launch has fewer than two workgroups per CU and each split keeps at least 16
+// steps of 32 k (measured on Ministral-3B shapes at 8 rows: 192 tiles x 4 takes 13.8 us where 192 x 1 took 18.7; at
+// 576 tiles a split no longer pays).
+int skinny_ksplit(int64_t k, int64_t n) {
+    const int64_t tiles = cdiv_s(n, 16);
+    if (tiles > (int64_t)kSkinnyTickets) return 1;
+    int ks = 1;
+    while (ks < 8 && tiles * ks < 512 && k / 32 / (ks * 2) >= 16) ks *= 2;
+    return ks;
+}
+size_t skinny_workspace_bytes(int64_t k, int64_t n, bool dual) {
+    const int ks = skinny_ksplit(k, n);
+    return ks > 1 ? (size_t)cdiv_s(n, 16) * ks * (dual ? 2 : 1) * 256 * sizeof(float) : 0;
+}
 void skinny_gemm(hipStream_t s, const SkinnyLinearArgs& a) {
-    const unsigned grid = (unsigned)cdiv_s(a.n, 16);
+    int ks = skinny_ksplit(a.k, a.n);
+    if (!a.part || !a.tickets || a.part_bytes < skinny_workspace_bytes(a.k, a.n, a.ws2 != nullptr)) ks = 1;
+    const dim3 grid((unsigned)cdiv_s(a.n, 16), (unsigned)ks);
     if (a.ws2)
         skinny_gemm_kernel<true><<<grid, 256, 0, s>>>((const bf16_t*)a.x, (const bf16_t*)a.ws, (const bf16_t*)a.ws2, (const bf16_t*)a.bias,
-                                                      (const bf16_t*)a.residual, (bf16_t*)a.y, (int)a.m, (int)a.k, (int)a.n, a.act);
+                                                      (const bf16_t*)a.residual, (bf16_t*)a.y, (int)a.m, (int)a.k, (int)a.n, a.act,
+                                                      (float*)a.part, a.tickets);
     else
         skinny_gemm_kernel<false><<<grid, 256, 0, s>>>((const bf16_t*)a.x, (const bf16_t*)a.ws, nullptr, (const bf16_t*)a.bias,
-                                                       (const bf16_t*)a.residual, (bf16_t*)a.y, (int)a.m, (int)a.k, (int)a.n, a.act);
+                                                       (const bf16_t*)a.residual, (bf16_t*)a.y, (int)a.m, (int)a.k, (int)a.n, a.act,
+                                                       (float*)a.part, a.tickets);
 }
 
 }  // namespace k

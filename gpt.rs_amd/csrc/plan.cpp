@@ -552,9 +552,11 @@ void Builder::describe(Step& st) {
                     if (in.act == 2) st.tiled_s2_input = pos(4);
                 }
             }
-            if (in.tiled && !in.quant && in.norm && x.dims[0] >= 2) {
-                // batched decode normalises into scratch first (the matrix-core kernel reads plain rows)
-                st.scratch_bytes = align_up((size_t)x.count() * dtype_size(x.dtype));
+            if (in.tiled && !in.quant && x.dims[0] >= 2) {
+                // batched decode normalises into scratch first (the matrix-core kernel reads plain rows); layers with
+                // few column tiles add the partial sums of their K splits
+                st.scratch_bytes = align_up(in.norm ? (size_t)x.count() * dtype_size(x.dtype) : 0) +
+                                   align_up(k::skinny_workspace_bytes(x.dims[1], w.dims[1], in.act == 2));
             }
             if (in.quant && !in.mfma) {
                 // stand-alone path of a quantised linear: (RMSNorm of x,) dequantised weights, then the generic kernel
@@ -1089,11 +1091,17 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
                 }
                 if (in.has_bias) sa.bias = src_ptr(st, cx, oi++);
                 if (in.has_residual) sa.residual = src_ptr(st, cx, oi++);
+                const size_t norm_bytes = in.norm ? align_up((size_t)x.count() * dtype_size(x.dtype)) : 0;
                 if (in.norm) {
                     void* xn = cx.ws + st.scratch_off;
                     k::rms_norm(s, (int)x.dtype, sa.x, src_ptr(st, cx, oi++), xn, sa.m, sa.k, in.scale, in.eps);
                     ++cx.launches;
                     sa.x = xn;
+                }
+                if (st.scratch_bytes > norm_bytes) {
+                    sa.part = cx.ws + st.scratch_off + norm_bytes;
+                    sa.part_bytes = st.scratch_bytes - norm_bytes;
+                    sa.tickets = cx.be->skinny_tickets();
                 }
                 sa.y = dst;
                 sa.act = in.act == 1 ? 1 : 0;

@@ -176,6 +176,8 @@ class Backend {
     // Device copy of a chain's phase table, cached by content (steady-state decode repeats a few tables).
     const k::ChainPhase* chain_table(const std::vector<k::ChainPhase>& phases);
     unsigned* chain_barrier() const { return d_chain_bar_; }
+    // kSkinnyTickets zeroed counters behind the chain's (split-K tickets of the batched-decode linear layers)
+    unsigned* skinny_tickets() const { return d_chain_bar_ + k::kChainBarrierBytes / sizeof(unsigned); }
     int* chain_abort_flag() const { return d_err_flag_ + 1; }
     bool opt_chain = true;
     int64_t n_chain_launches = 0, n_chain_phases = 0;

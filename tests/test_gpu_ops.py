@@ -293,7 +293,7 @@ def test_batched_decode_linear_on_matrix_cores(hip, m, k, n):
         assert_close(got, want, atol=3e-2, rtol=2e-2, what=f"m={m} k={k} n={n}")
 
 
-@pytest.mark.parametrize("m,k,n", [(8, 3072, 9216), (4, 256, 96)])
+@pytest.mark.parametrize("m,k,n", [(8, 3072, 9216), (4, 256, 96), (16, 3072, 9216), (12, 512, 256)])
 def test_batched_decode_norm_swiglu_on_matrix_cores(hip, m, k, n):
     from gptrs_amd.ptir import f32_to_bf16_bits
     r16 = lambda a: (f32_to_bf16_bits(np.asarray(a, np.float32)).astype(np.uint32) << 16).view(np.float32)  # noqa: E731
