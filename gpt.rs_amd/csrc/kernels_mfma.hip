@@ -82,7 +82,7 @@ template <int BM, int BN, bool DUAL>
 __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wk,
                                                              const bf16_t* __restrict__ wk2, const bf16_t* __restrict__ bias,
                                                              const bf16_t* __restrict__ residual, bf16_t* __restrict__ y,
-                                                             int M, int K, int N, int Npad, int act) {
+                                                             int M, int K, int N, int Npad, int act, int NT, int MT) {
     constexpr int SA = (BM + 1) * 16, SB = (BN + 1) * 16;     // bytes between k-groups
     constexpr int STAGE = kKb * (SA + SB);
     constexpr int TM = BM / 64, TN = BN / 64;
@@ -94,7 +94,22 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __res
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * NREAL;
+    // Tile order.  Consecutive workgroup ids go to the 8 XCDs in turn and each XCD has its own L2, so XCD c takes
+    // the contiguous range [c * per, (c + 1) * per) of a grouped order in which up to 8 row blocks of one column
+    // tile follow each other: the ~32 workgroups an XCD runs at a time then cover 8 row blocks x 4 column tiles, a
+    // weight tile is fetched from memory once for all its row blocks (with row-major ids the 1024 column tiles of an
+    // lm_head were each fetched once per row block) and an activation tile once per 4 column tiles.
+    int bx, by;
+    {
+        const int total = NT * MT, per = (total + 7) / 8;
+        const int v = (int)(blockIdx.x % 8) * per + (int)(blockIdx.x / 8);
+        if (blockIdx.x / 8 >= (unsigned)per || v >= total) return;
+        const int gsz = 8 * NT, g = v / gsz, first = g * 8;
+        const int gm = MT - first < 8 ? MT - first : 8;
+        by = first + (v % gsz) % gm;
+        bx = (v % gsz) / gm;
+    }
+    const int m0 = by * BM, n0 = bx * NREAL;
 
     // global -> LDS chunk assignment (16 bytes each)
     // A: chunk c -> kb = c % 8, row = c / 8: eight lanes read 128 contiguous bytes of one row
@@ -208,7 +223,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __res
 
 bool mfma_gemm_supported(int dtype, int64_t m, int64_t k, int64_t n) {
     return dtype == 2 && m > 16 && k >= kBK && k % kBK == 0 && n >= 1 && m < (1ll << 31) && n < (1ll << 31) - kBN &&
-           k < (1ll << 31);
+           k < (1ll << 31) && cdiv(m, 128) * cdiv(n, 64) < (1ll << 30);   // tile ids are ints
 }
 
 template <int BM, int BN, bool DUAL>
@@ -222,9 +237,11 @@ static void launch_mfma(hipStream_t s, const MfmaLinearArgs& a) {
     }
     const int64_t npad = mfma_padded_n(a.n);
     constexpr int nreal = DUAL ? BN / 2 : BN;
-    dim3 grid((unsigned)cdiv(npad, nreal), (unsigned)cdiv(a.m, BM));
+    const int64_t nt = cdiv(npad, nreal), mt = cdiv(a.m, BM);
+    const unsigned grid = (unsigned)(cdiv(nt * mt, 8) * 8);
     kern<<<grid, 256, lds_bytes, s>>>((const bf16_t*)a.x, (const bf16_t*)a.wk, (const bf16_t*)a.wk2, (const bf16_t*)a.bias,
-                                      (const bf16_t*)a.residual, (bf16_t*)a.y, (int)a.m, (int)a.k, (int)a.n, (int)npad, a.act);
+                                      (const bf16_t*)a.residual, (bf16_t*)a.y, (int)a.m, (int)a.k, (int)a.n, (int)npad, a.act,
+                                      (int)nt, (int)mt);
 }
 
 void mfma_gemm(hipStream_t s, const MfmaLinearArgs& a) {
