@@ -26,7 +26,8 @@ EXPORTS = [
     "gptrs_hip_to_literal", "gptrs_hip_tensor_retain", "gptrs_hip_tensor_release", "gptrs_hip_tensor_spec",
     "gptrs_hip_run_program", "gptrs_hip_run_program_donate", "gptrs_hip_execute_instruction",
     "gptrs_hip_param_get", "gptrs_hip_param_set", "gptrs_hip_supports_decode_sampling",
-    "gptrs_hip_sample_decode_token", "gptrs_hip_last_error", "gptrs_hip_synchronize", "gptrs_hip_set_option",
+    "gptrs_hip_sample_decode_token", "gptrs_hip_sample_decode_token_begin", "gptrs_hip_sample_decode_token_wait",
+    "gptrs_hip_decode_token_tensor", "gptrs_hip_last_error", "gptrs_hip_synchronize", "gptrs_hip_set_option",
     "gptrs_hip_counter",
 ]
 
@@ -77,6 +78,10 @@ def load_library(path: str = LIB_PATH):
     lib.gptrs_hip_supports_decode_sampling.argtypes = [vp, ctypes.c_float, ctypes.c_int, ctypes.c_int]
     lib.gptrs_hip_sample_decode_token.argtypes = [vp, vp, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_float,
                                                   ctypes.POINTER(ctypes.c_int64)]
+    lib.gptrs_hip_sample_decode_token_begin.argtypes = [vp, vp, ctypes.c_float, ctypes.c_int, ctypes.c_int, ctypes.c_float,
+                                                        ctypes.POINTER(ctypes.c_int64)]
+    lib.gptrs_hip_sample_decode_token_wait.argtypes = [vp, ctypes.c_int64, ctypes.POINTER(ctypes.c_int64)]
+    lib.gptrs_hip_decode_token_tensor.argtypes = [vp, pvp]
     lib.gptrs_hip_last_error.argtypes = []
     lib.gptrs_hip_last_error.restype = cp
     lib.gptrs_hip_synchronize.argtypes = [vp]
@@ -224,6 +229,25 @@ class HipBackend:
         self._check(self._lib.gptrs_hip_sample_decode_token(self._handle, logits.ptr, temperature, top_k is not None,
                                                             random_u is not None, random_u or 0.0, ctypes.byref(tok)))
         return None if tok.value < 0 else int(tok.value)
+
+    def sample_decode_token_begin(self, logits: TensorHandle, temperature: float = 0.0, top_k: Optional[int] = None,
+                                  random_u: Optional[float] = None) -> Optional[int]:
+        """Queues the sampling and returns a ticket at once (None: not served here); see sample_decode_token_wait."""
+        ticket = ctypes.c_int64(-1)
+        self._check(self._lib.gptrs_hip_sample_decode_token_begin(self._handle, logits.ptr, temperature, top_k is not None,
+                                                                  random_u is not None, random_u or 0.0, ctypes.byref(ticket)))
+        return None if ticket.value < 0 else int(ticket.value)
+
+    def sample_decode_token_wait(self, ticket: int) -> int:
+        tok = ctypes.c_int64(-1)
+        self._check(self._lib.gptrs_hip_sample_decode_token_wait(self._handle, ticket, ctypes.byref(tok)))
+        return int(tok.value)
+
+    def decode_token_tensor(self) -> TensorHandle:
+        """si32[1] handle over the device copy of the last sampled token."""
+        out = ctypes.c_void_p()
+        self._check(self._lib.gptrs_hip_decode_token_tensor(self._handle, ctypes.byref(out)))
+        return TensorHandle(self, out.value, self._spec_of(out.value))
 
     # -- extras ----------------------------------------------------------------------------
     def synchronize(self):

@@ -70,7 +70,9 @@ Backend::Backend(int dev) : device(dev) {
     GPTRS_HIP_CHECK(hipMalloc((void**)&d_counters_, k::kLinearCounters * sizeof(int)));
     GPTRS_HIP_CHECK(hipMalloc((void**)&d_argmax_val_, 1024 * sizeof(float)));
     GPTRS_HIP_CHECK(hipMalloc((void**)&d_argmax_idx_, 1024 * sizeof(int32_t)));
-    GPTRS_HIP_CHECK(hipMalloc((void**)&d_token_, 256));
+    token_buf_ = new_buffer(256);
+    d_token_ = (int64_t*)token_buf_->ptr;
+    GPTRS_HIP_CHECK(hipHostMalloc((void**)&h_token_ring_, kTokenRing * 2 * sizeof(int64_t), hipHostMallocDefault));
     GPTRS_HIP_CHECK(hipHostMalloc(&h_pinned_, 256, hipHostMallocDefault));
     GPTRS_HIP_CHECK(hipMalloc((void**)&d_chain_bar_, k::kChainBarrierBytes + k::kSkinnyTickets * sizeof(unsigned)));
     k::fill_zero(stream, d_chain_bar_, k::kChainBarrierBytes + k::kSkinnyTickets * sizeof(unsigned));
@@ -101,7 +103,10 @@ Backend::~Backend() {
     (void)hipFree(d_counters_);
     (void)hipFree(d_argmax_val_);
     (void)hipFree(d_argmax_idx_);
-    (void)hipFree(d_token_);
+    token_buf_.reset();
+    for (hipEvent_t e : token_events_)
+        if (e) (void)hipEventDestroy(e);
+    if (h_token_ring_) (void)hipHostFree(h_token_ring_);
     if (h_pinned_) (void)hipHostFree(h_pinned_);
     if (stream) (void)hipStreamDestroy(stream);
 }
@@ -279,27 +284,64 @@ void Backend::param_set(const std::array<uint8_t, 16>& id, gptrs_hip_tensor* t) 
     }
 }
 
-int64_t Backend::sample(const gptrs_hip_tensor* logits, float temperature, bool has_top_k, bool has_u, float u) {
+bool Backend::queue_sampling(const gptrs_hip_tensor* logits, float temperature, bool has_top_k, bool has_u, float u) {
     GPTRS_HIP_CHECK(hipSetDevice(device));
     if (logits->consumed) fail_exec("tensor handle was donated to run_program and can no longer be read");
     const Spec& s = logits->spec;
     if (!dtype_is_float(s.dtype) || s.rank() < 1 || s.rank() > 2 || s.count() == 0)
         fail_exec("sample_decode_token expects non-empty f32/bf16 logits of rank 1 or 2");
     const int64_t vocab = s.dims.back(), rows = s.rank() == 2 ? s.dims[0] : 1;
-    if (has_top_k) return -1;  // Ok(None): host sampler handles top-k
+    if (has_top_k) return false;  // Ok(None): host sampler handles top-k
     if (temperature <= 0.0f) {
         k::argmax_last_row(stream, (int)s.dtype, logits->data(), rows, vocab, d_token_, d_argmax_val_, d_argmax_idx_, 1024);
         n_launches += 2;
     } else {
-        if (!has_u) return -1;
+        if (!has_u) return false;
         k::sample_temperature_last_row(stream, (int)s.dtype, logits->data(), rows, vocab, temperature, u, d_token_);
         n_launches += 1;
     }
+    return true;
+}
+
+int64_t Backend::sample(const gptrs_hip_tensor* logits, float temperature, bool has_top_k, bool has_u, float u) {
+    if (!queue_sampling(logits, temperature, has_top_k, has_u, u)) return -1;
     int64_t* host = (int64_t*)h_pinned_;
     GPTRS_HIP_CHECK(hipMemcpyAsync(host, d_token_, sizeof(int64_t), hipMemcpyDeviceToHost, stream));
     GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
     check_device_errors();
     return *host;
+}
+
+int64_t Backend::sample_begin(const gptrs_hip_tensor* logits, float temperature, bool has_top_k, bool has_u, float u) {
+    if (!queue_sampling(logits, temperature, has_top_k, has_u, u)) return -1;
+    const int64_t ticket = next_ticket_++;
+    const int slot = (int)(ticket % kTokenRing);
+    if (!token_events_[slot]) GPTRS_HIP_CHECK(hipEventCreateWithFlags(&token_events_[slot], hipEventDisableTiming));
+    GPTRS_HIP_CHECK(hipMemcpyAsync(h_token_ring_ + 2 * slot, d_token_, sizeof(int64_t), hipMemcpyDeviceToHost, stream));
+    GPTRS_HIP_CHECK(hipMemcpyAsync(h_token_ring_ + 2 * slot + 1, d_err_flag_, 2 * sizeof(int), hipMemcpyDeviceToHost, stream));
+    GPTRS_HIP_CHECK(hipEventRecord(token_events_[slot], stream));
+    return ticket;
+}
+
+int64_t Backend::sample_wait(int64_t ticket) {
+    if (ticket < 0 || ticket >= next_ticket_ || ticket + kTokenRing <= next_ticket_)
+        fail_exec("sample_decode_token_wait: unknown or expired ticket");
+    GPTRS_HIP_CHECK(hipSetDevice(device));
+    const int slot = (int)(ticket % kTokenRing);
+    GPTRS_HIP_CHECK(hipEventSynchronize(token_events_[slot]));
+    if (h_token_ring_[2 * slot + 1] != 0) {   // a device-side error flag was up when the token was sampled
+        GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
+        check_device_errors();
+    }
+    return h_token_ring_[2 * slot];
+}
+
+gptrs_hip_tensor* Backend::token_tensor() {
+    auto* t = new gptrs_hip_tensor();
+    t->spec.dtype = DType::SI32;
+    t->spec.dims = {1};
+    t->buf = token_buf_;
+    return t;
 }
 
 std::shared_ptr<Plan> Backend::get_plan(const char* json, size_t len, uint64_t key, const uint8_t* donate, size_t n_in) {
@@ -732,6 +774,31 @@ int gptrs_hip_sample_decode_token(gptrs_hip_backend* b, const gptrs_hip_tensor* 
         if (!b || !logits || !token_out) gptrs::fail_exec("null argument");
         std::lock_guard<std::mutex> g(b->impl.mu);
         *token_out = b->impl.sample(logits, temperature, has_top_k != 0, has_random_u != 0, random_u);
+    });
+}
+
+int gptrs_hip_sample_decode_token_begin(gptrs_hip_backend* b, const gptrs_hip_tensor* logits, float temperature, int has_top_k,
+                                        int has_random_u, float random_u, int64_t* ticket_out) {
+    return guarded([&] {
+        if (!b || !logits || !ticket_out) gptrs::fail_exec("null argument");
+        std::lock_guard<std::mutex> g(b->impl.mu);
+        *ticket_out = b->impl.sample_begin(logits, temperature, has_top_k != 0, has_random_u != 0, random_u);
+    });
+}
+
+int gptrs_hip_sample_decode_token_wait(gptrs_hip_backend* b, int64_t ticket, int64_t* token_out) {
+    return guarded([&] {
+        if (!b || !token_out) gptrs::fail_exec("null argument");
+        std::lock_guard<std::mutex> g(b->impl.mu);
+        *token_out = b->impl.sample_wait(ticket);
+    });
+}
+
+int gptrs_hip_decode_token_tensor(gptrs_hip_backend* b, gptrs_hip_tensor** out) {
+    return guarded([&] {
+        if (!b || !out) gptrs::fail_exec("null argument");
+        std::lock_guard<std::mutex> g(b->impl.mu);
+        *out = b->impl.token_tensor();
     });
 }
 

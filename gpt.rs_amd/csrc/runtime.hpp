@@ -159,6 +159,13 @@ class Backend {
     gptrs_hip_tensor* param_get(const std::array<uint8_t, 16>& id);
     void param_set(const std::array<uint8_t, 16>& id, gptrs_hip_tensor* t);
     int64_t sample(const gptrs_hip_tensor* logits, float temperature, bool has_top_k, bool has_u, float u);
+    // sample() in two halves for a pipelined decode loop: begin queues the sampling kernels and the copies of the token
+    // and of the device error flags into a pinned ring and returns a ticket (-1: request not served here), wait blocks
+    // on that ticket's event only.  The token also stays in token_tensor() (si32[1] over the sampling output).
+    static constexpr int kTokenRing = 32;
+    int64_t sample_begin(const gptrs_hip_tensor* logits, float temperature, bool has_top_k, bool has_u, float u);
+    int64_t sample_wait(int64_t ticket);
+    gptrs_hip_tensor* token_tensor();
     void synchronize();
     void check_device_errors();
 
@@ -217,7 +224,12 @@ class Backend {
     int* d_counters_ = nullptr;
     float* d_argmax_val_ = nullptr;
     int32_t* d_argmax_idx_ = nullptr;
-    int64_t* d_token_ = nullptr;
+    int64_t* d_token_ = nullptr;       // = token_buf_->ptr: the sampled token as int64, little endian
+    BufferP token_buf_;
+    int64_t* h_token_ring_ = nullptr;  // pinned: kTokenRing x {token, error flags}
+    hipEvent_t token_events_[kTokenRing] = {};
+    int64_t next_ticket_ = 0;
+    bool queue_sampling(const gptrs_hip_tensor* logits, float temperature, bool has_top_k, bool has_u, float u);
     void* h_pinned_ = nullptr;  // 64 bytes of pinned host memory for readbacks
     struct Derived { std::weak_ptr<Buffer> src, src2; BufferP tiled; };
     std::map<std::array<uint64_t, 3>, Derived> tiled_cache_;

@@ -370,8 +370,16 @@ class Gpt(_ModelBase):
         """model/gpt.rs:585-751.  Returns the logits handle [T, V]; `caches` is updated in place."""
         return self.forward_batch([list(tokens)], position_offset, [caches], fixed_capacity)
 
+    def forward_decode_device_token(self, token_handle, position_offset: int, caches: List[Optional[DecodeKvCache]],
+                                    fixed_capacity: Optional[int] = None):
+        """One decode step whose token id is already on the device (a si32[1] handle, e.g.
+        backend.decode_token_tensor()): the same program as forward_with_decode_cache([token], ...), without the
+        host having to know the token yet.  An id outside the vocabulary raises at the next synchronising call."""
+        return self.forward_batch([[None]], position_offset, [caches], fixed_capacity, token_handle=token_handle)
+
     def forward_batch(self, token_rows: List[List[int]], position_offset: int,
-                      caches: List[List[Optional[DecodeKvCache]]], fixed_capacity: Optional[int] = None):
+                      caches: List[List[Optional[DecodeKvCache]]], fixed_capacity: Optional[int] = None,
+                      token_handle=None):
         """Independent sequences sharing the weights: row-stacked hidden states, one M=B*T
         GEMM per linear, per-sequence attention.  The reference has no batch dimension
         (ops/functional/attention.rs:189-203); with one row this is exactly its path."""
@@ -384,10 +392,13 @@ class Gpt(_ModelBase):
         total = position_offset + seq
         if total > cfg.context_length:
             raise ValueError(f"token sequence length {total} exceeds model context length {cfg.context_length}")
-        for row in token_rows:
-            for t in row:
-                if not 0 <= t < cfg.vocab_size:
-                    raise ValueError(f"token index {t} out of range")
+        if token_handle is None:
+            for row in token_rows:
+                for t in row:
+                    if not 0 <= t < cfg.vocab_size:
+                        raise ValueError(f"token index {t} out of range")
+        elif batch != 1 or seq != 1:
+            raise ValueError("a device token feeds one sequence, one step")
         if any(len(c) != cfg.num_layers for c in caches):
             raise ValueError(f"expected {cfg.num_layers} cache slots (one per layer)")
         if fixed_capacity is not None:
@@ -403,9 +414,9 @@ class Gpt(_ModelBase):
             raise ValueError("decode with an existing cache supports one token per sequence")
         L = cfg.num_layers
         prog, _ = self._build(seq, capacity, have, batch)
-        toks = [t for row in token_rows for t in row]
         poss = [position_offset + j for _ in range(batch) for j in range(seq)]
-        args = [self._upload_i32(toks), self._upload_i32(poss)]
+        tok_arg = token_handle if token_handle is not None else self._upload_i32([t for row in token_rows for t in row])
+        args = [tok_arg, self._upload_i32(poss)]
         if have:
             for c in caches:
                 for slot in c:
@@ -688,9 +699,15 @@ class Ministral(_ModelBase):
         """model/ministral.rs:613-766."""
         return self.forward_batch([list(tokens)], position_offset, [caches], fixed_capacity)
 
-    def forward_batch(self, token_rows, position_offset, caches, fixed_capacity=None):
+    def forward_decode_device_token(self, token_handle, position_offset, caches, fixed_capacity=None):
+        """See Gpt.forward_decode_device_token."""
+        return self.forward_batch([[None]], position_offset, [caches], fixed_capacity, token_handle=token_handle)
+
+    def forward_batch(self, token_rows, position_offset, caches, fixed_capacity=None, token_handle=None):
         cfg = self.config
         batch, seq = len(token_rows), len(token_rows[0])
+        if token_handle is not None and (batch != 1 or seq != 1):
+            raise ValueError("a device token feeds one sequence, one step")
         if seq == 0:
             raise ValueError("token sequence must contain at least one element")
         if any(len(r) != seq for r in token_rows):
@@ -713,8 +730,8 @@ class Ministral(_ModelBase):
         prog, _ = self._build(seq, capacity, have, batch)
         cos, sin = F.rotary_cos_sin_cache_slice(position_offset, seq, self.rope)   # ministral.rs:253-261
         half = cfg.rotary_dim // 2
-        toks = [t for row in token_rows for t in row]
-        args = [self._upload_i32(toks),
+        tok_arg = token_handle if token_handle is not None else self._upload_i32([t for row in token_rows for t in row])
+        args = [tok_arg,
                 self.backend.materialize(TensorSpec(self.dtype, [seq, half]), _np_to_bytes(cos, self.dtype)),
                 self.backend.materialize(TensorSpec(self.dtype, [seq, half]), _np_to_bytes(sin, self.dtype))]
         if have:
@@ -741,10 +758,16 @@ class Generator:
     With `device_sampling` the token comes from backend.sample_decode_token (spec.rs:1333-1348)
     and only 8 bytes cross PCIe per step; otherwise the last logits row is read back and
     arg-maxed on the host (sampler.rs:96-103).
+
+    `pipelined` (default: on when the backend offers sample_decode_token_begin / _wait and sampling is on the
+    device): a step queues the sampling of token t, then the forward of step t + 1 fed by the device copy of that
+    token, and only then waits for token t, so the device never idles for the host round trip.  Same tokens as
+    the unpipelined loop; an error of step t + 1's launch surfaces one step later.
     """
 
     def __init__(self, model, prompt: Sequence[int], kv_cache_capacity: Optional[int] = None,
-                 device_sampling: bool = True, temperature: float = 0.0, seed: int = 0):
+                 device_sampling: bool = True, temperature: float = 0.0, seed: int = 0,
+                 pipelined: Optional[bool] = None):
         if len(prompt) == 0:
             raise ValueError("prompt must be non-empty")
         self.model = model
@@ -755,6 +778,11 @@ class Generator:
         # step (DecodeSampleRequest.random_u, spec.rs:1270-1284; sampler.rs:83-93 draws it in (eps, 1 - eps))
         self.temperature = float(temperature)
         self._rng = np.random.default_rng(seed)
+        can_pipeline = device_sampling and hasattr(model.backend, "sample_decode_token_begin") and \
+            hasattr(model, "forward_decode_device_token")
+        if pipelined and not can_pipeline:
+            raise ValueError("pipelined generation needs device sampling and a backend with sample_decode_token_begin")
+        self.pipelined = can_pipeline if pipelined is None else bool(pipelined)
         self.caches: List[Optional[DecodeKvCache]] = [None] * model.num_layers
         self.window_start = max(0, len(self.tokens) - model.context_length)
         context = self.tokens[self.window_start:]
@@ -764,9 +792,7 @@ class Generator:
     def _sample(self) -> int:
         be = self.model.backend
         if self.temperature > 0.0:
-            eps = float(np.finfo(np.float32).eps)
-            u = float(np.float32(self._rng.uniform(eps, 1.0 - eps)))
-            tok = be.sample_decode_token(self.logits, temperature=self.temperature, random_u=u)
+            tok = be.sample_decode_token(self.logits, temperature=self.temperature, random_u=self._draw_u())
             if tok is None:
                 raise RuntimeError("backend declined temperature sampling")
             return tok
@@ -777,7 +803,35 @@ class Generator:
         row = be.to_numpy(self.logits)[-1]
         return int(np.argmax(row))
 
+    def _draw_u(self) -> float:
+        eps = float(np.finfo(np.float32).eps)
+        return float(np.float32(self._rng.uniform(eps, 1.0 - eps)))
+
+    def _step_pipelined(self) -> Optional[int]:
+        """Queue sampling + next forward, then wait for the token.  None: the backend declined (nothing queued)."""
+        be = self.model.backend
+        if self.temperature > 0.0:
+            state = self._rng.bit_generator.state
+            ticket = be.sample_decode_token_begin(self.logits, temperature=self.temperature, random_u=self._draw_u())
+            if ticket is None:
+                self._rng.bit_generator.state = state   # the unpipelined path draws again
+                return None
+        else:
+            ticket = be.sample_decode_token_begin(self.logits, temperature=0.0)
+            if ticket is None:
+                return None
+        self.logits = self.model.forward_decode_device_token(be.decode_token_tensor(), self.processed_len, self.caches,
+                                                             self.capacity)
+        self.processed_len += 1
+        nxt = be.sample_decode_token_wait(ticket)
+        self.tokens.append(nxt)
+        return nxt
+
     def step(self) -> int:
+        if self.pipelined and self.processed_len < self.model.context_length:
+            nxt = self._step_pipelined()
+            if nxt is not None:
+                return nxt
         nxt = self._sample()
         self.tokens.append(nxt)
         if self.processed_len >= self.model.context_length:

@@ -122,6 +122,21 @@ int gptrs_hip_supports_decode_sampling(const gptrs_hip_backend* b, float tempera
 int gptrs_hip_sample_decode_token(gptrs_hip_backend* b, const gptrs_hip_tensor* logits, float temperature,
                                   int has_top_k, int has_random_u, float random_u, int64_t* token_out);
 
+/* sample_decode_token in two halves, for a decode loop that queues step t+1 before it has seen token t.  No
+ * counterpart in the reference: its loop (crates/gpt-rs/src/inference/generate.rs:96-140) waits for each token
+ * before it builds the next step, which leaves the device idle for a host round trip per token.
+ * _begin queues the sampling of the last logits row (same rules and same kernels as sample_decode_token) and a copy
+ * of the token into pinned host memory, and returns at once with *ticket_out >= 0, or -1 for Ok(None).
+ * The sampled token also stays on the device: gptrs_hip_decode_token_tensor returns a new handle (si32[1]) over the
+ * sampling output, valid as the token-id input of the next step's program; it is overwritten by the next _begin or
+ * sample_decode_token, in stream order, so a program queued before that still reads its own token.
+ * _wait blocks until the token of `ticket` has arrived (not until the queue is empty) and reports device errors
+ * raised up to that point.  At most 32 tickets can be outstanding; older ones expire. */
+int gptrs_hip_sample_decode_token_begin(gptrs_hip_backend* b, const gptrs_hip_tensor* logits, float temperature,
+                                        int has_top_k, int has_random_u, float random_u, int64_t* ticket_out);
+int gptrs_hip_sample_decode_token_wait(gptrs_hip_backend* b, int64_t ticket, int64_t* token_out);
+int gptrs_hip_decode_token_tensor(gptrs_hip_backend* b, gptrs_hip_tensor** out);
+
 /* Message of the calling thread's most recent non-zero return (BackendError Display). */
 const char* gptrs_hip_last_error(void);
 

@@ -60,6 +60,52 @@ def test_tiny_gpt_temperature_sampling_matches_oracle(hip):
     assert len(set(t_hip)) > 3   # a sampled sequence, not one token repeated
 
 
+@pytest.mark.parametrize("temperature", [0.0, 0.8])
+def test_pipelined_generation_equals_unpipelined(hip, temperature):
+    """sample_decode_token_begin / _wait + the device token tensor: step t + 1 is queued before token t reaches the
+    host.  Same tokens and bit-identical logits as the loop that waits for every token, through cache-bucket growth
+    (no fixed capacity) and into the sliding window (context 32)."""
+    for cls, cfg in ((models.Gpt, TINY_GPT), (models.Ministral, TINY_MINISTRAL)):
+        m = cls.random(cfg, hip, seed=31, std=0.3)
+        runs = []
+        for pipelined in (False, True):
+            gen = models.Generator(m, PROMPT, temperature=temperature, seed=5, pipelined=pipelined)
+            assert gen.pipelined == pipelined
+            toks, rows = [], []
+            for _ in range(34):
+                toks.append(gen.step())
+                rows.append(hip.to_numpy(gen.logits)[-1].tobytes())
+            runs.append((toks, rows))
+        assert runs[0][0] == runs[1][0]
+        assert runs[0][1] == runs[1][1]
+    assert models.Generator(m, PROMPT).pipelined                      # the default on this backend
+    with pytest.raises(ValueError):
+        models.Generator(m, PROMPT, device_sampling=False, pipelined=True)
+
+
+def test_sampling_tickets(hip):
+    from parity import TensorSpec
+    from gptrs_amd.backend import BackendError
+    a = hip.materialize(TensorSpec("F32", [2, 5]), np.array([[9, 0, 0, 0, 0], [0, 1, 7, 3, 2]], np.float32).tobytes())
+    b = hip.materialize(TensorSpec("F32", [4]), np.array([0, 0, 0, 5], np.float32).tobytes())
+    t0 = hip.sample_decode_token_begin(a)
+    tok_dev = hip.decode_token_tensor()
+    assert tok_dev.spec.dtype == "Si32" and list(tok_dev.spec.dims) == [1]
+    assert hip.to_numpy(tok_dev).tolist() == [2]
+    t1 = hip.sample_decode_token_begin(b)
+    assert hip.sample_decode_token_wait(t1) == 3 and hip.sample_decode_token_wait(t0) == 2   # any order
+    assert hip.to_numpy(tok_dev).tolist() == [3]                       # the tensor follows the latest sample
+    assert hip.sample_decode_token_begin(a, temperature=0.7) is None   # no draw supplied: Ok(None), nothing queued
+    assert hip.sample_decode_token_begin(a, top_k=3) is None
+    with pytest.raises(BackendError):
+        hip.sample_decode_token_wait(t1 + 1000)
+    for _ in range(40):
+        last = hip.sample_decode_token_begin(a)
+    assert hip.sample_decode_token_wait(last) == 2
+    with pytest.raises(BackendError):                                  # 32 outstanding at most: t0 has expired
+        hip.sample_decode_token_wait(t0)
+
+
 def test_model_from_checkpoint_on_device(hip, tmp_path):
     """A GPTRSCHK v2 file written from one backend feeds the other (checkpoint/loader.rs, runtime/loader.rs:19-241):
     same greedy tokens, logits within the f32 bar; bf16 storage and on-load quantisation go through as well."""
