@@ -113,6 +113,66 @@ def cpu_baseline(cfg, seconds_budget: float = 25.0):
                       f"8 head slices; non-GEMV ops excluded"}
 
 
+def batched_decode(args, be, cfg, model, capacity):
+    """B independent sequences decoded together (models.forward_batch): tokens/s summed over the sequences.  The next
+    tokens are the row-wise argmax taken on the host (B x vocab bf16 logits cross PCIe each step, inside the timed
+    region), the linear layers are bracketed by HIP events in a second pass as in the batch-1 run."""
+    B = args.batch
+    rng = np.random.default_rng(6)
+    rows = [rng.integers(0, cfg.vocab_size, args.prompt).tolist() for _ in range(B)]
+    caches = [[None] * cfg.num_layers for _ in range(B)]
+    t0 = time.perf_counter()
+    state = {"logits": model.forward_batch(rows, 0, caches, capacity), "pos": args.prompt}
+    be.synchronize()
+    t_prefill = time.perf_counter() - t0
+
+    def step():
+        lg = be.to_numpy(state["logits"]).reshape(B, -1, cfg.vocab_size)[:, -1]
+        toks = [[int(np.argmax(lg[b]))] for b in range(B)]
+        state["logits"] = model.forward_batch(toks, state["pos"], caches, capacity)
+        state["pos"] += 1
+
+    for _ in range(args.warmup):
+        step()
+    be.synchronize()
+    start_len = state["pos"]
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    be.synchronize()
+    elapsed = time.perf_counter() - t0
+    launches = be.counter("last_program_launches")
+    prof_steps = min(8, capacity - state["pos"] - 1)
+    roof = None
+    if prof_steps > 0:
+        be.set_option("profile", 1)
+        for _ in range(prof_steps):
+            step()
+        t_ns, calls, nbytes = be.counter("linear_time_ns"), be.counter("linear_calls"), be.counter("linear_bytes")
+        be.set_option("profile", 0)
+        if t_ns > 0:
+            achieved = nbytes / (t_ns * 1e-9) / 1e9
+            roof = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                    "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                    "kernel": "skinny_gemm_kernel: all linear layers of a batched decode step (weights once, %d activation rows)" % B,
+                    "launches": calls, "avg_launch_us": round(t_ns / max(calls, 1) / 1e3, 2),
+                    "bytes_per_launch": round(nbytes / max(calls, 1))}
+    mid_len = start_len + args.steps // 2
+    kv_bytes = 2 * cfg.num_layers * cfg.num_kv_heads * cfg.head_dim * 2 * (mid_len + 1)
+    step_bytes = algorithmic_bytes_per_step(cfg, 2, mid_len, args.quant) + (B - 1) * kv_bytes   # weights once, every sequence's KV
+    print(json.dumps({
+        "metric": "decode tokens/s summed over %d sequences, Ministral-3B-shape bf16 (side workload: batched decode)" % B,
+        "value": round(B * args.steps / elapsed, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(elapsed / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "ministral-3b-shape bf16 decode, batch %d, prompt %d each, greedy (host argmax), KV capacity %d" % (B, args.prompt, capacity),
+                   "layers": cfg.num_layers, "cache_len_mid": mid_len},
+        "hbm_gbps": round(step_bytes / (elapsed / args.steps) / 1e9, 1),
+        "hbm_frac": round(step_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS, 4),
+        "algorithmic_bytes_per_step": step_bytes, "launches_per_step": launches,
+        "prefill_ms": round(t_prefill * 1e3, 2), "prefill_tokens": B * args.prompt, "roofline": roof, "cpu_baseline": None}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -123,6 +183,9 @@ def main():
     ap.add_argument("--quant", choices=["none", "w8", "w4g128"], default="none",
                     help="weight-only quantisation of every linear weight (BASELINE configs[4]: w8 = int8 per output channel, "
                          "w4g128 = int4 in groups of 128); activations, KV cache and embeddings stay bf16")
+    ap.add_argument("--batch", type=int, default=1,
+                    help="B > 1: batched decode of B independent sequences (rows stacked through the linear layers, one attention "
+                         "launch per layer for all of them); a side workload, NOT the headline metric (which is batch 1)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain elementwise kernel of known traffic (x + 0 over 2^28 f32: 1 GiB read, 1 GiB written, "
@@ -159,6 +222,8 @@ def main():
     model = models.Ministral.random(cfg, be, seed=5, dtype="Bf16", quant=None if args.quant == "none" else args.quant)
     t_init = time.perf_counter() - t0
     prompt = np.random.default_rng(6).integers(0, cfg.vocab_size, args.prompt).tolist()
+    if args.batch > 1:
+        return batched_decode(args, be, cfg, model, capacity)
 
     # prefill (reported separately, crates/gpt-rs-cli/src/main.rs:900-935): first call compiles the plan
     gen = models.Generator(model, prompt, kv_cache_capacity=capacity)
