@@ -157,15 +157,16 @@ def batched_decode(args, be, cfg, model, capacity):
                     "kernel": "skinny_gemm_kernel: all linear layers of a batched decode step (weights once, %d activation rows)" % B,
                     "launches": calls, "avg_launch_us": round(t_ns / max(calls, 1) / 1e3, 2),
                     "bytes_per_launch": round(nbytes / max(calls, 1))}
+    wname = {"none": "bf16", "w8": "int8-weight-only (per output channel) bf16", "w4g128": "int4-weight-only (groups of 128) bf16"}[args.quant]
     mid_len = start_len + args.steps // 2
     kv_bytes = 2 * cfg.num_layers * cfg.num_kv_heads * cfg.head_dim * 2 * (mid_len + 1)
     step_bytes = algorithmic_bytes_per_step(cfg, 2, mid_len, args.quant) + (B - 1) * kv_bytes   # weights once, every sequence's KV
     print(json.dumps({
-        "metric": "decode tokens/s summed over %d sequences, Ministral-3B-shape bf16 (side workload: batched decode)" % B,
+        "metric": "decode tokens/s summed over %d sequences, Ministral-3B-shape %s (side workload: batched decode)" % (B, wname),
         "value": round(B * args.steps / elapsed, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(elapsed / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "ministral-3b-shape bf16 decode, batch %d, prompt %d each, greedy (host argmax), KV capacity %d" % (B, args.prompt, capacity),
+        "config": {"workload": "ministral-3b-shape %s decode, batch %d, prompt %d each, greedy (host argmax), KV capacity %d" % (wname, B, args.prompt, capacity),
                    "layers": cfg.num_layers, "cache_len_mid": mid_len},
         "hbm_gbps": round(step_bytes / (elapsed / args.steps) / 1e9, 1),
         "hbm_frac": round(step_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS, 4),

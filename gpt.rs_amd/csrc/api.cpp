@@ -166,6 +166,9 @@ BufferP Backend::derived_weights(const BufferP& src, int kind, DType dtype, int6
     } else if (kind == 8) {                             // batched decode: 16-column tiles, k-grouped (kernels_skinny.hip)
         t = new_buffer(k::skinny_weight_bytes(k, n));
         k::skinny_pack_weights(stream, src->ptr, t->ptr, k, n);
+    } else if (kind == 9 || kind == 10) {               // batched decode: int8 / int4 codes in the 16-column tiled word order
+        t = new_buffer(k::skinny_codes_bytes(k, n, kind - 8));
+        k::skinny_pack_codes(stream, src->ptr, t->ptr, k, n, kind - 8);
     } else {                                            // 6 / 7: MFMA copy of dequantised int8 / int4 (src2: scales)
         if (!src2) fail_exec("quantised weight copy needs its scales");
         BufferP full = new_buffer((size_t)k * n * dtype_size(dtype));

@@ -801,8 +801,9 @@ struct Fuser {
                 in.mfma = true;
                 continue;
             }
-            if (in.quant) {   // decode: only the persistent chain reads the codes directly
-                in.tiled = k::chain_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1], in.act == 2, false, in.quant);
+            if (in.quant) {   // decode: the persistent chain (one row) and the batched matrix-core kernel read the codes directly
+                in.tiled = k::chain_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1], in.act == 2, false, in.quant) ||
+                           k::skinny_quant_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1], in.quant);
                 continue;
             }
             if (!k::gemv_tiled_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1])) continue;

@@ -119,7 +119,13 @@ struct SkinnyLinearArgs {
     // split-K over workgroups (layers with few tiles): part = skinny_workspace_bytes() of scratch, tickets =
     // kSkinnyTickets counters zeroed once (every launch leaves them zero); without them the layer runs unsplit
     void* part; size_t part_bytes; unsigned* tickets;
+    // weight-only quantised: quant 1 = int8 (scale [N]), 2 = int4 groups of 128 (scale [K/128, N]); ws / ws2 are then
+    // the code copies of skinny_pack_codes, scale / scale2 the scale tensors as the program holds them (bf16)
+    int quant; const void* scale; const void* scale2;
 };
+bool skinny_quant_supported(int dtype, int64_t m, int64_t k, int64_t n, int qf);
+size_t skinny_codes_bytes(int64_t k, int64_t n, int qf);
+void skinny_pack_codes(hipStream_t s, const void* codes, void* out, int64_t k, int64_t n, int qf);
 constexpr size_t kSkinnyTickets = 1024;
 int skinny_ksplit(int64_t k, int64_t n);
 size_t skinny_workspace_bytes(int64_t k, int64_t n, bool dual);

@@ -552,13 +552,13 @@ void Builder::describe(Step& st) {
                     if (in.act == 2) st.tiled_s2_input = pos(4);
                 }
             }
-            if (in.tiled && !in.quant && x.dims[0] >= 2) {
+            if (in.tiled && x.dims[0] >= 2) {
                 // batched decode normalises into scratch first (the matrix-core kernel reads plain rows); layers with
                 // few column tiles add the partial sums of their K splits
                 st.scratch_bytes = align_up(in.norm ? (size_t)x.count() * dtype_size(x.dtype) : 0) +
                                    align_up(k::skinny_workspace_bytes(x.dims[1], w.dims[1], in.act == 2));
             }
-            if (in.quant && !in.mfma) {
+            if (in.quant && !in.mfma && !(in.tiled && x.dims[0] >= 2)) {
                 // stand-alone path of a quantised linear: (RMSNorm of x,) dequantised weights, then the generic kernel
                 const size_t es = dtype_size(x.dtype);
                 st.scratch_bytes = align_up(in.norm ? (size_t)x.count() * es : 0) +
@@ -1075,19 +1075,24 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
                 ++cx.launches;
                 break;
             }
-            if (in.tiled && !in.quant && k::skinny_gemm_supported((int)x.dtype, x.dims[0], x.dims[1], w.dims[1]) &&
+            if (in.tiled &&
+                (in.quant ? k::skinny_quant_supported((int)x.dtype, x.dims[0], x.dims[1], w.dims[1], in.quant)
+                          : k::skinny_gemm_supported((int)x.dtype, x.dims[0], x.dims[1], w.dims[1])) &&
                 (!in.norm || st.scratch_bytes >= (size_t)x.count() * dtype_size(x.dtype))) {
                 k::SkinnyLinearArgs sa{};
                 sa.x = src_ptr(st, cx, 0);
                 sa.m = x.dims[0]; sa.k = x.dims[1]; sa.n = w.dims[1];
-                BufferP wsk = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], 8, x.dtype, sa.k, sa.n);
+                const int kind = in.quant == 0 ? 8 : (in.quant == 1 ? 9 : 10);   // bf16 copy, or the codes in the same tile order
+                BufferP wsk = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], kind, x.dtype, sa.k, sa.n);
                 BufferP wsk2;
                 sa.ws = wsk->ptr;
-                size_t oi = 2;
+                sa.quant = in.quant;
+                if (in.quant) sa.scale = src_ptr(st, cx, 2);
+                size_t oi = linear_extra_pos(in);
                 if (in.act == 2) {
-                    wsk2 = cx.be->derived_weights(cx.input_bufs[st.tiled_w2_input], 8, x.dtype, sa.k, sa.n);
+                    wsk2 = cx.be->derived_weights(cx.input_bufs[st.tiled_w2_input], kind, x.dtype, sa.k, sa.n);
                     sa.ws2 = wsk2->ptr;
-                    ++oi;
+                    if (in.quant) sa.scale2 = src_ptr(st, cx, 4);
                 }
                 if (in.has_bias) sa.bias = src_ptr(st, cx, oi++);
                 if (in.has_residual) sa.residual = src_ptr(st, cx, oi++);

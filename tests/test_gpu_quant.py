@@ -155,7 +155,23 @@ def test_prefill_linear_bf16(hip, scheme, m, k, n):
 
 
 @pytest.mark.parametrize("scheme", ["w8", "w4g128"])
-@pytest.mark.parametrize("m", [1, 64])
+@pytest.mark.parametrize("m,k,n", [(8, 3072, 6144), (8, 4096, 3072), (2, 9216, 3072), (16, 3072, 1000), (5, 512, 40), (8, 3072, 32768)])
+def test_batched_decode_linear_bf16(hip, scheme, m, k, n):
+    """2..16 bf16 rows: the matrix-core kernel streams the codes (biased codes are exact in bf16; the bias leaves through
+    a second product against a column of ones), K split over workgroups where the layer has few column tiles."""
+    x, w = bf16_round(rnd(21, (m, k))), rnd(22, (k, n), 2.0 / np.sqrt(k))
+    q, s = quantize(w, scheme)
+    specs = [("Bf16", [m, k]), code_spec(scheme, k, n), ("Bf16", scale_dims(scheme, k, n))]
+    built = hip.counter("derived_weights_built")
+    run_linear(hip, lambda fb, a, b, c: F.linear_quantized(a, b, c), specs, [x, q, s], 3e-2, 2e-2, expect_chain=False)
+    assert hip.counter("derived_weights_built") > built        # the code copy in tile order, not the generic fallback
+    # activations with a large common offset: the bias term 128 * sum(x) is then far larger than the result
+    x2 = bf16_round(rnd(23, (m, k)) + 3.0)
+    run_linear(hip, lambda fb, a, b, c: F.linear_quantized(a, b, c), specs, [x2, q, s], 6e-2, 2e-2, expect_chain=False)
+
+
+@pytest.mark.parametrize("scheme", ["w8", "w4g128"])
+@pytest.mark.parametrize("m", [1, 8, 64])
 def test_bias_gelu_residual(hip, scheme, m):
     k, n = 768, 3072
     x, w, b, r = bf16_round(rnd(10, (m, k))), rnd(11, (k, n), 2.0 / np.sqrt(k)), bf16_round(rnd(12, (n,))), bf16_round(rnd(13, (m, n)))
@@ -166,7 +182,7 @@ def test_bias_gelu_residual(hip, scheme, m):
 
 
 @pytest.mark.parametrize("scheme", ["w8", "w4g128"])
-@pytest.mark.parametrize("m,k,n", [(1, 3072, 9216), (1, 256, 96), (64, 512, 256)])
+@pytest.mark.parametrize("m,k,n", [(1, 3072, 9216), (1, 256, 96), (64, 512, 256), (8, 3072, 9216), (16, 256, 96)])
 def test_norm_swiglu_pair(hip, scheme, m, k, n):
     """RMSNorm -> gate / up -> SwiGLU: one phase of the chain (or one dual GEMM) over two quantised matrices."""
     x, g = bf16_round(rnd(6, (m, k), 3.0)), bf16_round(rnd(7, (k,)) + 1.5)
