@@ -194,6 +194,13 @@ class _ModelBase:
         return self.backend.run_program(program, list(args) + params, don)
 
 
+def _last_rows(hidden: Tensor, seq: int, batch: int) -> Tensor:
+    """Row seq - 1 of each of the `batch` stacked sequences."""
+    d = hidden.dims[1]
+    rows = [hidden.slice([b * seq + seq - 1, 0], [1, d]) for b in range(batch)]
+    return rows[0] if batch == 1 else Tensor.concat(0, rows)
+
+
 # ================================================================================ GPT-2
 @dataclass
 class GptConfig:
@@ -303,9 +310,11 @@ class Gpt(_ModelBase):
         ff = F.linear(act, P[p + "feed_forward.w_out"], P[p + "feed_forward.b_out"])
         return ff + residual
 
-    def _build(self, seq: int, capacity: int, decode: bool, batch: int = 1) -> Tuple[Program, dict]:
-        """One program for the whole forward (model/gpt.rs:585-751)."""
-        key = (seq, capacity, decode, batch)
+    def _build(self, seq: int, capacity: int, decode: bool, batch: int = 1, last_only: bool = False) -> Tuple[Program, dict]:
+        """One program for the whole forward (model/gpt.rs:585-751).  last_only: the head runs on the last row of
+        each sequence only (logits [batch, V] instead of [batch * seq, V])."""
+        last_only = last_only and seq > 1
+        key = (seq, capacity, decode, batch, last_only)
         if key in self._programs:
             return self._programs[key]
         cfg, L = self.config, self.config.num_layers
@@ -352,6 +361,8 @@ class Gpt(_ModelBase):
                 ctxs.append(ctx)
             ctx_all = ctxs[0] if batch == 1 else Tensor.concat(0, ctxs)
             hidden = self._block_tail(P, i, hidden, ctx_all)
+        if last_only:
+            hidden = _last_rows(hidden, seq, batch)
         normalized, *_ = F.layer_norm(hidden, P["final_ln.gamma"], P["final_ln.beta"], cfg.eps)
         logits = normalized.matmul(P["lm_head"])
         results = []
@@ -366,9 +377,12 @@ class Gpt(_ModelBase):
 
     # -- forward -----------------------------------------------------------------------
     def forward_with_decode_cache(self, tokens: Sequence[int], position_offset: int,
-                                  caches: List[Optional[DecodeKvCache]], fixed_capacity: Optional[int] = None):
-        """model/gpt.rs:585-751.  Returns the logits handle [T, V]; `caches` is updated in place."""
-        return self.forward_batch([list(tokens)], position_offset, [caches], fixed_capacity)
+                                  caches: List[Optional[DecodeKvCache]], fixed_capacity: Optional[int] = None,
+                                  last_logits_only: bool = False):
+        """model/gpt.rs:585-751.  Returns the logits handle [T, V]; `caches` is updated in place.
+        last_logits_only: the final norm and the lm_head run on the last position only and the handle is [1, V] (the
+        reference computes every row, gpt.rs:735-736, and its generation loop reads the last)."""
+        return self.forward_batch([list(tokens)], position_offset, [caches], fixed_capacity, last_logits_only=last_logits_only)
 
     def forward_decode_device_token(self, token_handle, position_offset: int, caches: List[Optional[DecodeKvCache]],
                                     fixed_capacity: Optional[int] = None):
@@ -379,7 +393,7 @@ class Gpt(_ModelBase):
 
     def forward_batch(self, token_rows: List[List[int]], position_offset: int,
                       caches: List[List[Optional[DecodeKvCache]]], fixed_capacity: Optional[int] = None,
-                      token_handle=None):
+                      token_handle=None, last_logits_only: bool = False):
         """Independent sequences sharing the weights: row-stacked hidden states, one M=B*T
         GEMM per linear, per-sequence attention.  The reference has no batch dimension
         (ops/functional/attention.rs:189-203); with one row this is exactly its path."""
@@ -413,7 +427,7 @@ class Gpt(_ModelBase):
         if have and (seq != 1):
             raise ValueError("decode with an existing cache supports one token per sequence")
         L = cfg.num_layers
-        prog, _ = self._build(seq, capacity, have, batch)
+        prog, _ = self._build(seq, capacity, have, batch, last_logits_only)
         poss = [position_offset + j for _ in range(batch) for j in range(seq)]
         tok_arg = token_handle if token_handle is not None else self._upload_i32([t for row in token_rows for t in row])
         args = [tok_arg, self._upload_i32(poss)]
@@ -629,8 +643,9 @@ class Ministral(_ModelBase):
             return F.linear_quantized(x, P[name + ".q"], P[name + ".s"])
         return F.linear(x, P[name])
 
-    def _build(self, seq: int, capacity: int, decode: bool, batch: int = 1) -> Tuple[Program, dict]:
-        key = (seq, capacity, decode, batch)
+    def _build(self, seq: int, capacity: int, decode: bool, batch: int = 1, last_only: bool = False) -> Tuple[Program, dict]:
+        last_only = last_only and seq > 1
+        key = (seq, capacity, decode, batch, last_only)
         if key in self._programs:
             return self._programs[key]
         cfg, L = self.config, self.config.num_layers
@@ -683,6 +698,8 @@ class Ministral(_ModelBase):
             act = F.swiglu(gate, up)
             ff = self._linear(P, p + "feed_forward.w_down", act)
             hidden = ff + residual
+        if last_only:
+            hidden = _last_rows(hidden, seq, batch)
         normalized, *_ = F.rms_norm(hidden, P["final_norm.gamma"], cfg.eps)
         logits = self._linear(P, "lm_head", normalized)
         results = []
@@ -695,15 +712,15 @@ class Ministral(_ModelBase):
         self._programs[key] = (prog, layout)
         return prog, layout
 
-    def forward_with_decode_cache(self, tokens, position_offset, caches, fixed_capacity=None):
-        """model/ministral.rs:613-766."""
-        return self.forward_batch([list(tokens)], position_offset, [caches], fixed_capacity)
+    def forward_with_decode_cache(self, tokens, position_offset, caches, fixed_capacity=None, last_logits_only=False):
+        """model/ministral.rs:613-766.  last_logits_only: see Gpt.forward_with_decode_cache."""
+        return self.forward_batch([list(tokens)], position_offset, [caches], fixed_capacity, last_logits_only=last_logits_only)
 
     def forward_decode_device_token(self, token_handle, position_offset, caches, fixed_capacity=None):
         """See Gpt.forward_decode_device_token."""
         return self.forward_batch([[None]], position_offset, [caches], fixed_capacity, token_handle=token_handle)
 
-    def forward_batch(self, token_rows, position_offset, caches, fixed_capacity=None, token_handle=None):
+    def forward_batch(self, token_rows, position_offset, caches, fixed_capacity=None, token_handle=None, last_logits_only=False):
         cfg = self.config
         batch, seq = len(token_rows), len(token_rows[0])
         if token_handle is not None and (batch != 1 or seq != 1):
@@ -727,7 +744,7 @@ class Ministral(_ModelBase):
         if have and seq != 1:
             raise ValueError("decode with an existing cache supports one token per sequence")
         L = cfg.num_layers
-        prog, _ = self._build(seq, capacity, have, batch)
+        prog, _ = self._build(seq, capacity, have, batch, last_logits_only)
         cos, sin = F.rotary_cos_sin_cache_slice(position_offset, seq, self.rope)   # ministral.rs:253-261
         half = cfg.rotary_dim // 2
         tok_arg = token_handle if token_handle is not None else self._upload_i32([t for row in token_rows for t in row])
@@ -767,7 +784,7 @@ class Generator:
 
     def __init__(self, model, prompt: Sequence[int], kv_cache_capacity: Optional[int] = None,
                  device_sampling: bool = True, temperature: float = 0.0, seed: int = 0,
-                 pipelined: Optional[bool] = None):
+                 pipelined: Optional[bool] = None, last_logits_only: bool = True):
         if len(prompt) == 0:
             raise ValueError("prompt must be non-empty")
         self.model = model
@@ -777,6 +794,9 @@ class Generator:
         # temperature > 0: the backend samples from softmax(logits / temperature) given a uniform draw per
         # step (DecodeSampleRequest.random_u, spec.rs:1270-1284; sampler.rs:83-93 draws it in (eps, 1 - eps))
         self.temperature = float(temperature)
+        # the loop only ever samples from the last row: prefill runs the head on that row alone (`self.logits` is then
+        # [1, V] after a prefill as after a decode step); False keeps every row as the reference's forward does
+        self.last_logits_only = bool(last_logits_only)
         self._rng = np.random.default_rng(seed)
         can_pipeline = device_sampling and hasattr(model.backend, "sample_decode_token_begin") and \
             hasattr(model, "forward_decode_device_token")
@@ -786,7 +806,7 @@ class Generator:
         self.caches: List[Optional[DecodeKvCache]] = [None] * model.num_layers
         self.window_start = max(0, len(self.tokens) - model.context_length)
         context = self.tokens[self.window_start:]
-        self.logits = model.forward_with_decode_cache(context, 0, self.caches, self.capacity)
+        self.logits = self._prefill(context)
         self.processed_len = len(context)
 
     def _sample(self) -> int:
@@ -802,6 +822,11 @@ class Generator:
                 return tok
         row = be.to_numpy(self.logits)[-1]
         return int(np.argmax(row))
+
+    def _prefill(self, context):
+        if self.last_logits_only:
+            return self.model.forward_with_decode_cache(context, 0, self.caches, self.capacity, last_logits_only=True)
+        return self.model.forward_with_decode_cache(context, 0, self.caches, self.capacity)
 
     def _draw_u(self) -> float:
         eps = float(np.finfo(np.float32).eps)
@@ -839,7 +864,7 @@ class Generator:
             self.caches = [None] * self.model.num_layers
             self.window_start = len(self.tokens) - self.model.context_length
             context = self.tokens[self.window_start:]
-            self.logits = self.model.forward_with_decode_cache(context, 0, self.caches, self.capacity)
+            self.logits = self._prefill(context)
             self.processed_len = len(context)
         else:
             self.logits = self.model.forward_with_decode_cache([nxt], self.processed_len, self.caches, self.capacity)

@@ -83,6 +83,27 @@ def test_pipelined_generation_equals_unpipelined(hip, temperature):
         models.Generator(m, PROMPT, device_sampling=False, pipelined=True)
 
 
+@pytest.mark.parametrize("cls,cfg", [(models.Gpt, TINY_GPT), (models.Ministral, MID_MINISTRAL)], ids=["gpt", "ministral"])
+def test_last_row_only_head(hip, cls, cfg):
+    """last_logits_only: final norm + lm_head on the last position only.  Equal to the last row of the full logits
+    (same f32 arithmetic per row; a different kernel serves one row, hence the 1e-5), same tokens from the generator."""
+    m = cls.random(cfg, hip, seed=41, std=0.1, dtype="F32")
+    prompt = [5, 9, 2, 77 % cfg.vocab_size, 31, 8, 1]
+    full = hip.to_numpy(m.forward_with_decode_cache(prompt, 0, [None] * cfg.num_layers, 32))
+    last = hip.to_numpy(m.forward_with_decode_cache(prompt, 0, [None] * cfg.num_layers, 32, last_logits_only=True))
+    assert full.shape == (len(prompt), cfg.vocab_size) and last.shape == (1, cfg.vocab_size)
+    assert rel_err(last[0], full[-1]) < 1e-5
+    ob = OracleBackend()
+    mo = cls.random(cfg, ob, seed=41, std=0.1, dtype="F32")
+    want = ob.to_numpy(mo.forward_with_decode_cache(prompt, 0, [None] * cfg.num_layers, 32, last_logits_only=True))
+    assert rel_err(last[0], want[0]) < 1e-4
+    rows = hip.to_numpy(m.forward_batch([prompt, prompt[::-1]], 0, [[None] * cfg.num_layers for _ in range(2)], 32, last_logits_only=True))
+    assert rows.shape == (2, cfg.vocab_size) and rel_err(rows[0], full[-1]) < 1e-5
+    a = models.Generator(m, prompt, kv_cache_capacity=32, last_logits_only=True).generate(8)
+    b = models.Generator(m, prompt, kv_cache_capacity=32, last_logits_only=False).generate(8)
+    assert a == b
+
+
 def test_sampling_tickets(hip):
     from parity import TensorSpec
     from gptrs_amd.backend import BackendError
