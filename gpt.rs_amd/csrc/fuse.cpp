@@ -816,7 +816,8 @@ struct Fuser {
         for (int r : fn.result_ids) is_result[r] = true;
         for (size_t i = 0; i < fn.body.size(); ++i) {
             Instr& nrm = fn.body[i];
-            if (nrm.dead || nrm.op != OpKind::FRmsNorm) continue;
+            if (nrm.dead || (nrm.op != OpKind::FRmsNorm && nrm.op != OpKind::FLayerNorm)) continue;
+            const bool ln = nrm.op == OpKind::FLayerNorm;   // folded into plain (unquantised) decode linears only
             const int nv = nrm.out_ids[0];
             if (is_result[nv] || nrm.out_specs[0].rank() != 2) continue;
             std::vector<Instr*> cons;
@@ -826,14 +827,16 @@ struct Fuser {
                 for (size_t o = 0; o < c.operands.size(); ++o) {
                     if (c.operands[o].value != nv) continue;
                     ++found;
-                    if (c.op == OpKind::FLinear && c.tiled && !c.norm && o == 0) cons.push_back(&c);
+                    if (c.op == OpKind::FLinear && c.tiled && !c.norm && o == 0 && !(ln && c.quant)) cons.push_back(&c);
                 }
             }
             if (cons.empty() || (int)cons.size() != found || found != uses[nv]) continue;
             for (Instr* c : cons) {
                 c->operands[0] = nrm.operands[0];
                 c->operands.push_back(nrm.operands[1]);
+                if (ln) c->operands.push_back(nrm.operands[2]);
                 c->norm = true;
+                c->norm_ln = ln;
                 c->eps = nrm.eps;
                 c->scale = nrm.scale;
             }

@@ -103,6 +103,7 @@ struct TiledLinearArgs {
     int64_t m, k, n;
     int act;
     float inv_n, eps;
+    const void* beta;   // with gamma: LayerNorm (normalization.rs:123-174) instead of RMSNorm
 };
 size_t tiled_weight_bytes(int dtype, int64_t k, int64_t n);
 void tile_weights(hipStream_t s, int dtype, const void* w, void* wt, int64_t k, int64_t n);

@@ -83,6 +83,7 @@ __device__ __forceinline__ float tiled_finish(float v, float v2, bool dual, int 
 template <typename T, int MT, int TP, int U, bool DUAL, bool NORM>
 __global__ __launch_bounds__(256) void gemv_tiled_kernel(const T* __restrict__ x, const T* __restrict__ wt,
                                                          const T* __restrict__ wt2, const T* __restrict__ gamma,
+                                                         const T* __restrict__ beta,
                                                          const T* __restrict__ bias, const T* __restrict__ residual,
                                                          T* __restrict__ y, int M, int64_t K, int64_t N, int64_t ntiles,
                                                          float inv_n, float eps, int act) {
@@ -93,6 +94,7 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(const T* __restrict__ x
     __shared__ T xs[MT][KT];
     __shared__ float red[4][NOUT];
     __shared__ float s_scale[MT];
+    __shared__ float s_mean[MT];
     __shared__ float s_tmp[16];
     const int t = threadIdx.x;
     const int64_t tile0 = (int64_t)blockIdx.x * TP;
@@ -126,18 +128,25 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(const T* __restrict__ x
     // RMSNorm prologue (normalization.rs:183-217): inv_rms = rsqrt(sum(x^2)*(1/N) + eps) per row.
     // When the whole row fits the staging buffer the same pass also stages x (raw); the scaling
     // pass below then touches only LDS and gamma.
+    // LayerNorm (beta given; normalization.rs:123-174): mean first, then the variance of the centred values, as the
+    // stand-alone kernel takes them.
     const bool one_chunk = K <= KT;
     if (NORM) {
         for (int m = 0; m < M; ++m) {
-            float q = 0.f;
+            float q = 0.f, mean = 0.f;
+            if (beta) {
+                float sm = 0.f;
+                for (int64_t kk = t; kk < K; kk += 256) sm += ldf(x, (int64_t)m * K + kk);
+                mean = block_sum(sm, s_tmp) * inv_n;
+            }
             for (int64_t kk = t; kk < K; kk += 256) {
                 const T raw = x[(int64_t)m * K + kk];
-                const float v = ldf(&raw, 0);
+                const float v = ldf(&raw, 0) - mean;
                 if (one_chunk) xs[m][kk] = raw;
                 q += v * v;
             }
             const float tot = block_sum(q, s_tmp);
-            if (t == 0) s_scale[m] = 1.0f / sqrtf(tot * inv_n + eps);
+            if (t == 0) { s_scale[m] = 1.0f / sqrtf(tot * inv_n + eps); s_mean[m] = mean; }
         }
         __syncthreads();
     }
@@ -161,7 +170,10 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(const T* __restrict__ x
                 // each thread re-reads only the slots it wrote itself in the prologue
                 float v = (NORM && one_chunk) ? ldf(&xs[m][0], kk) : ldf(x, (int64_t)m * K + k0 + kk);
                 // the value the stand-alone norm kernel would have stored: (x*inv_rms)*gamma, rounded to T
-                if (NORM) v = (v * s_scale[m]) * ldf(gamma, k0 + kk);
+                if (NORM) {
+                    v = ((v - s_mean[m]) * s_scale[m]) * ldf(gamma, k0 + kk);
+                    if (beta) v += ldf(beta, k0 + kk);
+                }
                 stf(&xs[m][0], kk, v);
             }
         __syncthreads();
@@ -242,7 +254,7 @@ static void launch_tiled(hipStream_t s, const TiledLinearArgs& a) {
     const unsigned grid = (unsigned)cdiv(ntiles, TP);
 #define GPTRS_GT(DUAL, NORM)                                                                                          \
     gemv_tiled_kernel<T, MT, TP, U, DUAL, NORM><<<grid, 256, 0, s>>>((const T*)a.x, (const T*)a.wt, (const T*)a.wt2,         \
-        (const T*)a.gamma, (const T*)a.bias, (const T*)a.residual, (T*)a.y, (int)a.m, a.k, a.n, ntiles, a.inv_n, a.eps, a.act)
+        (const T*)a.gamma, (const T*)a.beta, (const T*)a.bias, (const T*)a.residual, (T*)a.y, (int)a.m, a.k, a.n, ntiles, a.inv_n, a.eps, a.act)
     if (a.wt2) { if (a.gamma) GPTRS_GT(true, true); else GPTRS_GT(true, false); }
     else { if (a.gamma) GPTRS_GT(false, true); else GPTRS_GT(false, false); }
 #undef GPTRS_GT

@@ -770,6 +770,7 @@ void Builder::build() {
         const Spec& w = plan.values[st.src[1]].spec;
         if (x.rank() != 2 || w.rank() != 2) return 0;
         const bool dual = in.act == 2;
+        if (in.norm_ln) return 0;   // the chain stages RMSNorm only
         if (!k::chain_supported((int)x.dtype, x.dims[0], x.dims[1], w.dims[1], dual, in.norm, in.quant)) return 0;
         k::ChainPhase p{};
         return k::chain_fill_phase(p, x.dims[1], w.dims[1], dual, in.quant) ? 1 : 0;
@@ -1099,7 +1100,12 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
                 const size_t norm_bytes = in.norm ? align_up((size_t)x.count() * dtype_size(x.dtype)) : 0;
                 if (in.norm) {
                     void* xn = cx.ws + st.scratch_off;
-                    k::rms_norm(s, (int)x.dtype, sa.x, src_ptr(st, cx, oi++), xn, sa.m, sa.k, in.scale, in.eps);
+                    if (in.norm_ln) {
+                        k::layer_norm(s, (int)x.dtype, sa.x, src_ptr(st, cx, oi), src_ptr(st, cx, oi + 1), xn, sa.m, sa.k, in.scale, in.eps);
+                        oi += 2;
+                    } else {
+                        k::rms_norm(s, (int)x.dtype, sa.x, src_ptr(st, cx, oi++), xn, sa.m, sa.k, in.scale, in.eps);
+                    }
                     ++cx.launches;
                     sa.x = xn;
                 }
@@ -1143,6 +1149,7 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
                 if (in.has_bias) ta.bias = src_ptr(st, cx, oi++);
                 if (in.has_residual) ta.residual = src_ptr(st, cx, oi++);
                 if (in.norm) { ta.gamma = src_ptr(st, cx, oi++); ta.inv_n = in.scale; ta.eps = in.eps; }
+                if (in.norm_ln) ta.beta = src_ptr(st, cx, oi++);
                 ta.y = dst;
                 ta.act = in.act == 1 ? 1 : 0;
                 hipEvent_t e0 = nullptr, e1 = nullptr;

@@ -118,6 +118,7 @@ struct Instr {
     bool mfma = false;                       // FLinear: prefill GEMM over the k-grouped weight copy
     bool tiled = false;                      // FLinear: decode GEMV over the column-tiled weight copy
     bool norm = false;                       // FLinear: RMSNorm of x fused in (last operand = gamma; eps, scale)
+    bool norm_ln = false;                    // with norm: LayerNorm instead (last two operands = gamma, beta)
     // FLinear over weight-only quantised weights (0: none; 1: int8 per column, 2: int4 groups of 128): every
     // weight operand is then a (codes, scales) pair: (x, q, s, [q2, s2], [bias], [residual], [gamma]).
     // FQuant: 1 int8 scales, 2 int8 codes, 3 int4 scales, 4 int4 codes, 5 int8 dequantise, 6 int4 dequantise
