@@ -73,9 +73,15 @@ def cpu_baseline(cfg, seconds_budget: float = 25.0):
     lib.gptrs_ref_cache_free.argtypes = [ctypes.c_void_p]
     lib.gptrs_ref_matmul_f32_cached.argtypes = [fp, fp, fp, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_void_p]
     a = cfg.attention_config()
-    d, f = cfg.embed_dim, cfg.ffn_dim
+    d = cfg.embed_dim
     head_cols = cfg.vocab_size // 8
-    shapes = [(d, a.total_projection_dim), (a.query_projection_dim, d), (d, f), (d, f), (f, d), (d, head_cols)]
+    if hasattr(cfg, "ffn_dim"):     # Ministral: qkv, out, gate, up, down
+        f = cfg.ffn_dim
+        shapes = [(d, a.total_projection_dim), (a.query_projection_dim, d), (d, f), (d, f), (f, d), (d, head_cols)]
+    else:                           # GPT-2: qkv, out, fc1, fc2
+        f = cfg.mlp_ratio * d
+        shapes = [(d, a.total_projection_dim), (a.query_projection_dim, d), (d, f), (f, d), (d, head_cols)]
+    nl = len(shapes) - 1
     rng = np.random.default_rng(0)
     mats, caches, xs, ys = [], [], [], []
     for k, n in shapes:
@@ -96,10 +102,10 @@ def cpu_baseline(cfg, seconds_budget: float = 25.0):
     t_start = time.perf_counter()
     while reps < 3 or (time.perf_counter() - t_start < seconds_budget / 3 and reps < 20):
         t0 = time.perf_counter()
-        for i in range(5):
+        for i in range(nl):
             call(i)
         t1 = time.perf_counter()
-        call(5)
+        call(nl)
         t2 = time.perf_counter()
         t_layer += t1 - t0
         t_head += t2 - t1
@@ -108,9 +114,65 @@ def cpu_baseline(cfg, seconds_budget: float = 25.0):
         lib.gptrs_ref_cache_free(c)
     t_token = cfg.num_layers * t_layer / reps + 8 * t_head / reps
     return {"value": round(1.0 / t_token, 4), "unit": "tokens/s", "cores": 1, "kind": "reference",
-            "sample": f"{reps} reps of one layer's 5 f32 GEMVs + 1/8 of lm_head through {name} "
-                      f"(gpt_rs_c_matmul_f32_cached_b, m=1, packed-B cache warm); token time = 26 layers + "
+            "sample": f"{reps} reps of one layer's {nl} f32 GEMVs + 1/8 of lm_head through {name} "
+                      f"(gpt_rs_c_matmul_f32_cached_b, m=1, packed-B cache warm); token time = {cfg.num_layers} layers + "
                       f"8 head slices; non-GEMV ops excluded"}
+
+
+README_GPT2_TOKENS_PER_S = 74.71   # reference README.md:18-25: GPT-2 small f32, generate 64 tokens, C backend, 1 thread of a Ryzen 9 9950X3D
+
+
+def gpt2_generate(args, be):
+    """BASELINE configs[0]: GPT-2 small f32, weights N(0, 0.02) from seed 0, prompt of 16 ids (seed 1), greedy, 64 tokens
+    with KV cache (capacity 128).  Timed like the reference's published figure (README.md:27-50,
+    scripts/gptrs_eval/runner.py:24-56): each step is one WHOLE generate call, prefill included; tokens/s = 64 / mean
+    wall time.  The steady decode rate and its share of the HBM roofline are reported beside it."""
+    from gptrs_amd import models
+    cfg = models.GptConfig()
+    t0 = time.perf_counter()
+    model = models.Gpt.random(cfg, be, seed=0, dtype="F32")
+    t_init = time.perf_counter() - t0
+    prompt = np.random.default_rng(1).integers(0, cfg.vocab_size, 16).tolist()
+    new_tokens = 64
+
+    def generate():
+        gen = models.Generator(model, prompt, kv_cache_capacity=128)
+        out = gen.generate(new_tokens)
+        be.synchronize()
+        return out
+
+    for _ in range(max(args.warmup, 1)):
+        tokens = generate()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        assert generate() == tokens
+    elapsed = (time.perf_counter() - t0) / args.steps
+    gen = models.Generator(model, prompt, kv_cache_capacity=256)
+    for _ in range(8):
+        gen.step()
+    be.synchronize()
+    n, start = 128, gen.processed_len
+    t0 = time.perf_counter()
+    for _ in range(n):
+        gen.step()
+    be.synchronize()
+    t_step = (time.perf_counter() - t0) / n
+    d, L, V = cfg.embed_dim, cfg.num_layers, cfg.vocab_size
+    per_layer = d * 3 * d + d * d + 2 * d * cfg.mlp_ratio * d + (3 * d + d + cfg.mlp_ratio * d + d) + 4 * d   # weights, biases, LN
+    step_bytes = 4 * (L * per_layer + 2 * d + d * V + 2 * L * d * (start + n // 2 + 1) + V + 2 * d)
+    value = new_tokens / elapsed
+    print(json.dumps({
+        "metric": "tokens/s of a whole generate call (prefill 16 + 64 greedy tokens), GPT-2 small f32, batch 1",
+        "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": max(args.warmup, 1),
+        "ms_per_step": round(elapsed * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": round(value / README_GPT2_TOKENS_PER_S, 2), "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "gpt-2 small f32, prompt 16, greedy generate 64 with KV cache (capacity 128); a step is one generate call",
+                   "baseline": "74.71 tokens/s: reference C backend, one thread of a Ryzen 9 9950X3D, 1-token prompt, sampled (README.md:18-25)"},
+        "decode_steady_tokens_per_s": round(1.0 / t_step, 1), "decode_us_per_step": round(t_step * 1e6, 1),
+        "hbm_gbps": round(step_bytes / t_step / 1e9, 1), "hbm_frac": round(step_bytes / t_step / 1e9 / HBM_PEAK_GBPS, 4),
+        "algorithmic_bytes_per_step": step_bytes, "launches_per_step": be.counter("last_program_launches"),
+        "weight_init_s": round(t_init, 1), "roofline": None,
+        "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(cfg)}))
 
 
 def batched_decode(args, be, cfg, model, capacity):
@@ -187,6 +249,9 @@ def main():
     ap.add_argument("--batch", type=int, default=1,
                     help="B > 1: batched decode of B independent sequences (rows stacked through the linear layers, one attention "
                          "launch per layer for all of them); a side workload, NOT the headline metric (which is batch 1)")
+    ap.add_argument("--model", choices=["ministral", "gpt2"], default="ministral",
+                    help="gpt2: the reference's own published workload (GPT-2 small f32, generate 64 tokens); --steps then counts "
+                         "whole generate calls (default 8)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain elementwise kernel of known traffic (x + 0 over 2^28 f32: 1 GiB read, 1 GiB written, "
@@ -214,6 +279,10 @@ def main():
         be.synchronize()
         print(json.dumps({"copy_calibration": "10 launches of x + 0.0 over %d f32" % n, "bytes_read_per_launch": 4 * n, "bytes_written_per_launch": 4 * n}))
         return
+    if args.model == "gpt2":
+        if args.steps == 224:
+            args.steps, args.warmup = 8, 2
+        return gpt2_generate(args, be)
     cfg = models.MinistralConfig(num_layers=args.layers)
     total_len = args.prompt + args.warmup + args.steps + 1
     capacity = max(1280, (total_len + 255) // 256 * 256)
