@@ -343,7 +343,7 @@ __device__ __forceinline__ void lane_pair(float v, int off, float& a, float& b) 
 // this launch are requested BEFORE the grid barrier is awaited (they do not depend on the
 // previous phase); only the query row and this step's K/V row are read after it.
 __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const ChainPhase& P, GPTRS_LDS float* lds, int unit, int phase) {
-    constexpr int PP = 3;   // positions per lane group requested ahead of the barrier
+    constexpr int PP = 4;   // positions per lane group requested ahead of the barrier
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const bool control = wave == NWS;
     const int dh = P.head_dim, n_q = P.n_q, n_kv = P.n_kv, nch = P.nch, half = P.rot_half;
