@@ -800,6 +800,7 @@ __device__ void stream_waves(Shared& sh, const unsigned* xs, int nphases) {
     // load iterator: the next j-step (TP words per lane) to fetch
     int l_phase = -1, l_unit = 0, l_unit_end = 0, l_j = 0, l_wpt = 1, l_ntiles = 1;
     long l_Kw = 0;
+    int l_Kv = 0;   // words of a tile stream that hold weights; the padding behind them (up to a whole step) is never fetched
     const uint4* l_w = nullptr;
     bool l_active = true;
     const GPTRS_GLOBAL u32x4* l_base[TP];
@@ -824,14 +825,23 @@ __device__ void stream_waves(Shared& sh, const unsigned* xs, int nphases) {
             l_unit_end = min(l_unit + upb, units);
             if (l_unit < l_unit_end) {
                 l_wpt = uni(ph.wpt); l_ntiles = uni(ph.ntiles); l_Kw = uni(ph.Kw);
+                constexpr int kpw = FMT == kChainW16 ? 2 : (FMT == kChainW8 ? 4 : 8);
+                l_Kv = (uni(ph.K) + kpw - 1) / kpw;
                 l_w = (const uint4*)uni_ptr(ph.w);
             }
         }
         if (l_active) l_setbase();
     };
     auto l_fetch = [&](u32x4 (&dst)[TP]) {   // requires l_active
+        // the activations are zero beyond K, so a lane whose word is padding contributes nothing with any word
+        // (quantised formats only: their words hold 4 or 8 k, so K = 3072 leaves a quarter of a step as padding; bf16
+        // rows of the model shapes fill whole steps and keep the unconditional load)
+        const bool live = FMT == kChainW16 || l_j * NS + t < l_Kv;
 #pragma unroll
-        for (int p = 0; p < TP; ++p) dst[p] = l_base[p][(long)l_j * NS];
+        for (int p = 0; p < TP; ++p) {
+            if (live) dst[p] = l_base[p][(long)l_j * NS];
+            else { dst[p].x = 0u; dst[p].y = 0u; dst[p].z = 0u; dst[p].w = 0u; }
+        }
         if (++l_j == l_wpt) {
             ++l_unit;
             if (l_unit >= l_unit_end) l_seek(); else l_setbase();
