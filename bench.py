@@ -176,22 +176,21 @@ def gpt2_generate(args, be):
 
 
 def batched_decode(args, be, cfg, model, capacity):
-    """B independent sequences decoded together (models.forward_batch): tokens/s summed over the sequences.  The next
-    tokens are the row-wise argmax taken on the host (B x vocab bf16 logits cross PCIe each step, inside the timed
-    region), the linear layers are bracketed by HIP events in a second pass as in the batch-1 run."""
+    """B independent sequences decoded together (models.BatchGenerator): tokens/s summed over the sequences.  The next
+    tokens are the row-wise argmax taken on the device and fed to the next step there (4 B bytes reach the host per
+    step), the linear layers are bracketed by HIP events in a second pass as in the batch-1 run."""
     B = args.batch
+    from gptrs_amd import models
     rng = np.random.default_rng(6)
     rows = [rng.integers(0, cfg.vocab_size, args.prompt).tolist() for _ in range(B)]
-    caches = [[None] * cfg.num_layers for _ in range(B)]
     t0 = time.perf_counter()
-    state = {"logits": model.forward_batch(rows, 0, caches, capacity), "pos": args.prompt}
+    gen = models.BatchGenerator(model, rows, kv_cache_capacity=capacity)
     be.synchronize()
     t_prefill = time.perf_counter() - t0
+    state = {"pos": args.prompt}
 
     def step():
-        lg = be.to_numpy(state["logits"]).reshape(B, -1, cfg.vocab_size)[:, -1]
-        toks = [[int(np.argmax(lg[b]))] for b in range(B)]
-        state["logits"] = model.forward_batch(toks, state["pos"], caches, capacity)
+        gen.step()
         state["pos"] += 1
 
     for _ in range(args.warmup):
@@ -228,7 +227,7 @@ def batched_decode(args, be, cfg, model, capacity):
         "value": round(B * args.steps / elapsed, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(elapsed / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "ministral-3b-shape %s decode, batch %d, prompt %d each, greedy (host argmax), KV capacity %d" % (wname, B, args.prompt, capacity),
+        "config": {"workload": "ministral-3b-shape %s decode, batch %d, prompt %d each, greedy, KV capacity %d" % (wname, B, args.prompt, capacity),
                    "layers": cfg.num_layers, "cache_len_mid": mid_len},
         "hbm_gbps": round(step_bytes / (elapsed / args.steps) / 1e9, 1),
         "hbm_frac": round(step_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS, 4),

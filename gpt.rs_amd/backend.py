@@ -27,7 +27,8 @@ EXPORTS = [
     "gptrs_hip_run_program", "gptrs_hip_run_program_donate", "gptrs_hip_execute_instruction",
     "gptrs_hip_param_get", "gptrs_hip_param_set", "gptrs_hip_supports_decode_sampling",
     "gptrs_hip_sample_decode_token", "gptrs_hip_sample_decode_token_begin", "gptrs_hip_sample_decode_token_wait",
-    "gptrs_hip_decode_token_tensor", "gptrs_hip_last_error", "gptrs_hip_synchronize", "gptrs_hip_set_option",
+    "gptrs_hip_decode_token_tensor", "gptrs_hip_sample_decode_rows_begin", "gptrs_hip_sample_decode_rows_wait",
+    "gptrs_hip_decode_rows_tensor", "gptrs_hip_last_error", "gptrs_hip_synchronize", "gptrs_hip_set_option",
     "gptrs_hip_counter",
 ]
 
@@ -82,6 +83,9 @@ def load_library(path: str = LIB_PATH):
                                                         ctypes.POINTER(ctypes.c_int64)]
     lib.gptrs_hip_sample_decode_token_wait.argtypes = [vp, ctypes.c_int64, ctypes.POINTER(ctypes.c_int64)]
     lib.gptrs_hip_decode_token_tensor.argtypes = [vp, pvp]
+    lib.gptrs_hip_sample_decode_rows_begin.argtypes = [vp, vp, ctypes.POINTER(ctypes.c_int64)]
+    lib.gptrs_hip_sample_decode_rows_wait.argtypes = [vp, ctypes.c_int64, ctypes.POINTER(ctypes.c_int32), sz]
+    lib.gptrs_hip_decode_rows_tensor.argtypes = [vp, ctypes.c_int64, pvp]
     lib.gptrs_hip_last_error.argtypes = []
     lib.gptrs_hip_last_error.restype = cp
     lib.gptrs_hip_synchronize.argtypes = [vp]
@@ -247,6 +251,23 @@ class HipBackend:
         """si32[1] handle over the device copy of the last sampled token."""
         out = ctypes.c_void_p()
         self._check(self._lib.gptrs_hip_decode_token_tensor(self._handle, ctypes.byref(out)))
+        return TensorHandle(self, out.value, self._spec_of(out.value))
+
+    def sample_decode_rows_begin(self, logits: TensorHandle) -> int:
+        """Queues the greedy token of every row of logits [rows, vocab]; returns a ticket for sample_decode_rows_wait."""
+        ticket = ctypes.c_int64(-1)
+        self._check(self._lib.gptrs_hip_sample_decode_rows_begin(self._handle, logits.ptr, ctypes.byref(ticket)))
+        return int(ticket.value)
+
+    def sample_decode_rows_wait(self, ticket: int, rows: int) -> list:
+        buf = (ctypes.c_int32 * rows)()
+        self._check(self._lib.gptrs_hip_sample_decode_rows_wait(self._handle, ticket, buf, rows))
+        return [int(v) for v in buf]
+
+    def decode_rows_tensor(self, rows: int) -> TensorHandle:
+        """si32[rows] handle over the device copy of the tokens of the last sample_decode_rows_begin."""
+        out = ctypes.c_void_p()
+        self._check(self._lib.gptrs_hip_decode_rows_tensor(self._handle, rows, ctypes.byref(out)))
         return TensorHandle(self, out.value, self._spec_of(out.value))
 
     # -- extras ----------------------------------------------------------------------------

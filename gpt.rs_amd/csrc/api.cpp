@@ -72,7 +72,8 @@ Backend::Backend(int dev) : device(dev) {
     GPTRS_HIP_CHECK(hipMalloc((void**)&d_argmax_idx_, 1024 * sizeof(int32_t)));
     token_buf_ = new_buffer(256);
     d_token_ = (int64_t*)token_buf_->ptr;
-    GPTRS_HIP_CHECK(hipHostMalloc((void**)&h_token_ring_, kTokenRing * 2 * sizeof(int64_t), hipHostMallocDefault));
+    rows_buf_ = new_buffer(kMaxTokenRows * sizeof(int32_t));
+    GPTRS_HIP_CHECK(hipHostMalloc((void**)&h_token_ring_, kTokenRing * kRingSlot * sizeof(int64_t), hipHostMallocDefault));
     GPTRS_HIP_CHECK(hipHostMalloc(&h_pinned_, 256, hipHostMallocDefault));
     GPTRS_HIP_CHECK(hipMalloc((void**)&d_chain_bar_, k::kChainBarrierBytes + k::kSkinnyTickets * sizeof(unsigned)));
     k::fill_zero(stream, d_chain_bar_, k::kChainBarrierBytes + k::kSkinnyTickets * sizeof(unsigned));
@@ -104,6 +105,7 @@ Backend::~Backend() {
     (void)hipFree(d_argmax_val_);
     (void)hipFree(d_argmax_idx_);
     token_buf_.reset();
+    rows_buf_.reset();
     for (hipEvent_t e : token_events_)
         if (e) (void)hipEventDestroy(e);
     if (h_token_ring_) (void)hipHostFree(h_token_ring_);
@@ -320,10 +322,53 @@ int64_t Backend::sample_begin(const gptrs_hip_tensor* logits, float temperature,
     const int64_t ticket = next_ticket_++;
     const int slot = (int)(ticket % kTokenRing);
     if (!token_events_[slot]) GPTRS_HIP_CHECK(hipEventCreateWithFlags(&token_events_[slot], hipEventDisableTiming));
-    GPTRS_HIP_CHECK(hipMemcpyAsync(h_token_ring_ + 2 * slot, d_token_, sizeof(int64_t), hipMemcpyDeviceToHost, stream));
-    GPTRS_HIP_CHECK(hipMemcpyAsync(h_token_ring_ + 2 * slot + 1, d_err_flag_, 2 * sizeof(int), hipMemcpyDeviceToHost, stream));
+    ring_rows_[slot] = 0;
+    GPTRS_HIP_CHECK(hipMemcpyAsync(h_token_ring_ + kRingSlot * slot, d_token_, sizeof(int64_t), hipMemcpyDeviceToHost, stream));
+    GPTRS_HIP_CHECK(hipMemcpyAsync(h_token_ring_ + kRingSlot * slot + 1, d_err_flag_, 2 * sizeof(int), hipMemcpyDeviceToHost, stream));
     GPTRS_HIP_CHECK(hipEventRecord(token_events_[slot], stream));
     return ticket;
+}
+
+int64_t Backend::sample_rows_begin(const gptrs_hip_tensor* logits) {
+    GPTRS_HIP_CHECK(hipSetDevice(device));
+    if (logits->consumed) fail_exec("tensor handle was donated to run_program and can no longer be read");
+    const Spec& s = logits->spec;
+    if (!dtype_is_float(s.dtype) || s.rank() != 2 || s.count() == 0 || s.dims[0] > kMaxTokenRows)
+        fail_exec("sample_decode_rows expects non-empty f32/bf16 logits [rows <= 64, vocab]");
+    k::argmax_rows(stream, (int)s.dtype, logits->data(), s.dims[0], s.dims[1], (int32_t*)rows_buf_->ptr, d_argmax_val_, d_argmax_idx_, 1024);
+    n_launches += 2;
+    const int64_t ticket = next_ticket_++;
+    const int slot = (int)(ticket % kTokenRing);
+    if (!token_events_[slot]) GPTRS_HIP_CHECK(hipEventCreateWithFlags(&token_events_[slot], hipEventDisableTiming));
+    ring_rows_[slot] = (int)s.dims[0];
+    GPTRS_HIP_CHECK(hipMemcpyAsync(h_token_ring_ + kRingSlot * slot + 2, rows_buf_->ptr, (size_t)s.dims[0] * sizeof(int32_t),
+                                   hipMemcpyDeviceToHost, stream));
+    GPTRS_HIP_CHECK(hipMemcpyAsync(h_token_ring_ + kRingSlot * slot + 1, d_err_flag_, 2 * sizeof(int), hipMemcpyDeviceToHost, stream));
+    GPTRS_HIP_CHECK(hipEventRecord(token_events_[slot], stream));
+    return ticket;
+}
+
+void Backend::sample_rows_wait(int64_t ticket, int32_t* tokens_out, size_t n) {
+    if (ticket < 0 || ticket >= next_ticket_ || ticket + kTokenRing <= next_ticket_)
+        fail_exec("sample_decode_rows_wait: unknown or expired ticket");
+    GPTRS_HIP_CHECK(hipSetDevice(device));
+    const int slot = (int)(ticket % kTokenRing);
+    if (ring_rows_[slot] == 0 || (size_t)ring_rows_[slot] != n) fail_exec("sample_decode_rows_wait: the ticket holds a different number of rows");
+    GPTRS_HIP_CHECK(hipEventSynchronize(token_events_[slot]));
+    if (h_token_ring_[kRingSlot * slot + 1] != 0) {
+        GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
+        check_device_errors();
+    }
+    memcpy(tokens_out, h_token_ring_ + kRingSlot * slot + 2, n * sizeof(int32_t));
+}
+
+gptrs_hip_tensor* Backend::rows_tensor(int64_t rows) {
+    if (rows < 1 || rows > kMaxTokenRows) fail_exec("decode_rows_tensor: 1 to 64 rows");
+    auto* t = new gptrs_hip_tensor();
+    t->spec.dtype = DType::SI32;
+    t->spec.dims = {rows};
+    t->buf = rows_buf_;
+    return t;
 }
 
 int64_t Backend::sample_wait(int64_t ticket) {
@@ -331,12 +376,13 @@ int64_t Backend::sample_wait(int64_t ticket) {
         fail_exec("sample_decode_token_wait: unknown or expired ticket");
     GPTRS_HIP_CHECK(hipSetDevice(device));
     const int slot = (int)(ticket % kTokenRing);
+    if (ring_rows_[slot] != 0) fail_exec("sample_decode_token_wait: the ticket belongs to sample_decode_rows_begin");
     GPTRS_HIP_CHECK(hipEventSynchronize(token_events_[slot]));
-    if (h_token_ring_[2 * slot + 1] != 0) {   // a device-side error flag was up when the token was sampled
+    if (h_token_ring_[kRingSlot * slot + 1] != 0) {   // a device-side error flag was up when the token was sampled
         GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
         check_device_errors();
     }
-    return h_token_ring_[2 * slot];
+    return h_token_ring_[kRingSlot * slot];
 }
 
 gptrs_hip_tensor* Backend::token_tensor() {
@@ -794,6 +840,30 @@ int gptrs_hip_sample_decode_token_wait(gptrs_hip_backend* b, int64_t ticket, int
         if (!b || !token_out) gptrs::fail_exec("null argument");
         std::lock_guard<std::mutex> g(b->impl.mu);
         *token_out = b->impl.sample_wait(ticket);
+    });
+}
+
+int gptrs_hip_sample_decode_rows_begin(gptrs_hip_backend* b, const gptrs_hip_tensor* logits, int64_t* ticket_out) {
+    return guarded([&] {
+        if (!b || !logits || !ticket_out) gptrs::fail_exec("null argument");
+        std::lock_guard<std::mutex> g(b->impl.mu);
+        *ticket_out = b->impl.sample_rows_begin(logits);
+    });
+}
+
+int gptrs_hip_sample_decode_rows_wait(gptrs_hip_backend* b, int64_t ticket, int32_t* tokens_out, size_t n) {
+    return guarded([&] {
+        if (!b || !tokens_out) gptrs::fail_exec("null argument");
+        std::lock_guard<std::mutex> g(b->impl.mu);
+        b->impl.sample_rows_wait(ticket, tokens_out, n);
+    });
+}
+
+int gptrs_hip_decode_rows_tensor(gptrs_hip_backend* b, int64_t rows, gptrs_hip_tensor** out) {
+    return guarded([&] {
+        if (!b || !out) gptrs::fail_exec("null argument");
+        std::lock_guard<std::mutex> g(b->impl.mu);
+        *out = b->impl.rows_tensor(rows);
     });
 }
 

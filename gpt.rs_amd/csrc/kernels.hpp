@@ -59,6 +59,9 @@ struct DotDesc {
 void dot_generic(hipStream_t s, int dtype, const void* a, const void* b, void* c, const DotDesc& d);
 
 // last row of [rows][vocab] logits; ties -> smallest index; result (int64) written to *out
+// greedy token of every row (rows * partial blocks <= scratch_cap), ties to the smallest index; out: si32[rows]
+void argmax_rows(hipStream_t s, int dtype, const void* logits, int64_t rows, int64_t vocab, int32_t* out, float* scratch_val,
+                 int32_t* scratch_idx, int scratch_cap);
 void argmax_last_row(hipStream_t s, int dtype, const void* logits, int64_t rows, int64_t vocab, int64_t* out,
                      float* scratch_val, int32_t* scratch_idx, int scratch_cap);
 // temperature sampling with a caller-supplied uniform u (inverse-CDF over softmax(logits/T))

@@ -416,6 +416,59 @@ void argmax_last_row(hipStream_t s, int dtype, const void* logits, int64_t rows,
     argmax_stage2<<<1, 64, 0, s>>>(scratch_val, scratch_idx, nb, out);
 }
 
+// Greedy token of EVERY row (batched decode): the same two stages with the row in blockIdx.y; out[r] as si32.
+template <typename T>
+__global__ void argmax_rows_stage1(const T* __restrict__ logits, int64_t n, float* pv, int32_t* pi) {
+    __shared__ float sv[4];
+    __shared__ int32_t si[4];
+    const T* row = logits + (int64_t)blockIdx.y * n;
+    float best = -INFINITY;
+    int32_t bidx = 0x7fffffff;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        const float v = ldf(row, i);
+        if (v > best || (v == best && (int32_t)i < bidx)) { best = v; bidx = (int32_t)i; }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_down(best, off, 64);
+        const int32_t oi = __shfl_down(bidx, off, 64);
+        if (ov > best || (ov == best && oi < bidx)) { best = ov; bidx = oi; }
+    }
+    if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = best; si[threadIdx.x >> 6] = bidx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; ++w)
+            if (sv[w] > best || (sv[w] == best && si[w] < bidx)) { best = sv[w]; bidx = si[w]; }
+        pv[blockIdx.y * gridDim.x + blockIdx.x] = best;
+        pi[blockIdx.y * gridDim.x + blockIdx.x] = bidx;
+    }
+}
+__global__ void argmax_rows_stage2(const float* pv, const int32_t* pi, int nparts, int32_t* out) {
+    float best = -INFINITY;
+    int32_t bidx = 0x7fffffff;
+    for (int i = threadIdx.x; i < nparts; i += 64) {
+        const float v = pv[blockIdx.x * nparts + i];
+        const int32_t id = pi[blockIdx.x * nparts + i];
+        if (v > best || (v == best && id < bidx)) { best = v; bidx = id; }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_down(best, off, 64);
+        const int32_t oi = __shfl_down(bidx, off, 64);
+        if (ov > best || (ov == best && oi < bidx)) { best = ov; bidx = oi; }
+    }
+    if (threadIdx.x == 0) out[blockIdx.x] = bidx == 0x7fffffff ? 0 : bidx;
+}
+void argmax_rows(hipStream_t s, int dtype, const void* logits, int64_t rows, int64_t vocab, int32_t* out, float* scratch_val,
+                 int32_t* scratch_idx, int scratch_cap) {
+    if (rows <= 0) return;
+    int nb = (int)cdiv(vocab, 256 * 8);
+    if (nb > scratch_cap / (int)rows) nb = scratch_cap / (int)rows;
+    if (nb < 1) nb = 1;
+    const dim3 grid((unsigned)nb, (unsigned)rows);
+    if (dtype == 0) argmax_rows_stage1<float><<<grid, 256, 0, s>>>((const float*)logits, vocab, scratch_val, scratch_idx);
+    else argmax_rows_stage1<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)logits, vocab, scratch_val, scratch_idx);
+    argmax_rows_stage2<<<(unsigned)rows, 64, 0, s>>>(scratch_val, scratch_idx, nb, out);
+}
+
 // Temperature sampling, single block: softmax(logits/T) then inverse CDF at u.  The running
 // sum is taken in index order by one wave so the chosen token does not depend on launch shape.
 // Temperature sampling as the reference's device path does it

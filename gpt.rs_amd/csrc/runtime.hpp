@@ -166,6 +166,12 @@ class Backend {
     int64_t sample_begin(const gptrs_hip_tensor* logits, float temperature, bool has_top_k, bool has_u, float u);
     int64_t sample_wait(int64_t ticket);
     gptrs_hip_tensor* token_tensor();
+    // the same for a batch: the greedy token of EVERY row of logits [rows <= kMaxTokenRows, vocab]; the tokens stay on
+    // the device in rows_tensor(rows) (si32[rows]) and travel to the host through the same ring
+    static constexpr int kMaxTokenRows = 64;
+    int64_t sample_rows_begin(const gptrs_hip_tensor* logits);
+    void sample_rows_wait(int64_t ticket, int32_t* tokens_out, size_t n);
+    gptrs_hip_tensor* rows_tensor(int64_t rows);
     void synchronize();
     void check_device_errors();
 
@@ -226,7 +232,10 @@ class Backend {
     int32_t* d_argmax_idx_ = nullptr;
     int64_t* d_token_ = nullptr;       // = token_buf_->ptr: the sampled token as int64, little endian
     BufferP token_buf_;
-    int64_t* h_token_ring_ = nullptr;  // pinned: kTokenRing x {token, error flags}
+    int64_t* h_token_ring_ = nullptr;  // pinned: kTokenRing x kRingSlot int64: {token, error flags, kMaxTokenRows si32 tokens}
+    static constexpr int kRingSlot = 2 + kMaxTokenRows / 2;
+    BufferP rows_buf_;                 // si32[kMaxTokenRows]: the tokens of the last sample_rows_begin
+    int ring_rows_[kTokenRing] = {};   // rows behind each ticket (0: a single-token ticket)
     hipEvent_t token_events_[kTokenRing] = {};
     int64_t next_ticket_ = 0;
     bool queue_sampling(const gptrs_hip_tensor* logits, float temperature, bool has_top_k, bool has_u, float u);

@@ -411,8 +411,8 @@ class Gpt(_ModelBase):
                 for t in row:
                     if not 0 <= t < cfg.vocab_size:
                         raise ValueError(f"token index {t} out of range")
-        elif batch != 1 or seq != 1:
-            raise ValueError("a device token feeds one sequence, one step")
+        elif seq != 1:
+            raise ValueError("device tokens feed one step (one token per sequence)")
         if any(len(c) != cfg.num_layers for c in caches):
             raise ValueError(f"expected {cfg.num_layers} cache slots (one per layer)")
         if fixed_capacity is not None:
@@ -723,8 +723,8 @@ class Ministral(_ModelBase):
     def forward_batch(self, token_rows, position_offset, caches, fixed_capacity=None, token_handle=None, last_logits_only=False):
         cfg = self.config
         batch, seq = len(token_rows), len(token_rows[0])
-        if token_handle is not None and (batch != 1 or seq != 1):
-            raise ValueError("a device token feeds one sequence, one step")
+        if token_handle is not None and seq != 1:
+            raise ValueError("device tokens feed one step (one token per sequence)")
         if seq == 0:
             raise ValueError("token sequence must contain at least one element")
         if any(len(r) != seq for r in token_rows):
@@ -766,6 +766,56 @@ class Ministral(_ModelBase):
                 k, v = next(it), next(it)
                 caches[b][i] = DecodeKvCache(k, v, total, capacity)
         return outs[-1]
+
+
+# ================================================================================ BatchGenerator
+class BatchGenerator:
+    """Greedy generation for several independent sequences of equal prompt length at once (the reference decodes one
+    sequence per model call; its batch is a host-side loop): rows stacked through `forward_batch`, one attention launch
+    per layer for all of them.  On a backend with sample_decode_rows_begin / _wait the loop is pipelined like
+    `Generator`: the tokens of step t stay on the device as the input of step t + 1, which is queued before the host
+    has seen them; elsewhere the rows are arg-maxed on the host (sampler.rs:96-103, last maximum... first index wins
+    here as on the device).  The context window does not slide: generation stops at the context length."""
+
+    def __init__(self, model, prompts: Sequence[Sequence[int]], kv_cache_capacity: Optional[int] = None):
+        if len(prompts) == 0 or len(prompts[0]) == 0:
+            raise ValueError("prompts must be non-empty")
+        if any(len(p) != len(prompts[0]) for p in prompts):
+            raise ValueError("all prompts of a batch must have equal length")
+        self.model = model
+        self.batch = len(prompts)
+        self.tokens = [list(p) for p in prompts]
+        self.capacity = kv_cache_capacity
+        self.caches = [[None] * model.num_layers for _ in prompts]
+        self.pipelined = hasattr(model.backend, "sample_decode_rows_begin")
+        self.logits = model.forward_batch(self.tokens, 0, self.caches, self.capacity, last_logits_only=True)
+        self.processed_len = len(prompts[0])
+
+    def step(self) -> List[int]:
+        """Samples one token per sequence and runs the forward that consumes them."""
+        be, B = self.model.backend, self.batch
+        if self.processed_len >= self.model.context_length:
+            raise ValueError("context length reached")
+        if self.pipelined:
+            ticket = be.sample_decode_rows_begin(self.logits)
+            self.logits = self.model.forward_batch([[None]] * B, self.processed_len, self.caches, self.capacity,
+                                                   token_handle=be.decode_rows_tensor(B))
+            nxt = be.sample_decode_rows_wait(ticket, B)
+        else:
+            rows = be.to_numpy(self.logits)
+            nxt = [int(np.argmax(rows[b])) for b in range(B)]
+            self.logits = self.model.forward_batch([[t] for t in nxt], self.processed_len, self.caches, self.capacity)
+        self.processed_len += 1
+        for b in range(B):
+            self.tokens[b].append(nxt[b])
+        return nxt
+
+    def generate(self, max_new_tokens: int) -> List[List[int]]:
+        out = [[] for _ in range(self.batch)]
+        for _ in range(max_new_tokens):
+            for b, t in enumerate(self.step()):
+                out[b].append(t)
+        return out
 
 
 # ================================================================================ Generator

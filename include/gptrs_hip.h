@@ -137,6 +137,16 @@ int gptrs_hip_sample_decode_token_begin(gptrs_hip_backend* b, const gptrs_hip_te
 int gptrs_hip_sample_decode_token_wait(gptrs_hip_backend* b, int64_t ticket, int64_t* token_out);
 int gptrs_hip_decode_token_tensor(gptrs_hip_backend* b, gptrs_hip_tensor** out);
 
+/* The pipelined halves for a BATCH of independent sequences decoded together (the reference has no batch dimension,
+ * crates/gpt-rs/src/ops/functional/attention.rs:189-203, so this has no counterpart there either): _rows_begin queues
+ * the greedy token (largest logit, smallest index on ties, docs/backend.md:270) of EVERY row of logits [rows <= 64,
+ * vocab] and returns a ticket; the tokens stay on the device in the si32[rows] tensor of gptrs_hip_decode_rows_tensor,
+ * which the next step's program takes as its token-id input; _rows_wait copies the ticket's tokens out (n must equal
+ * the rows the ticket was drawn for).  Tickets share the ring of sample_decode_token_begin. */
+int gptrs_hip_sample_decode_rows_begin(gptrs_hip_backend* b, const gptrs_hip_tensor* logits, int64_t* ticket_out);
+int gptrs_hip_sample_decode_rows_wait(gptrs_hip_backend* b, int64_t ticket, int32_t* tokens_out, size_t n);
+int gptrs_hip_decode_rows_tensor(gptrs_hip_backend* b, int64_t rows, gptrs_hip_tensor** out);
+
 /* Message of the calling thread's most recent non-zero return (BackendError Display). */
 const char* gptrs_hip_last_error(void);
 

@@ -283,6 +283,51 @@ def test_batched_decode_matches_single_sequences(hip):
     assert toks == singles
 
 
+@pytest.mark.parametrize("cls,cfg,dtype", [(models.Gpt, TINY_GPT, "F32"), (models.Ministral, MID_MINISTRAL, "F32"),
+                                           (models.Ministral, MID_MINISTRAL, "Bf16")], ids=["gpt-f32", "ministral-f32", "ministral-bf16"])
+def test_batch_generator_pipelined_rows(hip, cls, cfg, dtype):
+    """BatchGenerator: the greedy tokens of all rows are taken on the device (sample_decode_rows_begin / _wait) and fed
+    to the next step from the device tensor.  f32: the same tokens as each sequence generated alone and as the
+    host-argmax loop over the same batch; bf16: the same tokens as the host-argmax loop (same programs, same logits)."""
+    m = cls.random(cfg, hip, seed=51, dtype=dtype, std=0.2)
+    prompts = [[1, 2, 3, 4], [9, 8, 7, 6], [5, 5, 5, 5], [11, 3, 30, 2], [6, 1, 6, 1]]
+    gen = models.BatchGenerator(m, prompts, kv_cache_capacity=16)
+    assert gen.pipelined
+    got = gen.generate(7)
+    host = models.BatchGenerator(m, prompts, kv_cache_capacity=16)
+    host.pipelined = False
+    assert host.generate(7) == got
+    if dtype == "F32":
+        for p, g in zip(prompts, got):
+            assert models.Generator(m, p, kv_cache_capacity=16).generate(7) == g
+    assert [t[len(prompts[0]):] for t in gen.tokens] == got
+
+
+def test_sample_rows_api(hip):
+    from parity import TensorSpec
+    from gptrs_amd.backend import BackendError
+    from gptrs_amd.ptir import f32_to_bf16_bits
+    rng = np.random.default_rng(3)
+    x = rng.normal(0, 2, (7, 50257)).astype(np.float32)
+    x[2, 100] = x[2, 40000] = 50.0                                   # a tie: the smaller index wins
+    for dtype, data in (("F32", x.tobytes()), ("Bf16", f32_to_bf16_bits(x).tobytes())):
+        h = hip.materialize(TensorSpec(dtype, [7, 50257]), data)
+        ref = x if dtype == "F32" else (f32_to_bf16_bits(x).astype(np.uint32) << 16).view(np.float32)
+        t = hip.sample_decode_rows_begin(h)
+        dev = hip.decode_rows_tensor(7)
+        want = [int(np.argmax(ref[r])) for r in range(7)]
+        assert want[2] == 100
+        assert hip.to_numpy(dev).tolist() == want
+        assert hip.sample_decode_rows_wait(t, 7) == want
+        with pytest.raises(BackendError):
+            hip.sample_decode_rows_wait(t, 5)                         # the ticket holds 7 rows
+        with pytest.raises(BackendError):
+            hip.sample_decode_token_wait(t)                           # and is not a single-token ticket
+    big = hip.materialize(TensorSpec("F32", [65, 8]), None)
+    with pytest.raises(BackendError):
+        hip.sample_decode_rows_begin(big)
+
+
 WIDE_HEAD_MINISTRAL = models.MinistralConfig(vocab_size=512, context_length=128, embed_dim=256, num_layers=2, num_heads=8,
                                              num_kv_heads=2, head_dim=64, ffn_dim=512, rotary_dim=64, rope_theta=1e6)
 
