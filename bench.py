@@ -320,7 +320,7 @@ def main():
     roof = None
     if prof_steps > 0:
         prof_start = gen.processed_len
-        chains0 = be.counter("chain_launches")
+        chains0, phases0 = be.counter("chain_launches"), be.counter("chain_phases")
         be.set_option("profile", 1)
         for _ in range(prof_steps):
             gen.step()
@@ -335,7 +335,7 @@ def main():
                 # the step's algorithmic bytes (weights once, valid KV once, logits once)
                 nbytes = sum(algorithmic_bytes_per_step(cfg, 2, prof_start + i, args.quant) for i in range(prof_steps))
                 kernel = "chain_kernel: persistent decode chain, %d phases per launch (all linear layers + decode attention of a step)" % (
-                    be.counter("chain_phases") // max(be.counter("chain_launches"), 1))
+                    (be.counter("chain_phases") - phases0) // max(chains, 1))
             else:
                 kernel = "gemv_tiled_kernel<bf16>: all linear layers of a decode step"
             achieved = nbytes / (t_ns * 1e-9) / 1e9
