@@ -30,6 +30,7 @@ sys.path.insert(0, ROOT)
 import __graft_entry__ as entry  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 # HBM bytes moved by one chain_kernel launch of the default workload (26 layers, prompt 1024, cache
 # length ~1040), from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a copy kernel of known size; the
 # commands and raw figures are in profiles/chain_kernel_ministral3b_bf16_b1_decode.md
@@ -117,6 +118,79 @@ def cpu_baseline(cfg, seconds_budget: float = 25.0):
             "sample": f"{reps} reps of one layer's {nl} f32 GEMVs + 1/8 of lm_head through {name} "
                       f"(gpt_rs_c_matmul_f32_cached_b, m=1, packed-B cache warm); token time = {cfg.num_layers} layers + "
                       f"8 head slices; non-GEMV ops excluded"}
+
+
+def microbench(args, be):
+    """BASELINE configs[1]: single-op PTIR programs, f32 and bf16: dot_general [M,K]x[K,N] for M in {1, 8, 64, 512} and
+    (K,N) in {(768,2304), (768,3072), (3072,768)}, softmax and layer_norm on [M,768]; plus the prefill GEMM shapes of
+    the Ministral-3B layer at M = 1024 (bf16, SwiGLU pair as one dual GEMM).  Inputs N(0,1) from seed 2 (weights scaled
+    by 1/sqrt(K)), resident on the device; each program runs `--steps` times after `--warmup`, wall clock with a device
+    sync at both ends (cached plan, graph replay where the plan has enough steps)."""
+    from gptrs_amd import functional as F
+    from gptrs_amd.ptir import FunctionBuilder, Program, TensorSpec, f32_to_bf16_bits
+    rng = np.random.default_rng(2)
+    steps, warmup = (50, 5) if args.steps == 224 else (args.steps, max(args.warmup, 1))
+
+    def upload(arr, dtype):
+        data = arr.astype(np.float32).tobytes() if dtype == "F32" else f32_to_bf16_bits(arr.astype(np.float32)).tobytes()
+        return be.materialize(TensorSpec(dtype, list(arr.shape)), data)
+
+    def timed(prog, handles):
+        for _ in range(warmup):
+            be.run_program(prog, handles)
+        be.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            be.run_program(prog, handles)
+        be.synchronize()
+        return (time.perf_counter() - t0) / steps
+
+    results = []
+    for dtype, es in (("F32", 4), ("Bf16", 2)):
+        for k, n in ((768, 2304), (768, 3072), (3072, 768)):
+            w = upload(rng.standard_normal((k, n), dtype=np.float32) / np.float32(np.sqrt(k)), dtype)
+            for m in (1, 8, 64, 512):
+                fb = FunctionBuilder("main", dtype)
+                x, wp = fb.param(dtype, [m, k]), fb.param(dtype, [k, n])
+                fb.set_results([x.matmul(wp)])
+                dt = timed(Program(fb), [upload(rng.standard_normal((m, k), dtype=np.float32), dtype), w])
+                nbytes, flops = (m * k + k * n + m * n) * es, 2.0 * m * k * n
+                results.append({"op": "dot_general", "dtype": dtype, "m": m, "k": k, "n": n, "us": round(dt * 1e6, 2),
+                                "gb_per_s": round(nbytes / dt / 1e9, 1), "tflop_per_s": round(flops / dt / 1e12, 3)})
+        for m in (1, 8, 64, 512):
+            for op in ("softmax", "layer_norm"):
+                fb = FunctionBuilder("main", dtype)
+                x = fb.param(dtype, [m, 768])
+                hs = [upload(rng.standard_normal((m, 768), dtype=np.float32), dtype)]
+                if op == "softmax":
+                    fb.set_results([F.softmax_last_axis(x)])
+                    nbytes = 2 * m * 768 * es
+                else:
+                    g, b = fb.param(dtype, [768]), fb.param(dtype, [768])
+                    hs += [upload(rng.standard_normal(768, dtype=np.float32), dtype), upload(rng.standard_normal(768, dtype=np.float32), dtype)]
+                    fb.set_results([F.layer_norm(x, g, b, 1e-5)[0]])
+                    nbytes = (2 * m * 768 + 2 * 768) * es
+                dt = timed(Program(fb), hs)
+                results.append({"op": op, "dtype": dtype, "m": m, "n": 768, "us": round(dt * 1e6, 2), "gb_per_s": round(nbytes / dt / 1e9, 1)})
+    m = 1024
+    for k, n, dual in ((3072, 6144, False), (4096, 3072, False), (3072, 9216, True), (9216, 3072, False)):
+        fb = FunctionBuilder("main", "Bf16")
+        x, wp = fb.param("Bf16", [m, k]), fb.param("Bf16", [k, n])
+        hs = [upload(rng.standard_normal((m, k), dtype=np.float32), "Bf16"),
+              upload(rng.standard_normal((k, n), dtype=np.float32) / np.float32(np.sqrt(k)), "Bf16")]
+        if dual:
+            w2 = fb.param("Bf16", [k, n])
+            hs.append(upload(rng.standard_normal((k, n), dtype=np.float32) / np.float32(np.sqrt(k)), "Bf16"))
+            fb.set_results([F.swiglu(x.matmul(wp), x.matmul(w2))])
+        else:
+            fb.set_results([x.matmul(wp)])
+        dt = timed(Program(fb), hs)
+        flops = 2.0 * m * k * n * (2 if dual else 1)
+        results.append({"op": "prefill_gemm" + ("_swiglu_pair" if dual else ""), "dtype": "Bf16", "m": m, "k": k, "n": n, "us": round(dt * 1e6, 2),
+                        "tflop_per_s": round(flops / dt / 1e12, 1), "mfma_frac": round(flops / dt / 1e12 / MFMA_PEAK_TFLOPS, 4)})
+    print(json.dumps({"metric": "single-op microbench (BASELINE configs[1]) + Ministral prefill GEMM shapes", "unit": "us per program run",
+                      "n_gpus": 1, "steps": steps, "warmup": warmup, "data": "synthetic", "peaks": {"hbm_gb_per_s": HBM_PEAK_GBPS,
+                      "bf16_mfma_tflop_per_s": MFMA_PEAK_TFLOPS}, "results": results}))
 
 
 README_GPT2_TOKENS_PER_S = 74.71   # reference README.md:18-25: GPT-2 small f32, generate 64 tokens, C backend, 1 thread of a Ryzen 9 9950X3D
@@ -251,6 +325,9 @@ def main():
     ap.add_argument("--model", choices=["ministral", "gpt2"], default="ministral",
                     help="gpt2: the reference's own published workload (GPT-2 small f32, generate 64 tokens); --steps then counts "
                          "whole generate calls (default 8)")
+    ap.add_argument("--microbench", action="store_true",
+                    help="single-op programs of BASELINE configs[1] (dot_general / softmax / layer_norm, f32 and bf16) and the "
+                         "Ministral prefill GEMM shapes; prints one JSON line with a result per shape")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain elementwise kernel of known traffic (x + 0 over 2^28 f32: 1 GiB read, 1 GiB written, "
@@ -278,6 +355,8 @@ def main():
         be.synchronize()
         print(json.dumps({"copy_calibration": "10 launches of x + 0.0 over %d f32" % n, "bytes_read_per_launch": 4 * n, "bytes_written_per_launch": 4 * n}))
         return
+    if args.microbench:
+        return microbench(args, be)
     if args.model == "gpt2":
         if args.steps == 224:
             args.steps, args.warmup = 8, 2
