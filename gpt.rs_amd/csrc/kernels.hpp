@@ -218,6 +218,7 @@ bool chain_launch(hipStream_t s, const ChainPhase* dev_table, int nphases, int l
 // Prefill GEMM (M > 16, bf16) on the matrix cores over a k-grouped copy of the weights,
 // Wk8[K/8][Npad][8] (kernels_mfma.hip).  wk2 != nullptr: SwiGLU pair.
 struct MfmaLinearArgs {
+    int dtype;   // 0 f32, 2 bf16
     const void* x; const void* wk; const void* wk2; const void* bias; const void* residual;
     void* y;
     int64_t m, k, n;

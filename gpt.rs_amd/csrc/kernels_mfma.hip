@@ -1,11 +1,12 @@
-// MFMA tile GEMM for prefill-sized linear layers (M > 16), bf16 in / f32 accumulate / bf16 out.
+// MFMA tile GEMM for prefill-sized linear layers (M > 16): bf16 in / f32 accumulate / bf16 out on
+// v_mfma_f32_32x32x16_bf16, and f32 throughout on v_mfma_f32_32x32x2_f32.
 //
-// v_mfma_f32_32x32x16_bf16 wants, per lane, 8 consecutive k of ONE row (A) or ONE column (B).
-// Activations x[M,K] are row-major, so A fragments are plain 16-byte loads.  Weights are stored
-// [in,out] row-major (nn/layers/linear.rs:50-71), the wrong way round for B, so the GEMM reads a
-// derived copy Wk8[K/8][Npad][8] (8 consecutive k of a column are adjacent; Npad = N rounded up to
-// the 128-column block tile, zero filled) that the backend builds once per weight and keeps beside
-// the original.  With it a block's B tile is, per group of 8 k, one contiguous 2 KiB run.
+// Per lane the matrix cores want consecutive k of ONE row (A) or ONE column (B).  Activations x[M,K] are row-major,
+// so A fragments are plain 16-byte loads.  Weights are stored [in,out] row-major (nn/layers/linear.rs:50-71), the
+// wrong way round for B, so the GEMM reads a derived copy Wk[K/KPC][Npad][KPC] in which the KPC consecutive k of a
+// column that fill 16 bytes (8 bf16 or 4 f32) are adjacent (Npad = N rounded up to the 128-column block tile, zero
+// filled); the backend builds it once per weight and keeps it beside the original.  With it a block's B tile is, per
+// 16-byte k-group, one contiguous 2 KiB run, and every data movement below is in 16-byte chunks whatever the type.
 #include "kernels.hpp"
 #include "device_utils.hpp"
 
@@ -13,42 +14,67 @@ namespace gptrs {
 namespace k {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+// Element types of the GEMM: KPC = k per 16-byte chunk; mma() multiplies one 32 x (2 KPC) A fragment by one
+// (2 KPC) x 32 B fragment (a lane holds the KPC values of its row / column in k-group lane / 32).
+template <typename T> struct Mma;
+template <> struct Mma<bf16_t> {
+    static constexpr int KPC = 8;
+    typedef bf16x8_t frag;
+    static __device__ __forceinline__ f32x16_t mma(const frag& a, const frag& b, f32x16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float ld(const bf16_t* p, int64_t i) { return bf16_to_f32(p[i]); }
+    static __device__ __forceinline__ void st(bf16_t* p, int64_t i, float v) { p[i] = f32_to_bf16(v); }
+};
+template <> struct Mma<float> {
+    static constexpr int KPC = 4;
+    typedef f32x4_t frag;
+    // four K = 2 products: element e of both fragments is k = 4 * (lane / 32) + e of the 8-k step
+    static __device__ __forceinline__ f32x16_t mma(const frag& a, const frag& b, f32x16_t c) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], c, 0, 0, 0);
+        return c;
+    }
+    static __device__ __forceinline__ float ld(const float* p, int64_t i) { return p[i]; }
+    static __device__ __forceinline__ void st(float* p, int64_t i, float v) { p[i] = v; }
+};
 
 static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
-constexpr int kBN = 128, kBK = 64;  // kBN: column padding unit of the derived weights
-constexpr int kKb = kBK / 8;                       // groups of 8 k per tile
+constexpr int kBN = 128;   // column padding unit of the derived weights
+constexpr int kKb = 8;     // 16-byte k-groups per k tile: 64 k of bf16, 32 k of f32
 
+static inline int kpc_of(int dtype) { return dtype == 0 ? 4 : 8; }
 int64_t mfma_padded_n(int64_t n) { return cdiv(n, kBN) * kBN; }
 size_t mfma_weight_bytes(int dtype, int64_t k, int64_t n) {
-    (void)dtype;
-    return (size_t)cdiv(k, 8) * (size_t)mfma_padded_n(n) * 8 * sizeof(bf16_t);
+    return (size_t)cdiv(k, kpc_of(dtype)) * (size_t)mfma_padded_n(n) * 16;
 }
 
-// Wk8[kb][n][i] = W[kb*8+i][n]; one thread per (kb, n); reads coalesced along n, one 16-byte store.
-__global__ __launch_bounds__(256) void k8_weights_kernel(const bf16_t* __restrict__ w, bf16_t* __restrict__ out, int64_t K,
-                                                         int64_t N, int64_t Npad) {
+// Wk[kb][n][i] = W[kb*KPC+i][n]; one thread per (kb, n); reads coalesced along n, one 16-byte store.
+template <typename T>
+__global__ __launch_bounds__(256) void k8_weights_kernel(const T* __restrict__ w, T* __restrict__ out, int64_t K, int64_t N,
+                                                         int64_t Npad) {
+    constexpr int KPC = Mma<T>::KPC;
     const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int64_t kb = blockIdx.y;
     if (n >= Npad) return;
-    uint32_t r[4] = {0, 0, 0, 0};
-    if (n < N) {
+    alignas(16) T r[KPC];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int64_t kx = kb * 8 + i;
-            const uint32_t v = kx < K ? (uint32_t)w[kx * N + n] : 0u;
-            r[i >> 1] |= v << ((i & 1) * 16);
-        }
+    for (int i = 0; i < KPC; ++i) {
+        const int64_t kx = kb * KPC + i;
+        r[i] = (n < N && kx < K) ? w[kx * N + n] : T(0);
     }
-    *reinterpret_cast<uint4*>(out + (kb * Npad + n) * 8) = make_uint4(r[0], r[1], r[2], r[3]);
+    *reinterpret_cast<uint4*>(out + (kb * Npad + n) * KPC) = *reinterpret_cast<const uint4*>(r);
 }
 
 void mfma_pack_weights(hipStream_t s, int dtype, const void* w, void* out, int64_t k, int64_t n) {
-    (void)dtype;
     const int64_t npad = mfma_padded_n(n);
-    dim3 grid((unsigned)cdiv(npad, 256), (unsigned)cdiv(k, 8));
-    k8_weights_kernel<<<grid, 256, 0, s>>>((const bf16_t*)w, (bf16_t*)out, k, n, npad);
+    dim3 grid((unsigned)cdiv(npad, 256), (unsigned)cdiv(k, kpc_of(dtype)));
+    if (dtype == 0) k8_weights_kernel<float><<<grid, 256, 0, s>>>((const float*)w, (float*)out, k, n, npad);
+    else k8_weights_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)w, (bf16_t*)out, k, n, npad);
 }
 
 __device__ __forceinline__ float mfma_finish(float v, float v2, bool dual, int act, float bias, bool has_res, float res) {
@@ -71,18 +97,21 @@ __device__ __forceinline__ float mfma_finish(float v, float v2, bool dual, int a
 // instead): with HIP's uint4 struct and a guarded load the compiler keeps the staging array in
 // scratch memory and waits for every load at once, which cost a factor of four.
 //
-// Requires K % 64 == 0; M and N are guarded (rows clamp on load, stores are masked; the derived
+// Requires K % (8 KPC) == 0 (64 for bf16, 32 for f32); M and N are guarded (rows clamp on load, stores are masked; the derived
 // weights are padded to whole 128-column tiles).
 // DUAL: SwiGLU pair silu(x.W) * (x.W2).  The block covers BN/2 real columns; the B tile holds, per
 // wave column, TN/2 fragments of W followed by the same columns of W2, so gate and up of one
 // output meet in the same lane.
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
-template <int BM, int BN, bool DUAL>
-__global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wk,
-                                                             const bf16_t* __restrict__ wk2, const bf16_t* __restrict__ bias,
-                                                             const bf16_t* __restrict__ residual, bf16_t* __restrict__ y,
-                                                             int M, int K, int N, int Npad, int act, int NT, int MT) {
+template <typename T, int BM, int BN, bool DUAL>
+__global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ x, const T* __restrict__ wk,
+                                                        const T* __restrict__ wk2, const T* __restrict__ bias,
+                                                        const T* __restrict__ residual, T* __restrict__ y,
+                                                        int M, int K, int N, int Npad, int act, int NT, int MT) {
+    constexpr int KPC = Mma<T>::KPC;
+    constexpr int kBK = kKb * KPC;                            // k per tile
+    typedef typename Mma<T>::frag frag_t;
     constexpr int SA = (BM + 1) * 16, SB = (BN + 1) * 16;     // bytes between k-groups
     constexpr int STAGE = kKb * (SA + SB);
     constexpr int TM = BM / 64, TN = BN / 64;
@@ -114,8 +143,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __res
     // global -> LDS chunk assignment (16 bytes each)
     // A: chunk c -> kb = c % 8, row = c / 8: eight lanes read 128 contiguous bytes of one row
     // B: chunk c -> tile column = c % BN, kb = c / BN: contiguous runs of the k-grouped weights
-    const bf16_t* a_src[CA];
-    const bf16_t* b_src[CB];
+    const T* a_src[CA];
+    const T* b_src[CB];
     int a_dst[CA], b_dst[CB];
 #pragma unroll
     for (int j = 0; j < CA; ++j) {
@@ -123,7 +152,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __res
         const int kb = c & 7, row = c >> 3;
         int m = m0 + row;
         if (m > M - 1) m = M - 1;
-        a_src[j] = x + (int64_t)m * K + kb * 8;
+        a_src[j] = x + (int64_t)m * K + kb * KPC;
         a_dst[j] = kb * SA + row * 16;
     }
 #pragma unroll
@@ -131,14 +160,14 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __res
         const int c = tid + 256 * j;
         const int bc = c % BN, bkb = c / BN;
         int col = n0 + bc;
-        const bf16_t* src = wk;
+        const T* src = wk;
         if (DUAL) {
             // tile column -> (wave column, gate|up, column inside the half)
             const int wcol = bc / WN, in_w = bc % WN, half = in_w / (WN / 2), cc = in_w % (WN / 2);
             col = n0 + wcol * (WN / 2) + cc;
             src = half ? wk2 : wk;
         }
-        b_src[j] = src + ((int64_t)bkb * Npad + col) * 8;
+        b_src[j] = src + ((int64_t)bkb * Npad + col) * KPC;
         b_dst[j] = kKb * SA + bkb * SB + bc * 16;
     }
 
@@ -152,7 +181,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __res
 
     u32x4_t ra[CA], rb[CB];
     const int nt = K / kBK;
-    const int64_t b_tile_step = (int64_t)kKb * Npad * 8;  // elements between consecutive k tiles of Wk8
+    const int64_t b_tile_step = (int64_t)kKb * Npad * KPC;  // elements between consecutive k tiles of Wk
     auto gload = [&](int t) {
 #pragma unroll
         for (int j = 0; j < CA; ++j) ra[j] = *reinterpret_cast<const u32x4_t*>(a_src[j] + (int64_t)t * kBK);
@@ -168,13 +197,13 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __res
     };
     const int a_rd = (wm * (BM / 2) + (lane & 31)) * 16 + (lane >> 5) * SA;
     const int b_rd = kKb * SA + (wn * WN + (lane & 31)) * 16 + (lane >> 5) * SB;
-    bf16x8_t af[2][TM], bfr[2][TN];
+    frag_t af[2][TM], bfr[2][TN];
     auto fread = [&](int buf, int kk, int slot) {
         const unsigned char* base = lds + buf * STAGE;
 #pragma unroll
-        for (int i = 0; i < TM; ++i) af[slot][i] = *reinterpret_cast<const bf16x8_t*>(base + a_rd + kk * 2 * SA + i * 32 * 16);
+        for (int i = 0; i < TM; ++i) af[slot][i] = *reinterpret_cast<const frag_t*>(base + a_rd + kk * 2 * SA + i * 32 * 16);
 #pragma unroll
-        for (int j = 0; j < TN; ++j) bfr[slot][j] = *reinterpret_cast<const bf16x8_t*>(base + b_rd + kk * 2 * SB + j * 32 * 16);
+        for (int j = 0; j < TN; ++j) bfr[slot][j] = *reinterpret_cast<const frag_t*>(base + b_rd + kk * 2 * SB + j * 32 * 16);
     };
 
     gload(0);
@@ -185,8 +214,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __res
         const int cur = t & 1;
         fread(cur, 0, 0);
 #pragma unroll
-        for (int kk = 0; kk < kBK / 16; ++kk) {
-            if (kk + 1 < kBK / 16) fread(cur, kk + 1, (kk + 1) & 1);
+        for (int kk = 0; kk < kKb / 2; ++kk) {
+            if (kk + 1 < kKb / 2) fread(cur, kk + 1, (kk + 1) & 1);
             if (kk == 1) {
                 lwrite(cur ^ 1);  // tile t+1; past the last tile this stores a copy nobody reads
                 gload(t + 2 < nt ? t + 2 : nt - 1);
@@ -195,7 +224,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __res
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], bfr[kk & 1][j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = Mma<T>::mma(af[kk & 1][i], bfr[kk & 1][j], acc[i][j]);
         }
         __syncthreads();
     }
@@ -208,28 +237,30 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const bf16_t* __res
         for (int j = 0; j < TNO; ++j) {
             const int n = n0 + wn * (NREAL / 2) + j * 32 + (lane & 31);
             if (n >= N) continue;
-            const float bv = bias ? bf16_to_f32(bias[n]) : 0.f;
+            const float bv = bias ? Mma<T>::ld(bias, n) : 0.f;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int m = m0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
                 if (m >= M) continue;
-                const float r = residual ? bf16_to_f32(residual[(int64_t)m * N + n]) : 0.f;
+                const float r = residual ? Mma<T>::ld(residual, (int64_t)m * N + n) : 0.f;
                 const float g = acc[i][j][v];
                 const float u = DUAL ? acc[i][DUAL ? j + TN / 2 : j][v] : 0.f;
-                y[(int64_t)m * N + n] = f32_to_bf16(mfma_finish(g, u, DUAL, act, bv, residual != nullptr, r));
+                Mma<T>::st(y, (int64_t)m * N + n, mfma_finish(g, u, DUAL, act, bv, residual != nullptr, r));
             }
         }
 }
 
 bool mfma_gemm_supported(int dtype, int64_t m, int64_t k, int64_t n) {
-    return dtype == 2 && m > 16 && k >= kBK && k % kBK == 0 && n >= 1 && m < (1ll << 31) && n < (1ll << 31) - kBN &&
-           k < (1ll << 31) && cdiv(m, 128) * cdiv(n, 64) < (1ll << 30);   // tile ids are ints
+    if (dtype != 0 && dtype != 2) return false;
+    const int64_t bk = kKb * kpc_of(dtype);
+    return m > 16 && k >= bk && k % bk == 0 && n >= 1 && m < (1ll << 31) && n < (1ll << 31) - kBN && k < (1ll << 31) &&
+           cdiv(m, 128) * cdiv(n, 64) < (1ll << 30);   // tile ids are ints
 }
 
-template <int BM, int BN, bool DUAL>
+template <typename T, int BM, int BN, bool DUAL>
 static void launch_mfma(hipStream_t s, const MfmaLinearArgs& a) {
     constexpr int lds_bytes = 2 * kKb * ((BM + 1) * 16 + (BN + 1) * 16);
-    auto kern = gemm_bf16_mfma_kernel<BM, BN, DUAL>;
+    auto kern = gemm_mfma_kernel<T, BM, BN, DUAL>;
     static bool configured = false;  // the attribute is per function, not per stream or device state
     if (!configured) {
         (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
@@ -239,14 +270,18 @@ static void launch_mfma(hipStream_t s, const MfmaLinearArgs& a) {
     constexpr int nreal = DUAL ? BN / 2 : BN;
     const int64_t nt = cdiv(npad, nreal), mt = cdiv(a.m, BM);
     const unsigned grid = (unsigned)(cdiv(nt * mt, 8) * 8);
-    kern<<<grid, 256, lds_bytes, s>>>((const bf16_t*)a.x, (const bf16_t*)a.wk, (const bf16_t*)a.wk2, (const bf16_t*)a.bias,
-                                      (const bf16_t*)a.residual, (bf16_t*)a.y, (int)a.m, (int)a.k, (int)a.n, (int)npad, a.act,
-                                      (int)nt, (int)mt);
+    kern<<<grid, 256, lds_bytes, s>>>((const T*)a.x, (const T*)a.wk, (const T*)a.wk2, (const T*)a.bias, (const T*)a.residual, (T*)a.y,
+                                      (int)a.m, (int)a.k, (int)a.n, (int)npad, a.act, (int)nt, (int)mt);
 }
 
 void mfma_gemm(hipStream_t s, const MfmaLinearArgs& a) {
-    if (a.wk2) launch_mfma<128, 128, true>(s, a);
-    else launch_mfma<128, 128, false>(s, a);
+    if (a.dtype == 0) {
+        if (a.wk2) launch_mfma<float, 128, 128, true>(s, a);
+        else launch_mfma<float, 128, 128, false>(s, a);
+    } else {
+        if (a.wk2) launch_mfma<bf16_t, 128, 128, true>(s, a);
+        else launch_mfma<bf16_t, 128, 128, false>(s, a);
+    }
 }
 
 }  // namespace k

@@ -1042,6 +1042,7 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
             const Spec& w = in_spec(1);
             if (in.mfma) {
                 k::MfmaLinearArgs ma{};
+                ma.dtype = (int)x.dtype;
                 ma.x = src_ptr(st, cx, 0);
                 ma.m = x.dims[0]; ma.k = x.dims[1]; ma.n = w.dims[1];
                 // quantised weights: the k-grouped copy is built once from the dequantised matrix
