@@ -166,8 +166,8 @@ BufferP Backend::derived_weights(const BufferP& src, int kind, DType dtype, int6
         t = new_buffer(k::chain_scale_bytes(k, n, src2 != nullptr));
         k::chain_pack_scales_w4(stream, (int)dtype, src->ptr, src2 ? src2->ptr : nullptr, t->ptr, k, n);
     } else if (kind == 8) {                             // batched decode: 16-column tiles, k-grouped (kernels_skinny.hip)
-        t = new_buffer(k::skinny_weight_bytes(k, n));
-        k::skinny_pack_weights(stream, src->ptr, t->ptr, k, n);
+        t = new_buffer(k::skinny_weight_bytes((int)dtype, k, n));
+        k::skinny_pack_weights(stream, (int)dtype, src->ptr, t->ptr, k, n);
     } else if (kind == 9 || kind == 10) {               // batched decode: int8 / int4 codes in the 16-column tiled word order
         t = new_buffer(k::skinny_codes_bytes(k, n, kind - 8));
         k::skinny_pack_codes(stream, src->ptr, t->ptr, k, n, kind - 8);

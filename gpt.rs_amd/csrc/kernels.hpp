@@ -113,9 +113,10 @@ void tile_weights(hipStream_t s, int dtype, const void* w, void* wt, int64_t k, 
 bool gemv_tiled_supported(int dtype, int64_t m, int64_t k, int64_t n);
 void gemv_tiled(hipStream_t s, const TiledLinearArgs& a);
 
-// Batched-decode linear layers (2 <= M <= 16, bf16) on the matrix cores over a 16-column tiled, k-grouped copy
-// of the weights, Ws[tile][K/8][16][8] (kernels_skinny.hip).  ws2 != nullptr: SwiGLU pair.  act: 0 none, 1 gelu.
+// Batched-decode linear layers (2 <= M <= 16, bf16 or f32) on the matrix cores over a 16-column tiled, k-grouped copy
+// of the weights, Ws[tile][K/KPC][16][KPC] with KPC = 8 (bf16) or 4 (f32) k per 16 bytes (kernels_skinny.hip).  ws2 != nullptr: SwiGLU pair.  act: 0 none, 1 gelu.
 struct SkinnyLinearArgs {
+    int dtype;   // 0 f32, 2 bf16
     const void* x; const void* ws; const void* ws2; const void* bias; const void* residual;
     void* y;
     int64_t m, k, n;
@@ -134,8 +135,8 @@ constexpr size_t kSkinnyTickets = 1024;
 int skinny_ksplit(int64_t k, int64_t n);
 size_t skinny_workspace_bytes(int64_t k, int64_t n, bool dual);
 bool skinny_gemm_supported(int dtype, int64_t m, int64_t k, int64_t n);
-size_t skinny_weight_bytes(int64_t k, int64_t n);
-void skinny_pack_weights(hipStream_t s, const void* w, void* out, int64_t k, int64_t n);
+size_t skinny_weight_bytes(int dtype, int64_t k, int64_t n);
+void skinny_pack_weights(hipStream_t s, int dtype, const void* w, void* out, int64_t k, int64_t n);
 void skinny_gemm(hipStream_t s, const SkinnyLinearArgs& a);
 
 // ---- weight-only quantisation (kernels_quant.hip) ------------------------------------------

@@ -1,4 +1,4 @@
-// Batched-decode linear layers (2 <= M <= 16 rows, bf16) on the matrix cores.
+// Batched-decode linear layers (2 <= M <= 16 rows, bf16 or f32) on the matrix cores.
 //
 // With a handful of rows a linear layer is still one pass over the weights, i.e. bound by HBM, but the
 // per-element work of a vector GEMV grows with M (M multiply-adds per weight element plus the activation reads)
@@ -11,6 +11,8 @@
 // the 32-k steps round-robin (so the workgroup reads 4 consecutive KiB per round) and add their partial products
 // through LDS.  The A operand (lane = 16 * k-group + row) comes straight from x, which is small and stays in L2.
 // DUAL computes silu(x.W) * (x.W2) (ops/functional/activation.rs:141-162) from two weight copies.
+// f32 takes the same route with 4 k per 16-byte lane word (Ws[tile][K/4][16][4], 16-k steps) on four
+// v_mfma_f32_16x16x4_f32 per word.
 //
 // Weight-only quantised layers (skinny_gemm_quant_kernel<QF, DUAL>) stream the CODES: a lane's 16-byte word holds 16
 // int8 codes (k = 64 S + 16 kg + 0..15 of its column: two MFMA steps) or 32 int4 codes (k = 128 Q + 32 kg + 0..31: four
@@ -37,24 +39,46 @@ typedef uint32_t u32x4_s __attribute__((ext_vector_type(4)));
 
 inline int64_t cdiv_s(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
-// Ws[tile][kb][c][i] = W[8 kb + i][16 tile + c], zero outside [K) x [N); one thread per 16-byte group
-__global__ __launch_bounds__(256) void skinny_pack_kernel(const bf16_t* __restrict__ w, bf16_t* __restrict__ out, int64_t K, int64_t N,
+// Element types: KPC = k per 16-byte lane word; a step of the K loop is 4 k-groups x KPC (32 k of bf16, 16 k of f32).
+// f32 runs on v_mfma_f32_16x16x4_f32: element e of both words is k = 4 * k-group + e of the step.
+template <typename T> struct SkinnyT;
+template <> struct SkinnyT<bf16_t> {
+    static constexpr int KPC = 8;
+    static __device__ __forceinline__ f32x4_s mma(const u32x4_s& a, const u32x4_s& b, f32x4_s c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_s, a), __builtin_bit_cast(bf16x8_s, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ float ld(const bf16_t* p, int64_t i) { return bf16_to_f32(p[i]); }
+    static __device__ __forceinline__ void st(bf16_t* p, int64_t i, float v) { p[i] = f32_to_bf16(v); }
+};
+template <> struct SkinnyT<float> {
+    static constexpr int KPC = 4;
+    static __device__ __forceinline__ f32x4_s mma(const u32x4_s& a, const u32x4_s& b, f32x4_s c) {
+        const f32x4_s af = __builtin_bit_cast(f32x4_s, a), bf = __builtin_bit_cast(f32x4_s, b);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_16x16x4f32(af[e], bf[e], c, 0, 0, 0);
+        return c;
+    }
+    static __device__ __forceinline__ float ld(const float* p, int64_t i) { return p[i]; }
+    static __device__ __forceinline__ void st(float* p, int64_t i, float v) { p[i] = v; }
+};
+
+// Ws[tile][kb][c][i] = W[KPC kb + i][16 tile + c], zero outside [K) x [N); one thread per 16-byte group
+template <typename T>
+__global__ __launch_bounds__(256) void skinny_pack_kernel(const T* __restrict__ w, T* __restrict__ out, int64_t K, int64_t N,
                                                           int64_t KB, int64_t ntiles) {
+    constexpr int KPC = SkinnyT<T>::KPC;
     const int64_t total = ntiles * KB * 16;
     for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < total; g += (int64_t)gridDim.x * blockDim.x) {
         const int c = (int)(g & 15);
         const int64_t kb = (g >> 4) % KB, tile = (g >> 4) / KB;
         const int64_t col = tile * 16 + c;
-        uint32_t r[4] = {0, 0, 0, 0};
-        if (col < N) {
+        alignas(16) T r[KPC];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int64_t kx = kb * 8 + i;
-                const uint32_t v = kx < K ? (uint32_t)w[kx * N + col] : 0u;
-                r[i >> 1] |= v << ((i & 1) * 16);
-            }
+        for (int i = 0; i < KPC; ++i) {
+            const int64_t kx = kb * KPC + i;
+            r[i] = (col < N && kx < K) ? w[kx * N + col] : T(0);
         }
-        *reinterpret_cast<uint4*>(out + g * 8) = make_uint4(r[0], r[1], r[2], r[3]);
+        *reinterpret_cast<uint4*>(out + g * KPC) = *reinterpret_cast<const uint4*>(r);
     }
 }
 
@@ -66,22 +90,23 @@ __device__ __forceinline__ float skinny_finish(float v, float v2, bool dual, int
     return v;
 }
 
-template <bool DUAL>
-__global__ __launch_bounds__(256) void skinny_gemm_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ ws,
-                                                          const bf16_t* __restrict__ ws2, const bf16_t* __restrict__ bias,
-                                                          const bf16_t* __restrict__ residual, bf16_t* __restrict__ y, int M, int K,
+template <typename T, bool DUAL>
+__global__ __launch_bounds__(256) void skinny_gemm_kernel(const T* __restrict__ x, const T* __restrict__ ws,
+                                                          const T* __restrict__ ws2, const T* __restrict__ bias,
+                                                          const T* __restrict__ residual, T* __restrict__ y, int M, int K,
                                                           int N, int act, float* __restrict__ part, unsigned* __restrict__ tickets) {
-    constexpr int U = 4;                         // 32-k steps per wave and round, all requested before the first is used
+    constexpr int U = 4;                         // steps per wave and round, all requested before the first is used
+    constexpr int KPC = SkinnyT<T>::KPC, KSTEP = 4 * KPC;
     __shared__ float red[4][DUAL ? 2 : 1][64][4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int c = lane & 15, kg = lane >> 4;     // B: column c, k-group kg; A: row c, k-group kg
     const int tile = blockIdx.x;
     const int ksplit = gridDim.y, ks = blockIdx.y;
-    const int s_begin = (int)((int64_t)(K / 32) * ks / ksplit), nsteps = (int)((int64_t)(K / 32) * (ks + 1) / ksplit);
-    const u32x4_s* bsrc = reinterpret_cast<const u32x4_s*>(ws) + (int64_t)tile * (K / 8) * 16 + lane;
-    const u32x4_s* bsrc2 = DUAL ? reinterpret_cast<const u32x4_s*>(ws2) + (int64_t)tile * (K / 8) * 16 + lane : nullptr;
+    const int s_begin = (int)((int64_t)(K / KSTEP) * ks / ksplit), nsteps = (int)((int64_t)(K / KSTEP) * (ks + 1) / ksplit);
+    const u32x4_s* bsrc = reinterpret_cast<const u32x4_s*>(ws) + (int64_t)tile * (K / KPC) * 16 + lane;
+    const u32x4_s* bsrc2 = DUAL ? reinterpret_cast<const u32x4_s*>(ws2) + (int64_t)tile * (K / KPC) * 16 + lane : nullptr;
     const int arow = c < M ? c : M - 1;          // rows beyond M re-read the last one; their products are never stored
-    const u32x4_s* asrc = reinterpret_cast<const u32x4_s*>(x + (int64_t)arow * K + 8 * kg);
+    const u32x4_s* asrc = reinterpret_cast<const u32x4_s*>(x + (int64_t)arow * K + KPC * kg);
 
     f32x4_s acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
     for (int s0 = s_begin + wave; s0 < nsteps; s0 += 4 * U) {
@@ -96,9 +121,8 @@ __global__ __launch_bounds__(256) void skinny_gemm_kernel(const bf16_t* __restri
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if (s0 + 4 * u < nsteps) {
-                const bf16x8_s av = __builtin_bit_cast(bf16x8_s, a[u]);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, __builtin_bit_cast(bf16x8_s, b[u]), acc, 0, 0, 0);
-                if (DUAL) acc2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, __builtin_bit_cast(bf16x8_s, b2[u]), acc2, 0, 0, 0);
+                acc = SkinnyT<T>::mma(a[u], b[u], acc);
+                if (DUAL) acc2 = SkinnyT<T>::mma(a[u], b2[DUAL ? u : 0], acc2);
             }
         }
     }
@@ -151,13 +175,13 @@ __global__ __launch_bounds__(256) void skinny_gemm_kernel(const bf16_t* __restri
     }
     const int n = tile * 16 + c;
     if (n >= N) return;
-    const float bv = bias ? bf16_to_f32(bias[n]) : 0.f;
+    const float bv = bias ? SkinnyT<T>::ld(bias, n) : 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int m = 4 * kg + i;                // D: lane holds rows 4 kg .. 4 kg + 3 of column c
         if (m >= M) continue;
-        const float r = residual ? bf16_to_f32(residual[(int64_t)m * N + n]) : 0.f;
-        y[(int64_t)m * N + n] = f32_to_bf16(skinny_finish(g[i], up[i], DUAL, act, bv, residual != nullptr, r));
+        const float r = residual ? SkinnyT<T>::ld(residual, (int64_t)m * N + n) : 0.f;
+        SkinnyT<T>::st(y, (int64_t)m * N + n, skinny_finish(g[i], up[i], DUAL, act, bv, residual != nullptr, r));
     }
 }
 
@@ -350,14 +374,20 @@ __global__ __launch_bounds__(256) void skinny_gemm_quant_kernel(const bf16_t* __
 }  // namespace
 
 bool skinny_gemm_supported(int dtype, int64_t m, int64_t k, int64_t n) {
-    return dtype == 2 && m >= 2 && m <= 16 && k >= 32 && k % 32 == 0 && n >= 1 && k < (1ll << 31) && n < (1ll << 31) - 16;
+    if (dtype != 0 && dtype != 2) return false;
+    const int64_t kstep = dtype == 0 ? 16 : 32;
+    return m >= 2 && m <= 16 && k >= kstep && k % kstep == 0 && n >= 1 && k < (1ll << 31) && n < (1ll << 31) - 16;
 }
-size_t skinny_weight_bytes(int64_t k, int64_t n) { return (size_t)(cdiv_s(n, 16) * cdiv_s(k, 8) * 16 * 8) * sizeof(bf16_t); }
-void skinny_pack_weights(hipStream_t s, const void* w, void* out, int64_t k, int64_t n) {
-    const int64_t ntiles = cdiv_s(n, 16), kb = cdiv_s(k, 8), total = ntiles * kb * 16;
+size_t skinny_weight_bytes(int dtype, int64_t k, int64_t n) {
+    const int64_t kpc = dtype == 0 ? 4 : 8;
+    return (size_t)(cdiv_s(n, 16) * cdiv_s(k, kpc) * 16) * 16;
+}
+void skinny_pack_weights(hipStream_t s, int dtype, const void* w, void* out, int64_t k, int64_t n) {
+    const int64_t ntiles = cdiv_s(n, 16), kb = cdiv_s(k, dtype == 0 ? 4 : 8), total = ntiles * kb * 16;
     if (total <= 0) return;
     const unsigned g = (unsigned)(cdiv_s(total, 256) > 65536 ? 65536 : cdiv_s(total, 256));
-    skinny_pack_kernel<<<g, 256, 0, s>>>((const bf16_t*)w, (bf16_t*)out, k, n, kb, ntiles);
+    if (dtype == 0) skinny_pack_kernel<float><<<g, 256, 0, s>>>((const float*)w, (float*)out, k, n, kb, ntiles);
+    else skinny_pack_kernel<bf16_t><<<g, 256, 0, s>>>((const bf16_t*)w, (bf16_t*)out, k, n, kb, ntiles);
 }
 // Workgroups per tile: doubled while the launch has fewer than two workgroups per CU and each split keeps at least 16
 // steps of 32 k (measured on Ministral-3B shapes at 8 rows: 192 tiles x 4 takes 13.8 us where 192 x 1 took 18.7; at
@@ -374,7 +404,7 @@ size_t skinny_workspace_bytes(int64_t k, int64_t n, bool dual) {
     return ks > 1 ? (size_t)cdiv_s(n, 16) * ks * (dual ? 2 : 1) * 256 * sizeof(float) : 0;
 }
 bool skinny_quant_supported(int dtype, int64_t m, int64_t k, int64_t n, int qf) {
-    if (qf != 1 && qf != 2) return false;
+    if ((qf != 1 && qf != 2) || dtype != 2) return false;
     return skinny_gemm_supported(dtype, m, k, n) && k % (qf == 1 ? 64 : 128) == 0;
 }
 size_t skinny_codes_bytes(int64_t k, int64_t n, int qf) { return (size_t)(cdiv_s(n, 16) * (k / (qf == 1 ? 64 : 128)) * 64 * 16); }
@@ -404,14 +434,12 @@ void skinny_gemm(hipStream_t s, const SkinnyLinearArgs& a) {
     int ks = skinny_ksplit(a.k, a.n);
     if (!a.part || !a.tickets || a.part_bytes < skinny_workspace_bytes(a.k, a.n, a.ws2 != nullptr)) ks = 1;
     const dim3 grid((unsigned)cdiv_s(a.n, 16), (unsigned)ks);
-    if (a.ws2)
-        skinny_gemm_kernel<true><<<grid, 256, 0, s>>>((const bf16_t*)a.x, (const bf16_t*)a.ws, (const bf16_t*)a.ws2, (const bf16_t*)a.bias,
-                                                      (const bf16_t*)a.residual, (bf16_t*)a.y, (int)a.m, (int)a.k, (int)a.n, a.act,
-                                                      (float*)a.part, a.tickets);
-    else
-        skinny_gemm_kernel<false><<<grid, 256, 0, s>>>((const bf16_t*)a.x, (const bf16_t*)a.ws, nullptr, (const bf16_t*)a.bias,
-                                                       (const bf16_t*)a.residual, (bf16_t*)a.y, (int)a.m, (int)a.k, (int)a.n, a.act,
-                                                       (float*)a.part, a.tickets);
+#define GPTRS_LAUNCH(T, DUAL)                                                                                               \
+    skinny_gemm_kernel<T, DUAL><<<grid, 256, 0, s>>>((const T*)a.x, (const T*)a.ws, (const T*)a.ws2, (const T*)a.bias,          \
+        (const T*)a.residual, (T*)a.y, (int)a.m, (int)a.k, (int)a.n, a.act, (float*)a.part, a.tickets)
+    if (a.dtype == 0) { if (a.ws2) GPTRS_LAUNCH(float, true); else GPTRS_LAUNCH(float, false); }
+    else { if (a.ws2) GPTRS_LAUNCH(bf16_t, true); else GPTRS_LAUNCH(bf16_t, false); }
+#undef GPTRS_LAUNCH
 }
 
 }  // namespace k

@@ -1082,6 +1082,7 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
                           : k::skinny_gemm_supported((int)x.dtype, x.dims[0], x.dims[1], w.dims[1])) &&
                 (!in.norm || st.scratch_bytes >= (size_t)x.count() * dtype_size(x.dtype))) {
                 k::SkinnyLinearArgs sa{};
+                sa.dtype = (int)x.dtype;
                 sa.x = src_ptr(st, cx, 0);
                 sa.m = x.dims[0]; sa.k = x.dims[1]; sa.n = w.dims[1];
                 const int kind = in.quant == 0 ? 8 : (in.quant == 1 ? 9 : 10);   // bf16 copy, or the codes in the same tile order

@@ -293,6 +293,22 @@ def test_batched_decode_linear_on_matrix_cores(hip, m, k, n):
         assert_close(got, want, atol=3e-2, rtol=2e-2, what=f"m={m} k={k} n={n}")
 
 
+@pytest.mark.parametrize("m,k,n", [(8, 768, 2304), (16, 3072, 768), (16, 768, 50257), (5, 512, 40), (2, 64, 24), (3, 48, 16)])
+def test_batched_decode_linear_f32_on_matrix_cores(hip, m, k, n):
+    """2..16 f32 rows: the same kernel on v_mfma_f32_16x16x4_f32 (weights in groups of 4 k); the reference suite's
+    tolerance (5e-4 + 1e-4 relative), plain, under LayerNorm + bias + exact GELU + residual, and as a SwiGLU pair."""
+    x, w = rng_uniform(60, (m, k)), rng_uniform(61, (k, n)) * (2.0 / np.sqrt(k))
+    b, r, g, be_ = rng_uniform(62, (n,)), rng_uniform(63, (m, n)), rng_uniform(64, (k,)) + 1.5, rng_uniform(65, (k,))
+    w2 = rng_uniform(66, (k, n)) * (2.0 / np.sqrt(k))
+    built = hip.counter("derived_weights_built")
+    check_program(hip, prog(lambda fb, a, c: a.matmul(c), [("F32", [m, k]), ("F32", [k, n])]), [x, w])
+    assert hip.counter("derived_weights_built") > built
+    check_program(hip, prog(lambda fb, a, gm, bt, c, d, e: F.gelu(F.linear(F.layer_norm(a, gm, bt, 1e-5)[0], c, d)) + e,
+                            [("F32", [m, k]), ("F32", [k]), ("F32", [k]), ("F32", [k, n]), ("F32", [n]), ("F32", [m, n])]), [x, g, be_, w, b, r])
+    check_program(hip, prog(lambda fb, a, c, d: F.swiglu(a.matmul(c), a.matmul(d)), [("F32", [m, k]), ("F32", [k, n]), ("F32", [k, n])]),
+                  [x, w, w2])
+
+
 @pytest.mark.parametrize("m,k,n", [(8, 3072, 9216), (4, 256, 96), (16, 3072, 9216), (12, 512, 256)])
 def test_batched_decode_norm_swiglu_on_matrix_cores(hip, m, k, n):
     from gptrs_amd.ptir import f32_to_bf16_bits
