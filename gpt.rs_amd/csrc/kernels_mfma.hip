@@ -275,11 +275,15 @@ static void launch_mfma(hipStream_t s, const MfmaLinearArgs& a) {
 }
 
 void mfma_gemm(hipStream_t s, const MfmaLinearArgs& a) {
+    // a problem with fewer 128 x 128 tiles than half the CUs runs on 64 x 64 tiles (four times the workgroups)
+    const bool small = cdiv(a.m, 128) * cdiv(a.n, a.wk2 ? 64 : 128) < 128;
     if (a.dtype == 0) {
         if (a.wk2) launch_mfma<float, 128, 128, true>(s, a);
+        else if (small) launch_mfma<float, 64, 64, false>(s, a);
         else launch_mfma<float, 128, 128, false>(s, a);
     } else {
         if (a.wk2) launch_mfma<bf16_t, 128, 128, true>(s, a);
+        else if (small) launch_mfma<bf16_t, 64, 64, false>(s, a);
         else launch_mfma<bf16_t, 128, 128, false>(s, a);
     }
 }
