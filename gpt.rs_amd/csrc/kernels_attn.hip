@@ -797,8 +797,155 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const bf16_t* __
     }
 }
 
+// The same kernel in f32 on v_mfma_f32_32x32x2_f32: a 16-byte fragment holds 4 consecutive d (scores) or 4 consecutive
+// keys (P.V), each fragment feeds four K = 2 products, and the probabilities stay f32.  V^T sits in LDS in plain key
+// order: the keys a lane holds of its query in score registers 4 i .. 4 i + 3 are 8 i + 4 (lane / 32) + 0..3, exactly
+// what fragment i of the second product covers.
+typedef float f32x4_v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ f32x16_v mma_f32x4(const f32x4_v& a, const f32x4_v& b, f32x16_v c) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e], b[e], c, 0, 0, 0);
+    return c;
+}
+
+template <int DH>
+__global__ __launch_bounds__(256) void attn_prefill_mfma_f32_kernel(const float* __restrict__ qkv, float* __restrict__ ctx, int T,
+                                                                    int n_q, int n_kv, float scale_log2e) {
+    constexpr int KT = 32;            // keys per tile
+    constexpr int KS = DH + 4;        // K tile row stride in elements (16 bytes of padding)
+    constexpr int VS = KT + 4;        // V^T row stride in elements
+    constexpr int ND = DH / 32;       // 32-row blocks of d in O^T
+    constexpr int NK = DH / 8;        // k-steps of the score product (8 d each)
+    constexpr int CH = KT * DH / 4;   // 16-byte chunks of a K (or V) tile
+    constexpr int CPT = (CH + 255) / 256;
+    __shared__ __align__(16) float ksm[2][KT * KS];
+    __shared__ __align__(16) float vsm[2][DH * VS];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, half = lane >> 5;
+    const int G = n_q / n_kv;
+    const int gw = G >= 4 ? 4 : G;
+    const int rtpb = 4 / gw;
+    const int kvh = blockIdx.y;
+    const int head = kvh * G + blockIdx.z * gw + wave % gw;
+    const int q0 = (blockIdx.x * rtpb + wave / gw) * 32;
+    const int64_t P = (int64_t)(n_q + 2 * n_kv) * DH;
+    const int64_t koff = (int64_t)n_q * DH + (int64_t)kvh * DH;
+    const int64_t voff = (int64_t)(n_q + n_kv) * DH + (int64_t)kvh * DH;
+    const int kend = min(T, (blockIdx.x * rtpb + rtpb) * 32);
+    const int ntiles = (kend + KT - 1) / KT;
+    const bool active = q0 < T;
+    const int my_tiles = active ? min(ntiles, (q0 + 31) / KT + 1) : 0;
+
+    f32x4_v qf[NK];
+    {
+        const int row = min(q0 + col, T - 1);
+        const float* qp = qkv + (int64_t)row * P + (int64_t)head * DH + 4 * half;
+#pragma unroll
+        for (int kk = 0; kk < NK; ++kk) qf[kk] = *reinterpret_cast<const f32x4_v*>(qp + 8 * kk);
+    }
+    f32x16_v acc_o[ND];
+#pragma unroll
+    for (int db = 0; db < ND; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc_o[db][v] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+
+    f32x4_v kreg[CPT], vreg[CPT];
+    auto gload = [&](int t) {
+#pragma unroll
+        for (int j = 0; j < CPT; ++j) {
+            const int c = tid + 256 * j;
+            if (CH % 256 == 0 || c < CH) {
+                const int r = c / (DH / 4), ch = c % (DH / 4);
+                const int64_t key = min(t * KT + r, T - 1);
+                kreg[j] = *reinterpret_cast<const f32x4_v*>(qkv + key * P + koff + ch * 4);
+                vreg[j] = *reinterpret_cast<const f32x4_v*>(qkv + key * P + voff + ch * 4);
+            }
+        }
+    };
+    auto lwrite = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < CPT; ++j) {
+            const int c = tid + 256 * j;
+            if (CH % 256 == 0 || c < CH) {
+                const int r = c / (DH / 4), ch = c % (DH / 4);
+                *reinterpret_cast<f32x4_v*>(&ksm[buf][r * KS + ch * 4]) = kreg[j];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) vsm[buf][(ch * 4 + e) * VS + r] = vreg[j][e];
+            }
+        }
+    };
+
+    gload(0);
+    lwrite(0);
+    __syncthreads();
+    for (int t = 0; t < ntiles; ++t) {
+        const int buf = t & 1;
+        if (t + 1 < ntiles) gload(t + 1);
+        if (t < my_tiles) {
+            f32x16_v sc;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) sc[v] = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < NK; ++kk) {
+                const f32x4_v kf = *reinterpret_cast<const f32x4_v*>(&ksm[buf][col * KS + 8 * kk + 4 * half]);
+                sc = mma_f32x4(kf, qf[kk], sc);
+            }
+            const int qrow = q0 + col;
+            const int kbase = t * KT + 4 * half;
+            float mx = -INFINITY;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int key = kbase + 8 * (v >> 2) + (v & 3);
+                const float x = key <= qrow ? sc[v] * scale_log2e : -INFINITY;
+                sc[v] = x;
+                mx = fmaxf(mx, x);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m_run, mx);
+            const float corr = exp2f(m_run - m_new);
+            float ls = 0.f;
+            f32x4_v pf[4];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const float pv = exp2f(sc[v] - m_new);
+                ls += pv;
+                pf[v >> 2][v & 3] = pv;
+            }
+            ls += __shfl_xor(ls, 32, 64);
+            l_run = l_run * corr + ls;
+            m_run = m_new;
+#pragma unroll
+            for (int db = 0; db < ND; ++db) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc_o[db][v] *= corr;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const f32x4_v vf = *reinterpret_cast<const f32x4_v*>(&vsm[buf][(db * 32 + col) * VS + 8 * i + 4 * half]);
+                    acc_o[db] = mma_f32x4(vf, pf[i], acc_o[db]);
+                }
+            }
+        }
+        if (t + 1 < ntiles) lwrite(buf ^ 1);
+        __syncthreads();
+    }
+    if (active && q0 + col < T) {
+        const float inv = 1.0f / l_run;
+        float* op = ctx + (int64_t)(q0 + col) * n_q * DH + (int64_t)head * DH;
+#pragma unroll
+        for (int db = 0; db < ND; ++db)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const int d = db * 32 + 8 * g4 + 4 * half;
+                *reinterpret_cast<float4*>(op + d) = make_float4(acc_o[db][4 * g4] * inv, acc_o[db][4 * g4 + 1] * inv,
+                                                                 acc_o[db][4 * g4 + 2] * inv, acc_o[db][4 * g4 + 3] * inv);
+            }
+    }
+}
+
 static bool attn_prefill_mfma_ok(const AttnPrefillArgs& a) {
-    if (a.dtype != 2 || a.n_kv <= 0 || a.n_q % a.n_kv != 0 || a.t >= (1ll << 30)) return false;
+    if ((a.dtype != 2 && a.dtype != 0) || a.n_kv <= 0 || a.n_q % a.n_kv != 0 || a.t >= (1ll << 30)) return false;
     if (a.head_dim != 32 && a.head_dim != 64 && a.head_dim != 128) return false;
     const int64_t g = a.n_q / a.n_kv;
     return g == 1 || g == 2 || g % 4 == 0;
@@ -811,6 +958,12 @@ void attn_prefill(hipStream_t s, const AttnPrefillArgs& a) {
         const int g = (int)(a.n_q / a.n_kv), gw = g >= 4 ? 4 : g;
         dim3 grid((unsigned)cdiv(cdiv(a.t, 32), 4 / gw), (unsigned)a.n_kv, (unsigned)(g >= 4 ? g / 4 : 1));
         const float sl = a.scale * 1.44269504088896f;
+        if (a.dtype == 0) {
+            if (a.head_dim == 32) attn_prefill_mfma_f32_kernel<32><<<grid, 256, 0, s>>>((const float*)a.qkv, (float*)a.ctx, (int)a.t, (int)a.n_q, (int)a.n_kv, sl);
+            else if (a.head_dim == 64) attn_prefill_mfma_f32_kernel<64><<<grid, 256, 0, s>>>((const float*)a.qkv, (float*)a.ctx, (int)a.t, (int)a.n_q, (int)a.n_kv, sl);
+            else attn_prefill_mfma_f32_kernel<128><<<grid, 256, 0, s>>>((const float*)a.qkv, (float*)a.ctx, (int)a.t, (int)a.n_q, (int)a.n_kv, sl);
+            return;
+        }
         if (a.head_dim == 32) attn_prefill_mfma_kernel<32><<<grid, 256, 0, s>>>((const bf16_t*)a.qkv, (bf16_t*)a.ctx, (int)a.t, (int)a.n_q, (int)a.n_kv, sl);
         else if (a.head_dim == 64) attn_prefill_mfma_kernel<64><<<grid, 256, 0, s>>>((const bf16_t*)a.qkv, (bf16_t*)a.ctx, (int)a.t, (int)a.n_q, (int)a.n_kv, sl);
         else attn_prefill_mfma_kernel<128><<<grid, 256, 0, s>>>((const bf16_t*)a.qkv, (bf16_t*)a.ctx, (int)a.t, (int)a.n_q, (int)a.n_kv, sl);
