@@ -392,11 +392,13 @@ def test_ministral_full_width_one_layer_bf16_vs_oracle(hip):
     (1) The op-by-op HIP path must reproduce the bf16 oracle (every op output rounded to bf16)
         BIT-EXACTLY on the prefill logits.
     (2) The fused HIP path is compared with the F32 oracle fed the same bf16-representable weights
-        (the reference's CPU backends execute f32 only).  North-star bar: 2e-2 absolute.  At this
-        width the logits reach |x| > 4, where one bf16 output quantum is already 3.1e-2 (half of it
-        1.6e-2), so the bar cannot hold for the largest logits: measured max error is 4.1e-2
-        (the per-op-rounded bf16 oracle itself is 6.4e-2 from f32).  Asserted here: 2e-2 wherever
-        |logit| < 2, and 5e-2 overall -- a documented miss of the stated bar, not a pass of it."""
+        (the reference's CPU backends execute f32 only).  North-star bar: 2e-2 absolute.  It does
+        NOT hold at this width, for any bf16 pipeline: a layer rounds about a dozen intermediate
+        tensors to bf16, each rounding moves a logit by ~1e-3 (std), and the maximum over 1M logits
+        lands at 4-6e-2 whatever the logit's own magnitude.  Measured: fused path 4.6e-2 from f32
+        (mean 6e-3), the per-op-rounded bf16 oracle 6.4e-2 from f32, and the two bf16 pipelines
+        7.8e-2 from each other.  Asserted here: 5e-2 overall and 1e-2 on average -- a documented
+        miss of the stated bar, not a pass of it; the numbers are printed (run with -s)."""
     cfg = models.MinistralConfig(num_layers=1)
     prompt = np.random.default_rng(6).integers(0, cfg.vocab_size, 8).tolist()
     ob = OracleBackend()
@@ -414,7 +416,16 @@ def test_ministral_full_width_one_layer_bf16_vs_oracle(hip):
         hip.set_option("fusion", 1)
     assert np.array_equal(generic, ref_bf16), "op-by-op bf16 path must match the bf16 oracle bit for bit"
     err = np.abs(fused - ref_f32)
-    print(f"ministral 1 layer bf16: max err {err.max():.4f} mean err {err.mean():.5f}, max |logit| {np.abs(ref_f32).max():.2f}")
+    small = np.abs(ref_f32) < 2.0
+    print(f"ministral 1 layer bf16: max err {err.max():.4f} mean err {err.mean():.5f}, max |logit| {np.abs(ref_f32).max():.2f}, "
+          f"max err where |logit| < 2: {err[small].max():.4f} ({small.mean() * 100:.1f} % of the logits); "
+          f"bf16 oracle vs f32 oracle: max {np.abs(ref_bf16 - ref_f32).max():.4f}")
+    eb = np.abs(fused - ref_bf16)
+    ulp = np.exp2(np.floor(np.log2(np.maximum(np.abs(ref_bf16), 1e-30))) - 7)
+    nu = eb / ulp
+    print(f"fused vs bf16 oracle: max {eb.max():.4f} mean {eb.mean():.6f}; equal {np.mean(eb == 0) * 100:.2f} %, "
+          f"<= 1 ulp {np.mean(nu <= 1.0) * 100:.3f} %, <= 2 ulp {np.mean(nu <= 2.0) * 100:.3f} %, max ulps {nu.max():.1f}, "
+          f"max err where |logit| >= 0.25: {eb[np.abs(ref_bf16) >= 0.25].max():.4f}")
     assert err.max() < 5e-2 and err.mean() < 1e-2
     # one decode step on top of the cache
     tok = int(np.argmax(ref_f32[-1]))
