@@ -171,14 +171,9 @@ BufferP Backend::derived_weights(const BufferP& src, int kind, DType dtype, int6
     } else if (kind == 9 || kind == 10) {               // batched decode: int8 / int4 codes in the 16-column tiled word order
         t = new_buffer(k::skinny_codes_bytes(k, n, kind - 8));
         k::skinny_pack_codes(stream, src->ptr, t->ptr, k, n, kind - 8);
-    } else {                                            // 6 / 7: MFMA copy of dequantised int8 / int4 (src2: scales)
-        if (!src2) fail_exec("quantised weight copy needs its scales");
-        BufferP full = new_buffer((size_t)k * n * dtype_size(dtype));
-        if (kind == 6) k::dequant_w8(stream, (int)dtype, (const int8_t*)src->ptr, src2->ptr, full->ptr, k, n);
-        else k::dequant_w4g128(stream, (int)dtype, (const uint8_t*)src->ptr, src2->ptr, full->ptr, k, n);
-        t = new_buffer(k::mfma_weight_bytes((int)dtype, k, n));
-        k::mfma_pack_weights(stream, (int)dtype, full->ptr, t->ptr, k, n);
-        // `full` returns to the pool here; later users are ordered behind the pack on the one stream
+    } else {                                            // 6 / 7: prefill GEMM: int8 / int4 codes, k-grouped (kernels_mfma.hip)
+        t = new_buffer(k::mfma_codes_bytes(k, n, kind - 5));
+        k::mfma_pack_codes(stream, src->ptr, t->ptr, k, n, kind - 5);
     }
     Derived d;
     d.src = src;

@@ -797,7 +797,7 @@ struct Fuser {
             if (!is_param(in.operands[1].value)) continue;
             if (in.act == 2 && !is_param(in.operands[linear_w2_pos(in)].value)) continue;
             if (in.quant && (!is_param(in.operands[2].value) || (in.act == 2 && !is_param(in.operands[4].value)))) continue;
-            if (k::mfma_gemm_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1])) {
+            if (k::mfma_gemm_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1], in.quant)) {
                 in.mfma = true;
                 continue;
             }

@@ -224,10 +224,16 @@ struct MfmaLinearArgs {
     void* y;
     int64_t m, k, n;
     int act;
+    // weight-only quantised (bf16 activations): quant 1 = int8 per column, 2 = int4 groups of 128; wk / wk2 are then
+    // the k-grouped CODE copies (mfma_pack_codes) and scale / scale2 the matrices' scale tensors
+    int quant;
+    const void* scale; const void* scale2;
 };
 size_t mfma_weight_bytes(int dtype, int64_t k, int64_t n);
 void mfma_pack_weights(hipStream_t s, int dtype, const void* w, void* out, int64_t k, int64_t n);
-bool mfma_gemm_supported(int dtype, int64_t m, int64_t k, int64_t n);
+size_t mfma_codes_bytes(int64_t k, int64_t n, int quant);
+void mfma_pack_codes(hipStream_t s, const void* q, void* out, int64_t k, int64_t n, int quant);
+bool mfma_gemm_supported(int dtype, int64_t m, int64_t k, int64_t n, int quant = 0);
 void mfma_gemm(hipStream_t s, const MfmaLinearArgs& a);
 
 // Rotate-half RoPE on packed [T, Q|K|V] rows (ops/functional/rotary.rs:430-536).

@@ -77,6 +77,59 @@ void mfma_pack_weights(hipStream_t s, int dtype, const void* w, void* out, int64
     else k8_weights_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)w, (bf16_t*)out, k, n, npad);
 }
 
+// Weight-only quantised weights (bf16 activations): the GEMM reads the CODES, in the same k-grouped order, and turns
+// them into the bf16 values of the dequantised matrix, bf16(code * scale), on the way into LDS; no dequantised copy
+// exists.  Ck[kb][n] holds the 8 codes of k-group kb of column n with the sign bias added (int8: 8 bytes of q + 128;
+// int4: one dword, nibble i = q(k = 8 kb + i) + 8), so a code converts with one unsigned-byte / bit-field instruction
+// and one fma (u * s - bias * s is exactly (u - bias) * s, rounded once like the product the dequantiser forms).
+// Padding (n >= N, k >= K) holds the code of zero.
+template <int QF>
+__global__ __launch_bounds__(256) void k8_codes_kernel(const uint8_t* __restrict__ q, uint32_t* __restrict__ out, int64_t K, int64_t N,
+                                                       int64_t Npad) {
+    const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t kb = blockIdx.y;
+    if (n >= Npad) return;
+    if (QF == 1) {
+        uint32_t w[2] = {0x80808080u, 0x80808080u};
+        if (n < N) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int64_t kx = kb * 8 + i;
+                const uint32_t u = kx < K ? (uint32_t)(uint8_t)(q[kx * N + n] + 128u) : 128u;   // si8 [K, N]
+                w[i >> 2] = (w[i >> 2] & ~(0xFFu << (8 * (i & 3)))) | (u << (8 * (i & 3)));
+            }
+        }
+        *reinterpret_cast<uint2*>(out + (kb * Npad + n) * 2) = make_uint2(w[0], w[1]);
+    } else {
+        uint32_t w = 0x88888888u;
+        if (n < N) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int64_t k2 = kb * 4 + j;   // ui8 [K / 2, N]: low nibble k = 2 k2, high nibble k = 2 k2 + 1
+                const uint32_t b = 2 * k2 < K ? (uint32_t)(q[k2 * N + n] ^ 0x88u) : 0x88u;
+                w = (w & ~(0xFFu << (8 * j))) | (b << (8 * j));
+            }
+        }
+        out[kb * Npad + n] = w;
+    }
+}
+size_t mfma_codes_bytes(int64_t k, int64_t n, int quant) {
+    return (size_t)cdiv(k, 8) * (size_t)mfma_padded_n(n) * (quant == 1 ? 8 : 4);
+}
+void mfma_pack_codes(hipStream_t s, const void* q, void* out, int64_t k, int64_t n, int quant) {
+    const int64_t npad = mfma_padded_n(n);
+    dim3 grid((unsigned)cdiv(npad, 256), (unsigned)cdiv(k, 8));
+    if (quant == 1) k8_codes_kernel<1><<<grid, 256, 0, s>>>((const uint8_t*)q, (uint32_t*)out, k, n, npad);
+    else k8_codes_kernel<2><<<grid, 256, 0, s>>>((const uint8_t*)q, (uint32_t*)out, k, n, npad);
+}
+__device__ __forceinline__ uint32_t mfma_pack_bf16(float lo, float hi) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    f32x2_t f;
+    f.x = lo; f.y = hi;
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));   // round to nearest even
+}
+
 __device__ __forceinline__ float mfma_finish(float v, float v2, bool dual, int act, float bias, bool has_res, float res) {
     if (dual) v = (v / (1.0f + expf(v * -1.0f))) * v2;        // activation.rs:141-162
     v += bias;                                                // tensor_ops.rs:42-56
@@ -104,11 +157,14 @@ __device__ __forceinline__ float mfma_finish(float v, float v2, bool dual, int a
 // output meet in the same lane.
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
-template <typename T, int BM, int BN, bool DUAL>
+// QF: 0 = wk / wk2 hold values; 1 / 2 = they hold int8 / int4 codes (see k8_codes_kernel) and `scale` / `scale2` the
+// scale tensors of the two matrices ([N] per column, or [K / 128, N] per group of 128 k), T = bf16 only.
+template <typename T, int BM, int BN, bool DUAL, int QF>
 __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ x, const T* __restrict__ wk,
                                                         const T* __restrict__ wk2, const T* __restrict__ bias,
                                                         const T* __restrict__ residual, T* __restrict__ y,
-                                                        int M, int K, int N, int Npad, int act, int NT, int MT) {
+                                                        int M, int K, int N, int Npad, int act, int NT, int MT,
+                                                        const T* __restrict__ scale, const T* __restrict__ scale2) {
     constexpr int KPC = Mma<T>::KPC;
     constexpr int kBK = kKb * KPC;                            // k per tile
     typedef typename Mma<T>::frag frag_t;
@@ -167,8 +223,28 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ x,
             col = n0 + wcol * (WN / 2) + cc;
             src = half ? wk2 : wk;
         }
-        b_src[j] = src + ((int64_t)bkb * Npad + col) * KPC;
+        // codes: 8 (int8) or 4 (int4) bytes per k-group and column instead of 16
+        constexpr int64_t CW = QF == 0 ? KPC * (int64_t)sizeof(T) : (QF == 1 ? 8 : 4);
+        b_src[j] = reinterpret_cast<const T*>(reinterpret_cast<const unsigned char*>(src) + ((int64_t)bkb * Npad + col) * CW);
         b_dst[j] = kKb * SA + bkb * SB + bc * 16;
+    }
+    // quantised: every chunk of a thread belongs to ONE tile column (256 % BN == 0), so one scale per thread (int8) or
+    // per thread and k tile (int4: a tile of 64 k lies inside one group of 128)
+    const T* s_src = nullptr;
+    float q_scale = 0.f, q_scale_next = 0.f;
+    if (QF != 0) {
+        static_assert(256 % BN == 0, "one tile column per thread");
+        const int bc = tid % BN;
+        int col = n0 + bc;
+        const T* sp = scale;
+        if (DUAL) {
+            const int wcol = bc / WN, in_w = bc % WN, half = in_w / (WN / 2), cc = in_w % (WN / 2);
+            col = n0 + wcol * (WN / 2) + cc;
+            sp = half ? scale2 : scale;
+        }
+        if (col > N - 1) col = N - 1;   // padding columns hold the code of zero
+        s_src = sp + col;
+        if (QF == 1) q_scale = Mma<T>::ld(s_src, 0);
     }
 
     f32x16_t acc[TM][TN];
@@ -179,21 +255,59 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ x,
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    u32x4_t ra[CA], rb[CB];
+    typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+    u32x4_t ra[CA], rb[QF == 0 ? CB : 1];
+    u32x2_t rq8[QF == 1 ? CB : 1];
+    uint32_t rq4[QF == 2 ? CB : 1];
     const int nt = K / kBK;
-    const int64_t b_tile_step = (int64_t)kKb * Npad * KPC;  // elements between consecutive k tiles of Wk
-    auto gload = [&](int t) {
+    // bytes between consecutive k tiles of Wk
+    const int64_t b_tile_step = (int64_t)kKb * Npad * (QF == 0 ? KPC * (int64_t)sizeof(T) : (QF == 1 ? 8 : 4));
+    auto gload = [&](int t, int part, int nparts) {
 #pragma unroll
-        for (int j = 0; j < CA; ++j) ra[j] = *reinterpret_cast<const u32x4_t*>(a_src[j] + (int64_t)t * kBK);
+        for (int j = 0; j < CA; ++j)
+            if (j % nparts == part) ra[j] = *reinterpret_cast<const u32x4_t*>(a_src[j] + (int64_t)t * kBK);
 #pragma unroll
-        for (int j = 0; j < CB; ++j) rb[j] = *reinterpret_cast<const u32x4_t*>(b_src[j] + (int64_t)t * b_tile_step);
+        for (int j = 0; j < CB; ++j) {
+            if (j % nparts != part) continue;
+            const unsigned char* p = reinterpret_cast<const unsigned char*>(b_src[j]) + (int64_t)t * b_tile_step;
+            if (QF == 0) rb[j] = *reinterpret_cast<const u32x4_t*>(p);
+            else if (QF == 1) rq8[j] = *reinterpret_cast<const u32x2_t*>(p);
+            else rq4[j] = *reinterpret_cast<const uint32_t*>(p);
+        }
+        if (QF == 2 && part == nparts - 1) q_scale_next = Mma<T>::ld(s_src, (int64_t)(t * kBK / 128) * N);
     };
-    auto lwrite = [&](int buf) {
+    // part p of NP: chunks j with j % NP == p
+    auto lwrite = [&](int buf, int part, int nparts) {
         unsigned char* base = lds + buf * STAGE;
 #pragma unroll
-        for (int j = 0; j < CA; ++j) *reinterpret_cast<u32x4_t*>(base + a_dst[j]) = ra[j];
+        for (int j = 0; j < CA; ++j)
+            if (j % nparts == part) *reinterpret_cast<u32x4_t*>(base + a_dst[j]) = ra[j];
 #pragma unroll
-        for (int j = 0; j < CB; ++j) *reinterpret_cast<u32x4_t*>(base + b_dst[j]) = rb[j];
+        for (int j = 0; j < CB; ++j) {
+            if (j % nparts != part) continue;
+            u32x4_t v;
+            if (QF == 0) {
+                v = rb[j];
+            } else if (QF == 1) {
+                const float nb = -128.0f * q_scale;
+                const uint32_t a = rq8[j].x, b = rq8[j].y;
+                v.x = mfma_pack_bf16(__builtin_fmaf((float)(a & 0xFFu), q_scale, nb), __builtin_fmaf((float)((a >> 8) & 0xFFu), q_scale, nb));
+                v.y = mfma_pack_bf16(__builtin_fmaf((float)((a >> 16) & 0xFFu), q_scale, nb), __builtin_fmaf((float)(a >> 24), q_scale, nb));
+                v.z = mfma_pack_bf16(__builtin_fmaf((float)(b & 0xFFu), q_scale, nb), __builtin_fmaf((float)((b >> 8) & 0xFFu), q_scale, nb));
+                v.w = mfma_pack_bf16(__builtin_fmaf((float)((b >> 16) & 0xFFu), q_scale, nb), __builtin_fmaf((float)(b >> 24), q_scale, nb));
+            } else {
+                const float nb = -8.0f * q_scale;
+                const uint32_t c = rq4[j];
+                float f[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) f[i] = __builtin_fmaf((float)((c >> (4 * i)) & 0xFu), q_scale, nb);
+                v.x = mfma_pack_bf16(f[0], f[1]);
+                v.y = mfma_pack_bf16(f[2], f[3]);
+                v.z = mfma_pack_bf16(f[4], f[5]);
+                v.w = mfma_pack_bf16(f[6], f[7]);
+            }
+            *reinterpret_cast<u32x4_t*>(base + b_dst[j]) = v;
+        }
     };
     const int a_rd = (wm * (BM / 2) + (lane & 31)) * 16 + (lane >> 5) * SA;
     const int b_rd = kKb * SA + (wn * WN + (lane & 31)) * 16 + (lane >> 5) * SB;
@@ -206,9 +320,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ x,
         for (int j = 0; j < TN; ++j) bfr[slot][j] = *reinterpret_cast<const frag_t*>(base + b_rd + kk * 2 * SB + j * 32 * 16);
     };
 
-    gload(0);
-    lwrite(0);
-    gload(nt > 1 ? 1 : 0);
+    gload(0, 0, 1);
+    if (QF == 2) q_scale = q_scale_next;
+    lwrite(0, 0, 1);
+    gload(nt > 1 ? 1 : 0, 0, 1);
     __syncthreads();
     for (int t = 0; t < nt; ++t) {
         const int cur = t & 1;
@@ -216,10 +331,11 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ x,
 #pragma unroll
         for (int kk = 0; kk < kKb / 2; ++kk) {
             if (kk + 1 < kKb / 2) fread(cur, kk + 1, (kk + 1) & 1);
-            if (kk == 1) {
-                lwrite(cur ^ 1);  // tile t+1; past the last tile this stores a copy nobody reads
-                gload(t + 2 < nt ? t + 2 : nt - 1);
-            }
+            // tile t+1 goes registers -> LDS (codes are converted on the way) and tile t+2 memory -> registers a quarter
+            // of the chunks per k-step, between the MFMAs; past the last tile this stores a copy nobody reads
+            if (QF == 2 && kk == 0) q_scale = q_scale_next;   // the scale that came with tile t+1
+            lwrite(cur ^ 1, kk, kKb / 2);
+            gload(t + 2 < nt ? t + 2 : nt - 1, kk, kKb / 2);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -250,17 +366,18 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ x,
         }
 }
 
-bool mfma_gemm_supported(int dtype, int64_t m, int64_t k, int64_t n) {
+bool mfma_gemm_supported(int dtype, int64_t m, int64_t k, int64_t n, int quant) {
     if (dtype != 0 && dtype != 2) return false;
+    if (quant != 0 && (dtype != 2 || (quant == 2 && k % 128 != 0))) return false;
     const int64_t bk = kKb * kpc_of(dtype);
     return m > 16 && k >= bk && k % bk == 0 && n >= 1 && m < (1ll << 31) && n < (1ll << 31) - kBN && k < (1ll << 31) &&
            cdiv(m, 128) * cdiv(n, 64) < (1ll << 30);   // tile ids are ints
 }
 
-template <typename T, int BM, int BN, bool DUAL>
+template <typename T, int BM, int BN, bool DUAL, int QF = 0>
 static void launch_mfma(hipStream_t s, const MfmaLinearArgs& a) {
     constexpr int lds_bytes = 2 * kKb * ((BM + 1) * 16 + (BN + 1) * 16);
-    auto kern = gemm_mfma_kernel<T, BM, BN, DUAL>;
+    auto kern = gemm_mfma_kernel<T, BM, BN, DUAL, QF>;
     static bool configured = false;  // the attribute is per function, not per stream or device state
     if (!configured) {
         (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
@@ -271,13 +388,21 @@ static void launch_mfma(hipStream_t s, const MfmaLinearArgs& a) {
     const int64_t nt = cdiv(npad, nreal), mt = cdiv(a.m, BM);
     const unsigned grid = (unsigned)(cdiv(nt * mt, 8) * 8);
     kern<<<grid, 256, lds_bytes, s>>>((const T*)a.x, (const T*)a.wk, (const T*)a.wk2, (const T*)a.bias, (const T*)a.residual, (T*)a.y,
-                                      (int)a.m, (int)a.k, (int)a.n, (int)npad, a.act, (int)nt, (int)mt);
+                                      (int)a.m, (int)a.k, (int)a.n, (int)npad, a.act, (int)nt, (int)mt, (const T*)a.scale, (const T*)a.scale2);
 }
 
 void mfma_gemm(hipStream_t s, const MfmaLinearArgs& a) {
     // a problem with fewer 128 x 128 tiles than half the CUs runs on 64 x 64 tiles (four times the workgroups)
     const bool small = cdiv(a.m, 128) * cdiv(a.n, a.wk2 ? 64 : 128) < 128;
-    if (a.dtype == 0) {
+    if (a.quant == 1) {
+        if (a.wk2) launch_mfma<bf16_t, 128, 128, true, 1>(s, a);
+        else if (small) launch_mfma<bf16_t, 64, 64, false, 1>(s, a);
+        else launch_mfma<bf16_t, 128, 128, false, 1>(s, a);
+    } else if (a.quant == 2) {
+        if (a.wk2) launch_mfma<bf16_t, 128, 128, true, 2>(s, a);
+        else if (small) launch_mfma<bf16_t, 64, 64, false, 2>(s, a);
+        else launch_mfma<bf16_t, 128, 128, false, 2>(s, a);
+    } else if (a.dtype == 0) {
         if (a.wk2) launch_mfma<float, 128, 128, true>(s, a);
         else if (small) launch_mfma<float, 64, 64, false>(s, a);
         else launch_mfma<float, 128, 128, false>(s, a);

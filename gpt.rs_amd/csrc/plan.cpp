@@ -1045,17 +1045,18 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
                 ma.dtype = (int)x.dtype;
                 ma.x = src_ptr(st, cx, 0);
                 ma.m = x.dims[0]; ma.k = x.dims[1]; ma.n = w.dims[1];
-                // quantised weights: the k-grouped copy is built once from the dequantised matrix
+                // quantised weights: the k-grouped copy holds the codes; the kernel applies the scales on the way into LDS
                 const int kind = in.quant == 0 ? 1 : (in.quant == 1 ? 6 : 7);
-                BufferP wk = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], kind, x.dtype, ma.k, ma.n,
-                                                    in.quant ? cx.input_bufs[st.tiled_s_input] : nullptr);
+                BufferP wk = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], kind, x.dtype, ma.k, ma.n);
                 BufferP wk2;
                 ma.wk = wk->ptr;
+                ma.quant = in.quant;
+                if (in.quant) ma.scale = cx.input_bufs[st.tiled_s_input]->ptr;
                 size_t oi = linear_extra_pos(in);
                 if (in.act == 2) {
-                    wk2 = cx.be->derived_weights(cx.input_bufs[st.tiled_w2_input], kind, x.dtype, ma.k, ma.n,
-                                                 in.quant ? cx.input_bufs[st.tiled_s2_input] : nullptr);
+                    wk2 = cx.be->derived_weights(cx.input_bufs[st.tiled_w2_input], kind, x.dtype, ma.k, ma.n);
                     ma.wk2 = wk2->ptr;
+                    if (in.quant) ma.scale2 = cx.input_bufs[st.tiled_s2_input]->ptr;
                 }
                 if (in.has_bias) ma.bias = src_ptr(st, cx, oi++);
                 if (in.has_residual) ma.residual = src_ptr(st, cx, oi++);
@@ -1180,7 +1181,7 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
             size_t i = linear_extra_pos(in);
             if (in.quant) {
                 // stand-alone path of a quantised linear: the weights are dequantised into scratch and the generic
-                // kernel runs over them (the decode chain and the cached MFMA copy are the fast paths)
+                // kernel runs over them (the decode chain and the matrix-core kernels over the codes are the fast paths)
                 const size_t es = dtype_size(x.dtype);
                 char* wsp = cx.ws + st.scratch_off;
                 const size_t wbytes = align_up((size_t)a.k * a.n * es);

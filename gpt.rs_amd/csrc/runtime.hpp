@@ -182,8 +182,8 @@ class Backend {
     // kind 2: 4-column / k-pair tiled copy for the persistent decode chain (kernels_chain.hip); with
     // src2 the SwiGLU pair (gate = src, up = src2) interleaved column by column in one copy.
     // Quantised weights: kind 3 / 4: chain copies of int8 / int4 codes (src2: the partner's codes); kind 5:
-    // chain copy of int4 group scales (src2: the partner's); kind 6 / 7: MFMA copy of the dequantised int8 /
-    // int4 matrix (src = codes, src2 = scales); kind 8: 16-column tiled k-grouped copy for batched decode
+    // chain copy of int4 group scales (src2: the partner's); kind 6 / 7: k-grouped copy of the int8 / int4
+    // codes for the MFMA GEMM, which applies the scales itself; kind 8: 16-column tiled k-grouped copy for batched decode
     // (kernels_skinny.hip); kind 9 / 10: int8 / int4 codes in that tile order.
     BufferP derived_weights(const BufferP& src, int kind, DType dtype, int64_t k, int64_t n, const BufferP& src2 = nullptr);
     // Device copy of a chain's phase table, cached by content (steady-state decode repeats a few tables).

@@ -4,8 +4,8 @@ The reference has no quantisation scheme (docs/backend.md:620-632 leaves Quantiz
 backend-defined, ref-cpu answers Unimplemented), so the yardstick is the oracle's closed form of the
 scheme this build defines: codes and scales must match it bit for bit, and a quantised linear must match
 "dequantise, then dot_general" as the oracle computes it, on every execution path of the backend (the
-persistent decode chain for one bf16 row, the cached MFMA copy for prefill-sized inputs, the generic
-kernels otherwise), alone and under the epilogues the fusion pass folds into it."""
+persistent decode chain for one bf16 row, the matrix-core kernels over the codes for 2..16 rows and for
+prefill-sized inputs, the generic kernels otherwise), alone and under the epilogues the fusion pass folds into it."""
 import numpy as np
 import pytest
 
@@ -147,11 +147,48 @@ def test_linear_f32(hip, scheme, m, k, n):
 @pytest.mark.parametrize("scheme", ["w8", "w4g128"])
 @pytest.mark.parametrize("m,k,n", [(128, 3072, 1024), (64, 512, 256), (7, 384, 40)])
 def test_prefill_linear_bf16(hip, scheme, m, k, n):
-    """Several bf16 rows: the MFMA GEMM over a cached copy of the dequantised matrix where it applies."""
+    """Several bf16 rows: the MFMA GEMM over the k-grouped codes where it applies."""
     x, w = bf16_round(rnd(5, (m, k))), rnd(6, (k, n), 2.0 / np.sqrt(k))
     q, s = quantize(w, scheme)
     specs = [("Bf16", [m, k]), code_spec(scheme, k, n), ("Bf16", scale_dims(scheme, k, n))]
     run_linear(hip, lambda fb, a, b, c: F.linear_quantized(a, b, c), specs, [x, q, s], 3e-2, 2e-2, expect_chain=False)
+
+
+def dequantize_host(q, s, scheme):
+    """bf16(code * scale), the dequantiser's value (one f32 product, rounded to nearest even)."""
+    if scheme == "w8":
+        return bf16_round(q.astype(np.float32) * s.astype(np.float32)[None, :])
+    lo = (q & 0xF).astype(np.int32)
+    hi = (q >> 4).astype(np.int32)
+    lo[lo > 7] -= 16
+    hi[hi > 7] -= 16
+    codes = np.empty((2 * q.shape[0], q.shape[1]), np.float32)
+    codes[0::2], codes[1::2] = lo, hi
+    return bf16_round(codes * np.repeat(s.astype(np.float32), 128, axis=0))
+
+
+@pytest.mark.parametrize("scheme", ["w8", "w4g128"])
+@pytest.mark.parametrize("m,k,n", [(128, 3072, 1024), (300, 1024, 3000), (17, 256, 40), (1024, 512, 200)])
+def test_prefill_codes_equal_dequantised_weights(hip, scheme, m, k, n):
+    """The MFMA GEMM over the codes forms bf16(code * scale) on the way into LDS: its result must equal, BIT FOR BIT,
+    the same GEMM over the dequantised matrix given as a plain bf16 weight (same kernel, same values, same order),
+    with and without the SwiGLU pairing; 128 x 128 and 64 x 64 tiles, ragged M and N, zero and extreme columns."""
+    x = bf16_round(rnd(31, (m, k)))
+    w = weights_with_corner_cases(32, k, n)
+    w2 = rnd(33, (k, n), 2.0 / np.sqrt(k))
+    (q, s), (q2, s2) = quantize(w, scheme), quantize(w2, scheme)
+    cs_, ss_ = code_spec(scheme, k, n), ("Bf16", scale_dims(scheme, k, n))
+    built = hip.counter("derived_weights_built")
+    (got,) = hip_run(hip, prog(lambda fb, a, b, c: F.linear_quantized(a, b, c), [("Bf16", [m, k]), cs_, ss_]), [x, q, s])
+    assert hip.counter("derived_weights_built") == built + 1     # one copy: the codes (no dequantised matrix)
+    (want,) = hip_run(hip, prog(lambda fb, a, b: a.matmul(b), [("Bf16", [m, k]), ("Bf16", [k, n])]), [x, dequantize_host(q, s, scheme)])
+    assert np.array_equal(got, want), f"max diff {np.max(np.abs(got - want))}"
+    (gotp,) = hip_run(hip, prog(lambda fb, a, b, bs, c, cs: F.swiglu(F.linear_quantized(a, b, bs), F.linear_quantized(a, c, cs)),
+                                [("Bf16", [m, k]), cs_, ss_, cs_, ss_]), [x, q, s, q2, s2])
+    (wantp,) = hip_run(hip, prog(lambda fb, a, b, c: F.swiglu(a.matmul(b), a.matmul(c)),
+                                 [("Bf16", [m, k]), ("Bf16", [k, n]), ("Bf16", [k, n])]),
+                       [x, dequantize_host(q, s, scheme), dequantize_host(q2, s2, scheme)])
+    assert np.array_equal(gotp, wantp), f"pair: max diff {np.max(np.abs(gotp - wantp))}"
 
 
 @pytest.mark.parametrize("scheme", ["w8", "w4g128"])
