@@ -654,12 +654,26 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const T* __restrict__
 // scalar, the rescaling of O^T is a per-lane multiply, and P^T needs no cross-lane movement to become the B operand:
 // the k-slots of the second product are simply numbered in the order the lane holds its keys, and V^T is written to
 // LDS in that order (key bits 2 and 3 swapped).
+// max / sum of a value over the two half-waves, in every lane: v_permlane32_swap leaves the low half's value in one
+// register and the high half's in the other (one VALU instruction instead of a round trip through the LDS crossbar)
+__device__ __forceinline__ float half_max(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float half_sum(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 template <int DH>
 __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ctx, int T,
                                                                 int n_q, int n_kv, float scale_log2e) {
     constexpr int KT = 32;            // keys per tile
     constexpr int KS = DH + 8;        // K tile row stride in elements (16 bytes of padding)
-    constexpr int VS = KT + 8;        // V^T row stride in elements
+    // V^T row stride in elements.  Row d starts 8 * ((d / 8) % 4) elements in: the 16 lanes that scatter one key's
+    // d-chunks into 16 rows would otherwise all hit one bank (8 rows = 640 bytes apart, a multiple of the 128-byte
+    // bank cycle); the skew keeps fragments 16-byte aligned and spreads them over 4 bank groups (16-way conflicts cost 20 us
+    // of 88 at 1024 tokens; spreading over all 8 groups changed nothing more).
+    constexpr int VS = KT + 8 + 24;
     constexpr int ND = DH / 32;       // 32-row blocks of d in O^T
     constexpr int NK = DH / 16;       // k-steps of the score product
     constexpr int CH = KT * DH / 8;   // 16-byte chunks of a K (or V) tile
@@ -723,7 +737,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const bf16_t* __
                 const uint32_t w[4] = {vreg[j].x, vreg[j].y, vreg[j].z, vreg[j].w};
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
-                    vsm[buf][(ch * 8 + e) * VS + pos] = (bf16_t)((w[e >> 1] >> ((e & 1) * 16)) & 0xFFFFu);
+                    vsm[buf][(ch * 8 + e) * VS + 8 * (ch & 3) + pos] = (bf16_t)((w[e >> 1] >> ((e & 1) * 16)) & 0xFFFFu);
             }
         }
     };
@@ -754,18 +768,18 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const bf16_t* __
                 sc[v] = x;
                 mx = fmaxf(mx, x);
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            mx = half_max(mx);
             const float m_new = fmaxf(m_run, mx);   // finite from the first tile on: key 0 is visible to every query
-            const float corr = exp2f(m_run - m_new);
+            const float corr = __builtin_amdgcn_exp2f(m_run - m_new);
             float ls = 0.f;
             bf16x8_v pb[2];
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const float pv = exp2f(sc[v] - m_new);
+                const float pv = __builtin_amdgcn_exp2f(sc[v] - m_new);
                 ls += pv;
                 pb[v >> 3][v & 7] = (__bf16)pv;
             }
-            ls += __shfl_xor(ls, 32, 64);
+            ls = half_sum(ls);
             l_run = l_run * corr + ls;
             m_run = m_new;
 #pragma unroll
@@ -774,7 +788,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const bf16_t* __
                 for (int v = 0; v < 16; ++v) acc_o[db][v] *= corr;
 #pragma unroll
                 for (int i = 0; i < 2; ++i) {
-                    const bf16x8_v vf = *reinterpret_cast<const bf16x8_v*>(&vsm[buf][(db * 32 + col) * VS + 16 * i + 8 * half]);
+                    const bf16x8_v vf = *reinterpret_cast<const bf16x8_v*>(&vsm[buf][(db * 32 + col) * VS + 8 * ((col >> 3) & 3) + 16 * i + 8 * half]);
                     acc_o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[i], acc_o[db], 0, 0, 0);
                 }
             }
