@@ -665,7 +665,7 @@ __device__ __forceinline__ float half_sum(float x) {
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 template <int DH>
-__global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ctx, int T,
+__global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ctx, int T,
                                                                 int n_q, int n_kv, float scale_log2e) {
     constexpr int KT = 32;            // keys per tile
     constexpr int KS = DH + 8;        // K tile row stride in elements (16 bytes of padding)
@@ -712,17 +712,18 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const bf16_t* __
         for (int v = 0; v < 16; ++v) acc_o[db][v] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;
 
-    uint4 kreg[CPT], vreg[CPT];
+    // native vectors and unconditional loads (the chunk index is clamped instead): with HIP's uint4 struct and a
+    // guarded load the compiler keeps these in scratch memory and waits for every load right where it is issued
+    typedef uint32_t u32x4_s __attribute__((ext_vector_type(4)));
+    u32x4_s kreg[CPT], vreg[CPT];
     auto gload = [&](int t) {
 #pragma unroll
         for (int j = 0; j < CPT; ++j) {
-            const int c = tid + 256 * j;
-            if (CH % 256 == 0 || c < CH) {
-                const int r = c / (DH / 8), ch = c % (DH / 8);
-                const int64_t key = min(t * KT + r, T - 1);
-                kreg[j] = *reinterpret_cast<const uint4*>(qkv + key * P + koff + ch * 8);
-                vreg[j] = *reinterpret_cast<const uint4*>(qkv + key * P + voff + ch * 8);
-            }
+            const int c = min(tid + 256 * j, CH - 1);
+            const int r = c / (DH / 8), ch = c % (DH / 8);
+            const int64_t key = min(t * KT + r, T - 1);
+            kreg[j] = *reinterpret_cast<const u32x4_s*>(qkv + key * P + koff + ch * 8);
+            vreg[j] = *reinterpret_cast<const u32x4_s*>(qkv + key * P + voff + ch * 8);
         }
     };
     auto lwrite = [&](int buf) {
@@ -731,10 +732,11 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const bf16_t* __
             const int c = tid + 256 * j;
             if (CH % 256 == 0 || c < CH) {
                 const int r = c / (DH / 8), ch = c % (DH / 8);
-                *reinterpret_cast<uint4*>(&ksm[buf][r * KS + ch * 8]) = kreg[j];
+                *reinterpret_cast<u32x4_s*>(&ksm[buf][r * KS + ch * 8]) = kreg[j];
                 // key r goes to k-slot position p: bits 2 and 3 of r swapped
                 const int pos = (r & 0x13) | ((r & 4) << 1) | ((r & 8) >> 1);
-                const uint32_t w[4] = {vreg[j].x, vreg[j].y, vreg[j].z, vreg[j].w};
+                const uint32_t w0 = vreg[j].x, w1 = vreg[j].y, w2 = vreg[j].z, w3 = vreg[j].w;
+                const uint32_t w[4] = {w0, w1, w2, w3};
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
                     vsm[buf][(ch * 8 + e) * VS + 8 * (ch & 3) + pos] = (bf16_t)((w[e >> 1] >> ((e & 1) * 16)) & 0xFFFFu);
@@ -760,32 +762,45 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(const bf16_t* __
             }
             const int qrow = q0 + col;
             const int kbase = t * KT + 4 * half;
+            // raw scores: the (positive) scale is applied inside the exponent's fma; only a tile that reaches past the
+            // wave's first row holds keys to mask
+            if (t * KT + KT - 1 > q0) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int key = kbase + 8 * (v >> 2) + (v & 3);
+                    if (key > qrow) sc[v] = -INFINITY;
+                }
+            }
             float mx = -INFINITY;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int key = kbase + 8 * (v >> 2) + (v & 3);
-                const float x = key <= qrow ? sc[v] * scale_log2e : -INFINITY;
-                sc[v] = x;
-                mx = fmaxf(mx, x);
-            }
-            mx = half_max(mx);
-            const float m_new = fmaxf(m_run, mx);   // finite from the first tile on: key 0 is visible to every query
-            const float corr = __builtin_amdgcn_exp2f(m_run - m_new);
+            for (int v = 0; v < 16; ++v) mx = fmaxf(mx, sc[v]);
+            mx = half_max(mx) * scale_log2e;
+            // The reference point of the exponentials follows the running maximum lazily: it moves only when the
+            // maximum has grown by more than 2^8 (probabilities then reach 2^8 at most, harmless in bf16 / f32, and
+            // the quotient O / l does not depend on the reference point).  Most tiles therefore leave O^T unscaled,
+            // and a wave skips the 64 multiplies (the accumulators live in AGPRs: 128 more moves) unless a lane moved.
+            const bool move = mx > m_run + 8.0f;    // first tile: m_run = -inf, key 0 is visible to every query
+            const float m_new = move ? mx : m_run;
+            const float corr = move ? __builtin_amdgcn_exp2f(m_run - m_new) : 1.0f;
             float ls = 0.f;
             bf16x8_v pb[2];
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const float pv = __builtin_amdgcn_exp2f(sc[v] - m_new);
+                const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[v], scale_log2e, -m_new));
                 ls += pv;
                 pb[v >> 3][v & 7] = (__bf16)pv;
             }
             ls = half_sum(ls);
             l_run = l_run * corr + ls;
             m_run = m_new;
+            if (__builtin_amdgcn_ballot_w64(move) != 0) {
+#pragma unroll
+                for (int db = 0; db < ND; ++db)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) acc_o[db][v] *= corr;
+            }
 #pragma unroll
             for (int db = 0; db < ND; ++db) {
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc_o[db][v] *= corr;
 #pragma unroll
                 for (int i = 0; i < 2; ++i) {
                     const bf16x8_v vf = *reinterpret_cast<const bf16x8_v*>(&vsm[buf][(db * 32 + col) * VS + 8 * ((col >> 3) & 3) + 16 * i + 8 * half]);
