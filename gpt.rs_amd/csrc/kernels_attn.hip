@@ -838,11 +838,13 @@ __device__ __forceinline__ f32x16_v mma_f32x4(const f32x4_v& a, const f32x4_v& b
 }
 
 template <int DH>
-__global__ __launch_bounds__(256) void attn_prefill_mfma_f32_kernel(const float* __restrict__ qkv, float* __restrict__ ctx, int T,
+__global__ __launch_bounds__(256, 2) void attn_prefill_mfma_f32_kernel(const float* __restrict__ qkv, float* __restrict__ ctx, int T,
                                                                     int n_q, int n_kv, float scale_log2e) {
     constexpr int KT = 32;            // keys per tile
     constexpr int KS = DH + 4;        // K tile row stride in elements (16 bytes of padding)
-    constexpr int VS = KT + 4;        // V^T row stride in elements
+    // V^T row stride in elements; row d starts 4 * ((d / 4) % 8) elements in, which spreads the lanes that scatter one
+    // key's d-chunks over the banks (as in the bf16 kernel)
+    constexpr int VS = KT + 4 + 28;
     constexpr int ND = DH / 32;       // 32-row blocks of d in O^T
     constexpr int NK = DH / 8;        // k-steps of the score product (8 d each)
     constexpr int CH = KT * DH / 4;   // 16-byte chunks of a K (or V) tile
@@ -884,13 +886,11 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_f32_kernel(const float*
     auto gload = [&](int t) {
 #pragma unroll
         for (int j = 0; j < CPT; ++j) {
-            const int c = tid + 256 * j;
-            if (CH % 256 == 0 || c < CH) {
-                const int r = c / (DH / 4), ch = c % (DH / 4);
-                const int64_t key = min(t * KT + r, T - 1);
-                kreg[j] = *reinterpret_cast<const f32x4_v*>(qkv + key * P + koff + ch * 4);
-                vreg[j] = *reinterpret_cast<const f32x4_v*>(qkv + key * P + voff + ch * 4);
-            }
+            const int c = min(tid + 256 * j, CH - 1);   // unconditional loads: see the bf16 kernel
+            const int r = c / (DH / 4), ch = c % (DH / 4);
+            const int64_t key = min(t * KT + r, T - 1);
+            kreg[j] = *reinterpret_cast<const f32x4_v*>(qkv + key * P + koff + ch * 4);
+            vreg[j] = *reinterpret_cast<const f32x4_v*>(qkv + key * P + voff + ch * 4);
         }
     };
     auto lwrite = [&](int buf) {
@@ -901,7 +901,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_f32_kernel(const float*
                 const int r = c / (DH / 4), ch = c % (DH / 4);
                 *reinterpret_cast<f32x4_v*>(&ksm[buf][r * KS + ch * 4]) = kreg[j];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) vsm[buf][(ch * 4 + e) * VS + r] = vreg[j][e];
+                for (int e = 0; e < 4; ++e) vsm[buf][(ch * 4 + e) * VS + 4 * (ch & 7) + r] = vreg[j][e];
             }
         }
     };
@@ -923,35 +923,43 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_f32_kernel(const float*
             }
             const int qrow = q0 + col;
             const int kbase = t * KT + 4 * half;
+            if (t * KT + KT - 1 > q0) {   // only a tile that reaches past the wave's first row holds keys to mask
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int key = kbase + 8 * (v >> 2) + (v & 3);
+                    if (key > qrow) sc[v] = -INFINITY;
+                }
+            }
             float mx = -INFINITY;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int key = kbase + 8 * (v >> 2) + (v & 3);
-                const float x = key <= qrow ? sc[v] * scale_log2e : -INFINITY;
-                sc[v] = x;
-                mx = fmaxf(mx, x);
-            }
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const float m_new = fmaxf(m_run, mx);
-            const float corr = exp2f(m_run - m_new);
+            for (int v = 0; v < 16; ++v) mx = fmaxf(mx, sc[v]);
+            mx = half_max(mx) * scale_log2e;
+            // lazy reference point and wave-wide skip of the rescaling, as in the bf16 kernel
+            const bool move = mx > m_run + 8.0f;
+            const float m_new = move ? mx : m_run;
+            const float corr = move ? __builtin_amdgcn_exp2f(m_run - m_new) : 1.0f;
             float ls = 0.f;
             f32x4_v pf[4];
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const float pv = exp2f(sc[v] - m_new);
+                const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[v], scale_log2e, -m_new));
                 ls += pv;
                 pf[v >> 2][v & 3] = pv;
             }
-            ls += __shfl_xor(ls, 32, 64);
+            ls = half_sum(ls);
             l_run = l_run * corr + ls;
             m_run = m_new;
+            if (__builtin_amdgcn_ballot_w64(move) != 0) {
+#pragma unroll
+                for (int db = 0; db < ND; ++db)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) acc_o[db][v] *= corr;
+            }
 #pragma unroll
             for (int db = 0; db < ND; ++db) {
 #pragma unroll
-                for (int v = 0; v < 16; ++v) acc_o[db][v] *= corr;
-#pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const f32x4_v vf = *reinterpret_cast<const f32x4_v*>(&vsm[buf][(db * 32 + col) * VS + 8 * i + 4 * half]);
+                    const f32x4_v vf = *reinterpret_cast<const f32x4_v*>(&vsm[buf][(db * 32 + col) * VS + 4 * ((col >> 2) & 7) + 8 * i + 4 * half]);
                     acc_o[db] = mma_f32x4(vf, pf[i], acc_o[db]);
                 }
             }
