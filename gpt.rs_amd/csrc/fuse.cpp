@@ -861,6 +861,84 @@ struct Fuser {
         }
     }
 
+    // DynamicUpdateSlice(base, view(x), starts), where view is a chain of Slice / Reshape / Transpose instructions
+    // that nothing else reads, copies straight out of x: the chain only renumbers elements, so its composition is a
+    // set of strides and an offset inside x.  (A prefill writes the K and V rows of the packed projection into the
+    // caches this way: four copies per layer become none.)
+    static bool reshape_view(const std::vector<int64_t>& od, const std::vector<int64_t>& os, const std::vector<int64_t>& nd,
+                             std::vector<int64_t>& ns) {
+        // strides of the new shape over the same elements, if the old view allows it without a copy
+        ns.assign(nd.size(), 0);
+        size_t oi = 0, ni = 0;
+        while (oi < od.size() && ni < nd.size()) {
+            // grow a group of old axes and a group of new axes until they hold the same number of elements
+            size_t oj = oi + 1, nj = ni + 1;
+            int64_t op = od[oi], np = nd[ni];
+            while (op != np) {
+                if (op < np) { if (oj >= od.size()) return false; op *= od[oj++]; }
+                else { if (nj >= nd.size()) return false; np *= nd[nj++]; }
+            }
+            // the old group must be contiguous in itself (axes of extent 1 carry no constraint)
+            for (size_t k = oi; k + 1 < oj; ++k)
+                if (od[k] != 1 && od[k + 1] != 1 && os[k] != os[k + 1] * od[k + 1]) return false;
+            int64_t inner = 1;
+            for (size_t k = oj; k-- > oi;) if (od[k] != 1) { inner = os[k]; break; }
+            for (size_t k = nj; k-- > ni;) { ns[k] = inner; inner *= nd[k]; }
+            oi = oj; ni = nj;
+        }
+        for (; oi < od.size(); ++oi) if (od[oi] != 1) return false;
+        for (; ni < nd.size(); ++ni) { if (nd[ni] != 1) return false; ns[ni] = 1; }
+        return true;
+    }
+    void pass_update_views() {
+        const std::vector<int> uses = count_uses();
+        for (auto& in : fn.body) {
+            if (in.dead || in.op != OpKind::DynamicUpdateSlice || !in.view_dims.empty()) continue;
+            // the chain, from the update up to its root
+            std::vector<const Instr*> chain;
+            int v = in.operands[1].value;
+            for (;;) {
+                const Instr* p = producer(v);
+                if (!p || uses[v] != 1 || p->operands.empty() || p->operands[0].value < 0) break;
+                if (p->op != OpKind::Slice && p->op != OpKind::Reshape && p->op != OpKind::Transpose) break;
+                chain.push_back(p);
+                v = p->operands[0].value;
+            }
+            bool copies = false;
+            for (const Instr* p : chain) copies = copies || p->op != OpKind::Reshape;
+            if (!copies) continue;   // reshapes alone cost nothing
+            const Spec* root = spec_of(v);
+            if (!root || root->rank() > k::kMaxRank) continue;
+            std::vector<int64_t> dims = root->dims, strides(root->rank(), 1);
+            for (int i = root->rank() - 2; i >= 0; --i) strides[i] = strides[i + 1] * dims[i + 1];
+            int64_t off = 0;
+            bool ok = true;
+            for (size_t c = chain.size(); ok && c-- > 0;) {
+                const Instr* p = chain[c];
+                if (p->op == OpKind::Slice) {
+                    for (size_t i = 0; i < dims.size(); ++i) off += p->a[i] * strides[i];
+                    dims = p->b;
+                } else if (p->op == OpKind::Transpose) {
+                    std::vector<int64_t> d2(dims.size()), s2(dims.size());
+                    for (size_t i = 0; i < dims.size(); ++i) { d2[i] = dims[p->a[i]]; s2[i] = strides[p->a[i]]; }
+                    dims = d2; strides = s2;
+                } else {
+                    std::vector<int64_t> s2;
+                    ok = reshape_view(dims, strides, p->out_specs[0].dims, s2);
+                    dims = p->out_specs[0].dims; strides = s2;
+                }
+                ok = ok && (int)dims.size() <= k::kMaxRank;
+            }
+            const Spec* upd = spec_of(in.operands[1].value);
+            if (!ok || !upd || dims != upd->dims) continue;
+            in.view_dims = dims;
+            in.view_strides = strides;
+            in.view_off = off;
+            in.operands[1].value = v;
+            ++fused;
+        }
+    }
+
     void dce() {
         std::vector<bool> live(fn.max_value_id + 1, false);
         for (int r : fn.result_ids) live[r] = true;
@@ -927,6 +1005,8 @@ int fuse_function(Function& fn) {
     f.pass_tiled_linear();
     f.dce();
     f.pass_scalar_rhs();
+    f.dce();
+    f.pass_update_views();
     f.dce();
     f.toposort();
     return f.fused;

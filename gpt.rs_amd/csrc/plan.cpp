@@ -267,11 +267,13 @@ void Builder::validate(Instr& in) {
             const Spec& x = spec_of(in, 0);
             const Spec& u = spec_of(in, 1);
             const Spec& st = spec_of(in, 2);
+            // after fusion operand 1 may be the tensor the update is a view of (in.view_dims is then the update's shape)
+            const std::vector<int64_t>& udims = in.view_dims.empty() ? u.dims : in.view_dims;
             expect(x.dtype == u.dtype, "dynamic_update_slice dtype mismatch");
-            expect(u.rank() == x.rank() && in.a == u.dims, "dynamic_update_slice sizes must match update shape");
+            expect((int)udims.size() == x.rank() && in.a == udims, "dynamic_update_slice sizes must match update shape");
             expect(st.dtype == DType::SI32 && st.rank() == 1 && st.dims[0] == x.rank(), "dynamic_update_slice starts must be si32[rank]");
             for (int i = 0; i < x.rank(); ++i)
-                if (u.dims[i] > x.dims[i]) fail_spec("dynamic_update_slice update exceeds base dimension");
+                if (udims[i] > x.dims[i]) fail_spec("dynamic_update_slice update exceeds base dimension");
             expect(out == x, "dynamic_update_slice output spec mismatch");
             break;
         }
@@ -451,13 +453,15 @@ void Builder::describe(Step& st) {
         }
         case OpKind::DynamicUpdateSlice: {
             const Spec& x = spec_of(in, 0);
-            const Spec& u = spec_of(in, 1);
+            // the update itself, or a view of operand 1 that the fusion pass composed (shape, strides, offset)
+            const bool view = !in.view_dims.empty();
+            const std::vector<int64_t> udims = view ? in.view_dims : spec_of(in, 1).dims;
             const auto xs = row_major_strides(x.dims);
-            k::CopyDesc c = make_copy(u.dims, xs, row_major_strides(u.dims), 0, 0);
+            k::CopyDesc c = make_copy(udims, xs, view ? in.view_strides : row_major_strides(udims), 0, view ? in.view_off : 0);
             c.dyn = 2;
             c.dyn_rank = x.rank();
             if (x.rank() > k::kMaxRank) fail_unimpl("dynamic_update_slice", "rank above 6");
-            for (int i = 0; i < x.rank(); ++i) { c.dyn_max[i] = x.dims[i] - u.dims[i]; c.dyn_stride[i] = c.dyn_max[i] ? xs[i] : 0; }
+            for (int i = 0; i < x.rank(); ++i) { c.dyn_max[i] = x.dims[i] - udims[i]; c.dyn_stride[i] = c.dyn_max[i] ? xs[i] : 0; }
             st.copies.push_back(c);
             st.elem_size = widen_copies(st.copies, es_of(out));
             break;

@@ -115,6 +115,10 @@ struct Instr {
     int act = 0;                      // FLinear epilogue: 0 none, 1 gelu, 2 swiglu (dual weights)
     bool has_bias = false, has_residual = false;
     float fparam[4] = {0.f, 0.f, 0.f, 0.f};  // FGelu: half, divisor, one
+    // DynamicUpdateSlice whose update is a view (Slice / Reshape / Transpose chain) of operand 1: the update's shape,
+    // and its element strides and offset inside operand 1; empty when operand 1 is the update itself
+    std::vector<int64_t> view_dims, view_strides;
+    int64_t view_off = 0;
     bool mfma = false;                       // FLinear: prefill GEMM over the k-grouped weight copy
     bool tiled = false;                      // FLinear: decode GEMV over the column-tiled weight copy
     bool norm = false;                       // FLinear: RMSNorm of x fused in (last operand = gamma; eps, scale)

@@ -7,7 +7,7 @@ import pytest
 
 from parity import FunctionBuilder, Program, assert_close, check_program, hip_run, oracle_run
 from gptrs_amd import functional as F
-from gptrs_amd.ptir import Tensor
+from gptrs_amd.ptir import Tensor, f32_to_bf16_bits
 
 pytestmark = pytest.mark.gpu
 
@@ -132,6 +132,39 @@ def test_dynamic_ops_rank3_exact(hip):
         p = prog(lambda fb, b, u, s: [b.dynamic_update_slice(u, s, [4, 1, 8]), b.dynamic_slice(s, [4, 2, 8])],
                  [("F32", [4, 16, 8]), ("F32", [4, 1, 8]), ("Si32", [3])])
         check_program(hip, p, [base, upd, st], atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", ["F32", "Bf16"])
+def test_update_from_a_view_exact(hip, dtype):
+    """DynamicUpdateSlice whose update is a Slice / Reshape / Transpose chain of another tensor: the fusion pass copies
+    straight out of that tensor (the K / V rows of a packed projection go into the caches this way).  Bit-exact against
+    the oracle, fusion on and off, including a chain whose reshape cannot be expressed as strides (merges transposed
+    axes) and one whose intermediate value is also a result."""
+    x = rng_uniform(11, (6, 20))
+    if dtype == "Bf16":
+        x = (f32_to_bf16_bits(x).astype(np.uint32) << 16).view(np.float32)
+    base = np.zeros((3, 10, 4), np.float32)
+    st = np.array([0, 2, 0], np.int32)
+    specs = [(dtype, [6, 20]), (dtype, [3, 10, 4]), ("Si32", [3])]
+
+    def heads(fb, a, b, s):          # columns 4..16 as 3 heads of 4, head-major
+        u = a.slice([0, 4], [6, 12]).reshape([6, 3, 4]).transpose([1, 0, 2])
+        return b.dynamic_update_slice(u, s, [3, 6, 4])
+
+    def merged(fb, a, b, s):         # transpose, then a reshape that merges the transposed axes: needs a real copy
+        u = a.slice([0, 0], [6, 12]).transpose([1, 0]).reshape([3, 6, 4])
+        return b.dynamic_update_slice(u, s, [3, 6, 4])
+
+    def shared(fb, a, b, s):         # the view is a result as well: it must still be materialised
+        u = a.slice([0, 8], [6, 12]).reshape([6, 3, 4]).transpose([1, 0, 2])
+        return [b.dynamic_update_slice(u, s, [3, 6, 4]), u]
+
+    def split(fb, a, b, s):          # a reshape that splits the sliced axis after a transpose of the outer ones
+        u = a.reshape([2, 3, 20]).transpose([1, 0, 2]).slice([0, 0, 4], [3, 2, 16]).reshape([3, 2, 4, 4]).reshape([3, 8, 4])
+        return b.dynamic_update_slice(u, s, [3, 8, 4])
+
+    for build in (heads, merged, shared, split):
+        check_program(hip, prog(build, specs), [x, base, st], atol=0, rtol=0)
 
 
 # ------------------------------------------------------------------ float ops
