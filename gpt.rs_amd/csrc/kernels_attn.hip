@@ -247,6 +247,16 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const T* __restrict__ 
     }
 }
 
+// max / sum of a value over the two half-waves, in every lane: v_permlane32_swap leaves the low half's value in one
+// register and the high half's in the other (one VALU instruction instead of a round trip through the LDS crossbar)
+__device__ __forceinline__ float half_max(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float half_sum(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 // bf16 decode attention with the scores on the matrix cores.  grid (n_kv, nsplit, batch), 256 threads; wave w of a
 // workgroup takes the 32-key tiles w, w+4, ... of the workgroup's chunk.  Per tile
 //   S^T[key, q] = K[key, :] . Q[q, :]   v_mfma_f32_32x32x16_bf16, A = cache rows straight from memory (lane = key row),
@@ -365,16 +375,16 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(const bf16_t* __r
                 sc[v] = x;
                 mx = fmaxf(mx, x);
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            mx = half_max(mx);
             const float m_new = fmaxf(m_run, mx);   // finite: the tile holds at least one attended key
-            const float corr = exp2f(m_run - m_new);
+            const float corr = __builtin_amdgcn_exp2f(m_run - m_new);
             float ls = 0.f;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                sc[v] = exp2f(sc[v] - m_new);
+                sc[v] = __builtin_amdgcn_exp2f(sc[v] - m_new);
                 ls += sc[v];
             }
-            ls += __shfl_xor(ls, 32, 64);
+            ls = half_sum(ls);
             l_run = l_run * corr + ls;
             m_run = m_new;
             if (col < G) {
@@ -654,16 +664,6 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const T* __restrict__
 // scalar, the rescaling of O^T is a per-lane multiply, and P^T needs no cross-lane movement to become the B operand:
 // the k-slots of the second product are simply numbered in the order the lane holds its keys, and V^T is written to
 // LDS in that order (key bits 2 and 3 swapped).
-// max / sum of a value over the two half-waves, in every lane: v_permlane32_swap leaves the low half's value in one
-// register and the high half's in the other (one VALU instruction instead of a round trip through the LDS crossbar)
-__device__ __forceinline__ float half_max(float x) {
-    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-__device__ __forceinline__ float half_sum(float x) {
-    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-}
 template <int DH>
 __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ctx, int T,
                                                                 int n_q, int n_kv, float scale_log2e) {
