@@ -205,7 +205,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ x,
 #pragma unroll
     for (int j = 0; j < CA; ++j) {
         const int c = tid + 256 * j;
-        const int kb = c & 7, row = c >> 3;
+        const int kb = c % kKb, row = c / kKb;
         int m = m0 + row;
         if (m > M - 1) m = M - 1;
         a_src[j] = x + (int64_t)m * K + kb * KPC;
