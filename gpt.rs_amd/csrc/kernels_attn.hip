@@ -669,11 +669,13 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const bf16_t*
                                                                 int n_q, int n_kv, float scale_log2e) {
     constexpr int KT = 32;            // keys per tile
     constexpr int KS = DH + 8;        // K tile row stride in elements (16 bytes of padding)
-    // V^T row stride in elements.  Row d starts 8 * ((d / 8) % 4) elements in: the 16 lanes that scatter one key's
-    // d-chunks into 16 rows would otherwise all hit one bank (8 rows = 640 bytes apart, a multiple of the 128-byte
-    // bank cycle); the skew keeps fragments 16-byte aligned and spreads them over 4 bank groups (16-way conflicts cost 20 us
-    // of 88 at 1024 tokens; spreading over all 8 groups changed nothing more).
-    constexpr int VS = KT + 8 + 24;
+    // V^T rows: stride VS elements, row d starts 8 * ((d / 8) % 8) elements in.  Two access patterns must spread over
+    // the 32 banks: a fragment read (8 lanes = 8 consecutive rows, 16 bytes each) wants the row stride to be an odd
+    // multiple of 16 bytes modulo 128 (104 elements = 208 bytes: rows land 20 banks apart), and the scatter of one key's
+    // d-chunks (16 lanes, 8 rows apart, same position) would hit a single bank whatever the stride (8 rows are a
+    // multiple of 128 bytes apart), which the skew spreads over 8 groups of 4 banks.  Measured at 1024 tokens: no skew
+    // 88 us per layer, skew with 128-byte rows (reads 8-way conflicting) 68 us.
+    constexpr int VS = 104;
     constexpr int ND = DH / 32;       // 32-row blocks of d in O^T
     constexpr int NK = DH / 16;       // k-steps of the score product
     constexpr int CH = KT * DH / 8;   // 16-byte chunks of a K (or V) tile
@@ -739,7 +741,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const bf16_t*
                 const uint32_t w[4] = {w0, w1, w2, w3};
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
-                    vsm[buf][(ch * 8 + e) * VS + 8 * (ch & 3) + pos] = (bf16_t)((w[e >> 1] >> ((e & 1) * 16)) & 0xFFFFu);
+                    vsm[buf][(ch * 8 + e) * VS + 8 * (ch & 7) + pos] = (bf16_t)((w[e >> 1] >> ((e & 1) * 16)) & 0xFFFFu);
             }
         }
     };
@@ -803,7 +805,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const bf16_t*
             for (int db = 0; db < ND; ++db) {
 #pragma unroll
                 for (int i = 0; i < 2; ++i) {
-                    const bf16x8_v vf = *reinterpret_cast<const bf16x8_v*>(&vsm[buf][(db * 32 + col) * VS + 8 * ((col >> 3) & 3) + 16 * i + 8 * half]);
+                    const bf16x8_v vf = *reinterpret_cast<const bf16x8_v*>(&vsm[buf][(db * 32 + col) * VS + 8 * (((db & 1) << 2) | (col >> 3)) + 16 * i + 8 * half]);
                     acc_o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[i], acc_o[db], 0, 0, 0);
                 }
             }
