@@ -907,6 +907,13 @@ struct Fuser {
             bool copies = false;
             for (const Instr* p : chain) copies = copies || p->op != OpKind::Reshape;
             if (!copies) continue;   // reshapes alone cost nothing
+            // a view of the base itself must be taken before the base is written (the update may run in place)
+            auto storage = [&](int x) {
+                for (const Instr* p = producer(x); p && p->op == OpKind::Reshape && p->operands[0].value >= 0; p = producer(x))
+                    x = p->operands[0].value;
+                return x;
+            };
+            if (storage(v) == storage(in.operands[0].value)) continue;
             const Spec* root = spec_of(v);
             if (!root || root->rank() > k::kMaxRank) continue;
             std::vector<int64_t> dims = root->dims, strides(root->rank(), 1);

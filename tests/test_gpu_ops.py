@@ -5,7 +5,7 @@ parity-case catalogue (crates/gpt-rs-backend-tests/src/lib.rs:99-261)."""
 import numpy as np
 import pytest
 
-from parity import FunctionBuilder, Program, assert_close, check_program, hip_run, oracle_run
+from parity import FunctionBuilder, Program, assert_close, check_program, hip_run, oracle_run, to_bytes
 from gptrs_amd import functional as F
 from gptrs_amd.ptir import Tensor, f32_to_bf16_bits
 
@@ -165,6 +165,27 @@ def test_update_from_a_view_exact(hip, dtype):
 
     for build in (heads, merged, shared, split):
         check_program(hip, prog(build, specs), [x, base, st], atol=0, rtol=0)
+
+    # a view of the base itself, overlapping the rows it is written to: the view must be taken before the write
+    own = rng_uniform(12, (3, 10, 4))
+    if dtype == "Bf16":
+        own = (f32_to_bf16_bits(own).astype(np.uint32) << 16).view(np.float32)
+
+    def overlap(fb, b, s):
+        return b.dynamic_update_slice(b.slice([0, 0, 0], [3, 6, 4]), s, [3, 6, 4])
+
+    def overlap_reshaped(fb, b, s):
+        flat = b.reshape([30, 4])
+        u = flat.reshape([3, 10, 4]).slice([0, 1, 0], [3, 6, 4])
+        return flat.reshape([3, 10, 4]).dynamic_update_slice(u, s, [3, 6, 4])
+
+    for build in (overlap, overlap_reshaped):
+        p = prog(build, [(dtype, [3, 10, 4]), ("Si32", [3])])
+        check_program(hip, p, [own, st], atol=0, rtol=0)
+        hs = [hip.materialize(sp, to_bytes(a, sp.dtype)) for sp, a in zip(p.param_specs, [own, st])]
+        (got,) = hip.run_program(p, hs, [True, False])          # donated base: the update runs in place
+        (want,) = oracle_run(p, [own, st])
+        assert np.array_equal(hip.to_numpy(got), want)
 
 
 # ------------------------------------------------------------------ float ops
