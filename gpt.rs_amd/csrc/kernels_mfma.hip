@@ -159,8 +159,12 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 // QF: 0 = wk / wk2 hold values; 1 / 2 = they hold int8 / int4 codes (see k8_codes_kernel) and `scale` / `scale2` the
 // scale tensors of the two matrices ([N] per column, or [K / 128, N] per group of 128 k), T = bf16 only.
-template <typename T, int BM, int BN, bool DUAL, int QF>
-__global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ x, const T* __restrict__ wk,
+// KW: wave groups per workgroup.  With KW = 2 a workgroup has 8 waves: both groups of four own the same 2 x 2 layout of
+// outputs, group g multiplies k-steps [2 g, 2 g + 2) of every tile, and the second group's accumulators reach the
+// first through LDS before the epilogue.  A launch with fewer tiles than two per CU then still has 8 waves per CU to
+// cover LDS and barrier waits (what two co-resident workgroups do for the launches with many tiles).
+template <typename T, int BM, int BN, bool DUAL, int QF, int KW>
+__global__ __launch_bounds__(256 * KW) void gemm_mfma_kernel(const T* __restrict__ x, const T* __restrict__ wk,
                                                         const T* __restrict__ wk2, const T* __restrict__ bias,
                                                         const T* __restrict__ residual, T* __restrict__ y,
                                                         int M, int K, int N, int Npad, int act, int NT, int MT,
@@ -171,14 +175,18 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ x,
     constexpr int SA = (BM + 1) * 16, SB = (BN + 1) * 16;     // bytes between k-groups
     constexpr int STAGE = kKb * (SA + SB);
     constexpr int TM = BM / 64, TN = BN / 64;
-    constexpr int CA = BM * kKb / 256, CB = BN * kKb / 256;   // 16-byte chunks per thread per tile
+    constexpr int NTH = 256 * KW;
+    constexpr int KSTEPS = kKb / 2 / KW;                      // k-steps (2 k-groups each) per wave and tile
+    constexpr int CA = BM * kKb / NTH, CB = BN * kKb / NTH;   // 16-byte chunks per thread per tile
+    static_assert(KW == 1 || (!DUAL && KSTEPS >= 1 && CA >= 1 && CB >= 1), "k-split layout");
     constexpr int WN = BN / 2;                                // B-tile columns per wave column
     constexpr int NREAL = DUAL ? BN / 2 : BN;                 // output columns per block
     static_assert(!DUAL || TN % 2 == 0, "dual tiles need an even number of column fragments");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wg = wave >> 2;               // wave group
+    const int wm = (wave >> 1) & 1, wn = wave & 1;
     // Tile order.  Consecutive workgroup ids go to the 8 XCDs in turn and each XCD has its own L2, so XCD c takes
     // the contiguous range [c * per, (c + 1) * per) of a grouped order in which up to 8 row blocks of one column
     // tile follow each other: the ~32 workgroups an XCD runs at a time then cover 8 row blocks x 4 column tiles, a
@@ -204,7 +212,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ x,
     int a_dst[CA], b_dst[CB];
 #pragma unroll
     for (int j = 0; j < CA; ++j) {
-        const int c = tid + 256 * j;
+        const int c = tid + NTH * j;
         const int kb = c % kKb, row = c / kKb;
         int m = m0 + row;
         if (m > M - 1) m = M - 1;
@@ -213,7 +221,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ x,
     }
 #pragma unroll
     for (int j = 0; j < CB; ++j) {
-        const int c = tid + 256 * j;
+        const int c = tid + NTH * j;
         const int bc = c % BN, bkb = c / BN;
         int col = n0 + bc;
         const T* src = wk;
@@ -233,7 +241,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ x,
     const T* s_src = nullptr;
     float q_scale = 0.f, q_scale_next = 0.f;
     if (QF != 0) {
-        static_assert(256 % BN == 0, "one tile column per thread");
+        static_assert(NTH % BN == 0, "one tile column per thread");
         const int bc = tid % BN;
         int col = n0 + bc;
         const T* sp = scale;
@@ -327,15 +335,15 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ x,
     __syncthreads();
     for (int t = 0; t < nt; ++t) {
         const int cur = t & 1;
-        fread(cur, 0, 0);
+        fread(cur, wg * KSTEPS, 0);
 #pragma unroll
-        for (int kk = 0; kk < kKb / 2; ++kk) {
-            if (kk + 1 < kKb / 2) fread(cur, kk + 1, (kk + 1) & 1);
+        for (int kk = 0; kk < KSTEPS; ++kk) {
+            if (kk + 1 < KSTEPS) fread(cur, wg * KSTEPS + kk + 1, (kk + 1) & 1);
             // tile t+1 goes registers -> LDS (codes are converted on the way) and tile t+2 memory -> registers a quarter
             // of the chunks per k-step, between the MFMAs; past the last tile this stores a copy nobody reads
             if (QF == 2 && kk == 0) q_scale = q_scale_next;   // the scale that came with tile t+1
-            lwrite(cur ^ 1, kk, kKb / 2);
-            gload(t + 2 < nt ? t + 2 : nt - 1, kk, kKb / 2);
+            lwrite(cur ^ 1, kk, KSTEPS);
+            gload(t + 2 < nt ? t + 2 : nt - 1, kk, KSTEPS);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -345,6 +353,27 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(const T* __restrict__ x,
         __syncthreads();
     }
 
+    if (KW == 2) {
+        // the second wave group hands its sums over through LDS (the tiles in it are dead: the loop ended on a barrier)
+        float* xch = reinterpret_cast<float*>(lds) + (wave & 3) * (TM * TN * 16 * 64);
+        static_assert(KW == 1 || 4 * TM * TN * 16 * 64 * 4 <= 2 * STAGE, "exchange area fits the staging buffers");
+        if (wg == 1) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) xch[((i * TN + j) * 16 + v) * 64 + lane] = acc[i][j][v];
+        }
+        __syncthreads();
+        if (wg == 1) return;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] += xch[((i * TN + j) * 16 + v) * 64 + lane];
+    }
     // epilogue: lane holds column (lane % 32), rows 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 tile
     constexpr int TNO = DUAL ? TN / 2 : TN;
 #pragma unroll
@@ -374,10 +403,10 @@ bool mfma_gemm_supported(int dtype, int64_t m, int64_t k, int64_t n, int quant) 
            cdiv(m, 128) * cdiv(n, 64) < (1ll << 30);   // tile ids are ints
 }
 
-template <typename T, int BM, int BN, bool DUAL, int QF = 0>
+template <typename T, int BM, int BN, bool DUAL, int QF = 0, int KW = 1>
 static void launch_mfma(hipStream_t s, const MfmaLinearArgs& a) {
     constexpr int lds_bytes = 2 * kKb * ((BM + 1) * 16 + (BN + 1) * 16);
-    auto kern = gemm_mfma_kernel<T, BM, BN, DUAL, QF>;
+    auto kern = gemm_mfma_kernel<T, BM, BN, DUAL, QF, KW>;
     static bool configured = false;  // the attribute is per function, not per stream or device state
     if (!configured) {
         (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
@@ -387,28 +416,37 @@ static void launch_mfma(hipStream_t s, const MfmaLinearArgs& a) {
     constexpr int nreal = DUAL ? BN / 2 : BN;
     const int64_t nt = cdiv(npad, nreal), mt = cdiv(a.m, BM);
     const unsigned grid = (unsigned)(cdiv(nt * mt, 8) * 8);
-    kern<<<grid, 256, lds_bytes, s>>>((const T*)a.x, (const T*)a.wk, (const T*)a.wk2, (const T*)a.bias, (const T*)a.residual, (T*)a.y,
+    kern<<<grid, 256 * KW, lds_bytes, s>>>((const T*)a.x, (const T*)a.wk, (const T*)a.wk2, (const T*)a.bias, (const T*)a.residual, (T*)a.y,
                                       (int)a.m, (int)a.k, (int)a.n, (int)npad, a.act, (int)nt, (int)mt, (const T*)a.scale, (const T*)a.scale2);
 }
 
 void mfma_gemm(hipStream_t s, const MfmaLinearArgs& a) {
-    // a problem with fewer 128 x 128 tiles than half the CUs runs on 64 x 64 tiles (four times the workgroups)
-    const bool small = cdiv(a.m, 128) * cdiv(a.n, a.wk2 ? 64 : 128) < 128;
+    // a problem with fewer 128 x 128 tiles than half the CUs runs on 64 x 64 tiles (four times the workgroups); one
+    // with at most one tile per CU on 8-wave workgroups that split every tile's k-steps between two wave groups
+    // (M = 1024, bf16: 192 tiles 46 -> 40 us at K = 4096 and 87 -> 72 us at K = 9216; 384 tiles 54 -> 56 us, not taken)
+    const int64_t tiles = cdiv(a.m, 128) * cdiv(a.n, a.wk2 ? 64 : 128);
+    const bool small = tiles < 128;
+    static const bool allow_split = [] { const char* e = getenv("GPTRS_HIP_GEMM_KSPLIT"); return !(e && e[0] == '0'); }();
+    const bool split = allow_split && !a.wk2 && !small && tiles <= 256;
     if (a.quant == 1) {
         if (a.wk2) launch_mfma<bf16_t, 128, 128, true, 1>(s, a);
         else if (small) launch_mfma<bf16_t, 64, 64, false, 1>(s, a);
+        else if (split) launch_mfma<bf16_t, 128, 128, false, 1, 2>(s, a);
         else launch_mfma<bf16_t, 128, 128, false, 1>(s, a);
     } else if (a.quant == 2) {
         if (a.wk2) launch_mfma<bf16_t, 128, 128, true, 2>(s, a);
         else if (small) launch_mfma<bf16_t, 64, 64, false, 2>(s, a);
+        else if (split) launch_mfma<bf16_t, 128, 128, false, 2, 2>(s, a);
         else launch_mfma<bf16_t, 128, 128, false, 2>(s, a);
     } else if (a.dtype == 0) {
         if (a.wk2) launch_mfma<float, 128, 128, true>(s, a);
         else if (small) launch_mfma<float, 64, 64, false>(s, a);
+        else if (split) launch_mfma<float, 128, 128, false, 0, 2>(s, a);
         else launch_mfma<float, 128, 128, false>(s, a);
     } else {
         if (a.wk2) launch_mfma<bf16_t, 128, 128, true>(s, a);
         else if (small) launch_mfma<bf16_t, 64, 64, false>(s, a);
+        else if (split) launch_mfma<bf16_t, 128, 128, false, 0, 2>(s, a);
         else launch_mfma<bf16_t, 128, 128, false>(s, a);
     }
 }
