@@ -664,8 +664,12 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const T* __restrict__
 // scalar, the rescaling of O^T is a per-lane multiply, and P^T needs no cross-lane movement to become the B operand:
 // the k-slots of the second product are simply numbered in the order the lane holds its keys, and V^T is written to
 // LDS in that order (key bits 2 and 3 swapped).
-template <int DH>
-__global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ctx, int T,
+// KG = 2: the workgroup has two groups of four waves; both serve the same queries, group g takes the key tiles
+// 2 s + g (it stages them itself, into its own LDS buffers), and the two online-softmax states meet through LDS at the
+// end.  A row tile then takes half as many steps, and a SIMD holds two waves whose matrix and vector phases overlap
+// (the launch has one wave-sized task per SIMD otherwise).
+template <int DH, int KG>
+__global__ __launch_bounds__(256 * KG, 2 / KG) void attn_prefill_mfma_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ ctx, int T,
                                                                 int n_q, int n_kv, float scale_log2e) {
     constexpr int KT = 32;            // keys per tile
     constexpr int KS = DH + 8;        // K tile row stride in elements (16 bytes of padding)
@@ -675,15 +679,19 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const bf16_t*
     // d-chunks (16 lanes, 8 rows apart, same position) would hit a single bank whatever the stride (8 rows are a
     // multiple of 128 bytes apart), which the skew spreads over 8 groups of 4 banks.  Measured at 1024 tokens: no skew
     // 88 us per layer, skew with 128-byte rows (reads 8-way conflicting) 68 us.
-    constexpr int VS = 104;
+    constexpr int VS = KG == 1 ? 104 : 72;   // two groups: 72 (rows 4 banks apart, 4 skews) keeps both sets of buffers in LDS
+    constexpr int SKEW = KG == 1 ? 7 : 3;
     constexpr int ND = DH / 32;       // 32-row blocks of d in O^T
     constexpr int NK = DH / 16;       // k-steps of the score product
     constexpr int CH = KT * DH / 8;   // 16-byte chunks of a K (or V) tile
     constexpr int CPT = (CH + 255) / 256;
-    __shared__ __align__(16) bf16_t ksm[2][KT * KS];
-    __shared__ __align__(16) bf16_t vsm[2][DH * VS];
+    __shared__ __align__(16) bf16_t ksm_all[KG][2][KT * KS];
+    __shared__ __align__(16) bf16_t vsm_all[KG][2][DH * VS];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kg = threadIdx.x / 256;                     // key group of this wave
+    const int tid = threadIdx.x % 256, lane = tid & 63, wave = tid >> 6;
+    bf16_t (*ksm)[KT * KS] = ksm_all[kg];
+    bf16_t (*vsm)[DH * VS] = vsm_all[kg];
     const int col = lane & 31, half = lane >> 5;
     const int G = n_q / n_kv;
     const int gw = G >= 4 ? 4 : G;                 // query heads of the group in this workgroup
@@ -741,17 +749,19 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const bf16_t*
                 const uint32_t w[4] = {w0, w1, w2, w3};
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
-                    vsm[buf][(ch * 8 + e) * VS + 8 * (ch & 7) + pos] = (bf16_t)((w[e >> 1] >> ((e & 1) * 16)) & 0xFFFFu);
+                    vsm[buf][(ch * 8 + e) * VS + 8 * (ch & SKEW) + pos] = (bf16_t)((w[e >> 1] >> ((e & 1) * 16)) & 0xFFFFu);
             }
         }
     };
 
-    gload(0);
-    lwrite(0);
+    // group kg visits tiles kg, kg + KG, ...; the step count is uniform over the workgroup (barriers)
+    const int nsteps = (ntiles + KG - 1) / KG;
+    if (kg < ntiles) { gload(kg); lwrite(0); }
     __syncthreads();
-    for (int t = 0; t < ntiles; ++t) {
-        const int buf = t & 1;
-        if (t + 1 < ntiles) gload(t + 1);
+    for (int st = 0; st < nsteps; ++st) {
+        const int buf = st & 1;
+        const int t = st * KG + kg;
+        if (t + KG < ntiles) gload(t + KG);
         if (t < my_tiles) {
             // scores, transposed: rows = keys of the tile, column = this lane's query
             f32x16_v sc;
@@ -805,13 +815,38 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(const bf16_t*
             for (int db = 0; db < ND; ++db) {
 #pragma unroll
                 for (int i = 0; i < 2; ++i) {
-                    const bf16x8_v vf = *reinterpret_cast<const bf16x8_v*>(&vsm[buf][(db * 32 + col) * VS + 8 * (((db & 1) << 2) | (col >> 3)) + 16 * i + 8 * half]);
+                    const bf16x8_v vf = *reinterpret_cast<const bf16x8_v*>(&vsm[buf][(db * 32 + col) * VS + 8 * ((((db & 1) << 2) | (col >> 3)) & SKEW) + 16 * i + 8 * half]);
                     acc_o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[i], acc_o[db], 0, 0, 0);
                 }
             }
         }
-        if (t + 1 < ntiles) lwrite(buf ^ 1);
+        if (t + KG < ntiles) lwrite(buf ^ 1);
         __syncthreads();
+    }
+    if (KG == 2) {
+        // merge the two groups' states: O = O0 c0 + O1 c1, l = l0 c0 + l1 c1 with c_g = 2^(m_g - max(m0, m1)); a group
+        // that saw no tile has m = -inf, l = 0, O = 0 and drops out.  The tiles in LDS are dead (the loop ended on a
+        // barrier); the exchange area is 66 floats per lane of the second group.
+        float* xch = reinterpret_cast<float*>(&vsm_all[0][0][0]) + (wave * 64 + lane);
+        static_assert(KG == 1 || (ND * 16 + 2) * 256 * 4 <= (int)sizeof(vsm_all), "exchange area fits the V buffers");
+        if (kg == 1) {
+#pragma unroll
+            for (int db = 0; db < ND; ++db)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) xch[(db * 16 + v) * 256] = acc_o[db][v];
+            xch[(ND * 16) * 256] = m_run;
+            xch[(ND * 16 + 1) * 256] = l_run;
+        }
+        __syncthreads();
+        if (kg == 1) return;
+        const float m1 = xch[(ND * 16) * 256], l1 = xch[(ND * 16 + 1) * 256];
+        const float mm = fmaxf(m_run, m1);
+        const float c0 = __builtin_amdgcn_exp2f(m_run - mm), c1 = __builtin_amdgcn_exp2f(m1 - mm);
+        l_run = l_run * c0 + l1 * c1;
+#pragma unroll
+        for (int db = 0; db < ND; ++db)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc_o[db][v] = acc_o[db][v] * c0 + xch[(db * 16 + v) * 256] * c1;
     }
     if (active && q0 + col < T) {
         const float inv = 1.0f / l_run;
@@ -1003,9 +1038,19 @@ void attn_prefill(hipStream_t s, const AttnPrefillArgs& a) {
             else attn_prefill_mfma_f32_kernel<128><<<grid, 256, 0, s>>>((const float*)a.qkv, (float*)a.ctx, (int)a.t, (int)a.n_q, (int)a.n_kv, sl);
             return;
         }
-        if (a.head_dim == 32) attn_prefill_mfma_kernel<32><<<grid, 256, 0, s>>>((const bf16_t*)a.qkv, (bf16_t*)a.ctx, (int)a.t, (int)a.n_q, (int)a.n_kv, sl);
-        else if (a.head_dim == 64) attn_prefill_mfma_kernel<64><<<grid, 256, 0, s>>>((const bf16_t*)a.qkv, (bf16_t*)a.ctx, (int)a.t, (int)a.n_q, (int)a.n_kv, sl);
-        else attn_prefill_mfma_kernel<128><<<grid, 256, 0, s>>>((const bf16_t*)a.qkv, (bf16_t*)a.ctx, (int)a.t, (int)a.n_q, (int)a.n_kv, sl);
+        // two key groups per workgroup once the launch is smaller than three workgroups per CU and rows are long
+        // enough to split
+        static const bool allow_kg = [] { const char* e = getenv("GPTRS_HIP_ATTN_KEYGROUPS"); return !(e && e[0] == '0'); }();
+        const bool kg2 = allow_kg && a.t >= 128 && (int64_t)grid.x * grid.y * grid.z < 768;
+#define GPTRS_PREFILL(DHV)                                                                                                   \
+        do {                                                                                                                 \
+            if (kg2) attn_prefill_mfma_kernel<DHV, 2><<<grid, 512, 0, s>>>((const bf16_t*)a.qkv, (bf16_t*)a.ctx, (int)a.t, (int)a.n_q, (int)a.n_kv, sl); \
+            else attn_prefill_mfma_kernel<DHV, 1><<<grid, 256, 0, s>>>((const bf16_t*)a.qkv, (bf16_t*)a.ctx, (int)a.t, (int)a.n_q, (int)a.n_kv, sl);     \
+        } while (0)
+        if (a.head_dim == 32) GPTRS_PREFILL(32);
+        else if (a.head_dim == 64) GPTRS_PREFILL(64);
+        else GPTRS_PREFILL(128);
+#undef GPTRS_PREFILL
         return;
     }
     dim3 grid((unsigned)cdiv(a.t, 4), (unsigned)a.n_q);
