@@ -228,7 +228,12 @@ struct MfmaLinearArgs {
     // the k-grouped CODE copies (mfma_pack_codes) and scale / scale2 the matrices' scale tensors
     int quant;
     const void* scale; const void* scale2;
+    // tail split: when the last round of 128 x 128 tiles would leave most CUs idle, those tiles are split over k between
+    // 2 or 4 workgroups that meet through `part` (mfma_workspace_bytes() of scratch) and `tickets` (kSkinnyTickets
+    // counters, zero before and after every launch); without them every tile runs whole
+    void* part = nullptr; size_t part_bytes = 0; unsigned* tickets = nullptr;
 };
+size_t mfma_workspace_bytes(int dtype, int64_t m, int64_t k, int64_t n, bool dual, int quant);
 size_t mfma_weight_bytes(int dtype, int64_t k, int64_t n);
 void mfma_pack_weights(hipStream_t s, int dtype, const void* w, void* out, int64_t k, int64_t n);
 size_t mfma_codes_bytes(int64_t k, int64_t n, int quant);

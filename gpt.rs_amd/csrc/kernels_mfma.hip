@@ -168,7 +168,9 @@ __global__ __launch_bounds__(256 * KW) void gemm_mfma_kernel(const T* __restrict
                                                         const T* __restrict__ wk2, const T* __restrict__ bias,
                                                         const T* __restrict__ residual, T* __restrict__ y,
                                                         int M, int K, int N, int Npad, int act, int NT, int MT,
-                                                        const T* __restrict__ scale, const T* __restrict__ scale2) {
+                                                        const T* __restrict__ scale, const T* __restrict__ scale2,
+                                                        int full_tiles, int splits, float* __restrict__ part,
+                                                        unsigned* __restrict__ tickets) {
     constexpr int KPC = Mma<T>::KPC;
     constexpr int kBK = kKb * KPC;                            // k per tile
     typedef typename Mma<T>::frag frag_t;
@@ -192,11 +194,27 @@ __global__ __launch_bounds__(256 * KW) void gemm_mfma_kernel(const T* __restrict
     // tile follow each other: the ~32 workgroups an XCD runs at a time then cover 8 row blocks x 4 column tiles, a
     // weight tile is fetched from memory once for all its row blocks (with row-major ids the 1024 column tiles of an
     // lm_head were each fetched once per row block) and an activation tile once per 4 column tiles.
+    //
+    // Tail split: tiles [full_tiles, total) of that order are the last, partly filled round of the launch; each is
+    // taken by `splits` workgroups (ids behind the whole tiles' ids, so the XCDs share them) that multiply a contiguous
+    // range of k tiles each and meet through `part` and a ticket per tile, see the end of the kernel.
     int bx, by;
+    int t_begin = 0, t_end = K / kBK, tail = -1, split = 0;
     {
-        const int total = NT * MT, per = (total + 7) / 8;
-        const int v = (int)(blockIdx.x % 8) * per + (int)(blockIdx.x / 8);
-        if (blockIdx.x / 8 >= (unsigned)per || v >= total) return;
+        const int total = NT * MT, per = (full_tiles + 7) / 8;
+        int v;
+        if (blockIdx.x < (unsigned)per * 8) {
+            v = (int)(blockIdx.x % 8) * per + (int)(blockIdx.x / 8);
+            if (v >= full_tiles) return;
+        } else {
+            const int u = (int)blockIdx.x - per * 8;
+            tail = u / splits;
+            split = u % splits;
+            v = full_tiles + tail;
+            if (v >= total) return;
+            t_begin = (int)((int64_t)split * t_end / splits);
+            t_end = (int)((int64_t)(split + 1) * t_end / splits);
+        }
         const int gsz = 8 * NT, g = v / gsz, first = g * 8;
         const int gm = MT - first < 8 ? MT - first : 8;
         by = first + (v % gsz) % gm;
@@ -267,7 +285,7 @@ __global__ __launch_bounds__(256 * KW) void gemm_mfma_kernel(const T* __restrict
     u32x4_t ra[CA], rb[QF == 0 ? CB : 1];
     u32x2_t rq8[QF == 1 ? CB : 1];
     uint32_t rq4[QF == 2 ? CB : 1];
-    const int nt = K / kBK;
+    const int nt = t_end;
     // bytes between consecutive k tiles of Wk
     const int64_t b_tile_step = (int64_t)kKb * Npad * (QF == 0 ? KPC * (int64_t)sizeof(T) : (QF == 1 ? 8 : 4));
     auto gload = [&](int t, int part, int nparts) {
@@ -328,13 +346,13 @@ __global__ __launch_bounds__(256 * KW) void gemm_mfma_kernel(const T* __restrict
         for (int j = 0; j < TN; ++j) bfr[slot][j] = *reinterpret_cast<const frag_t*>(base + b_rd + kk * 2 * SB + j * 32 * 16);
     };
 
-    gload(0, 0, 1);
+    gload(t_begin, 0, 1);
     if (QF == 2) q_scale = q_scale_next;
     lwrite(0, 0, 1);
-    gload(nt > 1 ? 1 : 0, 0, 1);
+    gload(t_begin + 1 < nt ? t_begin + 1 : t_begin, 0, 1);
     __syncthreads();
-    for (int t = 0; t < nt; ++t) {
-        const int cur = t & 1;
+    for (int t = t_begin; t < nt; ++t) {
+        const int cur = (t - t_begin) & 1;
         fread(cur, wg * KSTEPS, 0);
 #pragma unroll
         for (int kk = 0; kk < KSTEPS; ++kk) {
@@ -374,6 +392,46 @@ __global__ __launch_bounds__(256 * KW) void gemm_mfma_kernel(const T* __restrict
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[i][j][v] += xch[((i * TN + j) * 16 + v) * 64 + lane];
     }
+    if (KW == 1 && tail >= 0) {
+        // Partial sums of a split tile go to the workspace, [item][value][thread], through device-scope stores (coherent
+        // across the L2s of the XCDs without cache maintenance); once they are acknowledged the workgroup draws the
+        // tile's ticket.  The one that draws the last ticket adds all partials in split order, its own included, so
+        // the result does not depend on which workgroup that is, leaves the ticket at zero and runs the epilogue.
+        constexpr int E = TM * TN * 16;
+        float* mine = part + ((int64_t)(tail * splits + split) * E) * 256 + tid;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    __hip_atomic_store(mine + ((i * TN + j) * 16 + v) * 256, acc[i][j][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_s_waitcnt(0x0F70);                         // vmcnt(0)
+        asm volatile("" ::: "memory");
+        unsigned* flag = reinterpret_cast<unsigned*>(lds);          // the tiles in LDS are dead (the loop ended on a barrier)
+        __syncthreads();
+        if (tid == 0) *flag = __hip_atomic_fetch_add(&tickets[tail], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (*flag != (unsigned)(splits - 1)) return;
+        asm volatile("" ::: "memory");                              // the partials are read after the ticket is known
+        if (tid == 0) __hip_atomic_store(&tickets[tail], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+        for (int q = 0; q < splits; ++q) {
+            const float* src = part + ((int64_t)(tail * splits + q) * E) * 256 + tid;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        acc[i][j][v] += __hip_atomic_load(src + ((i * TN + j) * 16 + v) * 256, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
     // epilogue: lane holds column (lane % 32), rows 8*(v/4) + 4*(lane/32) + v%4 of each 32x32 tile
     constexpr int TNO = DUAL ? TN / 2 : TN;
 #pragma unroll
@@ -403,6 +461,28 @@ bool mfma_gemm_supported(int dtype, int64_t m, int64_t k, int64_t n, int quant) 
            cdiv(m, 128) * cdiv(n, 64) < (1ll << 30);   // tile ids are ints
 }
 
+// Tail split of a launch of 128 x 128 tiles on a chip of 256 CUs: the tiles beyond the last multiple of 256 would run
+// as a round of their own on a few CUs (576 pair tiles: 64 CUs work, 192 wait); split 2 or 4 ways over k they give
+// every CU a share.  Returns the number of whole tiles; `splits` = 1 means no split.
+static int64_t mfma_tail_plan(int64_t tiles, int64_t k_tiles, int* splits) {
+    *splits = 1;
+    static const bool allow = [] { const char* e = getenv("GPTRS_HIP_GEMM_TAILSPLIT"); return !(e && e[0] == '0'); }();
+    const int64_t tail = tiles % 256;
+    if (!allow || tiles <= 256 || tail == 0 || tail > 128 || tail > (int64_t)kSkinnyTickets) return tiles;
+    int sp = tail <= 64 ? 4 : 2;
+    while (sp > 1 && k_tiles < 4 * sp) sp /= 2;
+    if (sp < 2) return tiles;
+    *splits = sp;
+    return tiles - tail;
+}
+size_t mfma_workspace_bytes(int dtype, int64_t m, int64_t k, int64_t n, bool dual, int quant) {
+    if (!mfma_gemm_supported(dtype, m, k, n, quant)) return 0;
+    const int64_t tiles = cdiv(m, 128) * cdiv(mfma_padded_n(n), dual ? 64 : 128);
+    int sp = 1;
+    const int64_t full = mfma_tail_plan(tiles, k / (kKb * kpc_of(dtype)), &sp);
+    return sp > 1 ? (size_t)(tiles - full) * sp * 128 * 128 * sizeof(float) : 0;
+}
+
 template <typename T, int BM, int BN, bool DUAL, int QF = 0, int KW = 1>
 static void launch_mfma(hipStream_t s, const MfmaLinearArgs& a) {
     constexpr int lds_bytes = 2 * kKb * ((BM + 1) * 16 + (BN + 1) * 16);
@@ -415,9 +495,17 @@ static void launch_mfma(hipStream_t s, const MfmaLinearArgs& a) {
     const int64_t npad = mfma_padded_n(a.n);
     constexpr int nreal = DUAL ? BN / 2 : BN;
     const int64_t nt = cdiv(npad, nreal), mt = cdiv(a.m, BM);
-    const unsigned grid = (unsigned)(cdiv(nt * mt, 8) * 8);
+    int64_t full = nt * mt;
+    int splits = 1;
+    if (KW == 1 && BM == 128 && BN == 128 && a.part && a.tickets) {
+        int sp = 1;
+        const int64_t f = mfma_tail_plan(nt * mt, a.k / (kKb * Mma<T>::KPC), &sp);
+        if (sp > 1 && a.part_bytes >= (size_t)(nt * mt - f) * sp * BM * BN * sizeof(float)) { full = f; splits = sp; }
+    }
+    const unsigned grid = (unsigned)(cdiv(full, 8) * 8 + (nt * mt - full) * splits);
     kern<<<grid, 256 * KW, lds_bytes, s>>>((const T*)a.x, (const T*)a.wk, (const T*)a.wk2, (const T*)a.bias, (const T*)a.residual, (T*)a.y,
-                                      (int)a.m, (int)a.k, (int)a.n, (int)npad, a.act, (int)nt, (int)mt, (const T*)a.scale, (const T*)a.scale2);
+                                      (int)a.m, (int)a.k, (int)a.n, (int)npad, a.act, (int)nt, (int)mt, (const T*)a.scale, (const T*)a.scale2,
+                                      (int)full, splits, (float*)a.part, a.tickets);
 }
 
 void mfma_gemm(hipStream_t s, const MfmaLinearArgs& a) {

@@ -556,6 +556,7 @@ void Builder::describe(Step& st) {
                     if (in.act == 2) st.tiled_s2_input = pos(4);
                 }
             }
+            if (in.mfma) st.scratch_bytes = k::mfma_workspace_bytes((int)x.dtype, x.dims[0], x.dims[1], w.dims[1], in.act == 2, in.quant);
             if (in.tiled && x.dims[0] >= 2) {
                 // batched decode normalises into scratch first (the matrix-core kernel reads plain rows); layers with
                 // few column tiles add the partial sums of their K splits
@@ -1066,6 +1067,11 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
                 if (in.has_residual) ma.residual = src_ptr(st, cx, oi++);
                 ma.y = dst;
                 ma.act = in.act == 1 ? 1 : 0;
+                if (st.scratch_bytes) {
+                    ma.part = cx.ws + st.scratch_off;
+                    ma.part_bytes = st.scratch_bytes;
+                    ma.tickets = cx.be->skinny_tickets();
+                }
                 hipEvent_t e0 = nullptr, e1 = nullptr;
                 if (cx.profile) {
                     GPTRS_HIP_CHECK(hipEventCreate(&e0));

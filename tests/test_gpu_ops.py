@@ -7,7 +7,7 @@ import pytest
 
 from parity import FunctionBuilder, Program, assert_close, check_program, hip_run, oracle_run, to_bytes
 from gptrs_amd import functional as F
-from gptrs_amd.ptir import Tensor, f32_to_bf16_bits
+from gptrs_amd.ptir import Tensor, bf16_bits_to_f32, f32_to_bf16_bits
 
 pytestmark = pytest.mark.gpu
 
@@ -220,6 +220,28 @@ def test_prefill_linear_on_matrix_cores(hip, m, k, n):
     assert hip.counter("derived_weights_built") - before >= 4  # the fused legs took the derived-weight path
 
 
+@pytest.mark.parametrize("dtype", ["Bf16", "F32"])
+@pytest.mark.parametrize("m,k,n,pair", [(1024, 1024, 4860, False), (1100, 512, 5120, False), (1024, 1024, 2430, True), (1024, 256, 4864, False)])
+def test_prefill_linear_tail_tiles_split_over_k(hip, m, k, n, pair, dtype):
+    """Launches of more than 256 tiles whose last round holds at most 128: those tiles are split 4 or 2 ways over k
+    between workgroups that meet through a workspace and a ticket (304 tiles -> 48 x 4, 360 -> 104 x 2, the SwiGLU pair
+    with 64 real columns per tile, and K = 256 with too few k tiles to split).  Checked against the oracle, and a second
+    run (tickets must have returned to zero) must reproduce the first bit for bit."""
+    x = rng_uniform(50, (m, k))
+    w, w2 = rng_uniform(51, (k, n)) / np.sqrt(k) * 2, rng_uniform(52, (k, n)) / np.sqrt(k) * 2
+    b, r = rng_uniform(53, (n,)), rng_uniform(54, (m, n))
+    tol = dict(atol=3e-2, rtol=3e-2) if dtype == "Bf16" else dict(atol=5e-4, rtol=1e-4)
+    if pair:
+        p = prog(lambda fb, a, c, d: F.swiglu(a.matmul(c), a.matmul(d)), [(dtype, [m, k]), (dtype, [k, n]), (dtype, [k, n])])
+        args = [x, w, w2]
+    else:
+        p = prog(lambda fb, a, c, d, e: F.gelu(F.linear(a, c, d)) + e, [(dtype, [m, k]), (dtype, [k, n]), (dtype, [n]), (dtype, [m, n])])
+        args = [x, w, b, r]
+    check_program(hip, p, args, both_modes=False, **tol)
+    first, second = hip_run(hip, p, args)[0], hip_run(hip, p, args)[0]
+    assert np.array_equal(first, second)
+
+
 @pytest.mark.parametrize("b,m,k,n", [(1, 4, 5, 2), (2, 7, 13, 9), (8, 4, 8, 4), (3, 33, 65, 31)])
 def test_matmul_batched(hip, b, m, k, n):
     a, c = rng_uniform(9, (b, m, k)), rng_uniform(10, (b, k, n))
@@ -298,7 +320,7 @@ def test_layer_norm_constant_input_gives_beta(hip):
     assert np.allclose(out, np.broadcast_to(b, out.shape), atol=1e-6)
 
 
-@pytest.mark.parametrize("shape", [(2, 3, 4), (5, 16), (1, 3072), (8, 3072)])
+@pytest.mark.parametrize("shape", [(2, 3, 4), (5, 16), (1, 3072), (8, 3072), (3, 24), (2, 8192), (2, 8200), (70, 1000)])
 @pytest.mark.parametrize("dtype", ["F32", "Bf16"])
 def test_rms_norm(hip, shape, dtype):
     n = shape[-1]
@@ -318,6 +340,29 @@ def test_rope_packed(hip, hq, hkv, dh, rot, seq):
     out = check_program(hip, p, [qkv, cos, sin])[0]
     # rotation preserves the norm of each (first, second) pair; V passes through untouched
     assert np.array_equal(out[:, (hq + hkv) * dh:], qkv[:, (hq + hkv) * dh:])
+
+
+@pytest.mark.parametrize("hq,hkv,dh,rot,seq", [(32, 8, 128, 128, 7), (4, 2, 16, 16, 33), (2, 1, 64, 64, 300), (4, 2, 16, 8, 3), (4, 4, 8, 8, 5)])
+def test_rope_packed_bf16(hip, hq, hkv, dh, rot, seq):
+    """bf16 rows: heads whose halves are multiples of 8 take the 16-byte kernel, the rest the element-wise one."""
+    cfg = F.AttentionConfig(hq * dh, hq, hkv, dh)
+    cos, sin = F.rotary_cos_sin_cache_slice(5, seq, F.RopeConfig(rot, 10000.0))
+    qkv = rng_uniform(27, (seq, cfg.total_projection_dim))
+    p = prog(lambda fb, a, c, s: F.apply_rope_qkv_packed(cfg, a, c, s),
+             [("Bf16", [seq, cfg.total_projection_dim]), ("Bf16", [seq, rot // 2]), ("Bf16", [seq, rot // 2])])
+    check_program(hip, p, [qkv, cos, sin], atol=2e-2, rtol=2e-2)
+    # V passes through bit for bit; the rotated part equals the f32 closed form of the bf16 inputs to one bf16 ulp
+    r = lambda a: bf16_bits_to_f32(f32_to_bf16_bits(np.asarray(a, np.float32)))
+    out = np.asarray(hip_run(hip, p, [qkv, cos, sin])[0], np.float32)
+    x, c, s_ = r(qkv), r(cos), r(sin)
+    assert np.array_equal(out[:, (hq + hkv) * dh:], x[:, (hq + hkv) * dh:])
+    h = rot // 2
+    heads = x[:, :(hq + hkv) * dh].reshape(seq, hq + hkv, dh)
+    want = heads.copy()
+    want[:, :, :h] = heads[:, :, :h] * c[:, None, :] - heads[:, :, h:rot] * s_[:, None, :]
+    want[:, :, h:rot] = heads[:, :, h:rot] * c[:, None, :] + heads[:, :, :h] * s_[:, None, :]
+    got = out[:, :(hq + hkv) * dh].reshape(seq, hq + hkv, dh)
+    assert np.all(np.abs(got - want) <= np.abs(want) * 2.0 ** -7 + 1e-6)
 
 
 @pytest.mark.parametrize("hq,hkv,dh,seq", [(3, 3, 2, 4), (2, 2, 4, 1), (4, 4, 8, 8), (4, 4, 1, 3), (4, 1, 4, 5), (4, 2, 8, 6), (8, 2, 16, 33)])
