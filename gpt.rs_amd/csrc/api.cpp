@@ -749,16 +749,30 @@ int gptrs_hip_execute_instruction(gptrs_hip_backend* b, const char* instruction_
         }
         std::string params, ids;
         size_t nv = 0;
+        // inputs are positional, one per Value operand (spec.rs:1317); an id that repeats (x * x) names one parameter
+        std::vector<std::pair<int64_t, gptrs_hip_tensor*>> seen;
+        std::vector<gptrs_hip_tensor*> uniq;
         try {
             for (auto& od : j.at("operands").as_array())
                 if (const gptrs::Json* v = od.find("Value")) {
                     if (nv >= n_in) gptrs::fail_exec("execute_instruction: fewer inputs than Value operands");
-                    const gptrs::Spec& s = inputs[nv]->spec;
+                    if (!inputs[nv]) gptrs::fail_exec("null input handle");
+                    const int64_t id = v->as_int();
+                    bool dup = false;
+                    for (auto& pr : seen)
+                        if (pr.first == id) {
+                            if (pr.second != inputs[nv]) gptrs::fail_exec("execute_instruction: one value id bound to two tensors");
+                            dup = true;
+                        }
+                    ++nv;
+                    if (dup) continue;
+                    seen.push_back({id, inputs[nv - 1]});
+                    uniq.push_back(inputs[nv - 1]);
+                    const gptrs::Spec& s = inputs[nv - 1]->spec;
                     std::string dims;
                     for (size_t i = 0; i < s.dims.size(); ++i) dims += (i ? "," : "") + std::string("{\"Static\":") + std::to_string(s.dims[i]) + "}";
-                    params += (nv ? "," : "") + std::string("{\"Tensor\":{\"dtype\":\"") + gptrs::dtype_name(s.dtype) + "\",\"shape\":{\"dims\":[" + dims + "]}}}";
-                    ids += (nv ? "," : "") + std::to_string(v->as_int());
-                    ++nv;
+                    params += (uniq.size() > 1 ? "," : "") + std::string("{\"Tensor\":{\"dtype\":\"") + gptrs::dtype_name(s.dtype) + "\",\"shape\":{\"dims\":[" + dims + "]}}}";
+                    ids += (uniq.size() > 1 ? "," : "") + std::to_string(id);
                 }
         } catch (const gptrs::JsonError& e) {
             gptrs::fail_spec(e.what());
@@ -783,7 +797,7 @@ int gptrs_hip_execute_instruction(gptrs_hip_backend* b, const char* instruction_
                                  std::string(instruction_json, json_len) + "],\"hints\":[],\"result_ids\":[" +
                                  std::to_string(j.at("id").as_int()) + "]}],\"regions\":[]}";
         std::lock_guard<std::mutex> g(b->impl.mu);
-        b->impl.run_program(prog.data(), prog.size(), 0, inputs, nullptr, n_in, output, 1);
+        b->impl.run_program(prog.data(), prog.size(), 0, uniq.data(), nullptr, uniq.size(), output, 1);
     });
 }
 

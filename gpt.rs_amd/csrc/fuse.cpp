@@ -241,6 +241,27 @@ struct Fuser {
         return true;
     }
 
+    // Cast(bf16)(rms_norm(x f32, gamma f32)): the norm stores bf16 directly (one rounding of the f32 result, which is
+    // what the cast does).  The reference's rms_norm is f32-only (normalization.rs:183-217), so a bf16 model with an
+    // f32 residual stream reaches its bf16 projections through exactly this pair.
+    void pass_norm_cast() {
+        const std::vector<int> uses = count_uses();
+        for (auto& in : fn.body) {
+            if (in.dead || in.op != OpKind::Cast || in.out_specs[0].dtype != DType::BF16) continue;
+            const int src = in.operands[0].value;
+            if (src < 0 || def[src] < 0 || uses[src] != 1) continue;
+            Instr& nrm = fn.body[def[src]];
+            if (nrm.dead || nrm.op != OpKind::FRmsNorm || nrm.out_specs[0].dtype != DType::F32) continue;
+            Instr ni = nrm;
+            ni.out_ids = in.out_ids;
+            ni.out_specs = in.out_specs;
+            nrm.dead = true;
+            in = ni;
+            ++fused;
+        }
+        reindex();
+    }
+
     Instr make(OpKind op, const char* name, std::vector<int> ins, int out_id, const Spec& out_spec) const {
         Instr ni;
         ni.op = op;
@@ -664,6 +685,30 @@ struct Fuser {
         return uses;
     }
 
+    // 0: the generic kernels; 1: matrix-core GEMM over a k-grouped copy; 2: weight-streaming decode kernels over a
+    // tiled copy (the persistent chain, the batched matrix-core kernel, the tiled GEMV).  Needs weights (and scales)
+    // that are program inputs.  Works on a Dot as well as on an FLinear (operand 0 = x, 1 = W).
+    int linear_path(const Instr& in) const {
+        auto is_param = [&](int v) { return v >= 0 && def[v] < 0 && spec_of(v) != nullptr; };
+        const Spec* xs = spec_of(in.operands[0].value);
+        const Spec* ws = spec_of(in.operands[1].value);
+        if (!xs || !ws || xs->rank() != 2 || ws->rank() != 2) return 0;
+        const int64_t M = xs->dims[0], K = xs->dims[1], N = ws->dims[1];
+        // with a folded f32 norm x is f32 while the kernel computes in the weights' dtype
+        const int dt = in.quant ? (int)spec_of(in.operands[2].value)->dtype : (int)ws->dtype;
+        if (!is_param(in.operands[1].value)) return 0;
+        if (in.act == 2 && !is_param(in.operands[linear_w2_pos(in)].value)) return 0;
+        if (in.quant && (!is_param(in.operands[2].value) || (in.act == 2 && !is_param(in.operands[4].value)))) return 0;
+        if (k::mfma_gemm_supported(dt, M, K, N, in.quant)) return 1;
+        if (in.quant)   // decode: the persistent chain (one row) and the batched matrix-core kernel read the codes directly
+            return (k::chain_supported(dt, M, K, N, in.act == 2, false, in.quant) || k::skinny_quant_supported(dt, M, K, N, in.quant)) ? 2 : 0;
+        if (!k::gemv_tiled_supported(dt, M, K, N)) return 0;
+        // SwiGLU pairs: the vector kernel holds up to 8 rows, the matrix-core kernel of batched decode up to 16
+        if (in.act == 2 && M > 8 && !k::skinny_gemm_supported(dt, M, K, N)) return 0;
+        return 2;
+    }
+    bool fast_linear(const Instr& in) const { return linear_path(in) != 0; }
+
     void pass_linear() {
         // 1. x[M,K] . W[K,N] -> FLinear
         for (auto& in : fn.body) {
@@ -673,6 +718,8 @@ struct Fuser {
             const Spec* l = spec_of(in.operands[0].value);
             const Spec* r = spec_of(in.operands[1].value);
             if (!l || !r || l->rank() != 2 || r->rank() != 2 || !dtype_is_float(l->dtype)) continue;
+            // an f32 result over bf16 operands is stored by the weight-streaming and matrix-core kernels only
+            if (in.out_f32 && !fast_linear(in)) continue;
             in.op = OpKind::FLinear;
             in.op_name = "fused.linear";
             in.act = 0;
@@ -712,7 +759,7 @@ struct Fuser {
                     // bias: Add(linear, BroadcastTo(b[N]))  (tensor_ops.rs:42-56)
                     Instr* lin = linear_of(a);
                     int vec;
-                    if (lin && !lin->has_bias && !lin->has_residual && lin->act == 0 &&
+                    if (lin && !lin->has_bias && !lin->has_residual && lin->act == 0 && !lin->out_f32 &&
                         vector_bcast_last(b, in.out_specs[0].dims.back(), vec)) {
                         Instr ni = *lin;
                         Operand o; o.value = vec;
@@ -730,6 +777,7 @@ struct Fuser {
                         Instr* l2 = linear_of(side == 0 ? a : b);
                         const int other = side == 0 ? b : a;
                         if (!l2 || l2->has_residual || l2->act == 2) continue;
+                        if (l2->out_f32 && !fast_linear(*l2)) continue;   // (a quantised linear outside the fast kernels)
                         if (def[other] >= 0 && def[other] > def[l2->out_ids[0]]) {
                             // the residual is produced after the linear: fine, the fused op sits at the Add
                         }
@@ -747,7 +795,7 @@ struct Fuser {
                     }
                 } else if (in.op == OpKind::FGelu) {
                     Instr* lin = linear_of(in.operands[0].value);
-                    if (lin && lin->act == 0 && !lin->has_residual && in.fparam[0] == 0.5f && in.fparam[1] == 1.41421354f &&
+                    if (lin && lin->act == 0 && !lin->has_residual && !lin->out_f32 && in.fparam[0] == 0.5f && in.fparam[1] == 1.41421354f &&
                         in.fparam[2] == 1.0f) {
                         Instr ni = *lin;
                         ni.act = 1;
@@ -761,6 +809,7 @@ struct Fuser {
                     Instr* lg = linear_of(in.operands[0].value);
                     Instr* lu = linear_of(in.operands[1].value);
                     if (lg && lu && lg != lu && lg->act == 0 && lu->act == 0 && !lg->has_bias && !lu->has_bias &&
+                        !lg->out_f32 && !lu->out_f32 &&
                         !lg->has_residual && !lu->has_residual && lg->operands[0].value == lu->operands[0].value &&
                         lg->quant == lu->quant) {
                         const Spec* wg = spec_of(lg->operands[1].value);
@@ -787,29 +836,11 @@ struct Fuser {
     // an RMSNorm feeding only such linears is folded into them (every block reads the whole row of x
     // anyway, so the row statistic is free).
     void pass_tiled_linear() {
-        auto is_param = [&](int v) { return v >= 0 && def[v] < 0 && spec_of(v) != nullptr; };
         for (auto& in : fn.body) {
             if (in.dead || in.op != OpKind::FLinear) continue;
-            const Spec* xs = spec_of(in.operands[0].value);
-            const Spec* ws = spec_of(in.operands[1].value);
-            if (!xs || !ws) continue;
-            const int64_t M = xs->dims[0];
-            if (!is_param(in.operands[1].value)) continue;
-            if (in.act == 2 && !is_param(in.operands[linear_w2_pos(in)].value)) continue;
-            if (in.quant && (!is_param(in.operands[2].value) || (in.act == 2 && !is_param(in.operands[4].value)))) continue;
-            if (k::mfma_gemm_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1], in.quant)) {
-                in.mfma = true;
-                continue;
-            }
-            if (in.quant) {   // decode: the persistent chain (one row) and the batched matrix-core kernel read the codes directly
-                in.tiled = k::chain_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1], in.act == 2, false, in.quant) ||
-                           k::skinny_quant_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1], in.quant);
-                continue;
-            }
-            if (!k::gemv_tiled_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1])) continue;
-            // SwiGLU pairs: the vector kernel holds up to 8 rows, the matrix-core kernel of batched decode up to 16
-            if (in.act == 2 && M > 8 && !k::skinny_gemm_supported((int)xs->dtype, M, xs->dims[1], ws->dims[1])) continue;
-            in.tiled = true;
+            const int path = linear_path(in);
+            in.mfma = path == 1;
+            in.tiled = path == 2;
         }
         const std::vector<int> uses = count_uses();
         std::vector<bool> is_result(fn.max_value_id + 1, false);
@@ -820,6 +851,8 @@ struct Fuser {
             const bool ln = nrm.op == OpKind::FLayerNorm;   // folded into plain (unquantised) decode linears only
             const int nv = nrm.out_ids[0];
             if (is_result[nv] || nrm.out_specs[0].rank() != 2) continue;
+            const Spec* nx = spec_of(nrm.operands[0].value);
+            const bool xf32 = nx && nx->dtype == DType::F32 && nrm.out_specs[0].dtype == DType::BF16;
             std::vector<Instr*> cons;
             int found = 0;
             for (auto& c : fn.body) {
@@ -827,7 +860,7 @@ struct Fuser {
                 for (size_t o = 0; o < c.operands.size(); ++o) {
                     if (c.operands[o].value != nv) continue;
                     ++found;
-                    if (c.op == OpKind::FLinear && c.tiled && !c.norm && o == 0 && !(ln && c.quant)) cons.push_back(&c);
+                    if (c.op == OpKind::FLinear && c.tiled && !c.norm && o == 0 && !(ln && c.quant) && !(ln && xf32)) cons.push_back(&c);
                 }
             }
             if (cons.empty() || (int)cons.size() != found || found != uses[nv]) continue;
@@ -836,6 +869,7 @@ struct Fuser {
                 c->operands.push_back(nrm.operands[1]);
                 if (ln) c->operands.push_back(nrm.operands[2]);
                 c->norm = true;
+                c->x_f32 = xf32;
                 c->norm_ln = ln;
                 c->eps = nrm.eps;
                 c->scale = nrm.scale;
@@ -999,6 +1033,8 @@ int fuse_function(Function& fn) {
     Fuser f(fn);
     f.dce();
     f.pass_elementwise();
+    f.dce();
+    f.pass_norm_cast();
     f.dce();
     f.pass_rope();
     f.pass_attention();

@@ -56,7 +56,8 @@ struct DotDesc {
     int64_t b_sb, b_sk, b_sn;
     int64_t c_sb, c_sm;  // C is [b][m][n] with n contiguous
 };
-void dot_generic(hipStream_t s, int dtype, const void* a, const void* b, void* c, const DotDesc& d);
+// dtype: of A and B; out_f32: bf16 operands, the f32 accumulator is stored as f32 (DotGeneralSpec.out_dtype)
+void dot_generic(hipStream_t s, int dtype, const void* a, const void* b, void* c, const DotDesc& d, bool out_f32 = false);
 
 // last row of [rows][vocab] logits; ties -> smallest index; result (int64) written to *out
 // greedy token of every row (rows * partial blocks <= scratch_cap), ties to the smallest index; out: si32[rows]
@@ -76,6 +77,9 @@ void layer_norm(hipStream_t s, int dtype, const void* x, const void* gamma, cons
 // y = x * rsqrt(mean(x^2)+eps) * gamma: normalization.rs:183-217
 void rms_norm(hipStream_t s, int dtype, const void* x, const void* gamma, void* y, int64_t rows, int64_t n,
               float inv_n, float eps);
+// the same over f32 rows and gains with a bf16 result (the f32 value rounded once)
+void rms_norm_f32_to_bf16(hipStream_t s, const void* x, const void* gamma, void* y, int64_t rows, int64_t n, float inv_n,
+                          float eps);
 void softmax_rows(hipStream_t s, int dtype, const void* x, void* y, int64_t rows, int64_t n);
 void gelu(hipStream_t s, int dtype, const void* x, void* y, int64_t n, float half, float inv_div, float one);
 void swiglu(hipStream_t s, int dtype, const void* gate, const void* up, void* y, int64_t n);  // up==nullptr: silu
@@ -107,6 +111,9 @@ struct TiledLinearArgs {
     int act;
     float inv_n, eps;
     const void* beta;   // with gamma: LayerNorm (normalization.rs:123-174) instead of RMSNorm
+    // bf16 weights only.  out_f32: y and residual are f32 (the accumulator leaves unrounded).  x_f32 (with gamma, RMSNorm):
+    // x and gamma are f32, the normalised row is rounded to bf16 once as it is staged.
+    int out_f32 = 0, x_f32 = 0;
 };
 size_t tiled_weight_bytes(int dtype, int64_t k, int64_t n);
 void tile_weights(hipStream_t s, int dtype, const void* w, void* wt, int64_t k, int64_t n);
@@ -127,6 +134,7 @@ struct SkinnyLinearArgs {
     // weight-only quantised: quant 1 = int8 (scale [N]), 2 = int4 groups of 128 (scale [K/128, N]); ws / ws2 are then
     // the code copies of skinny_pack_codes, scale / scale2 the scale tensors as the program holds them (bf16)
     int quant; const void* scale; const void* scale2;
+    int out_f32 = 0;   // bf16 only: y and residual are f32
 };
 bool skinny_quant_supported(int dtype, int64_t m, int64_t k, int64_t n, int qf);
 size_t skinny_codes_bytes(int64_t k, int64_t n, int qf);
@@ -165,7 +173,9 @@ constexpr int kChainCounters = 16;        // striped arrival counters of the gri
 constexpr int kChainMaxPhases = 192;
 constexpr int kChainMaxXsWords = 16384;   // staged activation pairs: K <= 32768
 constexpr size_t kChainBarrierBytes = (kChainCounters * 64 + 64) * sizeof(unsigned);  // zero-initialised once
-enum : int { kChainNorm = 1, kChainDual = 2, kChainGelu = 4, kChainResidual = 8, kChainBias = 16 };
+// kChainOutF32: y and the residual are f32.  kChainXF32 (with kChainNorm): x and gamma are f32, the normalised row is
+// rounded to bf16 once as it is staged.
+enum : int { kChainNorm = 1, kChainDual = 2, kChainGelu = 4, kChainResidual = 8, kChainBias = 16, kChainOutF32 = 32, kChainXF32 = 64 };
 enum : int { kChainW16 = 0, kChainW8 = 1, kChainW4 = 2 };   // weight format of a linear phase
 enum : int { kChainLinear = 0, kChainAttnPartial = 1, kChainAttnCombine = 2 };
 // One phase of a chain.  Linear: y = act(norm?(x) . W + bias) (+ residual).  Decode attention
@@ -194,7 +204,7 @@ struct ChainPhase {
     int pad;
 };
 int chain_grid();  // workgroups per launch (one per CU), 0 when no device is current
-bool chain_supported(int dtype, int64_t m, int64_t k, int64_t n, bool dual, bool norm, int wfmt = kChainW16);
+bool chain_supported(int dtype, int64_t m, int64_t k, int64_t n, bool dual, bool norm, int wfmt = kChainW16, bool x_f32 = false);
 size_t chain_weight_bytes(int64_t k, int64_t n, bool dual, int wfmt = kChainW16);
 // w2 != nullptr: SwiGLU pair, columns of w (gate) and w2 (up) interleaved.  wfmt 0: w is bf16 [k,n];
 // 1: si8 [k,n]; 2: packed int4, ui8 [k/2,n]
@@ -232,6 +242,7 @@ struct MfmaLinearArgs {
     // 2 or 4 workgroups that meet through `part` (mfma_workspace_bytes() of scratch) and `tickets` (kSkinnyTickets
     // counters, zero before and after every launch); without them every tile runs whole
     void* part = nullptr; size_t part_bytes = 0; unsigned* tickets = nullptr;
+    int out_f32 = 0;   // bf16 only: y and residual are f32
 };
 size_t mfma_workspace_bytes(int dtype, int64_t m, int64_t k, int64_t n, bool dual, int quant);
 size_t mfma_weight_bytes(int dtype, int64_t k, int64_t n);

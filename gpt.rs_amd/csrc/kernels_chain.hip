@@ -140,7 +140,7 @@ struct Shared {
 
 // ---------------------------------------------------------------------------- staging (all waves)
 // xs[j] = (x[2j], x[2j+1]) as a bf16 pair, zero beyond K; with norm: the value the stand-alone
-// RMSNorm kernel stores, ((x * inv_rms) -> bf16) * gamma -> bf16 (normalization.rs:183-217).
+// RMSNorm kernels store, ((x * inv_rms) * gamma) -> bf16 (normalization.rs:183-217).
 __device__ void stage_block(const ChainPhase& P, unsigned* xs, float* ssq) {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int K = uni(P.K);
@@ -166,7 +166,49 @@ __device__ void stage_block(const ChainPhase& P, unsigned* xs, float* ssq) {
             sv[u] = i < sc_n ? gload2(sc_src + i) : make_uint2(0u, 0u);
         }
     }
-    if (uni(P.flags) & kChainNorm) {
+    if ((uni(P.flags) & (kChainNorm | kChainXF32)) == (kChainNorm | kChainXF32)) {
+        // f32 row and gains (a bf16 model whose residual stream is f32): the f32 norm, rounded to bf16 once
+        constexpr int MF = MAXI / 2;   // 16-byte items per thread: K <= 4 * MF * NT
+        const char* g = (const char*)uni_ptr(P.gamma);
+        uint4 v[MF], gg[MF];
+#pragma unroll
+        for (int u = 0; u < MF; ++u) {
+            const int i = u * NT + t;
+            v[u] = make_uint4(0u, 0u, 0u, 0u);
+            gg[u] = make_uint4(0u, 0u, 0u, 0u);
+            if (u * NT < n && i < n) {
+                const unsigned long long a = cload8(x + 16 * (size_t)i), b = cload8(x + 16 * (size_t)i + 8);
+                v[u] = make_uint4((unsigned)a, (unsigned)(a >> 32), (unsigned)b, (unsigned)(b >> 32));
+                gg[u] = gload4(g + 16 * (size_t)i);
+            }
+        }
+        float q = 0.f;
+#pragma unroll
+        for (int u = 0; u < MF; ++u) {
+            if (u * NT < n) {
+                const float a = __uint_as_float(v[u].x), b = __uint_as_float(v[u].y), c = __uint_as_float(v[u].z), d = __uint_as_float(v[u].w);
+                q += a * a; q += b * b; q += c * c; q += d * d;
+            }
+        }
+        const float ws = wave_sum(q);
+        if (lane == 0) ssq[wave] = ws;
+        lds_barrier();
+        float tot = 0.f;
+#pragma unroll
+        for (int w = 0; w < NT / 64; ++w) tot += ssq[w];
+        const float inv = 1.0f / sqrtf(tot * P.inv_n + P.eps);
+#pragma unroll
+        for (int u = 0; u < MF; ++u) {
+            const int i = u * NT + t;
+            if (u * NT < npad && i < npad) {
+                const unsigned o0 = pack_hw((__uint_as_float(v[u].x) * inv) * __uint_as_float(gg[u].x),
+                                            (__uint_as_float(v[u].y) * inv) * __uint_as_float(gg[u].y));
+                const unsigned o1 = pack_hw((__uint_as_float(v[u].z) * inv) * __uint_as_float(gg[u].z),
+                                            (__uint_as_float(v[u].w) * inv) * __uint_as_float(gg[u].w));
+                *reinterpret_cast<uint2*>(&xs[2 * i]) = make_uint2(o0, o1);
+            }
+        }
+    } else if (uni(P.flags) & kChainNorm) {
         const uint2* g = (const uint2*)uni_ptr(P.gamma);
         unsigned long long v[MAXI];
         uint2 gg[MAXI];
@@ -205,10 +247,9 @@ __device__ void stage_block(const ChainPhase& P, unsigned* xs, float* ssq) {
             const int i = u * NT + t;
             if (u * NT < npad && i < npad) {
                 const unsigned lo = (unsigned)v[u], hi = (unsigned)(v[u] >> 32);
-                // ((x * inv) -> bf16) * gamma -> bf16, two values per conversion
-                const unsigned n0 = pack_hw(bf16lo(lo) * inv, bf16hi(lo) * inv), n1 = pack_hw(bf16lo(hi) * inv, bf16hi(hi) * inv);
-                const unsigned o0 = pack_hw(bf16lo(n0) * bf16lo(gg[u].x), bf16hi(n0) * bf16hi(gg[u].x));
-                const unsigned o1 = pack_hw(bf16lo(n1) * bf16lo(gg[u].y), bf16hi(n1) * bf16hi(gg[u].y));
+                // (x * inv) * gamma in f32, rounded to bf16 once: what the stand-alone RMSNorm kernels store
+                const unsigned o0 = pack_hw((bf16lo(lo) * inv) * bf16lo(gg[u].x), (bf16hi(lo) * inv) * bf16hi(gg[u].x));
+                const unsigned o1 = pack_hw((bf16lo(hi) * inv) * bf16lo(gg[u].y), (bf16hi(hi) * inv) * bf16hi(gg[u].y));
                 *reinterpret_cast<uint2*>(&xs[2 * i]) = make_uint2(o0, o1);
             }
         }
@@ -662,11 +703,14 @@ __device__ void control_wave(Shared& sh, unsigned* xs, int nphases, unsigned* ba
             const unsigned* sg = wfmt == kChainW8 ? (const unsigned*)uni_ptr(P.wscale) : nullptr;
             const unsigned* su = wfmt == kChainW8 ? (const unsigned*)uni_ptr(P.wscale2) : nullptr;
             if (lane == 0) lds_st(&sh.go, ph);
+            const bool out_f32 = flags & kChainOutF32;   // y and the residual are f32
+            unsigned long long e_rf = 0ull;              // two f32 residual values
             auto epi_load = [&](int i, unsigned& bw, unsigned& rw, unsigned& ga, unsigned& gb) {
                 const int col = col0 + i;
                 const bool in = i < ncols && col < N;
                 bw = (bias && in) ? gload(bias + (col >> 1)) : 0u;
-                rw = (resid && in) ? cload4(resid + 2 * (size_t)col) : 0u;
+                if (out_f32) e_rf = (resid && in) ? cload8(resid + 4 * (size_t)col) : 0ull;
+                rw = (resid && in && !out_f32) ? cload4(resid + 2 * (size_t)col) : 0u;
                 ga = (sg && in) ? gload(sg + (col >> 1)) : 0u;
                 gb = (su && in) ? gload(su + (col >> 1)) : 0u;
             };
@@ -674,7 +718,8 @@ __device__ void control_wave(Shared& sh, unsigned* xs, int nphases, unsigned* ba
                 if (i >= ncols) return;
                 if (bias || resid) {
                     *reinterpret_cast<float2*>(&sh.epi_bias[i]) = make_float2(bf16lo(bw), bf16hi(bw));
-                    *reinterpret_cast<float2*>(&sh.epi_res[i]) = make_float2(bf16lo(rw), bf16hi(rw));
+                    *reinterpret_cast<float2*>(&sh.epi_res[i]) = out_f32 ? make_float2(__uint_as_float((unsigned)e_rf), __uint_as_float((unsigned)(e_rf >> 32)))
+                                                                          : make_float2(bf16lo(rw), bf16hi(rw));
                 }
                 if (sg) {
                     *reinterpret_cast<float2*>(&sh.epi_s[i]) = make_float2(bf16lo(ga), bf16hi(ga));
@@ -735,8 +780,13 @@ __device__ void control_wave(Shared& sh, unsigned* xs, int nphases, unsigned* ba
                         float o[4];
 #pragma unroll
                         for (int c = 0; c < 4; ++c) o[c] = finish(s[c], flags, sh.epi_bias[e + c], sh.epi_res[e + c]);
-                        cstore8(out + 2 * (size_t)(tile * 4),
-                                (unsigned long long)pack_bf16x2(o[0], o[1]) | ((unsigned long long)pack_bf16x2(o[2], o[3]) << 32));
+                        if (out_f32) {
+                            cstore8(out + 4 * (size_t)(tile * 4), (unsigned long long)__float_as_uint(o[0]) | ((unsigned long long)__float_as_uint(o[1]) << 32));
+                            cstore8(out + 4 * (size_t)(tile * 4) + 8, (unsigned long long)__float_as_uint(o[2]) | ((unsigned long long)__float_as_uint(o[3]) << 32));
+                        } else {
+                            cstore8(out + 2 * (size_t)(tile * 4),
+                                    (unsigned long long)pack_bf16x2(o[0], o[1]) | ((unsigned long long)pack_bf16x2(o[2], o[3]) << 32));
+                        }
                     }
                 }
             }
@@ -1073,8 +1123,9 @@ static inline int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 static inline int chain_kpw(int wfmt) { return wfmt == kChainW16 ? 2 : (wfmt == kChainW8 ? 4 : 8); }   // k per column of a word
 static inline int64_t chain_kw(int64_t k, int wfmt) { return cdiv64(cdiv64(k, chain_kpw(wfmt)), NS) * NS; }
 
-bool chain_supported(int dtype, int64_t m, int64_t k, int64_t n, bool dual, bool norm, int wfmt) {
+bool chain_supported(int dtype, int64_t m, int64_t k, int64_t n, bool dual, bool norm, int wfmt, bool x_f32) {
     if (dtype != 2 || m != 1 || k < 4 || n < 4) return false;
+    if (x_f32 && (!norm || k > 4 * (MAXI / 2) * NT)) return false;
     if (wfmt < kChainW16 || wfmt > kChainW4) return false;
     if (k % 4 != 0 || n % (dual ? 2 : 4) != 0) return false;
     if (wfmt == kChainW4 && k % 128 != 0) return false;

@@ -162,6 +162,48 @@ static void rms_norm_t(hipStream_t s, const T* x, const T* g, T* y, int64_t rows
     else if (per <= 16) rms_norm_kernel<T, 16><<<(unsigned)rows, block, 0, s>>>(x, g, y, n, inv_n, eps);
     else rms_norm_long_kernel<T><<<(unsigned)rows, 1024, 0, s>>>(x, g, y, n, inv_n, eps);
 }
+// f32 rows and gains, bf16 result: the f32 value of normalization.rs:183-217 rounded once (the pair
+// Cast(bf16)(rms_norm(x)) of a bf16 model whose residual stream is f32).  Rows whose length is a multiple of 8: two
+// 16-byte loads of x and of gamma and one 16-byte store per thread.
+__global__ void rms_norm_f32_bf16_kernel(const float* __restrict__ x, const float* __restrict__ gamma, bf16_t* __restrict__ y,
+                                         int64_t n, float inv_n, float eps) {
+    __shared__ float red[16];
+    const float* row = x + (int64_t)blockIdx.x * n;
+    bf16_t* out = y + (int64_t)blockIdx.x * n;
+    const bool vec = (n % 8) == 0 && ((((uintptr_t)x | (uintptr_t)gamma | (uintptr_t)y) & 15u) == 0);
+    float q = 0.f;
+    if (vec) {
+        for (int64_t c = threadIdx.x; c * 8 < n; c += blockDim.x) {
+            const float4 a = *reinterpret_cast<const float4*>(row + c * 8), b = *reinterpret_cast<const float4*>(row + c * 8 + 4);
+            q += a.x * a.x; q += a.y * a.y; q += a.z * a.z; q += a.w * a.w;
+            q += b.x * b.x; q += b.y * b.y; q += b.z * b.z; q += b.w * b.w;
+        }
+    } else {
+        for (int64_t i = threadIdx.x; i < n; i += blockDim.x) { const float v = row[i]; q += v * v; }
+    }
+    const float inv_rms = 1.0f / sqrtf(block_sum(q, red) * inv_n + eps);
+    if (vec) {
+        for (int64_t c = threadIdx.x; c * 8 < n; c += blockDim.x) {
+            const float4 a = *reinterpret_cast<const float4*>(row + c * 8), b = *reinterpret_cast<const float4*>(row + c * 8 + 4);
+            const float4 ga = *reinterpret_cast<const float4*>(gamma + c * 8), gb = *reinterpret_cast<const float4*>(gamma + c * 8 + 4);
+            fused_u32x4_t o;
+            o[0] = pack_bf16x2((a.x * inv_rms) * ga.x, (a.y * inv_rms) * ga.y);
+            o[1] = pack_bf16x2((a.z * inv_rms) * ga.z, (a.w * inv_rms) * ga.w);
+            o[2] = pack_bf16x2((b.x * inv_rms) * gb.x, (b.y * inv_rms) * gb.y);
+            o[3] = pack_bf16x2((b.z * inv_rms) * gb.z, (b.w * inv_rms) * gb.w);
+            *reinterpret_cast<fused_u32x4_t*>(out + c * 8) = o;
+        }
+    } else {
+        for (int64_t i = threadIdx.x; i < n; i += blockDim.x) out[i] = f32_to_bf16((row[i] * inv_rms) * gamma[i]);
+    }
+}
+void rms_norm_f32_to_bf16(hipStream_t s, const void* x, const void* gamma, void* y, int64_t rows, int64_t n, float inv_n,
+                          float eps) {
+    if (rows <= 0 || n <= 0) return;
+    const int64_t chunks = cdiv(n, 8);
+    const int threads = chunks <= 64 ? 64 : (chunks <= 256 ? 256 : (chunks <= 512 ? 512 : 1024));
+    rms_norm_f32_bf16_kernel<<<(unsigned)rows, threads, 0, s>>>((const float*)x, (const float*)gamma, (bf16_t*)y, n, inv_n, eps);
+}
 void rms_norm(hipStream_t s, int dtype, const void* x, const void* gamma, void* y, int64_t rows, int64_t n, float inv_n,
               float eps) {
     if (rows <= 0 || n <= 0) return;

@@ -86,7 +86,7 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(const T* __restrict__ x
                                                          const T* __restrict__ beta,
                                                          const T* __restrict__ bias, const T* __restrict__ residual,
                                                          T* __restrict__ y, int M, int64_t K, int64_t N, int64_t ntiles,
-                                                         float inv_n, float eps, int act) {
+                                                         float inv_n, float eps, int act, int out_f32, int x_f32) {
     constexpr int VEC = Word<T>::VEC;
     constexpr int KT = kXsBytes / (int)sizeof(T) / MT;   // rows of x staged at a time (kept as T)
     constexpr int PLANE = TP * MT * VEC;                 // outputs per block (per weight stream set)
@@ -130,7 +130,10 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(const T* __restrict__ x
     // pass below then touches only LDS and gamma.
     // LayerNorm (beta given; normalization.rs:123-174): mean first, then the variance of the centred values, as the
     // stand-alone kernel takes them.
-    const bool one_chunk = K <= KT;
+    // x_f32 (RMSNorm only): x and gamma are f32; the staged row is their f32 norm rounded to T once
+    const float* xf = reinterpret_cast<const float*>(x);
+    const float* gf = reinterpret_cast<const float*>(gamma);
+    const bool one_chunk = K <= KT && !x_f32;
     if (NORM) {
         for (int m = 0; m < M; ++m) {
             float q = 0.f, mean = 0.f;
@@ -140,6 +143,7 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(const T* __restrict__ x
                 mean = block_sum(sm, s_tmp) * inv_n;
             }
             for (int64_t kk = t; kk < K; kk += 256) {
+                if (x_f32) { const float v = xf[(int64_t)m * K + kk]; q += v * v; continue; }
                 const T raw = x[(int64_t)m * K + kk];
                 const float v = ldf(&raw, 0) - mean;
                 if (one_chunk) xs[m][kk] = raw;
@@ -168,10 +172,11 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(const T* __restrict__ x
         for (int m = 0; m < M; ++m)
             for (int64_t kk = t; kk < kt; kk += 256) {
                 // each thread re-reads only the slots it wrote itself in the prologue
-                float v = (NORM && one_chunk) ? ldf(&xs[m][0], kk) : ldf(x, (int64_t)m * K + k0 + kk);
+                float v = (NORM && x_f32) ? xf[(int64_t)m * K + k0 + kk]
+                                          : ((NORM && one_chunk) ? ldf(&xs[m][0], kk) : ldf(x, (int64_t)m * K + k0 + kk));
                 // the value the stand-alone norm kernel would have stored: (x*inv_rms)*gamma, rounded to T
                 if (NORM) {
-                    v = ((v - s_mean[m]) * s_scale[m]) * ldf(gamma, k0 + kk);
+                    v = ((v - s_mean[m]) * s_scale[m]) * (x_f32 ? gf[k0 + kk] : ldf(gamma, k0 + kk));
                     if (beta) v += ldf(beta, k0 + kk);
                 }
                 stf(&xs[m][0], kk, v);
@@ -238,8 +243,12 @@ __global__ __launch_bounds__(256) void gemv_tiled_kernel(const T* __restrict__ x
         const float tot = red[0][o] + red[1][o] + red[2][o] + red[3][o];
         const float tot2 = DUAL ? red[0][PLANE + o] + red[1][PLANE + o] + red[2][PLANE + o] + red[3][PLANE + o] : 0.f;
         const float b = bias ? ldf(bias, col) : 0.f;
-        const float r = residual ? ldf(residual, (int64_t)m * N + col) : 0.f;
-        stf(y, (int64_t)m * N + col, tiled_finish(tot, tot2, DUAL, act, b, residual != nullptr, r));
+        // out_f32: the f32 accumulator (plus an f32 residual) is stored as it is
+        const float r = residual ? (out_f32 ? reinterpret_cast<const float*>(residual)[(int64_t)m * N + col]
+                                            : ldf(residual, (int64_t)m * N + col)) : 0.f;
+        const float res = tiled_finish(tot, tot2, DUAL, act, b, residual != nullptr, r);
+        if (out_f32) reinterpret_cast<float*>(y)[(int64_t)m * N + col] = res;
+        else stf(y, (int64_t)m * N + col, res);
     }
 }
 
@@ -254,7 +263,8 @@ static void launch_tiled(hipStream_t s, const TiledLinearArgs& a) {
     const unsigned grid = (unsigned)cdiv(ntiles, TP);
 #define GPTRS_GT(DUAL, NORM)                                                                                          \
     gemv_tiled_kernel<T, MT, TP, U, DUAL, NORM><<<grid, 256, 0, s>>>((const T*)a.x, (const T*)a.wt, (const T*)a.wt2,         \
-        (const T*)a.gamma, (const T*)a.beta, (const T*)a.bias, (const T*)a.residual, (T*)a.y, (int)a.m, a.k, a.n, ntiles, a.inv_n, a.eps, a.act)
+        (const T*)a.gamma, (const T*)a.beta, (const T*)a.bias, (const T*)a.residual, (T*)a.y, (int)a.m, a.k, a.n, ntiles, a.inv_n, a.eps, a.act, \
+        sizeof(T) == 2 ? a.out_f32 : 0, sizeof(T) == 2 ? a.x_f32 : 0)
     if (a.wt2) { if (a.gamma) GPTRS_GT(true, true); else GPTRS_GT(true, false); }
     else { if (a.gamma) GPTRS_GT(false, true); else GPTRS_GT(false, false); }
 #undef GPTRS_GT

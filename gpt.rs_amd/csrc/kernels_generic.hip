@@ -324,8 +324,8 @@ void take(hipStream_t s, int elem_size, const void* table, const int32_t* idx, v
 // 32x32 output tile per 256-thread block, K stepped by 32 through LDS; arbitrary operand strides.
 // Correctness path for dots no tuned kernel claims (attention score / PV contractions in prefill,
 // odd shapes).  Accumulates in f32 in k order within a tile.
-template <typename T>
-__global__ void dot_generic_kernel(const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ c, DotDesc d) {
+template <typename T, typename TO>
+__global__ void dot_generic_kernel(const T* __restrict__ a, const T* __restrict__ b, TO* __restrict__ c, DotDesc d) {
     __shared__ float As[32][33];
     __shared__ float Bs[32][33];
     const int64_t bi = blockIdx.z;
@@ -356,11 +356,12 @@ __global__ void dot_generic_kernel(const T* __restrict__ a, const T* __restrict_
         if (m < d.m && n < d.n) stf(c, bi * d.c_sb + m * d.c_sm + n, acc[j]);
     }
 }
-void dot_generic(hipStream_t s, int dtype, const void* a, const void* b, void* c, const DotDesc& d) {
+void dot_generic(hipStream_t s, int dtype, const void* a, const void* b, void* c, const DotDesc& d, bool out_f32) {
     if (d.batch * d.m * d.n <= 0) return;
     dim3 grid((unsigned)cdiv(d.n, 32), (unsigned)cdiv(d.m, 32), (unsigned)d.batch);
-    if (dtype == 0) dot_generic_kernel<float><<<grid, 256, 0, s>>>((const float*)a, (const float*)b, (float*)c, d);
-    else dot_generic_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)a, (const bf16_t*)b, (bf16_t*)c, d);
+    if (dtype == 0) dot_generic_kernel<float, float><<<grid, 256, 0, s>>>((const float*)a, (const float*)b, (float*)c, d);
+    else if (out_f32) dot_generic_kernel<bf16_t, float><<<grid, 256, 0, s>>>((const bf16_t*)a, (const bf16_t*)b, (float*)c, d);
+    else dot_generic_kernel<bf16_t, bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)a, (const bf16_t*)b, (bf16_t*)c, d);
 }
 
 // ------------------------------------------------------------------------------ sampling

@@ -170,7 +170,7 @@ __global__ __launch_bounds__(256 * KW) void gemm_mfma_kernel(const T* __restrict
                                                         int M, int K, int N, int Npad, int act, int NT, int MT,
                                                         const T* __restrict__ scale, const T* __restrict__ scale2,
                                                         int full_tiles, int splits, float* __restrict__ part,
-                                                        unsigned* __restrict__ tickets) {
+                                                        unsigned* __restrict__ tickets, int out_f32) {
     constexpr int KPC = Mma<T>::KPC;
     constexpr int kBK = kKb * KPC;                            // k per tile
     typedef typename Mma<T>::frag frag_t;
@@ -445,10 +445,14 @@ __global__ __launch_bounds__(256 * KW) void gemm_mfma_kernel(const T* __restrict
             for (int v = 0; v < 16; ++v) {
                 const int m = m0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
                 if (m >= M) continue;
-                const float r = residual ? Mma<T>::ld(residual, (int64_t)m * N + n) : 0.f;
+                // out_f32: the f32 accumulator (plus an f32 residual) is stored as it is
+                const float r = residual ? (out_f32 ? reinterpret_cast<const float*>(residual)[(int64_t)m * N + n]
+                                                    : Mma<T>::ld(residual, (int64_t)m * N + n)) : 0.f;
                 const float g = acc[i][j][v];
                 const float u = DUAL ? acc[i][DUAL ? j + TN / 2 : j][v] : 0.f;
-                Mma<T>::st(y, (int64_t)m * N + n, mfma_finish(g, u, DUAL, act, bv, residual != nullptr, r));
+                const float o = mfma_finish(g, u, DUAL, act, bv, residual != nullptr, r);
+                if (out_f32) reinterpret_cast<float*>(y)[(int64_t)m * N + n] = o;
+                else Mma<T>::st(y, (int64_t)m * N + n, o);
             }
         }
 }
@@ -505,7 +509,7 @@ static void launch_mfma(hipStream_t s, const MfmaLinearArgs& a) {
     const unsigned grid = (unsigned)(cdiv(full, 8) * 8 + (nt * mt - full) * splits);
     kern<<<grid, 256 * KW, lds_bytes, s>>>((const T*)a.x, (const T*)a.wk, (const T*)a.wk2, (const T*)a.bias, (const T*)a.residual, (T*)a.y,
                                       (int)a.m, (int)a.k, (int)a.n, (int)npad, a.act, (int)nt, (int)mt, (const T*)a.scale, (const T*)a.scale2,
-                                      (int)full, splits, (float*)a.part, a.tickets);
+                                      (int)full, splits, (float*)a.part, a.tickets, a.dtype == 2 ? a.out_f32 : 0);
 }
 
 void mfma_gemm(hipStream_t s, const MfmaLinearArgs& a) {

@@ -94,7 +94,8 @@ template <typename T, bool DUAL>
 __global__ __launch_bounds__(256) void skinny_gemm_kernel(const T* __restrict__ x, const T* __restrict__ ws,
                                                           const T* __restrict__ ws2, const T* __restrict__ bias,
                                                           const T* __restrict__ residual, T* __restrict__ y, int M, int K,
-                                                          int N, int act, float* __restrict__ part, unsigned* __restrict__ tickets) {
+                                                          int N, int act, float* __restrict__ part, unsigned* __restrict__ tickets,
+                                                          int out_f32) {
     constexpr int U = 4;                         // steps per wave and round, all requested before the first is used
     constexpr int KPC = SkinnyT<T>::KPC, KSTEP = 4 * KPC;
     __shared__ float red[4][DUAL ? 2 : 1][64][4];
@@ -180,8 +181,12 @@ __global__ __launch_bounds__(256) void skinny_gemm_kernel(const T* __restrict__ 
     for (int i = 0; i < 4; ++i) {
         const int m = 4 * kg + i;                // D: lane holds rows 4 kg .. 4 kg + 3 of column c
         if (m >= M) continue;
-        const float r = residual ? SkinnyT<T>::ld(residual, (int64_t)m * N + n) : 0.f;
-        SkinnyT<T>::st(y, (int64_t)m * N + n, skinny_finish(g[i], up[i], DUAL, act, bv, residual != nullptr, r));
+        // out_f32: the f32 accumulator (plus an f32 residual) is stored as it is
+        const float r = residual ? (out_f32 ? reinterpret_cast<const float*>(residual)[(int64_t)m * N + n]
+                                            : SkinnyT<T>::ld(residual, (int64_t)m * N + n)) : 0.f;
+        const float o = skinny_finish(g[i], up[i], DUAL, act, bv, residual != nullptr, r);
+        if (out_f32) reinterpret_cast<float*>(y)[(int64_t)m * N + n] = o;
+        else SkinnyT<T>::st(y, (int64_t)m * N + n, o);
     }
 }
 
@@ -238,7 +243,8 @@ __global__ __launch_bounds__(256) void skinny_gemm_quant_kernel(const bf16_t* __
                                                                 const uint8_t* __restrict__ qs2, const bf16_t* __restrict__ sc,
                                                                 const bf16_t* __restrict__ sc2, const bf16_t* __restrict__ bias,
                                                                 const bf16_t* __restrict__ residual, bf16_t* __restrict__ y, int M, int K,
-                                                                int N, int act, float* __restrict__ part, unsigned* __restrict__ tickets) {
+                                                                int N, int act, float* __restrict__ part, unsigned* __restrict__ tickets,
+                                                                int out_f32) {
     constexpr int U = 4;                         // words per wave and round, all requested before the first is used
     constexpr int KPW = QF == 1 ? 64 : 128;      // k per word
     constexpr int SPW = KPW / 32;                // MFMA steps per word
@@ -366,8 +372,11 @@ __global__ __launch_bounds__(256) void skinny_gemm_quant_kernel(const bf16_t* __
     for (int i = 0; i < 4; ++i) {
         const int m = 4 * kg + i;
         if (m >= M) continue;
-        const float r = residual ? bf16_to_f32(residual[(int64_t)m * N + n]) : 0.f;
-        y[(int64_t)m * N + n] = f32_to_bf16(skinny_finish(g[i] * s1, up[i] * s2, DUAL, act, bv, residual != nullptr, r));
+        const float r = residual ? (out_f32 ? reinterpret_cast<const float*>(residual)[(int64_t)m * N + n]
+                                            : bf16_to_f32(residual[(int64_t)m * N + n])) : 0.f;
+        const float o = skinny_finish(g[i] * s1, up[i] * s2, DUAL, act, bv, residual != nullptr, r);
+        if (out_f32) reinterpret_cast<float*>(y)[(int64_t)m * N + n] = o;
+        else y[(int64_t)m * N + n] = f32_to_bf16(o);
     }
 }
 
@@ -425,7 +434,7 @@ void skinny_gemm(hipStream_t s, const SkinnyLinearArgs& a) {
 #define GPTRS_LAUNCH(QF, DUAL)                                                                                              \
         skinny_gemm_quant_kernel<QF, DUAL><<<grid, 256, 0, s>>>((const bf16_t*)a.x, (const uint8_t*)a.ws, (const uint8_t*)a.ws2,  \
             (const bf16_t*)a.scale, (const bf16_t*)a.scale2, (const bf16_t*)a.bias, (const bf16_t*)a.residual, (bf16_t*)a.y,   \
-            (int)a.m, (int)a.k, (int)a.n, a.act, (float*)a.part, a.tickets)
+            (int)a.m, (int)a.k, (int)a.n, a.act, (float*)a.part, a.tickets, a.out_f32)
         if (a.quant == 1) { if (a.ws2) GPTRS_LAUNCH(1, true); else GPTRS_LAUNCH(1, false); }
         else { if (a.ws2) GPTRS_LAUNCH(2, true); else GPTRS_LAUNCH(2, false); }
 #undef GPTRS_LAUNCH
@@ -436,7 +445,7 @@ void skinny_gemm(hipStream_t s, const SkinnyLinearArgs& a) {
     const dim3 grid((unsigned)cdiv_s(a.n, 16), (unsigned)ks);
 #define GPTRS_LAUNCH(T, DUAL)                                                                                               \
     skinny_gemm_kernel<T, DUAL><<<grid, 256, 0, s>>>((const T*)a.x, (const T*)a.ws, (const T*)a.ws2, (const T*)a.bias,          \
-        (const T*)a.residual, (T*)a.y, (int)a.m, (int)a.k, (int)a.n, a.act, (float*)a.part, a.tickets)
+        (const T*)a.residual, (T*)a.y, (int)a.m, (int)a.k, (int)a.n, a.act, (float*)a.part, a.tickets, a.dtype == 2 ? a.out_f32 : 0)
     if (a.dtype == 0) { if (a.ws2) GPTRS_LAUNCH(float, true); else GPTRS_LAUNCH(float, false); }
     else { if (a.ws2) GPTRS_LAUNCH(bf16_t, true); else GPTRS_LAUNCH(bf16_t, false); }
 #undef GPTRS_LAUNCH

@@ -85,6 +85,12 @@ static int widen_copies(std::vector<k::CopyDesc>& cs, int es) {
     return es;
 }
 
+// The dtype an FLinear computes in: its weights' (a quantised one: its scales').  x has it too unless an f32 norm was
+// folded in (Instr::x_f32); the result has it unless the accumulator leaves as f32 (Instr::out_f32).
+static inline DType linear_dtype(const Instr& in, const Spec& w, const Spec* scales) {
+    return in.quant && scales ? scales->dtype : w.dtype;
+}
+
 static int64_t norm_axis(int64_t axis, int rank, const char* op) {
     if (axis < 0) axis += rank;
     if (axis < 0 || axis >= rank) fail_exec(std::string(op) + " axis out of range");
@@ -310,7 +316,9 @@ void Builder::validate(Instr& in) {
             auto has = [](const std::vector<int64_t>& v, int64_t x) { return std::find(v.begin(), v.end(), x) != v.end(); };
             for (int i = 0; i < l.rank(); ++i) if (!has(in.a, i) && !has(in.c, i)) want.push_back(l.dims[i]);
             for (int i = 0; i < r.rank(); ++i) if (!has(in.b, i) && !has(in.d, i)) want.push_back(r.dims[i]);
-            expect(out.dtype == l.dtype && out.dims == want, "dot_general output shape mismatch");
+            // out_dtype = F32 on bf16 operands keeps the f32 accumulator (docs/backend.md:104-115)
+            in.out_f32 = in.out_f32 && l.dtype == DType::BF16;
+            expect((out.dtype == l.dtype || in.out_f32) && out.dims == want, "dot_general output shape mismatch");
             break;
         }
         case OpKind::CustomCall: {
@@ -337,7 +345,9 @@ void Builder::validate(Instr& in) {
                 const Spec& c = spec_of(in, 1);
                 expect(c.rank() == 2, in.target + ": codes must be a matrix");
                 check_pair(qd, c, spec_of(in, 2), x.dims[1], c.dims[1], x.dtype);
-                expect(out.dtype == x.dtype && out.dims == std::vector<int64_t>{x.dims[0], c.dims[1]}, in.target + ": output must be [M,N] of x's dtype");
+                in.out_f32 = x.dtype == DType::BF16 && out.dtype == DType::F32;   // the accumulator leaves as f32
+                expect((out.dtype == x.dtype || in.out_f32) && out.dims == std::vector<int64_t>{x.dims[0], c.dims[1]},
+                       in.target + ": output must be [M,N] of x's dtype (or f32)");
                 in.op = OpKind::FLinear;
                 in.op_name = qd == 1 ? "fused.linear_w8" : "fused.linear_w4g128";
                 in.quant = qd;
@@ -542,6 +552,7 @@ void Builder::describe(Step& st) {
         case OpKind::FLinear: {
             const Spec& x = spec_of(in, 0);
             const Spec& w = spec_of(in, 1);
+            const DType ldt = linear_dtype(in, w, in.quant ? &spec_of(in, 2) : nullptr);
             if (in.tiled || in.mfma) {
                 auto pos = [&](size_t op) {
                     const int v = in.operands[op].value;
@@ -556,7 +567,7 @@ void Builder::describe(Step& st) {
                     if (in.act == 2) st.tiled_s2_input = pos(4);
                 }
             }
-            if (in.mfma) st.scratch_bytes = k::mfma_workspace_bytes((int)x.dtype, x.dims[0], x.dims[1], w.dims[1], in.act == 2, in.quant);
+            if (in.mfma) st.scratch_bytes = k::mfma_workspace_bytes((int)ldt, x.dims[0], x.dims[1], w.dims[1], in.act == 2, in.quant);
             if (in.tiled && x.dims[0] >= 2) {
                 // batched decode normalises into scratch first (the matrix-core kernel reads plain rows); layers with
                 // few column tiles add the partial sums of their K splits
@@ -565,12 +576,12 @@ void Builder::describe(Step& st) {
             }
             if (in.quant && !in.mfma && !(in.tiled && x.dims[0] >= 2)) {
                 // stand-alone path of a quantised linear: (RMSNorm of x,) dequantised weights, then the generic kernel
-                const size_t es = dtype_size(x.dtype);
+                const size_t es = dtype_size(ldt);
                 st.scratch_bytes = align_up(in.norm ? (size_t)x.count() * es : 0) +
                                    align_up((size_t)x.dims[1] * w.dims[1] * es) * (in.act == 2 ? 2 : 1) +
-                                   k::linear_workspace_bytes((int)x.dtype, x.dims[0], x.dims[1], w.dims[1], in.act == 2);
+                                   k::linear_workspace_bytes((int)ldt, x.dims[0], x.dims[1], w.dims[1], in.act == 2);
             } else if (!in.tiled && !in.mfma) {
-                st.scratch_bytes = k::linear_workspace_bytes((int)x.dtype, x.dims[0], x.dims[1], w.dims[1], in.act == 2);
+                st.scratch_bytes = k::linear_workspace_bytes((int)ldt, x.dims[0], x.dims[1], w.dims[1], in.act == 2);
             }
             break;
         }
@@ -776,7 +787,8 @@ void Builder::build() {
         if (x.rank() != 2 || w.rank() != 2) return 0;
         const bool dual = in.act == 2;
         if (in.norm_ln) return 0;   // the chain stages RMSNorm only
-        if (!k::chain_supported((int)x.dtype, x.dims[0], x.dims[1], w.dims[1], dual, in.norm, in.quant)) return 0;
+        const DType ldt = linear_dtype(in, w, in.quant ? &plan.values[st.src[2]].spec : nullptr);
+        if (!k::chain_supported((int)ldt, x.dims[0], x.dims[1], w.dims[1], dual, in.norm, in.quant, in.x_f32)) return 0;
         k::ChainPhase p{};
         return k::chain_fill_phase(p, x.dims[1], w.dims[1], dual, in.quant) ? 1 : 0;
     };
@@ -817,8 +829,8 @@ static inline const void* src_ptr(const Step& st, const ExecCtx& cx, size_t i) {
 }
 
 // algorithmic bytes of the weights an FLinear reads once: codes and scales when quantised
-static int64_t linear_weight_bytes(const Instr& in, const Spec& x, const Spec& w) {
-    const int64_t K = x.dims[1], N = w.dims[1], es = (int64_t)dtype_size(x.dtype);
+static int64_t linear_weight_bytes(const Instr& in, DType ldt, const Spec& x, const Spec& w) {
+    const int64_t K = x.dims[1], N = w.dims[1], es = (int64_t)dtype_size(ldt);
     int64_t b = in.quant == 0 ? K * N * es : (in.quant == 1 ? K * N + N * es : K * N / 2 + (K / 128) * N * es);
     return b * (in.act == 2 ? 2 : 1);
 }
@@ -870,7 +882,8 @@ static bool run_chain(const Plan& plan, const Step& head, ExecCtx& cx) {
         k::ChainPhase p{};
         if (!k::chain_fill_phase(p, x.dims[1], w.dims[1], dual, in.quant)) { cx.chain = false; return false; }
         wfmt = in.quant;
-        BufferP wc = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], in.quant == 0 ? 2 : (in.quant == 1 ? 3 : 4), x.dtype,
+        const DType ldt = linear_dtype(in, w, in.quant ? &plan.values[st.src[2]].spec : nullptr);
+        BufferP wc = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], in.quant == 0 ? 2 : (in.quant == 1 ? 3 : 4), ldt,
                                             x.dims[1], w.dims[1], dual ? cx.input_bufs[st.tiled_w2_input] : nullptr);
         p.w = wc->ptr;
         p.x = src_ptr(st, cx, 0);
@@ -879,7 +892,7 @@ static bool run_chain(const Plan& plan, const Step& head, ExecCtx& cx) {
             if (dual) p.wscale2 = src_ptr(st, cx, 4);
             if (((uintptr_t)p.wscale | (uintptr_t)p.wscale2) & 3) fail_exec("decode chain: scale buffers must be 4-byte aligned");
         } else if (in.quant == 2) {  // group scales follow the tile order of the weights
-            BufferP sc = cx.be->derived_weights(cx.input_bufs[st.tiled_s_input], 5, x.dtype, x.dims[1], w.dims[1],
+            BufferP sc = cx.be->derived_weights(cx.input_bufs[st.tiled_s_input], 5, ldt, x.dims[1], w.dims[1],
                                                 dual ? cx.input_bufs[st.tiled_s2_input] : nullptr);
             p.wscale = sc->ptr;
         }
@@ -888,10 +901,13 @@ static bool run_chain(const Plan& plan, const Step& head, ExecCtx& cx) {
         if (in.has_residual) { p.residual = src_ptr(st, cx, oi++); p.flags |= k::kChainResidual; }
         if (in.norm) { p.gamma = src_ptr(st, cx, oi++); p.inv_n = in.scale; p.eps = in.eps; p.flags |= k::kChainNorm; }
         if (in.act == 1) p.flags |= k::kChainGelu;
+        if (in.out_f32) p.flags |= k::kChainOutF32;
+        if (in.x_f32) p.flags |= k::kChainXF32;
         p.y = cx.ptr[st.dst[0]];
         aligned8({p.x, p.y, p.residual, p.bias, p.gamma});
+        if (in.x_f32 && ((uintptr_t)p.gamma & 15)) fail_exec("decode chain: f32 gains must be 16-byte aligned");
         lds_bytes = std::max(lds_bytes, p.lds_total);
-        bytes += (int64_t)dtype_size(x.dtype) * (x.dims[1] + w.dims[1]) + linear_weight_bytes(in, x, w);
+        bytes += (int64_t)dtype_size(x.dtype) * x.dims[1] + (int64_t)(in.out_f32 ? 4 : dtype_size(ldt)) * w.dims[1] + linear_weight_bytes(in, ldt, x, w);
         phases.push_back(p);
     }
     const k::ChainPhase* table = cx.be->chain_table(phases);
@@ -991,7 +1007,8 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
         case OpKind::Dot: {
             const void* a = src_ptr(st, cx, 0);
             const void* b = src_ptr(st, cx, 1);
-            const int es = (int)dtype_size(out.dtype);
+            const DType idt = in_spec(0).dtype;   // the operands' dtype (the result's may be f32 over bf16 operands)
+            const int es = (int)dtype_size(idt);
             if (st.lhs_pack) {
                 void* p = cx.ws + st.scratch_off + st.pack_l_off;
                 k::copy_strided(s, p, a, es, st.pack_l, nullptr);
@@ -1004,7 +1021,7 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
                 b = p;
                 ++cx.launches;
             }
-            k::dot_generic(s, (int)out.dtype, a, b, dst, st.dot);
+            k::dot_generic(s, (int)idt, a, b, dst, st.dot, in.out_f32);
             ++cx.launches;
             break;
         }
@@ -1018,7 +1035,10 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
         case OpKind::FRmsNorm: {
             const Spec& x = in_spec(0);
             const int64_t n = x.dims.back();
-            k::rms_norm(s, (int)out.dtype, src_ptr(st, cx, 0), src_ptr(st, cx, 1), dst, n ? x.count() / n : 0, n, in.scale, in.eps);
+            if (x.dtype == DType::F32 && out.dtype == DType::BF16)   // Cast(bf16)(rms_norm(x f32)) folded
+                k::rms_norm_f32_to_bf16(s, src_ptr(st, cx, 0), src_ptr(st, cx, 1), dst, n ? x.count() / n : 0, n, in.scale, in.eps);
+            else
+                k::rms_norm(s, (int)out.dtype, src_ptr(st, cx, 0), src_ptr(st, cx, 1), dst, n ? x.count() / n : 0, n, in.scale, in.eps);
             ++cx.launches;
             break;
         }
@@ -1045,21 +1065,30 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
             if (cx.chain && st.chain_len > 0 && run_chain(plan, st, cx)) break;
             const Spec& x = in_spec(0);
             const Spec& w = in_spec(1);
+            const DType ldt = linear_dtype(in, w, in.quant ? &in_spec(2) : nullptr);
+            const int64_t io_bytes = (int64_t)dtype_size(x.dtype) * x.count() + (int64_t)dtype_size(out.dtype) * out.count();
+            // RMSNorm of x into scratch for the kernels that read plain rows of the compute dtype
+            auto norm_into = [&](const void* xp, const void* gp, void* to) {
+                if (in.x_f32) k::rms_norm_f32_to_bf16(s, xp, gp, to, x.dims[0], x.dims[1], in.scale, in.eps);
+                else k::rms_norm(s, (int)ldt, xp, gp, to, x.dims[0], x.dims[1], in.scale, in.eps);
+                ++cx.launches;
+            };
             if (in.mfma) {
                 k::MfmaLinearArgs ma{};
-                ma.dtype = (int)x.dtype;
+                ma.dtype = (int)ldt;
+                ma.out_f32 = in.out_f32;
                 ma.x = src_ptr(st, cx, 0);
                 ma.m = x.dims[0]; ma.k = x.dims[1]; ma.n = w.dims[1];
                 // quantised weights: the k-grouped copy holds the codes; the kernel applies the scales on the way into LDS
                 const int kind = in.quant == 0 ? 1 : (in.quant == 1 ? 6 : 7);
-                BufferP wk = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], kind, x.dtype, ma.k, ma.n);
+                BufferP wk = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], kind, ldt, ma.k, ma.n);
                 BufferP wk2;
                 ma.wk = wk->ptr;
                 ma.quant = in.quant;
                 if (in.quant) ma.scale = cx.input_bufs[st.tiled_s_input]->ptr;
                 size_t oi = linear_extra_pos(in);
                 if (in.act == 2) {
-                    wk2 = cx.be->derived_weights(cx.input_bufs[st.tiled_w2_input], kind, x.dtype, ma.k, ma.n);
+                    wk2 = cx.be->derived_weights(cx.input_bufs[st.tiled_w2_input], kind, ldt, ma.k, ma.n);
                     ma.wk2 = wk2->ptr;
                     if (in.quant) ma.scale2 = cx.input_bufs[st.tiled_s2_input]->ptr;
                 }
@@ -1083,28 +1112,29 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
                     GPTRS_HIP_CHECK(hipEventRecord(e1, s));
                     cx.be->prof_events.emplace_back(e0, e1);
                     ++cx.be->prof_linear_calls;
-                    cx.be->prof_linear_bytes += (int64_t)dtype_size(x.dtype) * (ma.m * ma.k + ma.m * ma.n) + linear_weight_bytes(in, x, w);
+                    cx.be->prof_linear_bytes += io_bytes + linear_weight_bytes(in, ldt, x, w);
                 }
                 ++cx.launches;
                 break;
             }
             if (in.tiled &&
-                (in.quant ? k::skinny_quant_supported((int)x.dtype, x.dims[0], x.dims[1], w.dims[1], in.quant)
-                          : k::skinny_gemm_supported((int)x.dtype, x.dims[0], x.dims[1], w.dims[1])) &&
+                (in.quant ? k::skinny_quant_supported((int)ldt, x.dims[0], x.dims[1], w.dims[1], in.quant)
+                          : k::skinny_gemm_supported((int)ldt, x.dims[0], x.dims[1], w.dims[1])) &&
                 (!in.norm || st.scratch_bytes >= (size_t)x.count() * dtype_size(x.dtype))) {
                 k::SkinnyLinearArgs sa{};
-                sa.dtype = (int)x.dtype;
+                sa.dtype = (int)ldt;
+                sa.out_f32 = in.out_f32;
                 sa.x = src_ptr(st, cx, 0);
                 sa.m = x.dims[0]; sa.k = x.dims[1]; sa.n = w.dims[1];
                 const int kind = in.quant == 0 ? 8 : (in.quant == 1 ? 9 : 10);   // bf16 copy, or the codes in the same tile order
-                BufferP wsk = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], kind, x.dtype, sa.k, sa.n);
+                BufferP wsk = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], kind, ldt, sa.k, sa.n);
                 BufferP wsk2;
                 sa.ws = wsk->ptr;
                 sa.quant = in.quant;
                 if (in.quant) sa.scale = src_ptr(st, cx, 2);
                 size_t oi = linear_extra_pos(in);
                 if (in.act == 2) {
-                    wsk2 = cx.be->derived_weights(cx.input_bufs[st.tiled_w2_input], kind, x.dtype, sa.k, sa.n);
+                    wsk2 = cx.be->derived_weights(cx.input_bufs[st.tiled_w2_input], kind, ldt, sa.k, sa.n);
                     sa.ws2 = wsk2->ptr;
                     if (in.quant) sa.scale2 = src_ptr(st, cx, 4);
                 }
@@ -1114,12 +1144,12 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
                 if (in.norm) {
                     void* xn = cx.ws + st.scratch_off;
                     if (in.norm_ln) {
-                        k::layer_norm(s, (int)x.dtype, sa.x, src_ptr(st, cx, oi), src_ptr(st, cx, oi + 1), xn, sa.m, sa.k, in.scale, in.eps);
+                        k::layer_norm(s, (int)ldt, sa.x, src_ptr(st, cx, oi), src_ptr(st, cx, oi + 1), xn, sa.m, sa.k, in.scale, in.eps);
                         oi += 2;
+                        ++cx.launches;
                     } else {
-                        k::rms_norm(s, (int)x.dtype, sa.x, src_ptr(st, cx, oi++), xn, sa.m, sa.k, in.scale, in.eps);
+                        norm_into(sa.x, src_ptr(st, cx, oi++), xn);
                     }
-                    ++cx.launches;
                     sa.x = xn;
                 }
                 if (st.scratch_bytes > norm_bytes) {
@@ -1140,22 +1170,24 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
                     GPTRS_HIP_CHECK(hipEventRecord(e1, s));
                     cx.be->prof_events.emplace_back(e0, e1);
                     ++cx.be->prof_linear_calls;
-                    cx.be->prof_linear_bytes += (int64_t)dtype_size(x.dtype) * (sa.m * sa.k + sa.m * sa.n) + linear_weight_bytes(in, x, w);
+                    cx.be->prof_linear_bytes += io_bytes + linear_weight_bytes(in, ldt, x, w);
                 }
                 ++cx.launches;
                 break;
             }
             if (in.tiled && !in.quant) {
                 k::TiledLinearArgs ta{};
-                ta.dtype = (int)x.dtype;
+                ta.dtype = (int)ldt;
+                ta.out_f32 = in.out_f32;
+                ta.x_f32 = in.x_f32;
                 ta.x = src_ptr(st, cx, 0);
                 ta.m = x.dims[0]; ta.k = x.dims[1]; ta.n = w.dims[1];
-                BufferP wt = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], 0, x.dtype, ta.k, ta.n);
+                BufferP wt = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], 0, ldt, ta.k, ta.n);
                 BufferP wt2;
                 ta.wt = wt->ptr;
                 size_t oi = 2;
                 if (in.act == 2) {
-                    wt2 = cx.be->derived_weights(cx.input_bufs[st.tiled_w2_input], 0, x.dtype, ta.k, ta.n);
+                    wt2 = cx.be->derived_weights(cx.input_bufs[st.tiled_w2_input], 0, ldt, ta.k, ta.n);
                     ta.wt2 = wt2->ptr;
                     ++oi;
                 }
@@ -1176,13 +1208,13 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
                     GPTRS_HIP_CHECK(hipEventRecord(e1, s));
                     cx.be->prof_events.emplace_back(e0, e1);
                     ++cx.be->prof_linear_calls;
-                    cx.be->prof_linear_bytes += (int64_t)dtype_size(x.dtype) * (ta.m * ta.k + ta.k * ta.n * (ta.wt2 ? 2 : 1) + ta.m * ta.n);
+                    cx.be->prof_linear_bytes += io_bytes + linear_weight_bytes(in, ldt, x, w);
                 }
                 ++cx.launches;
                 break;
             }
             k::LinearArgs a{};
-            a.dtype = (int)x.dtype;
+            a.dtype = (int)ldt;
             a.x = src_ptr(st, cx, 0);
             a.w = src_ptr(st, cx, 1);
             a.m = x.dims[0]; a.k = x.dims[1]; a.n = w.dims[1];
@@ -1192,18 +1224,17 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
             if (in.quant) {
                 // stand-alone path of a quantised linear: the weights are dequantised into scratch and the generic
                 // kernel runs over them (the decode chain and the matrix-core kernels over the codes are the fast paths)
-                const size_t es = dtype_size(x.dtype);
+                const size_t es = dtype_size(ldt);
                 char* wsp = cx.ws + st.scratch_off;
                 const size_t wbytes = align_up((size_t)a.k * a.n * es);
                 auto deq = [&](size_t codes, size_t scales, void* to) {
-                    if (in.quant == 1) k::dequant_w8(s, (int)x.dtype, (const int8_t*)src_ptr(st, cx, codes), src_ptr(st, cx, scales), to, a.k, a.n);
-                    else k::dequant_w4g128(s, (int)x.dtype, (const uint8_t*)src_ptr(st, cx, codes), src_ptr(st, cx, scales), to, a.k, a.n);
+                    if (in.quant == 1) k::dequant_w8(s, (int)ldt, (const int8_t*)src_ptr(st, cx, codes), src_ptr(st, cx, scales), to, a.k, a.n);
+                    else k::dequant_w4g128(s, (int)ldt, (const uint8_t*)src_ptr(st, cx, codes), src_ptr(st, cx, scales), to, a.k, a.n);
                     ++cx.launches;
                 };
                 if (in.norm) {
                     const size_t gi = i + (in.has_bias ? 1 : 0) + (in.has_residual ? 1 : 0);
-                    k::rms_norm(s, (int)x.dtype, a.x, src_ptr(st, cx, gi), wsp, a.m, a.k, in.scale, in.eps);
-                    ++cx.launches;
+                    norm_into(a.x, src_ptr(st, cx, gi), wsp);
                     a.x = wsp;
                     wsp += align_up((size_t)x.count() * es);
                 }
@@ -1221,6 +1252,20 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
             a.y = dst;
             a.act = in.act == 1 ? 1 : 0;
             a.counters = cx.counters;
+            if (in.out_f32) {
+                // f32 result over bf16 operands outside the fast kernels (a quantised linear with the chain switched off):
+                // the generic dot stores the accumulator, the f32 residual is added by the element-wise kernel
+                if (in.act != 0 || in.has_bias) fail_exec("linear: f32 result with an absorbed activation or bias");
+                k::DotDesc d{};
+                d.batch = 1; d.m = a.m; d.n = a.n; d.k = a.k;
+                d.a_sb = 0; d.a_sm = a.k; d.a_sk = 1;
+                d.b_sb = 0; d.b_sk = a.n; d.b_sn = 1;
+                d.c_sb = a.m * a.n; d.c_sm = a.n;
+                k::dot_generic(s, (int)ldt, a.x, a.w, dst, d, true);
+                ++cx.launches;
+                if (in.has_residual) { k::binary(s, 0, (int)BinaryOp::Add, dst, a.residual, dst, out.count()); ++cx.launches; }
+                break;
+            }
             hipEvent_t e0 = nullptr, e1 = nullptr;
             if (cx.profile) {
                 GPTRS_HIP_CHECK(hipEventCreate(&e0));
@@ -1233,7 +1278,7 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
                 cx.be->prof_events.emplace_back(e0, e1);
                 ++cx.be->prof_linear_calls;
                 // algorithmic bytes: activations in, every weight once, result out
-                cx.be->prof_linear_bytes += (int64_t)dtype_size(x.dtype) * (a.m * a.k + a.m * a.n) + linear_weight_bytes(in, x, w);
+                cx.be->prof_linear_bytes += io_bytes + linear_weight_bytes(in, ldt, x, w);
             }
             cx.launches += (in.act == 2 && a.m > 16) ? 3 : 1;
             break;

@@ -138,6 +138,7 @@ Instr parse_instruction(const Json& j, Function& fn) {
         in.c = int_list(attr->at("contract_lhs"));
         in.d = int_list(attr->at("contract_rhs"));
         reject_dtype_override(*attr, "dot_general", in.out_specs[0].dtype);
+        if (const Json* o = attr->find("out_dtype")) in.out_f32 = !o->is_null() && in.out_specs[0].dtype == DType::F32;
     } else if (name == "Reduce") {
         in.op = OpKind::Reduce; need(1);
         in.reduce = parse_enum<ReduceKind>(attr->at("kind"), {{"Sum", ReduceKind::Sum}, {"Max", ReduceKind::Max},

@@ -123,6 +123,12 @@ struct Instr {
     bool tiled = false;                      // FLinear: decode GEMV over the column-tiled weight copy
     bool norm = false;                       // FLinear: RMSNorm of x fused in (last operand = gamma; eps, scale)
     bool norm_ln = false;                    // with norm: LayerNorm instead (last two operands = gamma, beta)
+    // Dot / FLinear with bf16 operands whose f32 accumulator leaves as f32 (DotGeneralSpec.out_dtype = F32,
+    // spec.rs:354-361); an FLinear's residual operand is then f32 too
+    bool out_f32 = false;
+    // FLinear with norm whose x (and gamma) are f32 while the weights are bf16: the norm runs in f32 and its result is
+    // rounded to bf16 once (the fold of Cast(bf16)(rms_norm(x f32)) into the linear)
+    bool x_f32 = false;
     // FLinear over weight-only quantised weights (0: none; 1: int8 per column, 2: int4 groups of 128): every
     // weight operand is then a (codes, scales) pair: (x, q, s, [q2, s2], [bias], [residual], [gamma]).
     // FQuant: 1 int8 scales, 2 int8 codes, 3 int4 scales, 4 int4 codes, 5 int8 dequantise, 6 int4 dequantise

@@ -18,9 +18,9 @@ from .ptir import Tensor, TensorSpec
 
 
 # --------------------------------------------------------------------------- basics
-def matmul(a: Tensor, b: Tensor) -> Tensor:
-    """ops/functional/linalg.rs:109-127."""
-    return a.matmul(b)
+def matmul(a: Tensor, b: Tensor, out_dtype: Optional[str] = None) -> Tensor:
+    """ops/functional/linalg.rs:109-127; `out_dtype` sets DotGeneralSpec.out_dtype (spec.rs:354-361)."""
+    return a.matmul(b, out_dtype)
 
 
 def add_bias(x: Tensor, bias: Tensor) -> Tensor:
@@ -28,13 +28,14 @@ def add_bias(x: Tensor, bias: Tensor) -> Tensor:
     return x + bias.broadcast_to(x.dims)
 
 
-def linear(x: Tensor, weight: Tensor, bias: Optional[Tensor] = None) -> Tensor:
-    """nn/layers/linear.rs:50-71: x[T,in] . W[in,out] (+ b)."""
+def linear(x: Tensor, weight: Tensor, bias: Optional[Tensor] = None, out_dtype: Optional[str] = None) -> Tensor:
+    """nn/layers/linear.rs:50-71: x[T,in] . W[in,out] (+ b).  `out_dtype`: the product leaves the f32 accumulator in that
+    dtype (docs/backend.md:104-115) instead of x's."""
     if x.spec.rank != 2:
         raise ValueError(f"linear expects 2D input, got shape {x.dims}")
     if x.dims[1] != weight.dims[0]:
         raise ValueError(f"input features ({x.dims[1]}) must match weight rows ({weight.dims[0]})")
-    out = matmul(x, weight)
+    out = matmul(x, weight, out_dtype)
     if bias is not None:
         out = add_bias(out, bias)
     return out
@@ -82,8 +83,9 @@ def dequantize_weight(q: Tensor, s: Tensor) -> Tensor:
     raise ValueError(f"codes must be Si8 (w8) or Ui8 (w4g128), got {q.dtype}")
 
 
-def linear_quantized(x: Tensor, q: Tensor, s: Tensor, bias: Optional[Tensor] = None) -> Tensor:
-    """x[T,K] . dequantise(q, s)[K,N] (+ b) without materialising the matrix: f32 accumulation, result in x's dtype."""
+def linear_quantized(x: Tensor, q: Tensor, s: Tensor, bias: Optional[Tensor] = None, out_dtype: Optional[str] = None) -> Tensor:
+    """x[T,K] . dequantise(q, s)[K,N] (+ b) without materialising the matrix: f32 accumulation, result in x's dtype
+    (or in `out_dtype`, the declared dtype of the call's output)."""
     if x.spec.rank != 2:
         raise ValueError(f"linear expects 2D input, got shape {x.dims}")
     if q.dtype == "Si8":
@@ -94,7 +96,7 @@ def linear_quantized(x: Tensor, q: Tensor, s: Tensor, bias: Optional[Tensor] = N
         raise ValueError(f"codes must be Si8 (w8) or Ui8 (w4g128), got {q.dtype}")
     if x.dims[1] != k:
         raise ValueError(f"input features ({x.dims[1]}) must match weight rows ({k})")
-    out = x.fb.custom_call(target, [x, q, s], TensorSpec(x.dtype, [x.dims[0], q.dims[1]]))
+    out = x.fb.custom_call(target, [x, q, s], TensorSpec(out_dtype or x.dtype, [x.dims[0], q.dims[1]]))
     if bias is not None:
         out = add_bias(out, bias)
     return out

@@ -135,9 +135,9 @@ class _ModelBase:
         self.set_param_handle(name + ".s", s)
 
     # -- checkpoints -----------------------------------------------------------------
-    def _load_tensors(self, ck, expected: Dict[str, tuple]):
+    def _load_tensors(self, ck, expected: Dict[str, tuple], dtype: Optional[str] = None):
         """Upload every expected tensor from an open checkpoint (checkpoint/loader.rs: by name, shape checked),
-        one at a time out of the file mapping."""
+        one at a time out of the file mapping; `dtype` overrides the model's storage dtype."""
         from .checkpoint import CheckpointError
         for name, dims in expected.items():
             e = ck.entry(name)
@@ -150,7 +150,7 @@ class _ModelBase:
                 host = bf16_bits_to_f32(np.asarray(arr))
             else:
                 raise CheckpointError(f"tensor `{name}`: dtype {e.dtype} cannot feed a model parameter")
-            self.set_param(name, host)
+            self.set_param(name, host, dtype)
 
     def save_checkpoint(self, path: str, kind: str, config: Dict[str, object]):
         """Write the parameters back as a GPTRSCHK v2 file (checkpoint/saver.rs), in their storage dtype."""
@@ -500,15 +500,28 @@ class Ministral(_ModelBase):
 
     namespace = "ministral"
 
-    def __init__(self, config: MinistralConfig, backend, dtype: str = "Bf16"):
+    def __init__(self, config: MinistralConfig, backend, dtype: str = "Bf16", residual_dtype: Optional[str] = None):
+        """`residual_dtype="F32"` on a bf16 model keeps the residual stream, the norms and the logits in f32: the
+        embedding rows are cast up, RMSNorm runs on f32 (what the reference's rms_norm requires,
+        ops/functional/normalization.rs:183-217) and is cast to bf16 for the projection that follows, the two
+        projections that feed a residual add (attention out, feed-forward down) and the lm_head leave their f32
+        accumulator as f32 (DotGeneralSpec.out_dtype, spec.rs:354-361; docs/backend.md:104-115).  Matmul operands,
+        RoPE, attention and the KV cache stay bf16.  Norm gains are then stored as f32."""
         super().__init__(backend, dtype)
         self.config = config
         self.attn = config.attention_config()
         self.rope = F.RopeConfig(config.rotary_dim, config.rope_theta, config.rope_scaling)
+        if residual_dtype is not None and residual_dtype not in ("F32",):
+            raise ValueError("residual_dtype must be None or 'F32'")
+        self.residual_dtype = residual_dtype if (residual_dtype and residual_dtype != dtype) else None
+
+    @property
+    def norm_dtype(self) -> str:
+        return self.residual_dtype or self.dtype
 
     @classmethod
     def random(cls, config: MinistralConfig, backend, seed: int = 0, dtype: str = "Bf16", std: float = 0.02,
-               bf16_values: bool = False, quant: Optional[str] = None):
+               bf16_values: bool = False, quant: Optional[str] = None, residual_dtype: Optional[str] = None):
         """Shapes and constant inits of Ministral::random (model/ministral.rs:262-330).  Every
         tensor draws from its own numpy stream SeedSequence([seed, index]), so the weights do not
         depend on the order or the number of worker threads that generate them.  `bf16_values`
@@ -516,7 +529,7 @@ class Ministral(_ModelBase):
         model can be given exactly the weights of a bf16 one.  `quant` ("w8" / "w4g128") quantises
         every linear weight (projections, feed-forward, lm_head) as it arrives on the device."""
         from concurrent.futures import ThreadPoolExecutor
-        m = cls(config, backend, dtype)
+        m = cls(config, backend, dtype, residual_dtype)
         d, a = config.embed_dim, config.attention_config()
         plan = [("tok_embeddings.weight", (config.vocab_size, d), "randn")]
         for i in range(config.num_layers):
@@ -533,13 +546,13 @@ class Ministral(_ModelBase):
         def make(idx):
             name, shape, kind = plan[idx]
             if kind == "ones":
-                arr = np.ones(shape, np.float32)
+                return name, shape, m.norm_dtype, _np_to_bytes(np.ones(shape, np.float32), m.norm_dtype)
             else:
                 arr = np.random.default_rng(np.random.SeedSequence([seed, idx])).standard_normal(shape, dtype=np.float32)
                 arr *= np.float32(std)
                 if bf16_values and dtype != "Bf16":
                     arr = bf16_bits_to_f32(f32_to_bf16_bits(arr))
-            return name, shape, _np_to_bytes(arr, dtype)
+            return name, shape, dtype, _np_to_bytes(arr, dtype)
 
         workers = max(1, min(16, (os.cpu_count() or 1)))
         with ThreadPoolExecutor(max_workers=workers) as ex:
@@ -549,8 +562,8 @@ class Ministral(_ModelBase):
                 while nxt < len(plan) and len(pending) < 2 * workers:
                     pending.append(ex.submit(make, nxt))
                     nxt += 1
-                name, shape, data = pending.pop(0).result()
-                m.set_param_bytes(name, TensorSpec(dtype, shape), data)
+                name, shape, dt, data = pending.pop(0).result()
+                m.set_param_bytes(name, TensorSpec(dt, shape), data)
                 if quant and len(shape) == 2 and name != "tok_embeddings.weight":
                     m.quantize_param(name, quant)
         return m
@@ -583,7 +596,8 @@ class Ministral(_ModelBase):
         raise ValueError(f"unknown rope scaling kind {js['kind']!r}")
 
     @classmethod
-    def from_checkpoint(cls, path: str, backend, dtype: str = "Bf16", quant: Optional[str] = None) -> "Ministral":
+    def from_checkpoint(cls, path: str, backend, dtype: str = "Bf16", quant: Optional[str] = None,
+                        residual_dtype: Optional[str] = None) -> "Ministral":
         """runtime/loader.rs:19-241 for kind "ministral" (MinistralConfig, model/ministral.rs:13-30)."""
         from .checkpoint import Checkpoint, CheckpointError
         with Checkpoint(path) as ck:
@@ -598,9 +612,9 @@ class Ministral(_ModelBase):
                                   head_dim=head_dim, ffn_dim=int(c["mlp_hidden_dim"]), rotary_dim=int(c["rotary_dim"]),
                                   rope_theta=float(c["rope_theta"]), eps=float(c["rms_norm_eps"]),
                                   rope_scaling=cls._scaling_from_json(c.get("rope_scaling")))
-            m = cls(cfg, backend, dtype)
+            m = cls(cfg, backend, dtype, residual_dtype)
             for name, dims in m.expected_params().items():
-                m._load_tensors(ck, {name: dims})
+                m._load_tensors(ck, {name: dims}, m.norm_dtype if name.endswith(".gamma") else None)
                 if quant and len(dims) == 2 and name != "tok_embeddings.weight":
                     m.quantize_param(name, quant)
         return m
@@ -637,11 +651,16 @@ class Ministral(_ModelBase):
     @property
     def context_length(self): return self.config.context_length
 
-    def _linear(self, P, name: str, x: Tensor) -> Tensor:
+    def _linear(self, P, name: str, x: Tensor, out_dtype: Optional[str] = None) -> Tensor:
         """nn/layers/linear.rs:50-71 without bias; quantised weights are read as codes and scales."""
         if name + ".q" in P:
-            return F.linear_quantized(x, P[name + ".q"], P[name + ".s"])
-        return F.linear(x, P[name])
+            return F.linear_quantized(x, P[name + ".q"], P[name + ".s"], out_dtype=out_dtype)
+        return F.linear(x, P[name], out_dtype=out_dtype)
+
+    def _norm(self, x: Tensor, gamma: Tensor) -> Tensor:
+        """RMSNorm in the residual stream's dtype, handed on in the matmul dtype."""
+        out, *_ = F.rms_norm(x, gamma, self.config.eps)
+        return out.cast(self.dtype) if self.residual_dtype else out
 
     def _build(self, seq: int, capacity: int, decode: bool, batch: int = 1, last_only: bool = False) -> Tuple[Program, dict]:
         last_only = last_only and seq > 1
@@ -669,11 +688,14 @@ class Ministral(_ModelBase):
         layout["n_args"] = len(fb.params)
         P = self._declare_params(fb)
 
+        rdt = self.residual_dtype   # None: every tensor in the model dtype
         hidden = F.embedding_lookup(P["tok_embeddings.weight"], tok)
+        if rdt:
+            hidden = hidden.cast(rdt)
         new_caches = [[None] * L for _ in range(batch)]
         for i in range(L):
             p = f"blocks.{i}."
-            normed, *_ = F.rms_norm(hidden, P[p + "norm_1.gamma"], cfg.eps)
+            normed = self._norm(hidden, P[p + "norm_1.gamma"])
             qkv = self._linear(P, p + "attention.w_qkv", normed)
             ctxs = []
             for b in range(batch):
@@ -690,18 +712,18 @@ class Ministral(_ModelBase):
                 new_caches[b][i] = (k2, v2)
                 ctxs.append(ctx)
             ctx_all = ctxs[0] if batch == 1 else Tensor.concat(0, ctxs)
-            attn_out = self._linear(P, p + "attention.w_out", ctx_all)
+            attn_out = self._linear(P, p + "attention.w_out", ctx_all, rdt)
             residual = attn_out + hidden
-            normed2, *_ = F.rms_norm(residual, P[p + "norm_2.gamma"], cfg.eps)
+            normed2 = self._norm(residual, P[p + "norm_2.gamma"])
             gate = self._linear(P, p + "feed_forward.w_gate", normed2)     # nn/layers/feed_forward.rs GatedFeedForward
             up = self._linear(P, p + "feed_forward.w_up", normed2)
             act = F.swiglu(gate, up)
-            ff = self._linear(P, p + "feed_forward.w_down", act)
+            ff = self._linear(P, p + "feed_forward.w_down", act, rdt)
             hidden = ff + residual
         if last_only:
             hidden = _last_rows(hidden, seq, batch)
-        normalized, *_ = F.rms_norm(hidden, P["final_norm.gamma"], cfg.eps)
-        logits = self._linear(P, "lm_head", normalized)
+        normalized = self._norm(hidden, P["final_norm.gamma"])
+        logits = self._linear(P, "lm_head", normalized, rdt)
         results = []
         for b in range(batch):
             for i in range(L):

@@ -207,8 +207,10 @@ class Tensor:
     def reduce_min(self, axes, keepdims=True): return self._reduce("Min", axes, keepdims)
 
     def dot_general(self, rhs: "Tensor", batch: Sequence[int], contract_lhs: Sequence[int],
-                    contract_rhs: Sequence[int], batch_rhs: Optional[Sequence[int]] = None) -> "Tensor":
-        """DotGeneral with DotAttrs::default() (accum/out dtype None; docs/backend.md:104-115).
+                    contract_rhs: Sequence[int], batch_rhs: Optional[Sequence[int]] = None,
+                    out_dtype: Optional[str] = None) -> "Tensor":
+        """DotGeneral; DotAttrs::default() (accum/out dtype None; docs/backend.md:104-115) unless `out_dtype` names
+        the result dtype (DotGeneralSpec.out_dtype, spec.rs:354-361: accumulate in f32, cast to out_dtype).
 
         Output dims: batch, lhs free, rhs free (docs/backend.md:287-291).
         """
@@ -227,15 +229,15 @@ class Tensor:
         out += [d for i, d in enumerate(self.dims) if i not in batch_l and i not in cl]
         out += [d for i, d in enumerate(rhs.dims) if i not in batch_r and i not in cr]
         op = {"DotGeneral": {"batch_lhs": batch_l, "batch_rhs": batch_r, "contract_lhs": cl,
-                             "contract_rhs": cr, "accum_dtype": None, "out_dtype": None}}
-        return self.fb.emit(op, [self, rhs], TensorSpec(self.dtype, tuple(out)))
+                             "contract_rhs": cr, "accum_dtype": None, "out_dtype": out_dtype}}
+        return self.fb.emit(op, [self, rhs], TensorSpec(out_dtype or self.dtype, tuple(out)))
 
-    def matmul(self, rhs: "Tensor") -> "Tensor":
+    def matmul(self, rhs: "Tensor", out_dtype: Optional[str] = None) -> "Tensor":
         """functional::matmul (ops/functional/linalg.rs:53-127): 2-D or batched 3-D."""
         if self.spec.rank == 2 and rhs.spec.rank == 2:
-            return self.dot_general(rhs, [], [1], [0])
+            return self.dot_general(rhs, [], [1], [0], out_dtype=out_dtype)
         if self.spec.rank == 3 and rhs.spec.rank == 3:
-            return self.dot_general(rhs, [0], [2], [1])
+            return self.dot_general(rhs, [0], [2], [1], out_dtype=out_dtype)
         raise ValueError("matmul expects rank-2 or rank-3 operands of equal rank")
 
     # -- indexing ------------------------------------------------------------

@@ -78,6 +78,24 @@ def _fp(a: np.ndarray):
     return a.ctypes.data_as(ctypes.POINTER(ctypes.c_float))
 
 
+# Contractions of at least this many multiply-adds run through numpy's f32 matmul (a blocked BLAS sum) instead of the
+# sequential-k loop of cpu.rs:2190-2236.  None (the default) keeps every dot on the reference's summation order.  Tests
+# of full-size shapes (0.25 TFLOP for one Ministral layer at 1024 tokens) set it: the two orders differ by a few f32
+# ulps of the sum, far inside the tolerances those tests state, and the sequential loop would take minutes.
+BLAS_DOT_MIN_MACS = None
+
+
+def _bmm(a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    """c[B,M,N] = a[B,M,K] . b[B,K,N] in f32."""
+    B, M, K = a.shape
+    N = b.shape[2]
+    if BLAS_DOT_MIN_MACS is not None and B * M * K * N >= BLAS_DOT_MIN_MACS:
+        return np.matmul(a, b).astype(np.float32, copy=False)
+    c = np.empty((B, M, N), dtype=np.float32)
+    _lib().oracle_bmm_f32(_fp(a), _fp(b), _fp(c), B, M, K, N)
+    return c
+
+
 # ----------------------------------------------------------------------------- tensors
 NP_DTYPES = {"F32": np.float32, "Si32": np.int32, "I1": np.uint8, "Bf16": np.float32,
              "Si8": np.int8, "Ui8": np.uint8}
@@ -320,8 +338,7 @@ def op_dot_general(l: OTensor, r: OTensor, spec) -> OTensor:          # cpu.rs:2
     N = int(np.prod(rshape, dtype=np.int64))
     a = np.ascontiguousarray(np.transpose(l.a, bl + lf + cl).reshape(B, M, K))
     b = np.ascontiguousarray(np.transpose(r.a, br + cr + rf).reshape(B, K, N))
-    c = np.empty((B, M, N), dtype=np.float32)
-    _lib().oracle_bmm_f32(_fp(a), _fp(b), _fp(c), B, M, K, N)
+    c = _bmm(a, b)
     out_dtype = spec.get("out_dtype") or l.dtype
     return _finish(out_dtype, c.reshape(bshape + lshape + rshape))
 
@@ -436,12 +453,10 @@ def _custom_call(target: str, attrs, ins: List[OTensor], out_dtype: str, out_dim
     else:
         raise OracleError("unimplemented", f"custom_call target {target}")
     # reference semantics for "dequantize + dot_general": f32 accumulate, output rounded
-    c = np.empty((x.a.shape[0], w.shape[1]), dtype=np.float32)
     a = np.ascontiguousarray(x.a, dtype=np.float32)
     wb = round_bf16(w) if x.dtype == "Bf16" else w
     wb = np.ascontiguousarray(wb, dtype=np.float32)
-    _lib().oracle_bmm_f32(_fp(a), _fp(wb), _fp(c), 1, a.shape[0], a.shape[1], wb.shape[1])
-    return _finish(out_dtype, c)
+    return _finish(out_dtype, _bmm(a[None], wb[None])[0])
 
 
 # ----------------------------------------------------------------------------- interpreter

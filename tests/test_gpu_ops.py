@@ -517,6 +517,51 @@ def test_decode_equals_prefill_row(hip):
     assert_close(ck[:, :T], k_full)
 
 
+# ------------------------------------------------------------------ execute_instruction
+def test_execute_instruction_single_ops(hip):
+    """PortableBackend::execute_instruction (spec.rs:1317): one instruction, operands positional.  Take (the embedding
+    gather, bit-exact), DotGeneral (the reference-held 2x2 vector, smoke.rs:12-24), DynamicUpdateSlice with a clamped
+    start (dynamic_ops_gpu.rs:35-104), a literal operand, and an operand that repeats."""
+    import json
+    from gptrs_amd.backend import BackendError
+    from gptrs_amd.ptir import TensorSpec
+
+    def instr_of(build, specs):
+        p = prog(build, specs)
+        body = p.obj["functions"][0]["body"]
+        return p, json.dumps(body[-1], separators=(",", ":")).encode()
+
+    def mat(dtype, arr):
+        arr = np.asarray(arr)
+        return hip.materialize(TensorSpec(dtype, arr.shape), arr)
+
+    # Take
+    table = np.arange(40, dtype=np.float32).reshape(10, 4)
+    idx = np.array([7, 0, 7, 9], np.int32)
+    p, js = instr_of(lambda fb, t, i: t.take(i), [("F32", [10, 4]), ("Si32", [4])])
+    out = hip.execute_instruction(js, [mat("F32", table), mat("Si32", idx)])
+    assert np.array_equal(hip.to_numpy(out), oracle_run(p, [table, idx])[0]) and np.array_equal(hip.to_numpy(out), table[idx])
+    # DotGeneral: [[1,2],[3,4]] . [[5,6],[7,8]] = [[19,22],[43,50]]
+    a, b = np.array([[1, 2], [3, 4]], np.float32), np.array([[5, 6], [7, 8]], np.float32)
+    p, js = instr_of(lambda fb, x, y: x.matmul(y), [("F32", [2, 2]), ("F32", [2, 2])])
+    assert hip.to_numpy(hip.execute_instruction(js, [mat("F32", a), mat("F32", b)])).tolist() == [[19, 22], [43, 50]]
+    # DynamicUpdateSlice, start 8 clamps to 3
+    p, js = instr_of(lambda fb, base, u, s: base.dynamic_update_slice(u, s, [2]), [("F32", [5]), ("F32", [2]), ("Si32", [1])])
+    base_h = mat("F32", np.array([10, 11, 12, 13, 14], np.float32))
+    out = hip.execute_instruction(js, [base_h, mat("F32", np.array([99, 88], np.float32)), mat("Si32", np.array([8], np.int32))])
+    assert hip.to_numpy(out).tolist() == [10, 11, 12, 99, 88] and hip.to_numpy(base_h).tolist() == [10, 11, 12, 13, 14]
+    # a literal operand travels inside the JSON: BroadcastTo(Literal 1.0)
+    p, js = instr_of(lambda fb, x: x + 1.0, [("F32", [4])])
+    lit = json.dumps(p.obj["functions"][0]["body"][0], separators=(",", ":")).encode()
+    assert hip.to_numpy(hip.execute_instruction(lit, [])).tolist() == [1, 1, 1, 1]
+    # one value on both sides of a product
+    p, js = instr_of(lambda fb, x: x * x, [("F32", [4])])
+    h = mat("F32", np.array([1, 2, 3, 4], np.float32))
+    assert hip.to_numpy(hip.execute_instruction(js, [h, h])).tolist() == [1, 4, 9, 16]
+    with pytest.raises(BackendError):
+        hip.execute_instruction(js, [h])              # fewer inputs than Value operands
+
+
 # ------------------------------------------------------------------ error surface
 def test_unknown_custom_call_is_unimplemented(hip):
     from gptrs_amd.backend import BackendError

@@ -167,12 +167,20 @@ def dequantize_host(q, s, scheme):
     return bf16_round(codes * np.repeat(s.astype(np.float32), 128, axis=0))
 
 
+# 64 x 64 tiles (fewer than 128 tiles of 128 x 128): (128, 3072, 1024), (300, 1024, 3000), (17, 256, 40), (1024, 512, 200).
+# 8-wave workgroups that split every tile's k-steps (128..256 tiles): (1024, 1024, 2048).  Tail split with tickets: 304
+# tiles, the last 48 split four ways over 18 k tiles, so the second and fourth splits start in the middle of an int4
+# scale group: (1024, 1152, 4860).  Plain 128 x 128 tiles, 512 of them: (1024, 3072, 8192).  Tail split at the
+# gate / up / down width: (1024, 3072, 9216).
 @pytest.mark.parametrize("scheme", ["w8", "w4g128"])
-@pytest.mark.parametrize("m,k,n", [(128, 3072, 1024), (300, 1024, 3000), (17, 256, 40), (1024, 512, 200)])
+@pytest.mark.parametrize("m,k,n", [(128, 3072, 1024), (300, 1024, 3000), (17, 256, 40), (1024, 512, 200),
+                                   (1024, 1024, 2048), (1024, 1152, 4860), (1024, 3072, 8192), (1024, 3072, 9216)])
 def test_prefill_codes_equal_dequantised_weights(hip, scheme, m, k, n):
     """The MFMA GEMM over the codes forms bf16(code * scale) on the way into LDS: its result must equal, BIT FOR BIT,
     the same GEMM over the dequantised matrix given as a plain bf16 weight (same kernel, same values, same order),
-    with and without the SwiGLU pairing; 128 x 128 and 64 x 64 tiles, ragged M and N, zero and extreme columns."""
+    with and without the SwiGLU pairing; every tile shape and split of the kernel, ragged M and N, zero and extreme
+    columns.  The single-matrix GEMM is also checked against the oracle's "dequantise, then dot_general", and run
+    twice: split tiles meet through tickets that every launch must leave at zero."""
     x = bf16_round(rnd(31, (m, k)))
     w = weights_with_corner_cases(32, k, n)
     w2 = rnd(33, (k, n), 2.0 / np.sqrt(k))
@@ -183,6 +191,15 @@ def test_prefill_codes_equal_dequantised_weights(hip, scheme, m, k, n):
     assert hip.counter("derived_weights_built") == built + 1     # one copy: the codes (no dequantised matrix)
     (want,) = hip_run(hip, prog(lambda fb, a, b: a.matmul(b), [("Bf16", [m, k]), ("Bf16", [k, n])]), [x, dequantize_host(q, s, scheme)])
     assert np.array_equal(got, want), f"max diff {np.max(np.abs(got - want))}"
+    pq = prog(lambda fb, a, b, c: F.linear_quantized(a, b, c), [("Bf16", [m, k]), cs_, ss_])
+    (again,) = hip_run(hip, pq, [x, q, s])
+    assert np.array_equal(again, got), "a second launch of the same GEMM differs (tickets not returned to zero?)"
+    po.BLAS_DOT_MIN_MACS, old_min = 1 << 27, po.BLAS_DOT_MIN_MACS
+    try:
+        (ref,) = oracle_run(pq, [x, q, s])
+    finally:
+        po.BLAS_DOT_MIN_MACS = old_min
+    assert_close(got, ref, atol=1e-4 * np.sqrt(k), rtol=2.0 ** -8, what="quantised GEMM vs oracle")
     (gotp,) = hip_run(hip, prog(lambda fb, a, b, bs, c, cs: F.swiglu(F.linear_quantized(a, b, bs), F.linear_quantized(a, c, cs)),
                                 [("Bf16", [m, k]), cs_, ss_, cs_, ss_]), [x, q, s, q2, s2])
     (wantp,) = hip_run(hip, prog(lambda fb, a, b, c: F.swiglu(a.matmul(b), a.matmul(c)),

@@ -413,6 +413,109 @@ def test_int8_and_int4_pack_round_trip():
     assert lo == int(np.clip(np.rint(w[0, 0] / s4[0, 0]), -7, 7))
 
 
+# -- independent pin of the quantisers: pure-Python per-element loops (no numpy arithmetic shared with the oracle) over
+# hand-placed cases, and hand-written expected bytes
+def _f32(v: float) -> float:
+    import struct
+    return struct.unpack("<f", struct.pack("<f", v))[0]
+
+
+def _bf16_rne(v: float) -> float:
+    """f32 -> bf16 (round to nearest, ties to even) -> f32, on the integer bit pattern."""
+    import struct
+    u = struct.unpack("<I", struct.pack("<f", v))[0]
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return struct.unpack("<f", struct.pack("<I", u))[0]
+
+
+def _py_quant_column(col, qmax):
+    """One scale group: s = bf16(max |w| / qmax) (1 when that is 0), q = clamp(round_half_even(f32(w / s)), +-qmax).
+    The f32 quotient is the f64 quotient rounded once to f32 (exact for f32 operands: 53 >= 2 * 24 + 2 bits)."""
+    amax = 0.0
+    for w in col:
+        amax = max(amax, abs(w))
+    s = _bf16_rne(_f32(amax / float(qmax)))
+    if s == 0.0:
+        s = 1.0
+    q = []
+    for w in col:
+        r = round(_f32(w / s))       # Python rounds halves to even
+        q.append(max(-qmax, min(qmax, r)))
+    return q, s
+
+
+def test_int8_quantiser_hand_vectors():
+    # column 0: all zero -> scale 1, codes 0.  column 1: max 127 -> scale exactly 1, so 0.5 / 1.5 / -2.5 are exact ties:
+    # half-even gives 0, 2, -2 (half-away would give 1, 2, -3).  column 2: max 254 -> scale 2: -254 -> -127, 3 -> 1.5 -> 2,
+    # -5 -> -2.5 -> -2, 1 -> 0.5 -> 0.
+    w = np.array([[0.0, 127.0, -254.0],
+                  [0.0, 0.5, 3.0],
+                  [0.0, 1.5, -5.0],
+                  [0.0, -2.5, 1.0]], np.float32)
+    q, s = po.quantize_int8_per_channel(w)
+    assert s.tolist() == [1.0, 1.0, 2.0]
+    assert q.tobytes() == bytes([0x00, 0x7F, 0x81, 0x00, 0x00, 0x02, 0x00, 0x02, 0xFE, 0x00, 0xFE, 0x00])
+    assert po.dequantize_int8(q, s).tolist() == [[0.0, 127.0, -254.0], [0.0, 0.0, 4.0], [0.0, 2.0, -4.0], [0.0, -2.0, 0.0]]
+
+
+def test_int8_quantiser_vs_python_loop():
+    rng = np.random.default_rng(77)
+    w = (rng.standard_normal((96, 7)) * 0.02).astype(np.float32)
+    w[:, 3] = 0.0                                   # an all-zero column
+    w[5, 0], w[6, 0] = 1.0, -1.0                    # scale bf16(1/127) is rounded DOWN: 1/s = 127.008 must stay 127
+    q, s = po.quantize_int8_per_channel(w)
+    for n in range(w.shape[1]):
+        pq, ps = _py_quant_column([float(v) for v in w[:, n]], 127)
+        assert ps == float(s[n]), f"scale of column {n}"
+        assert pq == [int(v) for v in q[:, n]], f"codes of column {n}"
+    assert int(q[5, 0]) == 127 and int(q[6, 0]) == -127 and float(s[3]) == 1.0
+    # the clamp is unreachable with the scheme's own scales: bf16 rounding moves s by at most 2^-9 relative, so
+    # |w| / s <= 127 * (1 + 2^-9) < 127.5; it guards scales handed in by a caller
+    assert float(np.max(np.abs(w[:, 0])) / s[0]) < 127.5
+
+
+def test_int4_quantiser_hand_vectors():
+    w = np.zeros((256, 2), np.float32)
+    # column 0, group 0 (k < 128): max 7 -> scale 1; ties 0.5 -> 0, 1.5 -> 2, -2.5 -> -2, and -3.5 -> -4 in the group's
+    # LAST row (k = 127).  group 1 starts at k = 128: max 14 -> scale 2: 14 -> 7, -14 -> -7, 3 -> 1.5 -> 2.
+    w[0, 0], w[1, 0], w[2, 0], w[3, 0], w[127, 0] = 7.0, 0.5, 1.5, -2.5, -3.5
+    w[128, 0], w[129, 0], w[130, 0] = 14.0, -14.0, 3.0
+    # column 1: group 0 all zero -> scale 1.  group 1: max 0.875 -> scale 0.125: -0.875 -> -7, 0.0625 -> 0.5 -> 0, 0.1875 -> 1.5 -> 2
+    w[255, 1], w[254, 1], w[253, 1] = -0.875, 0.0625, 0.1875
+    pk, s = po.quantize_int4_g128(w)
+    assert s.tolist() == [[1.0, 1.0], [2.0, 0.125]]
+    exp = np.zeros((128, 2), np.uint8)
+    exp[0, 0] = 0x07      # k0 = 7 (low nibble), k1 = 0
+    exp[1, 0] = 0xE2      # k2 = 2, k3 = -2 -> 0xE (high nibble)
+    exp[63, 0] = 0xC0     # k126 = 0, k127 = -4 -> 0xC
+    exp[64, 0] = 0x97     # k128 = 7, k129 = -7 -> 0x9: first byte of the second group
+    exp[65, 0] = 0x02     # k130 = 2
+    exp[126, 1] = 0x20    # k252 = 0, k253 = 2
+    exp[127, 1] = 0x90    # k254 = 0, k255 = -7
+    assert pk.tobytes() == exp.tobytes()
+    deq = po.dequantize_int4_g128(pk, s)
+    assert deq[127, 0] == -4.0 and deq[128, 0] == 14.0 and deq[129, 0] == -14.0 and deq[130, 0] == 4.0
+    assert deq[255, 1] == -0.875 and deq[253, 1] == 0.25 and deq[1, 0] == 0.0
+
+
+def test_int4_quantiser_vs_python_loop():
+    rng = np.random.default_rng(78)
+    w = (rng.standard_normal((384, 5)) * 0.02).astype(np.float32)
+    w[128:256, 2] = 0.0                             # an all-zero group between two live ones
+    pk, s = po.quantize_int4_g128(w)
+    deq = po.dequantize_int4_g128(pk, s)
+    for n in range(w.shape[1]):
+        for g in range(3):
+            pq, ps = _py_quant_column([float(v) for v in w[128 * g:128 * g + 128, n]], 7)
+            assert ps == float(s[g, n])
+            for j in range(64):                     # both nibbles of every byte, by integer arithmetic
+                b = int(pk[64 * g + j, n])
+                lo, hi = b & 0xF, b >> 4
+                lo, hi = (lo - 16 if lo > 7 else lo), (hi - 16 if hi > 7 else hi)
+                assert (lo, hi) == (pq[2 * j], pq[2 * j + 1]), f"byte {64 * g + j} of column {n}"
+                assert float(deq[128 * g + 2 * j, n]) == _f32(lo * ps) and float(deq[128 * g + 2 * j + 1, n]) == _f32(hi * ps)
+
+
 # ---------------------------------------------------------------------------------- temperature sampling
 def _gumbel_score_reference(i, seed, logit, temperature):
     """The per-index arithmetic of sample_temperature_last_axis_f32.triton:44-60 with Python integers and
