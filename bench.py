@@ -1,8 +1,9 @@
 #!/usr/bin/env python3
 """Decode throughput of the HIP PTIR backend on one MI355X.
 
-Workload (BASELINE.json configs[3], batch 1): Ministral-3B-shaped decoder, bf16, random-init
-N(0, 0.02) weights from a seed, prompt of 1024 random token ids, greedy decode with a
+Workload (BASELINE.json configs[3], batch 1): Ministral-3B-shaped decoder, bf16 weights and matmul
+operands with an f32 residual stream and f32 logits (`--residual bf16`: every tensor bf16),
+random-init N(0, 0.02) weights from a seed, prompt of 1024 random token ids, greedy decode with a
 fixed-capacity KV cache.  One "step" = one decode token: upload of the per-step scalars, one
 `run_program` over the whole model, on-device argmax and the 8-byte token readback -- the
 reference's decode-steady protocol (crates/gpt-rs-cli/src/main.rs:976-1051).
@@ -11,15 +12,20 @@ Prints ONE JSON line; `value` = tokens/s with all weights and the KV cache resid
 `roofline` covers the dominant kernel, the persistent decode chain (one launch per step: every
 linear layer and the decode attention): the step's algorithmic bytes (every weight element once,
 the valid KV rows once, activations and logits once) over the HIP-event time of those launches on
-the backend's stream.  `cpu_baseline` times the reference C backend's own GEMV kernels
-(oracle/_ref, built from the reference checkout) on one host core over a bounded sample.
+the backend's stream.  `prefill` prices the 1024-token prefill against the bf16 MFMA peak, `gpt2_f32`
+is the other half of the metric (GPT-2 small f32: whole generate calls of 64 tokens, and steady
+decode against the HBM roofline).  `cpu_baseline` (and `gpt2_f32.cpu_baseline`) time the reference C
+backend's own kernels (oracle/_ref, built from the reference checkout) on the host, before the GPU
+is touched: one core, the reference's own setting, and one process per core.
 """
 from __future__ import annotations
 
 import argparse
 import ctypes
+import hashlib
 import json
 import os
+import struct
 import sys
 import time
 
@@ -31,16 +37,27 @@ import __graft_entry__ as entry  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
-# HBM bytes moved by one chain_kernel launch of the default workload (26 layers, prompt 1024, cache
-# length ~1040), from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a copy kernel of known size; the
-# commands and raw figures are in profiles/chain_kernel_ministral3b_bf16_b1_decode.md
-MEASURED_CHAIN_TRAFFIC_BYTES = 7.010e9 + 0.0216e9
+# HBM bytes moved by one chain_kernel launch of the default workload (26 layers, prompt 1024, cache length ~1040), from
+# rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a copy kernel of known size (commands and raw figures: `profile`).  The
+# figure belongs to ONE version of the kernel: `source_sha256` is the hash of gpt.rs_amd/csrc/kernels_chain.hip it was
+# measured on, and `roofline.traffic` is null whenever the file in the tree hashes differently.
+CHAIN_TRAFFIC = {"bytes": 7.010e9 + 0.0216e9, "source_sha256": "unmeasured",
+                 "profile": "profiles/chain_kernel_ministral3b_bf16_b1_decode.md"}
 
 
-def algorithmic_bytes_per_step(cfg, dtype_bytes: int, cache_len: int, quant: str = "none") -> int:
+def chain_traffic_bytes():
+    try:
+        with open(os.path.join(ROOT, "gpt.rs_amd", "csrc", "kernels_chain.hip"), "rb") as f:
+            return CHAIN_TRAFFIC["bytes"] if hashlib.sha256(f.read()).hexdigest() == CHAIN_TRAFFIC["source_sha256"] else None
+    except OSError:
+        return None
+
+
+def algorithmic_bytes_per_step(cfg, dtype_bytes: int, cache_len: int, quant: str = "none", f32_stream: bool = False) -> int:
     """Minimum HBM traffic of one decode token: every weight once, the valid KV once, the new KV
     row and the logits written once.  Quantised linear weights count their codes (1 or 1/2 byte per
-    element) plus their scales (one per column, or one per column and 128 rows)."""
+    element) plus their scales (one per column, or one per column and 128 rows).  f32_stream: norm
+    gains and logits are f32."""
     a = cfg.attention_config()
     mats = cfg.num_layers * [(cfg.embed_dim, a.total_projection_dim), (a.query_projection_dim, cfg.embed_dim),
                              (cfg.embed_dim, cfg.ffn_dim), (cfg.embed_dim, cfg.ffn_dim), (cfg.ffn_dim, cfg.embed_dim)]
@@ -53,35 +70,78 @@ def algorithmic_bytes_per_step(cfg, dtype_bytes: int, cache_len: int, quant: str
             return k * n // 2 + (k // 128) * n * dtype_bytes
         return k * n * dtype_bytes
 
-    weights = sum(mat_bytes(k, n) for k, n in mats) + dtype_bytes * (cfg.num_layers * 2 * cfg.embed_dim + cfg.embed_dim)
+    sb = 4 if f32_stream else dtype_bytes
+    weights = sum(mat_bytes(k, n) for k, n in mats) + sb * (cfg.num_layers * 2 * cfg.embed_dim + cfg.embed_dim)
     kv_row = cfg.num_layers * 2 * cfg.num_kv_heads * cfg.head_dim
-    return weights + dtype_bytes * (kv_row * (cache_len + 1) + cfg.vocab_size + cfg.embed_dim)
+    return weights + dtype_bytes * (kv_row * (cache_len + 1) + cfg.embed_dim) + sb * cfg.vocab_size
 
 
-def cpu_baseline(cfg, seconds_budget: float = 25.0):
-    """Reference C kernels (gpt_rs_c_matmul_f32_cached_b, GEMV path, packed-B cache warm) on one
-    core, f32 (the reference executes no bf16).  Sample: ONE layer's five weight matrices plus a
-    1/8 column slice of lm_head; a token = 26 layers + the full lm_head, extrapolated linearly."""
+def _ref_lib():
+    """oracle/_ref: the reference C backend's kernels compiled from the reference checkout (test infrastructure)."""
     ref_dir = os.path.join(ROOT, "oracle", "_ref")
     flags = open("/proc/cpuinfo").read()
     name = "libgptrs_c_ref_avx512.so" if (" avx512f" in flags and " fma" in flags) else "libgptrs_c_ref_avx2.so"
     path = os.path.join(ref_dir, name)
     if not os.path.exists(path):
-        return None
+        return None, name
     lib = ctypes.CDLL(path)
     fp = ctypes.POINTER(ctypes.c_float)
     lib.gptrs_ref_cache_new.restype = ctypes.c_void_p
     lib.gptrs_ref_cache_free.argtypes = [ctypes.c_void_p]
     lib.gptrs_ref_matmul_f32_cached.argtypes = [fp, fp, fp, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_void_p]
+    return lib, name
+
+
+def host_cores() -> int:
+    """Worker processes for the all-cores figures: the cores this process may run on, capped by the share the
+    environment grants (OMP_NUM_THREADS is set to it on the GPU box)."""
+    n = len(os.sched_getaffinity(0))
+    cap = os.environ.get("OMP_NUM_THREADS", "")
+    if cap.isdigit() and int(cap) > 0:
+        n = min(n, int(cap))
+    return max(n, 1)
+
+
+def _fork_all(n: int, work):
+    """Runs work(i) -> float in n forked children at once (the parent's weights and packed caches are shared
+    copy-on-write) and returns their results.  Only called before the process has touched the GPU."""
+    pipes = []
+    for i in range(n):
+        r, w = os.pipe()
+        pid = os.fork()
+        if pid == 0:
+            code = 0
+            try:
+                os.close(r)
+                os.write(w, struct.pack("<d", float(work(i))))
+            except BaseException:
+                code = 1
+            os._exit(code)
+        os.close(w)
+        pipes.append((pid, r))
+    out = []
+    for pid, r in pipes:
+        data = os.read(r, 8)
+        os.close(r)
+        os.waitpid(pid, 0)
+        out.append(struct.unpack("<d", data)[0] if len(data) == 8 else float("nan"))
+    return out
+
+
+def cpu_baseline(cfg, seconds_budget: float = 20.0):
+    """Reference C kernels (gpt_rs_c_matmul_f32_cached_b, GEMV path, packed-B cache warm), f32 (the reference executes no
+    bf16).  Sample: ONE layer's five weight matrices plus a 1/8 column slice of lm_head; a token = 26 layers + the full
+    lm_head, extrapolated linearly.  One core (the C backend is single-threaded: the faithful figure), then the same
+    loop in one process per core at once (independent sequences), with the core count stated."""
+    lib, name = _ref_lib()
+    if lib is None:
+        return None
+    fp = ctypes.POINTER(ctypes.c_float)
     a = cfg.attention_config()
     d = cfg.embed_dim
     head_cols = cfg.vocab_size // 8
-    if hasattr(cfg, "ffn_dim"):     # Ministral: qkv, out, gate, up, down
-        f = cfg.ffn_dim
-        shapes = [(d, a.total_projection_dim), (a.query_projection_dim, d), (d, f), (d, f), (f, d), (d, head_cols)]
-    else:                           # GPT-2: qkv, out, fc1, fc2
-        f = cfg.mlp_ratio * d
-        shapes = [(d, a.total_projection_dim), (a.query_projection_dim, d), (d, f), (f, d), (d, head_cols)]
+    f = cfg.ffn_dim
+    shapes = [(d, a.total_projection_dim), (a.query_projection_dim, d), (d, f), (d, f), (f, d), (d, head_cols)]
     nl = len(shapes) - 1
     rng = np.random.default_rng(0)
     mats, caches, xs, ys = [], [], [], []
@@ -99,25 +159,130 @@ def cpu_baseline(cfg, seconds_budget: float = 25.0):
 
     for i in range(len(shapes)):
         call(i)  # packs B once (gpt_rs_c_prepare warms this cache in the reference)
-    t_layer, t_head, reps = 0.0, 0.0, 0
-    t_start = time.perf_counter()
-    while reps < 3 or (time.perf_counter() - t_start < seconds_budget / 3 and reps < 20):
-        t0 = time.perf_counter()
-        for i in range(nl):
-            call(i)
-        t1 = time.perf_counter()
-        call(nl)
-        t2 = time.perf_counter()
-        t_layer += t1 - t0
-        t_head += t2 - t1
-        reps += 1
+
+    def token_time(budget, max_reps):
+        t_layer, t_head, reps = 0.0, 0.0, 0
+        t_start = time.perf_counter()
+        while reps < 2 or (time.perf_counter() - t_start < budget and reps < max_reps):
+            t0 = time.perf_counter()
+            for i in range(nl):
+                call(i)
+            t1 = time.perf_counter()
+            call(nl)
+            t2 = time.perf_counter()
+            t_layer += t1 - t0
+            t_head += t2 - t1
+            reps += 1
+        return cfg.num_layers * t_layer / reps + 8 * t_head / reps, reps
+
+    t_token, reps = token_time(seconds_budget / 3, 20)
+    cores = host_cores()
+    all_cores = None
+    if cores > 1:
+        times = _fork_all(cores, lambda i: token_time(seconds_budget / 3, 20)[0])
+        if all(t == t and t > 0 for t in times):
+            all_cores = {"value": round(sum(1.0 / t for t in times), 3), "unit": "tokens/s", "cores": cores, "nproc": os.cpu_count(),
+                         "how": "one process per core at once, each an independent sequence over the shared weights"}
     for c in caches:
         lib.gptrs_ref_cache_free(c)
-    t_token = cfg.num_layers * t_layer / reps + 8 * t_head / reps
     return {"value": round(1.0 / t_token, 4), "unit": "tokens/s", "cores": 1, "kind": "reference",
             "sample": f"{reps} reps of one layer's {nl} f32 GEMVs + 1/8 of lm_head through {name} "
                       f"(gpt_rs_c_matmul_f32_cached_b, m=1, packed-B cache warm); token time = {cfg.num_layers} layers + "
-                      f"8 head slices; non-GEMV ops excluded"}
+                      f"8 head slices; non-GEMV ops excluded", "all_cores": all_cores}
+
+
+class _HostParams:
+    """Backend stand-in that keeps materialised parameters on the host (weights for the CPU baseline come out of the
+    same seeded initialiser the device model uses)."""
+
+    def __init__(self):
+        self.arrays = []
+
+    def materialize(self, spec, data):
+        self.arrays.append(np.frombuffer(bytes(data), "<f4").reshape(spec.dims).copy())
+        return len(self.arrays) - 1
+
+    def param_resolver(self):
+        return self
+
+    def set(self, sid, handle):
+        pass
+
+
+def cpu_gpt2_baseline(prompt, new_tokens: int, capacity: int = 128):
+    """BASELINE.md's CPU workload (ii): GPT-2 small f32 greedy decode with a KV cache on the reference C kernels
+    (oracle/ref_harness.c: every matrix product through gpt_rs_c_matmul_f32_cached_b with a warm packed-B cache, the
+    other ops as plain C loops), same seeded weights and prompt as the device run.  The prompt goes through token by
+    token (the harness has no batched prefill); timed: the last `new_tokens` steps, steady decode.  One core, then one
+    process per core at once."""
+    lib, name = _ref_lib()
+    if lib is None or not hasattr(lib, "gptrs_ref_gpt2_generate"):
+        return None
+    from gptrs_amd import models
+    cfg = models.GptConfig()
+    host = _HostParams()
+    m = models.Gpt.random(cfg, host, seed=0, dtype="F32")
+    P = dict(zip(m.param_names, host.arrays))
+    L, d, f = cfg.num_layers, cfg.embed_dim, cfg.embed_dim * cfg.mlp_ratio
+    fp = ctypes.POINTER(ctypes.c_float)
+    fpp = ctypes.POINTER(fp)
+
+    def ptr(a):
+        return a.ctypes.data_as(fp)
+
+    def per_layer(fmt):
+        arr = (fp * L)(*[ptr(P[fmt.format(i)]) for i in range(L)])
+        return arr
+
+    class W(ctypes.Structure):
+        _fields_ = [("tok_emb", fp), ("pos_emb", fp), ("ln1_g", fpp), ("ln1_b", fpp), ("w_qkv", fpp), ("b_qkv", fpp),
+                    ("w_out", fpp), ("b_out", fpp), ("ln2_g", fpp), ("ln2_b", fpp), ("w_in", fpp), ("b_in", fpp),
+                    ("w_o2", fpp), ("b_o2", fpp), ("lnf_g", fp), ("lnf_b", fp), ("lm_head", fp),
+                    ("caches", ctypes.POINTER(ctypes.c_void_p)), ("layers", ctypes.c_int), ("d", ctypes.c_int),
+                    ("heads", ctypes.c_int), ("f", ctypes.c_int), ("vocab", ctypes.c_int), ("capacity", ctypes.c_int),
+                    ("eps", ctypes.c_float)]
+
+    keep = [per_layer(x) for x in ("blocks.{}.ln_1.gamma", "blocks.{}.ln_1.beta", "blocks.{}.attention.w_qkv", "blocks.{}.attention.b_qkv",
+                                   "blocks.{}.attention.w_out", "blocks.{}.attention.b_out", "blocks.{}.ln_2.gamma", "blocks.{}.ln_2.beta",
+                                   "blocks.{}.feed_forward.w_in", "blocks.{}.feed_forward.b_in", "blocks.{}.feed_forward.w_out",
+                                   "blocks.{}.feed_forward.b_out")]
+    ncache = 4 * L + 1
+    caches = (ctypes.c_void_p * ncache)(*[lib.gptrs_ref_cache_new() for _ in range(ncache)])
+    w = W(ptr(P["tok_embeddings.weight"]), ptr(P["pos_embeddings"]), *[ctypes.cast(k, fpp) for k in keep],
+          ptr(P["final_ln.gamma"]), ptr(P["final_ln.beta"]), ptr(P["lm_head"]), caches, L, d, cfg.num_heads, f, cfg.vocab_size,
+          capacity, cfg.eps)
+    lib.gptrs_ref_gpt2_generate.restype = ctypes.c_double
+    lib.gptrs_ref_gpt2_generate.argtypes = [ctypes.POINTER(W), ctypes.POINTER(ctypes.c_int), ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                            fp, fp, fp, ctypes.POINTER(ctypes.c_int)]
+    n_prompt = len(prompt)
+    if n_prompt + new_tokens > capacity:
+        return None
+    prompt_arr = (ctypes.c_int * n_prompt)(*prompt)
+
+    def run(n_new):
+        kc = np.zeros(L * cfg.num_heads * capacity * (d // cfg.num_heads), np.float32)
+        vc = np.zeros_like(kc)
+        scratch = np.zeros(4 * d + 3 * d + f + capacity + cfg.vocab_size, np.float32)
+        toks = (ctypes.c_int * n_new)()
+        sec = lib.gptrs_ref_gpt2_generate(ctypes.byref(w), prompt_arr, n_prompt, n_new, n_new - 1, ptr(kc), ptr(vc), ptr(scratch), toks)
+        return sec, list(toks)
+
+    run(2)                       # packs every B once (the reference warms the caches in gpt_rs_c_prepare)
+    sec, tokens = run(new_tokens)
+    steps = new_tokens - 1
+    cores = host_cores()
+    all_cores = None
+    if cores > 1:
+        times = _fork_all(cores, lambda i: run(new_tokens)[0])
+        if all(t == t and t > 0 for t in times):
+            all_cores = {"value": round(sum(steps / t for t in times), 1), "unit": "tokens/s", "cores": cores, "nproc": os.cpu_count(),
+                         "how": "one process per core at once, each generating the same sequence over the shared weights"}
+    for c in caches:
+        lib.gptrs_ref_cache_free(c)
+    return {"value": round(steps / sec, 2), "unit": "tokens/s", "cores": 1, "kind": "reference",
+            "sample": f"{steps} steady decode steps (cache length {n_prompt + 1}..{n_prompt + steps}) of GPT-2 small f32 through {name}: "
+                      f"49 GEMVs per step via gpt_rs_c_matmul_f32_cached_b (packed-B caches warm), LayerNorm / bias / GELU / attention / "
+                      f"argmax as plain C loops", "all_cores": all_cores, "tokens": tokens}
 
 
 def microbench(args, be):
@@ -196,7 +361,7 @@ def microbench(args, be):
 README_GPT2_TOKENS_PER_S = 74.71   # reference README.md:18-25: GPT-2 small f32, generate 64 tokens, C backend, 1 thread of a Ryzen 9 9950X3D
 
 
-def gpt2_generate(args, be):
+def gpt2_record(be, steps: int, warmup: int, cpu=None):
     """BASELINE configs[0]: GPT-2 small f32, weights N(0, 0.02) from seed 0, prompt of 16 ids (seed 1), greedy, 64 tokens
     with KV cache (capacity 128).  Timed like the reference's published figure (README.md:27-50,
     scripts/gptrs_eval/runner.py:24-56): each step is one WHOLE generate call, prefill included; tokens/s = 64 / mean
@@ -215,12 +380,12 @@ def gpt2_generate(args, be):
         be.synchronize()
         return out
 
-    for _ in range(max(args.warmup, 1)):
+    for _ in range(max(warmup, 1)):
         tokens = generate()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         assert generate() == tokens
-    elapsed = (time.perf_counter() - t0) / args.steps
+    elapsed = (time.perf_counter() - t0) / steps
     gen = models.Generator(model, prompt, kv_cache_capacity=256)
     for _ in range(8):
         gen.step()
@@ -235,18 +400,21 @@ def gpt2_generate(args, be):
     per_layer = d * 3 * d + d * d + 2 * d * cfg.mlp_ratio * d + (3 * d + d + cfg.mlp_ratio * d + d) + 4 * d   # weights, biases, LN
     step_bytes = 4 * (L * per_layer + 2 * d + d * V + 2 * L * d * (start + n // 2 + 1) + V + 2 * d)
     value = new_tokens / elapsed
-    print(json.dumps({
+    if cpu is not None:
+        cpu = dict(cpu)
+        cpu["same_tokens_as_device"] = cpu.pop("tokens", None) == tokens
+    return {
         "metric": "tokens/s of a whole generate call (prefill 16 + 64 greedy tokens), GPT-2 small f32, batch 1",
-        "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": max(args.warmup, 1),
-        "ms_per_step": round(elapsed * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "value": round(value, 2), "unit": "tokens/s", "steps": steps, "warmup": max(warmup, 1),
+        "ms_per_step": round(elapsed * 1e3, 4),
         "vs_baseline": round(value / README_GPT2_TOKENS_PER_S, 2), "dtype": "f32", "data": "synthetic",
         "config": {"workload": "gpt-2 small f32, prompt 16, greedy generate 64 with KV cache (capacity 128); a step is one generate call",
                    "baseline": "74.71 tokens/s: reference C backend, one thread of a Ryzen 9 9950X3D, 1-token prompt, sampled (README.md:18-25)"},
         "decode_steady_tokens_per_s": round(1.0 / t_step, 1), "decode_us_per_step": round(t_step * 1e6, 1),
         "hbm_gbps": round(step_bytes / t_step / 1e9, 1), "hbm_frac": round(step_bytes / t_step / 1e9 / HBM_PEAK_GBPS, 4),
         "algorithmic_bytes_per_step": step_bytes, "launches_per_step": be.counter("last_program_launches"),
-        "weight_init_s": round(t_init, 1), "roofline": None,
-        "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(cfg)}))
+        "chain_launches_per_step": None,
+        "weight_init_s": round(t_init, 1), "cpu_baseline": cpu}
 
 
 def batched_decode(args, be, cfg, model, capacity):
@@ -301,7 +469,7 @@ def batched_decode(args, be, cfg, model, capacity):
     wname = {"none": "bf16", "w8": "int8-weight-only (per output channel) bf16", "w4g128": "int4-weight-only (groups of 128) bf16"}[args.quant]
     mid_len = start_len + args.steps // 2
     kv_bytes = 2 * cfg.num_layers * cfg.num_kv_heads * cfg.head_dim * 2 * (mid_len + 1)
-    step_bytes = algorithmic_bytes_per_step(cfg, 2, mid_len, args.quant) + (B - 1) * kv_bytes   # weights once, every sequence's KV
+    step_bytes = algorithmic_bytes_per_step(cfg, 2, mid_len, args.quant, args.residual == "f32") + (B - 1) * kv_bytes   # weights once, every sequence's KV
     print(json.dumps({
         "metric": "decode tokens/s summed over %d sequences, Ministral-3B-shape %s (side workload: batched decode)" % (B, wname),
         "value": round(B * args.steps / elapsed, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -335,6 +503,10 @@ def main():
                     help="single-op programs of BASELINE configs[1] (dot_general / softmax / layer_norm, f32 and bf16) and the "
                          "Ministral prefill GEMM shapes; prints one JSON line with a result per shape")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--residual", choices=["f32", "bf16"], default="f32",
+                    help="f32 (default): bf16 weights and matmul operands with an f32 residual stream, f32 norms and f32 logits "
+                         "(DotGeneral out_dtype); bf16: every tensor of the program is bf16")
+    ap.add_argument("--no-gpt2", action="store_true", help="skip the GPT-2 small f32 sub-record of the default run")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain elementwise kernel of known traffic (x + 0 over 2^28 f32: 1 GiB read, 1 GiB written, "
                          "kernel binary_scalar_kernel) so FETCH_SIZE / WRITE_SIZE can be scaled to bytes")
@@ -346,6 +518,15 @@ def main():
     entry.load_package()
     from gptrs_amd import models
     from gptrs_amd.backend import HipBackend
+
+    # CPU baselines first: they fork one worker per core, which must happen before this process touches the GPU
+    plain_run = not (args.copy_calibration or args.microbench)
+    cpu_main = cpu_gpt2 = None
+    if plain_run and not args.no_cpu_baseline:
+        if args.model == "gpt2" or (args.batch == 1 and not args.no_gpt2):
+            cpu_gpt2 = cpu_gpt2_baseline(np.random.default_rng(1).integers(0, models.GptConfig().vocab_size, 16).tolist(), 64)
+        if args.model == "ministral" and args.batch == 1:
+            cpu_main = cpu_baseline(models.MinistralConfig(num_layers=args.layers))
 
     be = HipBackend(0)
     if args.copy_calibration:
@@ -366,14 +547,19 @@ def main():
     if args.model == "gpt2":
         if args.steps == 224:
             args.steps, args.warmup = 8, 2
-        return gpt2_generate(args, be)
+        rec = gpt2_record(be, args.steps, args.warmup, cpu_gpt2)
+        rec.update({"n_gpus": 1, "higher_is_better": True, "scaling": "weak", "roofline": None})
+        print(json.dumps(rec))
+        return
     cfg = models.MinistralConfig(num_layers=args.layers)
+    f32_stream = args.residual == "f32"
     total_len = args.prompt + args.warmup + args.steps + 1
     capacity = max(1280, (total_len + 255) // 256 * 256)
     if capacity > cfg.context_length:
         raise SystemExit(f"prompt + warmup + steps = {total_len} exceeds the context length {cfg.context_length}")
     t0 = time.perf_counter()
-    model = models.Ministral.random(cfg, be, seed=5, dtype="Bf16", quant=None if args.quant == "none" else args.quant)
+    model = models.Ministral.random(cfg, be, seed=5, dtype="Bf16", quant=None if args.quant == "none" else args.quant,
+                                    residual_dtype="F32" if f32_stream else None)
     t_init = time.perf_counter() - t0
     prompt = np.random.default_rng(6).integers(0, cfg.vocab_size, args.prompt).tolist()
     if args.batch > 1:
@@ -421,7 +607,7 @@ def main():
             if chains == calls:
                 # the timed launches are whole decode steps minus embedding and argmax: price them with
                 # the step's algorithmic bytes (weights once, valid KV once, logits once)
-                nbytes = sum(algorithmic_bytes_per_step(cfg, 2, prof_start + i, args.quant) for i in range(prof_steps))
+                nbytes = sum(algorithmic_bytes_per_step(cfg, 2, prof_start + i, args.quant, f32_stream) for i in range(prof_steps))
                 kernel = "chain_kernel: persistent decode chain, %d phases per launch (all linear layers + decode attention of a step)" % (
                     (be.counter("chain_phases") - phases0) // max(chains, 1))
             else:
@@ -430,15 +616,32 @@ def main():
             default_workload = chains == calls and args.layers == 26 and args.prompt == 1024 and args.quant == "none"
             roof = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                    "traffic": MEASURED_CHAIN_TRAFFIC_BYTES if default_workload else None,
+                    "traffic": chain_traffic_bytes() if default_workload else None,
                     "kernel": kernel,
                     "launches": calls, "avg_launch_us": round(t_ns / max(calls, 1) / 1e3, 2),
                     "bytes_per_launch": round(nbytes / max(calls, 1))}
 
     mid_len = start_len + args.steps // 2
-    step_bytes = algorithmic_bytes_per_step(cfg, 2, mid_len, args.quant)
+    step_bytes = algorithmic_bytes_per_step(cfg, 2, mid_len, args.quant, f32_stream)
     wname = {"none": "bf16", "w8": "int8-weight-only (per output channel) bf16", "w4g128": "int4-weight-only (groups of 128) bf16"}[args.quant]
+    if f32_stream:
+        wname += " (f32 residual stream and logits)"
     ms_per_step = elapsed / args.steps * 1e3
+    # prefill against the matrix-core peak: the linear layers over every prompt row, causal attention (half of the
+    # T x T products), the head on the last row
+    a_ = cfg.attention_config()
+    lin = cfg.embed_dim * a_.total_projection_dim + a_.query_projection_dim * cfg.embed_dim + 3 * cfg.embed_dim * cfg.ffn_dim
+    prefill_flops = cfg.num_layers * (2.0 * args.prompt * lin + 4.0 * cfg.num_heads * args.prompt * args.prompt * cfg.head_dim / 2) + \
+        2.0 * cfg.embed_dim * cfg.vocab_size
+    prefill = {"ms": round(t_prefill * 1e3, 2), "tokens": args.prompt, "tflop": round(prefill_flops / 1e12, 3),
+               "tflop_per_s": round(prefill_flops / t_prefill / 1e12, 1),
+               "mfma_frac": round(prefill_flops / t_prefill / 1e12 / MFMA_PEAK_TFLOPS, 4), "peak_tflop_per_s": MFMA_PEAK_TFLOPS,
+               "what": "wall time of one 1024-token prefill call (median of three; head on the last row), all launches included"}
+    bytes_allocated = be.counter("bytes_allocated")
+    gpt2 = None
+    if not args.no_gpt2:
+        del gen, model
+        gpt2 = gpt2_record(be, 8, 2, cpu_gpt2)
     out = {
         "metric": "decode tokens/s, Ministral-3B-shape %s batch 1 (HBM GB/s as %% of 8 TB/s in hbm_frac)" % wname,
         "value": round(args.steps / elapsed, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
@@ -452,9 +655,11 @@ def main():
         "algorithmic_bytes_per_step": step_bytes,
         "launches_per_step": launches,
         "prefill_ms": round(t_prefill * 1e3, 2), "prefill_tokens": args.prompt,
-        "weight_init_s": round(t_init, 1),
+        "weight_init_s": round(t_init, 1), "device_bytes_allocated": bytes_allocated,
         "roofline": roof,
-        "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(cfg),
+        "cpu_baseline": cpu_main,
+        "prefill": prefill,
+        "gpt2_f32": gpt2,
     }
     print(json.dumps(out))
 

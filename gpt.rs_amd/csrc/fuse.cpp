@@ -737,6 +737,8 @@ struct Fuser {
             in.op_name = q == 1 ? "fused.linear_w8" : "fused.linear_w4g128";
             in.quant = q;
             in.act = 0;
+            const Spec* xs = spec_of(in.operands[0].value);   // the accumulator leaves as f32 when the call's output is declared so
+            in.out_f32 = xs && xs->dtype == DType::BF16 && in.out_specs[0].dtype == DType::F32;
         }
         reindex();
         // 2. epilogues, each absorbed only when the linear's value has no other reader

@@ -8,12 +8,14 @@ execute f32 only).  The chain keeps f32 inside a linear and rounds its output to
 per-op-rounded bf16 oracle is further away from f32 than the chain is (its RMSNorm scale alone is
 rounded to 8 bits), so it is not the yardstick here.
 
-Tolerances against the f32 oracle: rtol = 2^-8 (the one bf16 rounding of the result, a full ulp to be
-safe) plus an absolute term for the inputs the kernel itself rounds to bf16 on the way (the
-normalised row, the intermediate vectors of a multi-phase chain): 4 sigma of the sum of K independent
-roundings, stated per test.  Against the one-kernel-per-linear path of the same backend, whose
-rounding points are the same, only the f32 summation order differs: rtol 2^-8 with a far smaller
-absolute term, which a dropped or doubled weight word (2 of K products) exceeds."""
+Tolerances against the f32 oracle: rtol = 2^-8 (the one bf16 rounding of the result: half an ulp is
+2^-9 .. 2^-8 of the value, depending on where in its binade it lies) plus an absolute term for the
+inputs the kernel itself rounds to bf16 on the way (the normalised row, the intermediate vectors of a
+multi-phase chain): about 4 sigma of the sum of K independent roundings, stated per test.  Against the
+one-kernel-per-linear path of the same backend, whose rounding points are the same, only the f32
+summation order differs, which now and then moves a result across a rounding boundary: one ulp,
+rtol 2^-7, with a far smaller absolute term, which a dropped or doubled weight word (2 of K products)
+exceeds."""
 import numpy as np
 import pytest
 
@@ -40,16 +42,17 @@ def bf16_round(a):
     return (f32_to_bf16_bits(np.asarray(a, np.float32)).astype(np.uint32) << 16).view(np.float32)
 
 
-ULP = 2.0 ** -8   # one bf16 ulp, relative
+HALF_ULP = 2.0 ** -8   # largest relative size of half a bf16 ulp: one rounding of an exact value
+ULP = 2.0 ** -7        # largest relative size of one bf16 ulp: two roundings of nearly equal values
 
 
 def _report(what, g, w):
     g, w = np.asarray(g, np.float64), np.asarray(w, np.float64)
     d = np.abs(g - w)
-    print(f"{what}: max abs {d.max():.3e}, max beyond {ULP:.1e} rel {np.max(d - ULP * np.maximum(np.abs(g), np.abs(w))):.3e}, max |ref| {np.abs(w).max():.2f}")
+    print(f"{what}: max abs {d.max():.3e}, max beyond {HALF_ULP:.1e} rel {np.max(d - HALF_ULP * np.maximum(np.abs(g), np.abs(w))):.3e}, max |ref| {np.abs(w).max():.2f}")
 
 
-def run_both(hip, build, specs, arrays, atol, atol_self):
+def run_both(hip, build, specs, arrays, atol, atol_self, rtol=HALF_ULP):
     """chain on vs the f32 oracle, and chain on vs chain off (same backend, one kernel per linear)."""
     p = prog(build, [("Bf16", d) for d in specs])
     before = hip.counter("chain_launches")
@@ -64,7 +67,7 @@ def run_both(hip, build, specs, arrays, atol, atol_self):
     for i, (g, w, q) in enumerate(zip(got, want, plain)):
         _report(f"result {i} vs oracle", g, w)
         _report(f"result {i} vs per-linear kernels", g, q)
-        assert_close(g, w, atol=atol, rtol=ULP, what=f"result {i} vs oracle")
+        assert_close(g, w, atol=atol, rtol=rtol, what=f"result {i} vs oracle")
         assert_close(g, q, atol=atol_self, rtol=ULP, what=f"result {i} vs per-linear kernels")
 
 
@@ -80,7 +83,7 @@ def test_norm_linear(hip, k, n):
     x, g, w = rnd(3, (1, k), 3.0), rnd(4, (k,)) + 1.5, rnd(5, (k, n), 2.0 / np.sqrt(k))
     # the normalised row (|v| up to 4.3, rms 2) is rounded to bf16 as it is staged: K roundings of relative 2^-9 against
     # weights of rms 1.15 / sqrt(K) move a result by 3e-3 (sigma)
-    run_both(hip, lambda fb, a, gm, b: F.rms_norm(a, gm, 1e-5)[0].matmul(b), [[1, k], [k], [k, n]], [x, g, w], 1.5e-2, 2e-3)
+    run_both(hip, lambda fb, a, gm, b: F.rms_norm(a, gm, 1e-5)[0].matmul(b), [[1, k], [k], [k, n]], [x, g, w], 2e-2, 2e-3)
 
 
 @pytest.mark.parametrize("k,n", [(3072, 9216), (256, 96)])
@@ -92,14 +95,20 @@ def test_swiglu_pair(hip, k, n):
         h = F.rms_norm(a, gm, 1e-5)[0]
         return F.swiglu(h.matmul(b), h.matmul(c))
 
-    # as above for gate and up; silu(g) * u roughly doubles the absolute effect (|u|, |silu'| of order 2)
-    run_both(hip, build, [[1, k], [k], [k, n], [k, n]], [x, g, wg, wu], 4e-2, 4e-3)
+    # as above for gate and up; silu(g) * u multiplies the effect by the other factor (|u|, |silu'| up to 7: results up
+    # to 41), so it enters relative to the result as well
+    run_both(hip, build, [[1, k], [k], [k, n], [k, n]], [x, g, wg, wu], 3e-2, 4e-3, rtol=ULP)
 
 
 @pytest.mark.parametrize("k,n", [(9216, 3072), (768, 3072), (128, 64)])
 def test_bias_gelu_residual(hip, k, n):
     x, w, b, r = rnd(10, (1, k)), rnd(11, (k, n), 2.0 / np.sqrt(k)), rnd(12, (n,)), rnd(13, (1, n))
-    run_both(hip, lambda fb, a, c, d, e: F.gelu(F.linear(a, c, d)) + e, [[1, k], [k, n], [n], [1, n]], [x, w, b, r], 2e-5, 2e-5)
+    # the scalar literals of a bf16 program are bf16: its GELU divides by bf16(sqrt 2) = 1.4140625, which the linear kernel's
+    # exact-erf epilogue (1.41421354) does not serve, so the GELU runs as its own kernel and the result carries three
+    # roundings (linear + bias, GELU, residual add) against the f32 oracle's none
+    run_both(hip, lambda fb, a, c, d, e: F.gelu(F.linear(a, c, d)) + e, [[1, k], [k, n], [n], [1, n]], [x, w, b, r], 2.5e-2, 2e-5)
+    # bias and residual alone are absorbed: the f32 sum + bias + residual, rounded once
+    run_both(hip, lambda fb, a, c, d, e: F.linear(a, c, d) + e, [[1, k], [k, n], [n], [1, n]], [x, w, b, r], 2e-5, 2e-5)
 
 
 @pytest.mark.parametrize("d,f", [(3072, 9216), (256, 640)])
@@ -121,7 +130,7 @@ def test_block_tail_chain(hip, d, f):
     specs = [[1, qp], [1, d], [qp, d], [d, f], [d, f], [f, d], [d, 2 * d], [d], [d]]
     before = hip.counter("chain_phases")
     # four vectors are rounded to bf16 between the phases (h, the SwiGLU output, ff, the normalised rows)
-    run_both(hip, build, specs, [ctx, x, wo, wg, wu, wd, wq, g1, g2], 6e-2, 1e-2)
+    run_both(hip, build, specs, [ctx, x, wo, wg, wu, wd, wq, g1, g2], 6e-2, 1e-3)
     assert hip.counter("chain_phases") - before >= 4
 
 

@@ -397,8 +397,10 @@ def test_ministral_full_width_one_layer_bf16_vs_oracle(hip):
         tensors to bf16, each rounding moves a logit by ~1e-3 (std), and the maximum over 1M logits
         lands at 4-6e-2 whatever the logit's own magnitude.  Measured: fused path 4.6e-2 from f32
         (mean 6e-3), the per-op-rounded bf16 oracle 6.4e-2 from f32, and the two bf16 pipelines
-        7.8e-2 from each other.  Asserted here: 5e-2 overall and 1e-2 on average -- a documented
-        miss of the stated bar, not a pass of it; the numbers are printed (run with -s)."""
+        7.8e-2 from each other.  The test is reported as an expected failure with the measured
+        numbers while the bar of 2e-2 is missed; the bound asserted before that (5e-2, 1e-2 on
+        average) only guards against regressions.  The variant with an f32 residual stream and f32
+        logits is measured in tests/test_gpu_configs.py."""
     cfg = models.MinistralConfig(num_layers=1)
     prompt = np.random.default_rng(6).integers(0, cfg.vocab_size, 8).tolist()
     ob = OracleBackend()
@@ -426,13 +428,16 @@ def test_ministral_full_width_one_layer_bf16_vs_oracle(hip):
     print(f"fused vs bf16 oracle: max {eb.max():.4f} mean {eb.mean():.6f}; equal {np.mean(eb == 0) * 100:.2f} %, "
           f"<= 1 ulp {np.mean(nu <= 1.0) * 100:.3f} %, <= 2 ulp {np.mean(nu <= 2.0) * 100:.3f} %, max ulps {nu.max():.1f}, "
           f"max err where |logit| >= 0.25: {eb[np.abs(ref_bf16) >= 0.25].max():.4f}")
-    assert err.max() < 5e-2 and err.mean() < 1e-2
+    assert err.max() < 5e-2 and err.mean() < 1e-2          # regression guard, not the bar
     # one decode step on top of the cache
     tok = int(np.argmax(ref_f32[-1]))
     d_hip = hip.to_numpy(mh.forward_with_decode_cache([tok], 8, ch, 16))
     d_ref = ob.to_numpy(mf.forward_with_decode_cache([tok], 8, cf, 16))
     derr = np.abs(d_hip - d_ref)
-    assert derr.max() < 5e-2 and derr.mean() < 1e-2
+    assert derr.max() < 5e-2 and derr.mean() < 1e-2        # regression guard, not the bar
+    if max(err.max(), derr.max()) >= 2e-2:
+        pytest.xfail(f"BASELINE bar 2e-2 absolute NOT met by the all-bf16 program: prefill max {err.max():.4f} "
+                     f"(mean {err.mean():.5f}), decode max {derr.max():.4f} (mean {derr.mean():.5f})")
 
 
 def test_ministral_full_size_fused_vs_generic_and_cache_invariant(hip):
@@ -454,10 +459,15 @@ def test_ministral_full_size_fused_vs_generic_and_cache_invariant(hip):
         hip.set_option("fusion", 1)
     # bf16 noise floor at this width and depth (see the one-layer test): compare in the mean, and
     # bound the max loosely
-    if toks[:5] == toks2:
-        d = np.abs(last - last2)
-        print(f"fused vs generic, 4 layers bf16: max {d.max():.4f} mean {d.mean():.5f}")
-        assert d.max() < 0.3 and d.mean() < 4e-2
+    # the two paths see the same token history only while their greedy tokens agree; compare the logits of the last
+    # step they share (at least the prefill's, whose input is the prompt alone)
+    assert toks[0] == toks2[0], "fused and op-by-op paths disagree on the first token"
+    if toks[:5] != toks2:
+        pytest.skip(f"greedy tokens diverge inside bf16 noise (fused {toks[:5]} vs op-by-op {toks2}): the logits of "
+                    "step 5 come from different histories and cannot be compared")
+    d = np.abs(last - last2)
+    print(f"fused vs generic, 4 layers bf16: max {d.max():.4f} mean {d.mean():.5f}")
+    assert d.max() < 0.3 and d.mean() < 4e-2
     # full-context forward over prompt + generated tokens reproduces the cached decode logits
     caches = [None] * cfg.num_layers
     full = hip.to_numpy(m.forward_with_decode_cache(prompt + toks[:5], 0, caches, 64))[-1]

@@ -199,7 +199,8 @@ def test_prefill_codes_equal_dequantised_weights(hip, scheme, m, k, n):
         (ref,) = oracle_run(pq, [x, q, s])
     finally:
         po.BLAS_DOT_MIN_MACS = old_min
-    assert_close(got, ref, atol=1e-4 * np.sqrt(k), rtol=2.0 ** -8, what="quantised GEMM vs oracle")
+    # both sides round an f32 sum to bf16: where the two summation orders straddle a rounding boundary, one ulp (2^-7)
+    assert_close(got, ref, atol=1e-4 * np.sqrt(k), rtol=2.0 ** -7, what="quantised GEMM vs oracle")
     (gotp,) = hip_run(hip, prog(lambda fb, a, b, bs, c, cs: F.swiglu(F.linear_quantized(a, b, bs), F.linear_quantized(a, c, cs)),
                                 [("Bf16", [m, k]), cs_, ss_, cs_, ss_]), [x, q, s, q2, s2])
     (wantp,) = hip_run(hip, prog(lambda fb, a, b, c: F.swiglu(a.matmul(b), a.matmul(c)),
