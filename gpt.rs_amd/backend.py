@@ -28,7 +28,7 @@ EXPORTS = [
     "gptrs_hip_param_get", "gptrs_hip_param_set", "gptrs_hip_supports_decode_sampling",
     "gptrs_hip_sample_decode_token", "gptrs_hip_sample_decode_token_begin", "gptrs_hip_sample_decode_token_wait",
     "gptrs_hip_decode_token_tensor", "gptrs_hip_sample_decode_rows_begin", "gptrs_hip_sample_decode_rows_wait",
-    "gptrs_hip_decode_rows_tensor", "gptrs_hip_last_error", "gptrs_hip_synchronize", "gptrs_hip_set_option",
+    "gptrs_hip_decode_rows_tensor", "gptrs_hip_sample_decode_rows_into", "gptrs_hip_last_error", "gptrs_hip_synchronize", "gptrs_hip_set_option",
     "gptrs_hip_counter",
 ]
 
@@ -86,6 +86,7 @@ def load_library(path: str = LIB_PATH):
     lib.gptrs_hip_sample_decode_rows_begin.argtypes = [vp, vp, ctypes.POINTER(ctypes.c_int64)]
     lib.gptrs_hip_sample_decode_rows_wait.argtypes = [vp, ctypes.c_int64, ctypes.POINTER(ctypes.c_int32), sz]
     lib.gptrs_hip_decode_rows_tensor.argtypes = [vp, ctypes.c_int64, pvp]
+    lib.gptrs_hip_sample_decode_rows_into.argtypes = [vp, vp, vp]
     lib.gptrs_hip_last_error.argtypes = []
     lib.gptrs_hip_last_error.restype = cp
     lib.gptrs_hip_synchronize.argtypes = [vp]
@@ -263,6 +264,11 @@ class HipBackend:
         buf = (ctypes.c_int32 * rows)()
         self._check(self._lib.gptrs_hip_sample_decode_rows_wait(self._handle, ticket, buf, rows))
         return [int(v) for v in buf]
+
+    def sample_decode_rows_into(self, logits: TensorHandle, tokens_out: TensorHandle):
+        """Queues the greedy token of every row of logits [rows <= 64, vocab] into tokens_out (si32[rows]); the call
+        allocates nothing on the device."""
+        self._check(self._lib.gptrs_hip_sample_decode_rows_into(self._handle, logits.ptr, tokens_out.ptr))
 
     def decode_rows_tensor(self, rows: int) -> TensorHandle:
         """si32[rows] handle over the device copy of the tokens of the last sample_decode_rows_begin."""

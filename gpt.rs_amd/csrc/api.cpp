@@ -68,6 +68,7 @@ Backend::Backend(int dev) : device(dev) {
     GPTRS_HIP_CHECK(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
     GPTRS_HIP_CHECK(hipMalloc((void**)&d_err_flag_, 256));
     GPTRS_HIP_CHECK(hipMalloc((void**)&d_counters_, k::kLinearCounters * sizeof(int)));
+    GPTRS_HIP_CHECK(k::argmax_noalloc_init(device));   // address of the no-allocation sampling scratch on this GPU
     GPTRS_HIP_CHECK(hipMalloc((void**)&d_argmax_val_, 1024 * sizeof(float)));
     GPTRS_HIP_CHECK(hipMalloc((void**)&d_argmax_idx_, 1024 * sizeof(int32_t)));
     token_buf_ = new_buffer(256);
@@ -341,6 +342,26 @@ int64_t Backend::sample_rows_begin(const gptrs_hip_tensor* logits) {
     GPTRS_HIP_CHECK(hipMemcpyAsync(h_token_ring_ + kRingSlot * slot + 1, d_err_flag_, 2 * sizeof(int), hipMemcpyDeviceToHost, stream));
     GPTRS_HIP_CHECK(hipEventRecord(token_events_[slot], stream));
     return ticket;
+}
+
+// The allocation-free variant of sample_rows_begin: kernels only, partial maxima in the library's fixed device array.
+void Backend::sample_rows_into(const gptrs_hip_tensor* logits, gptrs_hip_tensor* tokens_out) {
+    GPTRS_HIP_CHECK(hipSetDevice(device));
+    if (logits->consumed || tokens_out->consumed) fail_exec("tensor handle was donated to run_program and can no longer be used");
+    const Spec& s = logits->spec;
+    const int max_rows = k::argmax_noalloc_max_rows();
+    if (!dtype_is_float(s.dtype) || s.rank() != 2 || s.count() == 0)
+        fail_exec("sample_decode_rows_into expects non-empty f32/bf16 logits [rows, vocab]");
+    if (s.dims[0] > max_rows)
+        fail_exec("sample_decode_rows_into: " + std::to_string(s.dims[0]) + " rows exceed the fixed scratch of " + std::to_string(max_rows) + " rows");
+    if (s.dims[1] > INT32_MAX) fail_exec("sample_decode_rows_into: vocabulary exceeds the si32 token range");
+    const Spec& o = tokens_out->spec;
+    if (o.dtype != DType::SI32 || o.count() != s.dims[0] || !tokens_out->data())
+        fail_exec("sample_decode_rows_into: tokens_out must be si32[rows]");
+    if (!k::argmax_rows_noalloc(stream, device, (int)s.dtype, logits->data(), s.dims[0], s.dims[1], (int32_t*)tokens_out->data()))
+        fail_exec("sample_decode_rows_into: the scratch of this device is not initialised");
+    if (tokens_out->buf) tokens_out->buf->id = next_buffer_id_++;   // the contents changed
+    n_launches += 2;
 }
 
 void Backend::sample_rows_wait(int64_t ticket, int32_t* tokens_out, size_t n) {
@@ -857,6 +878,14 @@ int gptrs_hip_sample_decode_rows_begin(gptrs_hip_backend* b, const gptrs_hip_ten
         if (!b || !logits || !ticket_out) gptrs::fail_exec("null argument");
         std::lock_guard<std::mutex> g(b->impl.mu);
         *ticket_out = b->impl.sample_rows_begin(logits);
+    });
+}
+
+int gptrs_hip_sample_decode_rows_into(gptrs_hip_backend* b, const gptrs_hip_tensor* logits, gptrs_hip_tensor* tokens_out) {
+    return guarded([&] {
+        if (!b || !logits || !tokens_out) gptrs::fail_exec("null argument");
+        std::lock_guard<std::mutex> g(b->impl.mu);
+        b->impl.sample_rows_into(logits, tokens_out);
     });
 }
 

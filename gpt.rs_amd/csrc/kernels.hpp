@@ -65,6 +65,12 @@ void argmax_rows(hipStream_t s, int dtype, const void* logits, int64_t rows, int
                  int32_t* scratch_idx, int scratch_cap);
 void argmax_last_row(hipStream_t s, int dtype, const void* logits, int64_t rows, int64_t vocab, int64_t* out,
                      float* scratch_val, int32_t* scratch_idx, int scratch_cap);
+// argmax_rows over a fixed device array of the library instead of caller scratch: no allocation anywhere.
+// argmax_noalloc_init: once per device, with that device current (resolves the array's address on that GPU).
+// argmax_rows_noalloc: false when the device was not initialised or rows is outside [1, argmax_noalloc_max_rows()].
+hipError_t argmax_noalloc_init(int device);
+int argmax_noalloc_max_rows();
+bool argmax_rows_noalloc(hipStream_t s, int device, int dtype, const void* logits, int64_t rows, int64_t vocab, int32_t* out);
 // temperature sampling with a caller-supplied uniform u (inverse-CDF over softmax(logits/T))
 void sample_temperature_last_row(hipStream_t s, int dtype, const void* logits, int64_t rows, int64_t vocab,
                                  float temperature, float u, int64_t* out);

@@ -4,6 +4,8 @@
 // bit-exact, float ops compute in f32 and round once to the output dtype.
 #include <cstring>
 
+#include <mutex>
+
 #include "kernels.hpp"
 #include "device_utils.hpp"
 
@@ -468,6 +470,45 @@ void argmax_rows(hipStream_t s, int dtype, const void* logits, int64_t rows, int
     if (dtype == 0) argmax_rows_stage1<float><<<grid, 256, 0, s>>>((const float*)logits, vocab, scratch_val, scratch_idx);
     else argmax_rows_stage1<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)logits, vocab, scratch_val, scratch_idx);
     argmax_rows_stage2<<<(unsigned)rows, 64, 0, s>>>(scratch_val, scratch_idx, nb, out);
+}
+
+// The same two stages for callers that must not allocate: the per-block partial maxima (value, index) live in a
+// file-scope device array instead of a buffer the backend allocated.  Each GPU holds its own copy of the array at its
+// own address until the process ends; argmax_noalloc_init() resolves that address once per device (with the device
+// current), and the launcher hands it to the kernels as an ordinary pointer argument.  Stage 1 overwrites every
+// partial that stage 2 reads, so nothing has to start at zero; two calls that overlap on one GPU (two streams) race
+// on the array.
+constexpr int kNoAllocPartials = 4096;   // rows * blocks per row
+static __device__ __align__(256) unsigned char scratch[kNoAllocPartials * (sizeof(float) + sizeof(int32_t))];
+constexpr int kNoAllocMaxDevices = 64;
+static void* g_noalloc_ptr[kNoAllocMaxDevices] = {};
+static std::mutex g_noalloc_mu;
+
+hipError_t argmax_noalloc_init(int device) {
+    if (device < 0 || device >= kNoAllocMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> g(g_noalloc_mu);
+    if (g_noalloc_ptr[device]) return hipSuccess;
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!p) return hipErrorInvalidSymbol;
+    // load the kernels' code now, so that the first call does not do it
+    hipFuncAttributes fa{};
+    (void)hipFuncGetAttributes(&fa, (const void*)argmax_rows_stage1<float>);
+    (void)hipFuncGetAttributes(&fa, (const void*)argmax_rows_stage1<bf16_t>);
+    (void)hipFuncGetAttributes(&fa, (const void*)argmax_rows_stage2);
+    g_noalloc_ptr[device] = p;
+    return hipSuccess;
+}
+int argmax_noalloc_max_rows() { return 64; }
+bool argmax_rows_noalloc(hipStream_t s, int device, int dtype, const void* logits, int64_t rows, int64_t vocab, int32_t* out) {
+    if (device < 0 || device >= kNoAllocMaxDevices || rows < 1 || rows > argmax_noalloc_max_rows()) return false;
+    void* p = g_noalloc_ptr[device];   // the device address, never the array's name (a host-side stand-in)
+    if (!p) return false;
+    float* val = reinterpret_cast<float*>(p);
+    int32_t* idx = reinterpret_cast<int32_t*>(reinterpret_cast<unsigned char*>(p) + kNoAllocPartials * sizeof(float));
+    argmax_rows(s, dtype, logits, rows, vocab, out, val, idx, kNoAllocPartials);
+    return true;
 }
 
 // Temperature sampling, single block: softmax(logits/T) then inverse CDF at u.  The running

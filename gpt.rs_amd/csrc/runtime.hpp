@@ -171,6 +171,8 @@ class Backend {
     static constexpr int kMaxTokenRows = 64;
     int64_t sample_rows_begin(const gptrs_hip_tensor* logits);
     void sample_rows_wait(int64_t ticket, int32_t* tokens_out, size_t n);
+    // greedy token of every row into a caller's si32[rows] tensor; launches only, allocates nothing
+    void sample_rows_into(const gptrs_hip_tensor* logits, gptrs_hip_tensor* tokens_out);
     gptrs_hip_tensor* rows_tensor(int64_t rows);
     void synchronize();
     void check_device_errors();

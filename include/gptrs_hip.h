@@ -147,6 +147,17 @@ int gptrs_hip_sample_decode_rows_begin(gptrs_hip_backend* b, const gptrs_hip_ten
 int gptrs_hip_sample_decode_rows_wait(gptrs_hip_backend* b, int64_t ticket, int32_t* tokens_out, size_t n);
 int gptrs_hip_decode_rows_tensor(gptrs_hip_backend* b, int64_t rows, gptrs_hip_tensor** out);
 
+/* No counterpart in the reference.  For callers that cannot allocate device memory: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  The device half of gptrs_hip_sample_decode_rows_begin with the output
+ * handed in: queues, on the backend's stream, the greedy token (largest logit, smallest index on ties) of every row of
+ * logits [rows, vocab] (f32 or bf16) into tokens_out, a si32 tensor of `rows` elements that the caller materialised
+ * beforehand, and returns without waiting.  It launches two kernels and calls no hipMalloc / hipFree or any other
+ * allocating routine; the per-block partial maxima go to a fixed 32 KiB array that the library holds on each GPU for
+ * the life of the process (4096 partials), which limits rows to 64; more rows are rejected with an Execution error and
+ * nothing is launched.  All calls on one GPU share that array: calls that overlap in time on one GPU (two backends on
+ * one device) race.  Read the tokens with gptrs_hip_to_literal or feed tokens_out to the next program. */
+int gptrs_hip_sample_decode_rows_into(gptrs_hip_backend* b, const gptrs_hip_tensor* logits, gptrs_hip_tensor* tokens_out);
+
 /* Message of the calling thread's most recent non-zero return (BackendError Display). */
 const char* gptrs_hip_last_error(void);
 
