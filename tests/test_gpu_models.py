@@ -441,32 +441,26 @@ def test_ministral_full_width_one_layer_bf16_vs_oracle(hip):
 
 
 def test_ministral_full_size_fused_vs_generic_and_cache_invariant(hip):
-    """All 26 layers at full width are too slow for the CPU oracle; at that size the fused path is
-    checked against the op-by-op generic path (itself oracle-checked per op) and through the
+    """Four layers at full width: the fused path against the op-by-op generic path (itself oracle-checked per op) on
+    the prefill logits, whose only input is the prompt (later steps depend on each path's own greedy tokens, and at
+    bf16 noise of 0.08 the largest of 131072 near-tied random logits is not the same on both paths), and the
     decode == full-context invariant (crates/gpt-rs/tests/ministral.rs:65-89)."""
     cfg = models.MinistralConfig(num_layers=4)
     prompt = np.random.default_rng(6).integers(0, cfg.vocab_size, 24).tolist()
     m = models.Ministral.random(cfg, hip, seed=5, dtype="Bf16")
     gen = models.Generator(m, prompt, kv_cache_capacity=64)
+    first = hip.to_numpy(gen.logits)[-1].copy()
     toks = gen.generate(6)
     last = hip.to_numpy(gen.logits)[-1]
     hip.set_option("fusion", 0)
     try:
         gen2 = models.Generator(m, prompt, kv_cache_capacity=64)
-        toks2 = [gen2.step() for _ in range(5)]
-        last2 = hip.to_numpy(gen2.logits)[-1]
+        first2 = hip.to_numpy(gen2.logits)[-1].copy()
     finally:
         hip.set_option("fusion", 1)
-    # bf16 noise floor at this width and depth (see the one-layer test): compare in the mean, and
-    # bound the max loosely
-    # the two paths see the same token history only while their greedy tokens agree; compare the logits of the last
-    # step they share (at least the prefill's, whose input is the prompt alone)
-    assert toks[0] == toks2[0], "fused and op-by-op paths disagree on the first token"
-    if toks[:5] != toks2:
-        pytest.skip(f"greedy tokens diverge inside bf16 noise (fused {toks[:5]} vs op-by-op {toks2}): the logits of "
-                    "step 5 come from different histories and cannot be compared")
-    d = np.abs(last - last2)
-    print(f"fused vs generic, 4 layers bf16: max {d.max():.4f} mean {d.mean():.5f}")
+    d = np.abs(first - first2)
+    print(f"fused vs generic prefill, 4 layers bf16: max {d.max():.4f} mean {d.mean():.5f}; same first token: "
+          f"{int(np.argmax(first)) == int(np.argmax(first2))}")
     assert d.max() < 0.3 and d.mean() < 4e-2
     # full-context forward over prompt + generated tokens reproduces the cached decode logits
     caches = [None] * cfg.num_layers
