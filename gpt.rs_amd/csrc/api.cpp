@@ -244,7 +244,14 @@ void Backend::check_device_errors() {
         // a grid barrier of the persistent decode chain gave up: its counters are mid-phase
         k::fill_zero(stream, d_err_flag_, 256);
         k::fill_zero(stream, d_chain_bar_, k::kChainBarrierBytes);
-        fail_exec("decode chain: grid barrier timed out (workgroups of one launch were not all resident)");
+        GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
+        if (chain_stall_phase >= 0) {   // the stall was asked for (set_option "chain_stall_phase"): one launch, then back to normal
+            chain_stall_phase = -1;
+            fail_exec("decode chain: grid barrier timed out (a stall was requested for this launch); the outputs of the program are invalid");
+        }
+        opt_chain = false;              // whatever kept the workgroups from meeting would do so again: one kernel per layer from here on
+        fail_exec("decode chain: grid barrier timed out (workgroups of one launch were not all resident); the outputs of the program are "
+                  "invalid, and this backend runs decode steps one kernel per layer from now on");
     }
     if (flag[0]) {
         k::fill_zero(stream, d_err_flag_, 256);
@@ -476,7 +483,7 @@ Plan::~Plan() {
 // allocated while recording.  Returns false when the caller must run the steps eagerly.
 bool Backend::run_graphed(Plan& plan, ExecCtx& cx, const std::vector<BufferP>& out_bufs) {
     constexpr size_t kMaxGraphs = 8, kSeenRing = 32;
-    if (!opt_graphs || opt_profile || !plan.cacheable || plan.steps.size() < 4) return false;
+    if (!opt_graphs || opt_profile || chain_stall_phase >= 0 || !plan.cacheable || plan.steps.size() < 4) return false;
     if (plan.graph_builds >= 16 && plan.graph_hits < 4 * plan.graph_builds) return false;  // addresses never settle
     std::vector<uint64_t> key;
     key.reserve(cx.input_bufs.size() + out_bufs.size() + 8);
@@ -930,6 +937,7 @@ int gptrs_hip_set_option(gptrs_hip_backend* b, const char* name, int64_t value) 
         if (!strcmp(name, "fusion")) b->impl.opt_fusion = value != 0;
         else if (!strcmp(name, "graphs")) b->impl.opt_graphs = value != 0;
         else if (!strcmp(name, "chain")) b->impl.opt_chain = value != 0;
+        else if (!strcmp(name, "chain_stall_phase")) b->impl.chain_stall_phase = value < 0 ? -1 : (int)std::min<int64_t>(value, 1 << 20);
         else if (!strcmp(name, "profile")) { b->impl.profile_reset(); b->impl.opt_profile = value != 0; }
         else gptrs::fail_spec(std::string("unknown option `") + name + "`");
     });

@@ -177,7 +177,7 @@ void dequant_w4g128(hipStream_t s, int dtype, const uint8_t* packed, const void*
 // the same launch.
 constexpr int kChainCounters = 16;        // striped arrival counters of the grid barrier
 constexpr int kChainMaxPhases = 192;
-constexpr int kChainMaxXsWords = 16384;   // staged activation pairs: K <= 32768
+constexpr int kChainMaxXsWords = 12288;   // staged activation words (48 KiB): K <= 24576 for bf16 weights
 constexpr size_t kChainBarrierBytes = (kChainCounters * 64 + 64) * sizeof(unsigned);  // zero-initialised once
 // kChainOutF32: y and the residual are f32.  kChainXF32 (with kChainNorm): x and gamma are f32, the normalised row is
 // rounded to bf16 once as it is staged.
@@ -229,8 +229,9 @@ void chain_fill_attn(ChainPhase& partial, ChainPhase& combine, int64_t n_q, int6
                      int64_t rot_half, float scale);
 // bar: kChainBarrierBytes of device memory zeroed once; abort_flag: raised when a barrier wait
 // gives up (every wave then leaves the kernel).  false: launch not possible (caller falls back).
+// stall_phase >= 0 (tests of the give-up path): every workgroup expects one arrival too many at that phase's barrier.
 bool chain_launch(hipStream_t s, const ChainPhase* dev_table, int nphases, int lds_bytes, unsigned* bar, int* abort_flag,
-                  int wfmt = kChainW16);   // wfmt: the weight format of EVERY linear phase of the table
+                  int wfmt = kChainW16, int stall_phase = -1);   // wfmt: the weight format of EVERY linear phase of the table
 
 // Prefill GEMM (M > 16, bf16) on the matrix cores over a k-grouped copy of the weights,
 // Wk8[K/8][Npad][8] (kernels_mfma.hip).  wk2 != nullptr: SwiGLU pair.

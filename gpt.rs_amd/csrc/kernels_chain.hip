@@ -5,18 +5,28 @@
 // every GEMV pays a launch gap, a cold start and a tail; here the whole run executes inside one
 // kernel of one workgroup per CU, phases separated by a grid-wide barrier:
 //
-//   * 8 streaming waves per workgroup only load weight words and issue v_dot2 (bf16 pairs): a
-//     workgroup owns groups of TP tiles of 4 output columns for the whole of K, lane t reading word
-//     t, t+512, ... of each tile stream (Wc[tile][k/2][4 cols][2 k], 16-byte words).  The next
-//     j-step (TP words) is always in flight while the current one is consumed, across unit AND phase
-//     boundaries: weights do not depend on activations, so the first words of the next layer are
-//     already in registers when its input becomes ready.
+//   * 8 compute waves per workgroup stream the workgroup's weight words from HBM straight into LDS
+//     (global_load_lds_dwordx4: no registers), each wave into a ring of its own (3 KiB per j-step: one 16-byte
+//     word per lane and tile of the unit), in the order they are consumed: phase by phase, unit by unit (TP
+//     tiles of 4 output columns for the whole of K), j-step by j-step.  Weights do not depend on activations,
+//     so a wave's requests run RING_D j-steps ahead of its reads across unit AND phase boundaries: while the
+//     wave stands at the grid barrier, stages the next input or runs an attention phase, HBM keeps delivering
+//     the next phase's first words.  Loads of a wave return in order, so "j-step g has landed" is a wait on
+//     the count of loads in flight: a ring private to the wave needs no flags and no barrier.  The loop
+//     around a j-step is kept to a few dozen instructions (uniform bookkeeping in scalar registers, one vector
+//     add and clamp per request): with three waves per SIMD a longer loop body, not HBM, sets the pace.
+//   * the compute lanes read their words from the ring (lane t owns word t of each tile stream,
+//     Wc[tile][k/2][4 cols][2 k]) and issue v_dot2 (bf16 pairs) against the activation vector staged in LDS.
 //   * 1 control wave per workgroup sums the 8 waves' partial sums of a unit out of LDS, applies the
 //     epilogue (SwiGLU pair, bias, GELU, residual), stores through to memory, and runs the grid
 //     barrier (16 striped arrival counters, one poll instruction).
 //   * Activations cross workgroups through agent-scope (sc1) loads and stores only, so no
 //     L2 write-back / invalidate is needed between phases; a phase's input vector is staged into
-//     LDS by all 9 waves together right after the barrier (RMSNorm statistics included).
+//     LDS by the 9 compute and control waves together right after the barrier (RMSNorm statistics
+//     included).
+//   * Phase descriptors are read from the table in memory ahead of the wait that precedes their use (scalar
+//     loads in the compute waves, one vector load with a lane per dword in the control wave), so a phase opens
+//     the moment its barrier is seen.
 //
 // Decode attention (T = 1 over the KV cache) runs inside the same launch as two more phase kinds,
 // executed by all 9 waves of a workgroup together: "partial" (one workgroup per kv head and
@@ -30,10 +40,11 @@
 // exact); the bias is taken out per word (-128 or -8 times the sum of the word's activations), the
 // per-column int8 scale is applied by the control wave.
 //
-// Every wait is bounded: a barrier that does not complete raises the abort flag, every wave
-// leaves the kernel, and the host reports an execution error.
+// Every wait is bounded by wall-clock time: a barrier that does not complete raises the abort flag, every
+// wave leaves the kernel, and the host reports an execution error.
 #include <algorithm>
 #include <climits>
+#include <cstddef>
 #include <cstdlib>
 
 #include "kernels.hpp"
@@ -44,18 +55,23 @@ namespace k {
 
 namespace {
 
-constexpr int NS = 512;          // streaming threads
-constexpr int NT = NS + 64;      // + control wave
+constexpr int NS = 512;          // compute threads
+constexpr int NT = NS + 64;      // + control wave: the threads that stage inputs and run attention phases
 constexpr int NWS = NS / 64;
 constexpr int TP = 3;            // tiles (of 4 columns) per unit
-constexpr int NSLOT = 4;         // unit hand-off slots between streaming waves and control wave
+constexpr int NSLOT = 4;         // unit hand-off slots between compute waves and control wave
 constexpr int NC = kChainCounters;
-constexpr int EPI_MAX = 2048;    // bias/residual values staged per workgroup and phase
+constexpr int EPI_MAX = 640;     // bias/residual values staged per workgroup and phase: N <= 160 * grid columns
 constexpr int MAXI = 8;          // 8-byte items per thread in the norm staging: K <= 4*MAXI*NT
-
+constexpr int SLOT_BYTES = TP * NS * 16;     // one j-step of a workgroup: a word per compute lane and tile
+constexpr int RING_D = 4;                    // j-steps a wave's ring holds: its requests run that far ahead of its reads
+constexpr int LDS_BYTES = 160 * 1024;        // per workgroup on gfx950
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+// The thread index behind an opaque barrier: values derived from it are recomputed by the phase that uses them instead of
+// being computed once per launch and held in registers (or spilled) across every other phase.
+__device__ __forceinline__ int local_tid() { int t = (int)threadIdx.x; asm volatile("" : "+v"(t)); return t; }
 template <typename T> __device__ __forceinline__ T* uni_ptr(T* p) {
     const unsigned long long v = (unsigned long long)p;
     const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)v);
@@ -105,25 +121,6 @@ template <typename P> __device__ __forceinline__ int lds_ld(P p) { return __hip_
 template <typename P> __device__ __forceinline__ void lds_st(P p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
 #define GPTRS_LDS_RELEASE() __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local")
 #define GPTRS_LDS_ACQUIRE() __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local")
-// workgroup barrier that waits for LDS traffic only: outstanding weight loads stay in flight
-__device__ __forceinline__ void lds_barrier() {
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
-    __builtin_amdgcn_s_barrier();
-}
-
-#ifdef GPTRS_CHAIN_STAMPS
-__device__ unsigned long long* g_chain_stamps = nullptr;   // lab builds: [phase][8] wall-clock stamps of workgroup 0
-#define GPTRS_STAMP(i) do { if (g_chain_stamps && blockIdx.x == 0 && (threadIdx.x & 63) == 0) g_chain_stamps[ph * 16 + (i)] = wall_clock64(); } while (0)
-#define GPTRS_STAMP_W0(i) do { if (g_chain_stamps && blockIdx.x == 0 && threadIdx.x == 0) g_chain_stamps[phase * 16 + (i)] = wall_clock64(); } while (0)
-#define GPTRS_STAMP_C(i) do { if (g_chain_stamps && blockIdx.x == 0 && threadIdx.x == NS) g_chain_stamps[phase * 16 + (i)] = wall_clock64(); } while (0)
-__device__ int g_chain_stage_phase = 0;
-#define GPTRS_STAMP_S(i) do { if (g_chain_stamps && blockIdx.x == 0 && threadIdx.x == NS) g_chain_stamps[g_chain_stage_phase * 16 + (i)] = wall_clock64(); } while (0)
-#else
-#define GPTRS_STAMP(i) do { } while (0)
-#define GPTRS_STAMP_W0(i) do { } while (0)
-#define GPTRS_STAMP_C(i) do { } while (0)
-#define GPTRS_STAMP_S(i) do { } while (0)
-#endif
 
 struct Shared {
     float red[NSLOT][NWS][16];
@@ -135,18 +132,59 @@ struct Shared {
     float ssq[16];
     int red_cnt[NSLOT];
     int go, consumed, abort, pad;
-    ChainPhase ph[kChainMaxPhases];
 };
+
+// The table of phases is read-only for the whole launch: reading it through the constant address space lets the
+// compiler use scalar loads (uniform addresses), which do not queue behind a wave's vector memory traffic.
+#define GPTRS_CONST __attribute__((address_space(4)))
+typedef const GPTRS_CONST ChainPhase* PhaseTable;
+static_assert(sizeof(Shared) + (size_t)kChainMaxXsWords * 4 + (size_t)RING_D * SLOT_BYTES <= (size_t)LDS_BYTES, "the largest launch fits a CU's LDS");
+constexpr int kPhaseDwords = (int)(sizeof(ChainPhase) / 4);
+static_assert(kPhaseDwords <= 64, "one lane of the control wave per dword of a phase descriptor");
+
+// Workgroup barrier that waits for this wave's LDS traffic only: the weight loads in flight stay in flight.
+__device__ __forceinline__ void wg_barrier() {
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+}
+
+// Uniform copy (scalar registers) of the descriptor fields that the staging and the epilogue read.  The compute waves
+// fill it with scalar loads from the table before they wait for the phase to open; the control wave reads the table with
+// one vector load (a lane per dword) before it waits for the grid barrier and picks the fields out of the lanes.  Either
+// way nothing is fetched between the barrier and the first use.
+struct PhaseRegs {
+    int K, N, Kw, ntiles, upb, units, lds_bytes, flags, wfmt;
+    float inv_n, eps;
+    const void *x, *gamma, *bias, *residual, *wscale, *wscale2;
+    void* y;
+};
+__device__ __forceinline__ void regs_from_table(PhaseRegs& R, const GPTRS_CONST ChainPhase* D) {
+    R.K = uni(D->K); R.N = uni(D->N); R.Kw = uni(D->Kw); R.ntiles = uni(D->ntiles); R.upb = uni(D->upb); R.units = uni(D->units);
+    R.lds_bytes = uni(D->lds_bytes); R.flags = uni(D->flags); R.wfmt = uni(D->wfmt);
+    R.inv_n = __int_as_float(uni(__float_as_int(D->inv_n))); R.eps = __int_as_float(uni(__float_as_int(D->eps)));
+    R.x = uni_ptr(D->x); R.gamma = uni_ptr(D->gamma); R.bias = uni_ptr(D->bias); R.residual = uni_ptr(D->residual);
+    R.wscale = uni_ptr(D->wscale); R.wscale2 = uni_ptr(D->wscale2); R.y = uni_ptr(D->y);
+}
+#define GPTRS_PD_INT(field) __builtin_amdgcn_readlane(pd, (int)(offsetof(ChainPhase, field) / 4))
+#define GPTRS_PD_PTR(field) ((const void*)(((unsigned long long)(unsigned)__builtin_amdgcn_readlane(pd, (int)(offsetof(ChainPhase, field) / 4) + 1) << 32) | \
+                                          (unsigned)__builtin_amdgcn_readlane(pd, (int)(offsetof(ChainPhase, field) / 4))))
+__device__ __forceinline__ void regs_from_lanes(PhaseRegs& R, int pd) {   // pd: dword `lane` of the descriptor
+    R.K = GPTRS_PD_INT(K); R.N = GPTRS_PD_INT(N); R.Kw = GPTRS_PD_INT(Kw); R.ntiles = GPTRS_PD_INT(ntiles); R.upb = GPTRS_PD_INT(upb);
+    R.units = GPTRS_PD_INT(units); R.lds_bytes = GPTRS_PD_INT(lds_bytes); R.flags = GPTRS_PD_INT(flags); R.wfmt = GPTRS_PD_INT(wfmt);
+    R.inv_n = __int_as_float(GPTRS_PD_INT(inv_n)); R.eps = __int_as_float(GPTRS_PD_INT(eps));
+    R.x = GPTRS_PD_PTR(x); R.gamma = GPTRS_PD_PTR(gamma); R.bias = GPTRS_PD_PTR(bias); R.residual = GPTRS_PD_PTR(residual);
+    R.wscale = GPTRS_PD_PTR(wscale); R.wscale2 = GPTRS_PD_PTR(wscale2); R.y = const_cast<void*>(GPTRS_PD_PTR(y));
+}
 
 // ---------------------------------------------------------------------------- staging (all waves)
 // xs[j] = (x[2j], x[2j+1]) as a bf16 pair, zero beyond K; with norm: the value the stand-alone
 // RMSNorm kernels store, ((x * inv_rms) * gamma) -> bf16 (normalization.rs:183-217).
-__device__ void stage_block(const ChainPhase& P, unsigned* xs, float* ssq) {
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int K = uni(P.K);
+__device__ __forceinline__ void stage_block(const PhaseRegs& P, unsigned* xs, float* ssq) {
+    const int t = local_tid(), lane = t & 63, wave = uni(t >> 6);
+    const int K = P.K;
     const int n = K / 4;                     // 8-byte items holding data (K % 4 == 0)
-    const int npad = uni(P.lds_bytes) >> 3;  // items to write: the words of every lane read zeros beyond K
-    const char* x = (const char*)uni_ptr(P.x);
+    const int npad = P.lds_bytes >> 3;  // items to write: the words of every lane read zeros beyond K
+    const char* x = (const char*)P.x;
     // int4: the group scales of this workgroup's tiles, one contiguous range of the tile-ordered copy
     // sc[tile][group][4] (bf16, 8 bytes per entry), go behind the activations; the first round of
     // loads is in flight while the activations are staged
@@ -155,21 +193,21 @@ __device__ void stage_block(const ChainPhase& P, unsigned* xs, float* ssq) {
     const uint2* sc_src = nullptr;
     uint2* sc_dst = reinterpret_cast<uint2*>(xs + 2 * npad);
     uint2 sv[SB];
-    if (uni(P.wfmt) == kChainW4) {
-        const int G = uni(P.Kw) >> 4, upb = uni(P.upb);
-        const int t0 = (int)blockIdx.x * upb * TP, t1 = min(min(t0 + upb * TP, uni(P.units) * TP), uni(P.ntiles));
+    if (P.wfmt == kChainW4) {
+        const int G = P.Kw >> 4, upb = P.upb;
+        const int t0 = (int)blockIdx.x * upb * TP, t1 = min(min(t0 + upb * TP, P.units * TP), P.ntiles);
         sc_n = max(t1 - t0, 0) * G;
-        sc_src = (const uint2*)uni_ptr(P.wscale) + (long)t0 * G;
+        sc_src = (const uint2*)P.wscale + (long)t0 * G;
 #pragma unroll
         for (int u = 0; u < SB; ++u) {
             const int i = u * NT + t;
             sv[u] = i < sc_n ? gload2(sc_src + i) : make_uint2(0u, 0u);
         }
     }
-    if ((uni(P.flags) & (kChainNorm | kChainXF32)) == (kChainNorm | kChainXF32)) {
+    if ((P.flags & (kChainNorm | kChainXF32)) == (kChainNorm | kChainXF32)) {
         // f32 row and gains (a bf16 model whose residual stream is f32): the f32 norm, rounded to bf16 once
         constexpr int MF = MAXI / 2;   // 16-byte items per thread: K <= 4 * MF * NT
-        const char* g = (const char*)uni_ptr(P.gamma);
+        const char* g = (const char*)P.gamma;
         uint4 v[MF], gg[MF];
 #pragma unroll
         for (int u = 0; u < MF; ++u) {
@@ -192,7 +230,7 @@ __device__ void stage_block(const ChainPhase& P, unsigned* xs, float* ssq) {
         }
         const float ws = wave_sum(q);
         if (lane == 0) ssq[wave] = ws;
-        lds_barrier();
+        wg_barrier();
         float tot = 0.f;
 #pragma unroll
         for (int w = 0; w < NT / 64; ++w) tot += ssq[w];
@@ -208,8 +246,8 @@ __device__ void stage_block(const ChainPhase& P, unsigned* xs, float* ssq) {
                 *reinterpret_cast<uint2*>(&xs[2 * i]) = make_uint2(o0, o1);
             }
         }
-    } else if (uni(P.flags) & kChainNorm) {
-        const uint2* g = (const uint2*)uni_ptr(P.gamma);
+    } else if (P.flags & kChainNorm) {
+        const uint2* g = (const uint2*)P.gamma;
         unsigned long long v[MAXI];
         uint2 gg[MAXI];
 #pragma unroll
@@ -232,16 +270,13 @@ __device__ void stage_block(const ChainPhase& P, unsigned* xs, float* ssq) {
                 q += a * a; q += b * b; q += c * c; q += d * d;
             }
         }
-        GPTRS_STAMP_S(6);
         const float ws = wave_sum(q);
         if (lane == 0) ssq[wave] = ws;
-        lds_barrier();
-        GPTRS_STAMP_S(7);
+        wg_barrier();
         float tot = 0.f;
 #pragma unroll
         for (int w = 0; w < NT / 64; ++w) tot += ssq[w];
         const float inv = 1.0f / sqrtf(tot * P.inv_n + P.eps);
-        GPTRS_STAMP_S(15);
 #pragma unroll
         for (int u = 0; u < MAXI; ++u) {
             const int i = u * NT + t;
@@ -268,7 +303,6 @@ __device__ void stage_block(const ChainPhase& P, unsigned* xs, float* ssq) {
             }
         }
     }
-    GPTRS_STAMP_S(14);
     if (sc_n > 0) {
 #pragma unroll
         for (int u = 0; u < SB; ++u) {
@@ -288,7 +322,7 @@ __device__ void stage_block(const ChainPhase& P, unsigned* xs, float* ssq) {
             }
         }
     }
-    lds_barrier();
+    wg_barrier();
 }
 
 
@@ -333,13 +367,27 @@ __device__ __forceinline__ void unpack_u4(const uint4& v, float (&o)[8]) {
     o[0] = bf16lo(v.x); o[1] = bf16hi(v.x); o[2] = bf16lo(v.y); o[3] = bf16hi(v.y);
     o[4] = bf16lo(v.z); o[5] = bf16hi(v.z); o[6] = bf16lo(v.w); o[7] = bf16hi(v.w);
 }
-// streaming waves wait here until the control wave has seen the grid barrier of `phase`
+// Waits inside the kernel are bounded by wall-clock time (wall_clock64 ticks at 100 MHz): the control wave's wait for the
+// grid barrier by the launch's budget, the waits on it inside the workgroup by a multiple of that, so that the control
+// wave is the one to give up and say why.
+struct Patience {
+    unsigned long long t0, ticks;
+    unsigned spins;
+    __device__ __forceinline__ Patience(unsigned long long budget) : t0(0), ticks(budget), spins(0) {}
+    __device__ __forceinline__ bool spent() {   // call once per poll; reads the clock every 64th time
+        if ((++spins & 63u) != 0) return false;
+        const unsigned long long now = wall_clock64();
+        if (t0 == 0) { t0 = now; return false; }
+        return now - t0 > ticks;
+    }
+};
+// compute waves wait here until the control wave has seen the grid barrier of `phase`
 template <typename IP>
-__device__ __forceinline__ bool wait_go(IP go, IP abort, int phase) {
-    unsigned spins = 0;
+__device__ __forceinline__ bool wait_go(IP go, IP abort, int phase, unsigned long long budget) {
+    Patience pat(8 * budget);
     while (uni(lds_ld(go)) < phase) {
         __builtin_amdgcn_s_sleep(1);
-        if (uni(lds_ld(abort)) || ++spins > (1u << 24)) return false;
+        if (uni(lds_ld(abort)) || pat.spent()) return false;
     }
     return true;
 }
@@ -383,9 +431,10 @@ __device__ __forceinline__ void lane_pair(float v, int off, float& a, float& b) 
 // the waves of different heads re-read the same rows out of the caches.  Cache rows older than
 // this launch are requested BEFORE the grid barrier is awaited (they do not depend on the
 // previous phase); only the query row and this step's K/V row are read after it.
-__device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const ChainPhase& P, GPTRS_LDS float* lds, int unit, int phase) {
+__device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const ChainPhase& P, GPTRS_LDS float* lds, int unit, int phase,
+                             unsigned long long budget) {
     constexpr int PP = 4;   // positions per lane group requested ahead of the barrier
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int t = local_tid(), lane = t & 63, wave = uni(t >> 6);
     const bool control = wave == NWS;
     const int dh = P.head_dim, n_q = P.n_q, n_kv = P.n_kv, nch = P.nch, half = P.rot_half;
     const int G = n_q / n_kv, nparts = NWS / G;
@@ -408,8 +457,6 @@ __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
     const bf16_t* knew = qkv + (long)n_q * dh + (long)kvh * dh;
     const bf16_t* vnew = qkv + (long)(n_q + n_kv) * dh + (long)kvh * dh;
     const int c0 = li * 8;
-
-    GPTRS_STAMP_W0(8);
     uint4 kraw[PP], vraw[PP];
 #pragma unroll
     for (int j = 0; j < PP; ++j) {
@@ -423,9 +470,7 @@ __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
             vraw[j] = make_uint4(0, 0, 0, 0);
         }
     }
-    GPTRS_STAMP_W0(9);
-    if (!control && !wait_go(go, abort, phase)) return false;
-    GPTRS_STAMP_W0(10);
+    if (!control && !wait_go(go, abort, phase, budget)) return false;
 
     float m = -INFINITY, l = 0.f, o[8];
 #pragma unroll
@@ -465,7 +510,6 @@ __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
         };
         float qf[8];
         rope(qa, qb, qf);
-        GPTRS_STAMP_W0(11);
 
         auto visit = [&](const float (&kf)[8], const float (&vf)[8]) {
             float sc = 0.f;
@@ -509,7 +553,6 @@ __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
             }
             if (upd >= p0 && upd < p1) visit(kf, vf);
         }
-        GPTRS_STAMP_W0(12);
         // merge the lane groups of this wave
         for (int off = lpr; off < 64; off <<= 1) {
             float ma, mb, la, lb;
@@ -537,10 +580,7 @@ __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
 #pragma unroll
         for (int v = 0; v < 8; ++v) so[wave * dh + c0 + v] = o[v];
     }
-    GPTRS_STAMP_W0(13);
-    lds_barrier();
-    GPTRS_STAMP_W0(14);
-    GPTRS_STAMP_C(6);
+    wg_barrier();
     float* partp = P.part;
     for (int idx = t; idx < G * dh; idx += NT) {
         const int gg = idx / dh, d = idx - gg * dh;
@@ -558,20 +598,19 @@ __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
         if (d == 0) { cstore4(rec, __float_as_uint(mn)); cstore4(rec + 1, __float_as_uint(Ls)); }
         cstore4(rec + 2 + d, __float_as_uint(O));
     }
-    GPTRS_STAMP_W0(15);
-    lds_barrier();
-    GPTRS_STAMP_C(7);
+    wg_barrier();
     return true;
 }
 
 // unit = query head: softmax-merge of its nch chunk records into the context row.  Thread
 // (sg, d2) reads the records of the chunks s = sg, sg + NW, ... for the dims (2 d2, 2 d2 + 1) in
 // one round of loads and merges them locally; the NW subsets meet in LDS.
-__device__ bool attn_combine(GPTRS_LDS int* go, GPTRS_LDS int* abort, const ChainPhase& P, GPTRS_LDS float* lds, int hq, int phase) {
+__device__ bool attn_combine(GPTRS_LDS int* go, GPTRS_LDS int* abort, const ChainPhase& P, GPTRS_LDS float* lds, int hq, int phase,
+                             unsigned long long budget) {
     constexpr int MAXC = 8;   // chunks per thread: nch <= MAXC * NW
-    const int t = threadIdx.x, wave = t >> 6;
+    const int t = local_tid(), wave = uni(t >> 6);
     const int dh = P.head_dim, nch = P.nch;
-    if (wave != NWS && !wait_go(go, abort, phase)) return false;
+    if (wave != NWS && !wait_go(go, abort, phase, budget)) return false;
     const float* base = P.part + (long)hq * nch * (dh + 2);
     bf16_t* ctx = (bf16_t*)P.y;
     const int h2 = dh / 2;
@@ -603,7 +642,7 @@ __device__ bool attn_combine(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
         }
         GPTRS_LDS f32x4* rec = (GPTRS_LDS f32x4*)lds;
         { f32x4 r4; r4.x = mn; r4.y = Ls; r4.z = o0; r4.w = o1; rec[wave * 64 + (t & 63)] = r4; }
-        lds_barrier();
+        wg_barrier();
         if (wave == 0 && act) {
             float M = -INFINITY;
 #pragma unroll
@@ -617,27 +656,30 @@ __device__ bool attn_combine(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
             }
             cstore4(ctx + (long)hq * dh + 2 * d2, pack_bf16x2(a0 / Lt, a1 / Lt));
         }
-        lds_barrier();
+        wg_barrier();
     }
     return true;
 }
 
-// All waves of the workgroup: the units blk, blk + grid, ... of an attention phase.  Kept out of
-// line (its register needs must not leak into the streaming loop); the LDS operands travel as
-// explicit local-address-space pointers so their accesses stay ds_* instructions.
-__device__ __forceinline__ bool run_attn_phase(GPTRS_LDS const ChainPhase* php, GPTRS_LDS float* lds, GPTRS_LDS int* go, GPTRS_LDS int* abort, int phase) {
+// The 9 compute and control waves of the workgroup: the units blk, blk + grid, ... of an attention phase.  Kept out of
+// line (its register needs must not leak into the compute loop); the LDS operands travel as explicit
+// local-address-space pointers so their accesses stay ds_* instructions.
+// The descriptor comes straight from the table in memory (scalar loads): the compute waves enter an attention phase, and
+// request the cache rows it needs, before the control wave has seen the barrier and filled the LDS copy.
+__device__ __forceinline__ bool run_attn_phase(const GPTRS_CONST ChainPhase* php, GPTRS_LDS float* lds, GPTRS_LDS int* go, GPTRS_LDS int* abort, int phase,
+                                               unsigned long long budget) {
     ChainPhase P;
     {
         int* dst = reinterpret_cast<int*>(&P);
-        GPTRS_LDS const int* src = (GPTRS_LDS const int*)php;
+        const GPTRS_CONST int* src = (const GPTRS_CONST int*)php;
 #pragma unroll
-        for (int i = 0; i < (int)(sizeof(ChainPhase) / 4); ++i) dst[i] = uni(src[i]);
+        for (int i = 0; i < kPhaseDwords; ++i) dst[i] = uni(src[i]);
     }
     const int kind = P.kind, units = P.units;
     for (int u = blockIdx.x; u < units; u += gridDim.x) {
         bool ok;
-        if (kind == kChainAttnCombine) ok = attn_combine(go, abort, P, lds, u, phase);
-        else ok = attn_partial(go, abort, P, lds, u, phase);
+        if (kind == kChainAttnCombine) ok = attn_combine(go, abort, P, lds, u, phase, budget);
+        else ok = attn_partial(go, abort, P, lds, u, phase, budget);
         if (!ok) return false;
     }
     return true;
@@ -652,29 +694,32 @@ __device__ __forceinline__ float finish(float v, int flags, float bias, float re
 }
 
 template <int FMT>
-__device__ void control_wave(Shared& sh, unsigned* xs, int nphases, unsigned* bar, int* abort_flag) {
+__device__ void control_wave(Shared& sh, unsigned* xs, const ChainPhase* phases, int nphases, unsigned* bar, int* abort_flag,
+                             unsigned long long budget, int stall_phase) {
+    PhaseTable table = (PhaseTable)phases;
     const int lane = threadIdx.x & 63;
     const int blk = blockIdx.x, per = gridDim.x / NC;
     const unsigned epoch = gload(bar + NC * 64);   // written by the previous launch, stable during this one
     int ucount = 0;
     for (int ph = 0; ph < nphases; ++ph) {
-        const ChainPhase& P = sh.ph[ph];
-        const int kind = uni(P.kind);
-        const int upb = uni(P.upb), units = uni(P.units);
+        // the phase's descriptor is requested before the wait for the barrier and lands in LDS after it, ahead of `go`
+        const int pd = lane < kPhaseDwords ? gload(reinterpret_cast<const int*>(phases + ph) + lane) : 0;
+        const GPTRS_CONST ChainPhase* D = table + ph;
+        const int kind = uni(D->kind);
+        const int upb = uni(D->upb), units = uni(D->units);
         const int u0 = kind == kChainLinear ? blk * upb : 0;
         const int u1 = kind == kChainLinear ? min(u0 + upb, units) : 0;
-        GPTRS_STAMP(0);
         if (ph > 0) {
-            const unsigned target = epoch + (unsigned)ph * per;
-            unsigned spins = 0;
+            // stall_phase (a test hook, -1 otherwise): one arrival more than the grid can deliver is expected at that
+            // phase, so this wait runs out of time and the give-up path below is taken
+            const unsigned target = epoch + (unsigned)ph * per + (ph == stall_phase ? 1u : 0u);
+            Patience pat(budget);
             bool ok = true;
             for (;;) {
                 const unsigned v = lane < NC ? __hip_atomic_load(as_global(bar) + lane * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : target;
                 if (__builtin_amdgcn_ballot_w64((int)(v - target) < 0) == 0) break;
                 __builtin_amdgcn_s_sleep(1);
-                if ((++spins & 63u) == 0) {
-                    if (__hip_atomic_load(as_global(abort_flag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) || spins > (1u << 19)) { ok = false; break; }
-                }
+                if (pat.spent() || ((pat.spins & 63u) == 0 && __hip_atomic_load(as_global(abort_flag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) { ok = false; break; }
             }
             if (!ok) {
                 __hip_atomic_store(as_global(abort_flag), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -682,14 +727,17 @@ __device__ void control_wave(Shared& sh, unsigned* xs, int nphases, unsigned* ba
                 return;
             }
         }
-        GPTRS_STAMP(1);
+        // the compute waves hold their own copy of the descriptor: the phase opens the moment the barrier is seen
         if (kind != kChainLinear) {
             if (blk < units) {
                 if (lane == 0) lds_st(&sh.go, ph);
-                run_attn_phase((GPTRS_LDS const ChainPhase*)&sh.ph[ph], (GPTRS_LDS float*)xs, (GPTRS_LDS int*)&sh.go, (GPTRS_LDS int*)&sh.abort, ph);
+                run_attn_phase(table + ph, (GPTRS_LDS float*)xs, (GPTRS_LDS int*)&sh.go, (GPTRS_LDS int*)&sh.abort, ph, budget);
             }
         } else if (u0 < u1) {
-            const int flags = uni(P.flags), ntiles = uni(P.ntiles), N = uni(P.N);
+            if (lane == 0) lds_st(&sh.go, ph);
+            PhaseRegs P;
+            regs_from_lanes(P, pd);
+            const int flags = P.flags, ntiles = P.ntiles, N = P.N;
             const bool dual = flags & kChainDual;
             const int cpt = dual ? 2 : 4;              // output columns per tile
             const int col0 = u0 * TP * cpt;
@@ -697,12 +745,11 @@ __device__ void control_wave(Shared& sh, unsigned* xs, int nphases, unsigned* ba
             // bias / residual / int8 scales of this workgroup's columns: the first round is requested before the
             // staging loads and written to LDS after the staging, so that its latency hides behind the staging
             // instead of holding up the workgroup's barrier inside it
-            const unsigned* bias = (const unsigned*)uni_ptr(P.bias);
-            const char* resid = (const char*)uni_ptr(P.residual);
+            const unsigned* bias = (const unsigned*)P.bias;
+            const char* resid = (const char*)P.residual;
             constexpr int wfmt = FMT;   // every linear phase of a launch has the kernel's weight format
-            const unsigned* sg = wfmt == kChainW8 ? (const unsigned*)uni_ptr(P.wscale) : nullptr;
-            const unsigned* su = wfmt == kChainW8 ? (const unsigned*)uni_ptr(P.wscale2) : nullptr;
-            if (lane == 0) lds_st(&sh.go, ph);
+            const unsigned* sg = wfmt == kChainW8 ? (const unsigned*)P.wscale : nullptr;
+            const unsigned* su = wfmt == kChainW8 ? (const unsigned*)P.wscale2 : nullptr;
             const bool out_f32 = flags & kChainOutF32;   // y and the residual are f32
             unsigned long long e_rf = 0ull;              // two f32 residual values
             auto epi_load = [&](int i, unsigned& bw, unsigned& rw, unsigned& ga, unsigned& gb) {
@@ -729,12 +776,7 @@ __device__ void control_wave(Shared& sh, unsigned* xs, int nphases, unsigned* ba
             const bool has_epi = bias || resid || sg;
             unsigned e_bw = 0u, e_rw = 0u, e_ga = 0u, e_gb = 0u;
             if (has_epi) epi_load(lane * 2, e_bw, e_rw, e_ga, e_gb);
-#ifdef GPTRS_CHAIN_STAMPS
-            if (blockIdx.x == 0 && lane == 0) g_chain_stage_phase = ph;
-            GPTRS_STAMP(3);
-#endif
             stage_block(P, xs, sh.ssq);
-            GPTRS_STAMP(2);
             if (has_epi) {
                 epi_store(lane * 2, e_bw, e_rw, e_ga, e_gb);
                 for (int i = lane * 2 + 128; i < ncols; i += 128) {
@@ -742,13 +784,13 @@ __device__ void control_wave(Shared& sh, unsigned* xs, int nphases, unsigned* ba
                     epi_store(i, e_bw, e_rw, e_ga, e_gb);
                 }
             }
-            char* out = (char*)uni_ptr(P.y);
+            char* out = (char*)P.y;
             for (int u = u0; u < u1; ++u, ++ucount) {
                 const int slot = ucount % NSLOT;
-                unsigned spins = 0;
+                Patience pat(8 * budget);
                 while (lds_ld(&sh.red_cnt[slot]) < NWS) {
                     __builtin_amdgcn_s_sleep(1);
-                    if (++spins > (1u << 24)) {
+                    if (pat.spent()) {
                         lds_st(&sh.abort, 1);
                         __hip_atomic_store(as_global(abort_flag), 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                         return;
@@ -791,11 +833,9 @@ __device__ void control_wave(Shared& sh, unsigned* xs, int nphases, unsigned* ba
                 }
             }
         }
-        GPTRS_STAMP(4);
         // this workgroup's outputs have left the CU before it arrives at the barrier
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         asm volatile("" ::: "memory");
-        GPTRS_STAMP(5);
         if (lane == 0) __hip_atomic_fetch_add(as_global(bar) + (blk % NC) * 64, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     // every launch advances each counter by nphases * per: the next launch starts from there
@@ -841,108 +881,147 @@ __device__ __forceinline__ float reduce_unit(const float (&acc)[TP][4], int lane
     return sidx == 0 ? q[0] : (sidx == 1 ? q[1] : q[2]);
 }
 
-// ---------------------------------------------------------------------------- streaming waves
+// ---------------------------------------------------------------------------- compute waves
+// s_waitcnt that waits until at most 3 * steps vector memory operations of the wave are in flight (and for nothing else);
+// the count is an immediate of the instruction
+template <int N> __device__ __forceinline__ void wait_vm_imm() { __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14)); }
+__device__ __forceinline__ void wait_vm_steps(int steps) {   // the last steps of a launch only: the ring runs empty
+    if (steps <= 0) wait_vm_imm<0>();
+    else if (steps == 1) wait_vm_imm<3>();
+    else if (steps == 2) wait_vm_imm<6>();
+    else if (steps == 3) wait_vm_imm<9>();
+    else wait_vm_imm<12>();
+    static_assert(RING_D - 1 <= 4, "cases above");
+}
+
 template <int FMT>
-__device__ void stream_waves(Shared& sh, const unsigned* xs, int nphases) {
+__device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, int nphases, const unsigned char* ring, unsigned long long budget) {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int blk = blockIdx.x;
+    constexpr int kpw = FMT == kChainW16 ? 2 : (FMT == kChainW8 ? 4 : 8);
+    constexpr unsigned STEP = NS * 16;   // bytes of a tile stream per j-step
 
-    // load iterator: the next j-step (TP words per lane) to fetch
-    int l_phase = -1, l_unit = 0, l_unit_end = 0, l_j = 0, l_wpt = 1, l_ntiles = 1;
-    long l_Kw = 0;
-    int l_Kv = 0;   // words of a tile stream that hold weights; the padding behind them (up to a whole step) is never fetched
-    const uint4* l_w = nullptr;
-    bool l_active = true;
-    const GPTRS_GLOBAL u32x4* l_base[TP];
+    // ---- request side: the wave's next j-step to ask for, in the order the steps are consumed.  Everything but r_off is
+    // uniform: a request costs one vector add and clamp, three scalar moves and three loads.
+    int r_phase = -1, r_unit = 0, r_unit_end = 0, r_j = 0, r_wpt = 1, r_ntiles = 1;
+    unsigned r_last = 0;              // byte offset of a tile stream's last weight word
+    unsigned r_tile_bytes = 0;        // bytes of a tile stream
+    unsigned long long r_w = 0, r_base[TP] = {0, 0, 0};   // tile streams of the unit
+    unsigned r_off = 0;               // this lane's byte offset in a tile stream at step r_j
+    const unsigned ring_lds = (unsigned)uni((int)((unsigned)(size_t)(GPTRS_LDS unsigned char*)ring + (unsigned)(wave * 1024)));
+    const unsigned ring_end = ring_lds + RING_D * SLOT_BYTES;
+    unsigned r_dst = ring_lds;        // LDS address of lane 0's word of tile 0 in the next slot to fill
+    int inflight = 0;                 // j-steps requested and not yet read
+    auto r_unit_setup = [&]() {
+        // a group's last tiles may not exist: the last tile is re-read in their place, never stored
 #pragma unroll
-    for (int p = 0; p < TP; ++p) l_base[p] = nullptr;
-    auto l_setbase = [&]() {
-#pragma unroll
-        for (int p = 0; p < TP; ++p) {
-            const int tile = min(l_unit * TP + p, l_ntiles - 1);   // a group's last tiles may not exist: re-read, never stored
-            l_base[p] = (const GPTRS_GLOBAL u32x4*)l_w + (long)tile * l_Kw + t;
-        }
-        l_j = 0;
+        for (int p = 0; p < TP; ++p) r_base[p] = r_w + (unsigned long long)(unsigned)min(r_unit * TP + p, r_ntiles - 1) * r_tile_bytes;
+        r_off = (unsigned)t * 16u;
+        r_j = 0;
     };
-    auto l_seek = [&]() {
-        while (l_active && l_unit >= l_unit_end) {
-            ++l_phase;
-            if (l_phase >= nphases) { l_active = false; break; }
-            const ChainPhase& ph = sh.ph[l_phase];
-            if (uni(ph.kind) != kChainLinear) continue;   // no weights to stream
-            const int upb = uni(ph.upb), units = uni(ph.units);
-            l_unit = blk * upb;
-            l_unit_end = min(l_unit + upb, units);
-            if (l_unit < l_unit_end) {
-                l_wpt = uni(ph.wpt); l_ntiles = uni(ph.ntiles); l_Kw = uni(ph.Kw);
-                constexpr int kpw = FMT == kChainW16 ? 2 : (FMT == kChainW8 ? 4 : 8);
-                l_Kv = (uni(ph.K) + kpw - 1) / kpw;
-                l_w = (const uint4*)uni_ptr(ph.w);
-            }
-        }
-        if (l_active) l_setbase();
-    };
-    auto l_fetch = [&](u32x4 (&dst)[TP]) {   // requires l_active
-        // the activations are zero beyond K, so a lane whose word is padding contributes nothing with any word
-        // (quantised formats only: their words hold 4 or 8 k, so K = 3072 leaves a quarter of a step as padding; bf16
-        // rows of the model shapes fill whole steps and keep the unconditional load)
-        const bool live = FMT == kChainW16 || l_j * NS + t < l_Kv;
-#pragma unroll
-        for (int p = 0; p < TP; ++p) {
-            if (live) dst[p] = l_base[p][(long)l_j * NS];
-            else { dst[p].x = 0u; dst[p].y = 0u; dst[p].z = 0u; dst[p].w = 0u; }
-        }
-        if (++l_j == l_wpt) {
-            ++l_unit;
-            if (l_unit >= l_unit_end) l_seek(); else l_setbase();
+    auto r_seek = [&]() -> bool {   // next linear phase in which this workgroup has units
+        for (;;) {
+            ++r_phase;
+            if (r_phase >= nphases) return false;
+            const GPTRS_CONST ChainPhase* D = table + r_phase;
+            if (uni(D->kind) != kChainLinear) continue;
+            const int upb = uni(D->upb);
+            r_unit = blk * upb;
+            r_unit_end = min(r_unit + upb, uni(D->units));
+            if (r_unit >= r_unit_end) continue;
+            r_wpt = uni(D->wpt);
+            r_ntiles = uni(D->ntiles);
+            r_tile_bytes = (unsigned)uni(D->Kw) * 16u;
+            r_last = (unsigned)((uni(D->K) + kpw - 1) / kpw - 1) * 16u;
+            r_w = (unsigned long long)uni_ptr(D->w);
+            r_unit_setup();
+            return true;
         }
     };
+    bool r_more = r_seek();
+    // asks for one j-step: three loads, always three, so that the count of loads in flight tells which steps have landed.
+    // Lanes whose word is padding behind K re-read the stream's last weight word (the reader zeroes them).
+    auto request = [&]() {
+        const unsigned off = min(r_off, r_last);
+#pragma unroll
+        for (int p = 0; p < TP; ++p)   // M0: LDS address of lane 0's word
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(off), "s"((unsigned long long)uni_ptr((const char*)r_base[p])), "s"((unsigned)uni((int)(r_dst + (unsigned)(p * NS * 16)))) : "memory", "m0");
+        r_off += STEP;
+        r_dst += SLOT_BYTES;
+        if (r_dst == ring_end) r_dst = ring_lds;
+        ++inflight;
+        if (++r_j == r_wpt) {
+            if (++r_unit < r_unit_end) r_unit_setup();
+            else r_more = r_seek();
+        }
+    };
+    for (int i = 0; i < RING_D && r_more; ++i) request();
 
-    // compute iterator
-    int c_phase = -1, c_unit = 0, c_unit_end = 0, c_j = 0, c_wpt = 1, c_sidx = 0, c_G = 0, c_soff = 0, ucount = 0;
+    // ---- read side
+    int c_phase = -1, c_unit = 0, c_unit_end = 0, c_j = 0, c_wpt = 1, c_sidx = 0, c_G = 0, c_soff = 0, c_Kv = 0, ucount = 0;
     constexpr int c_fmt = FMT;
     // advance to this workgroup's next linear unit, taking part in attention phases on the way
     auto c_seek = [&]() -> bool {
         for (;;) {
             ++c_phase;
             if (c_phase >= nphases) return false;
-            const ChainPhase& ph = sh.ph[c_phase];
-            const int units = uni(ph.units);
-            if (uni(ph.kind) != kChainLinear) {
+            const GPTRS_CONST ChainPhase* D = table + c_phase;   // the fields that decide this workgroup's part, before the wait
+            const int units = uni(D->units);
+            if (uni(D->kind) != kChainLinear) {
                 if (blk >= units) continue;
-                if (!run_attn_phase((GPTRS_LDS const ChainPhase*)&sh.ph[c_phase], (GPTRS_LDS float*)xs, (GPTRS_LDS int*)&sh.go, (GPTRS_LDS int*)&sh.abort, c_phase)) return false;
+                if (!run_attn_phase(table + c_phase, (GPTRS_LDS float*)xs, (GPTRS_LDS int*)&sh.go, (GPTRS_LDS int*)&sh.abort, c_phase,
+                                    budget)) return false;
                 continue;
             }
-            const int upb = uni(ph.upb);
+            const int upb = uni(D->upb);
             c_unit = blk * upb;
             c_unit_end = min(c_unit + upb, units);
             if (c_unit >= c_unit_end) continue;
-            c_wpt = uni(ph.wpt);
-            c_G = uni(ph.Kw) >> 4;
+            c_wpt = uni(D->wpt);
+            c_G = uni(D->Kw) >> 4;
+            c_Kv = (uni(D->K) + kpw - 1) / kpw;
             c_sidx = 0;   // int4: entry of the unit's first tile and group in the staged scales ...
-            c_soff = uni(ph.lds_bytes) >> 2;   // ... which sit behind the activations
-            if (!wait_go(&sh.go, &sh.abort, c_phase)) return false;
-            stage_block(ph, const_cast<unsigned*>(xs), sh.ssq);
-            c_j = 0;
+            c_soff = uni(D->lds_bytes) >> 2;   // ... which sit behind the activations
+            PhaseRegs R;
+            regs_from_table(R, D);
+            if (!wait_go(&sh.go, &sh.abort, c_phase, budget)) return false;
+            stage_block(R, const_cast<unsigned*>(xs), sh.ssq);
             return true;
         }
     };
 
-    u32x4 cur[TP], nxt[TP];
-    bool have_nxt = false;
-    l_seek();
-    if (l_active) { l_fetch(nxt); have_nxt = true; }
     float acc[TP][4];
 #pragma unroll
     for (int p = 0; p < TP; ++p)
 #pragma unroll
         for (int c = 0; c < 4; ++c) acc[p][c] = 0.f;
+    int slot = 0;
+    const GPTRS_LDS u32x4* mine = (const GPTRS_LDS u32x4*)ring + t;   // this lane's word of tile 0 in slot 0
 
-    bool alive = c_seek();
-    while (alive && have_nxt) {
+    // A request can hold its wave for a microsecond (the memory pipeline of a CU takes a limited number of requests, and one
+    // beyond that waits for an older one to land), so the request that a read frees is made after the step's arithmetic
+    // and, at the end of a unit, after the partial sums are handed over: nothing the workgroup waits for stands behind it.
+    // phases (rare code: seek, attention, staging) around units around j-steps (the loop that has to be tight)
+    bool alive = true;
+    while (alive && c_seek()) {
+      for (; c_unit < c_unit_end; ++c_unit) {
+        for (c_j = 0; c_j < c_wpt; ++c_j) {
+        const GPTRS_LDS u32x4* wp = mine + slot * (SLOT_BYTES / 16);
+        // the loads of this j-step are the oldest in flight: they have landed once no more than the younger ones remain
+        if (__builtin_expect(inflight == RING_D, 1)) wait_vm_imm<3 * (RING_D - 1)>();
+        else wait_vm_steps(inflight - 1);
+        asm volatile("" ::: "memory");
+        u32x4 cur[TP];
 #pragma unroll
-        for (int p = 0; p < TP; ++p) cur[p] = nxt[p];
-        if (l_active) l_fetch(nxt); else have_nxt = false;
+        for (int p = 0; p < TP; ++p) cur[p] = wp[p * NS];
+        if ((c_j + 1) * NS > c_Kv) {   // the stream's last step: lanes whose words are padding count as zeros
+            if (c_j * NS + t >= c_Kv) {
+#pragma unroll
+                for (int p = 0; p < TP; ++p) { cur[p].x = 0u; cur[p].y = 0u; cur[p].z = 0u; cur[p].w = 0u; }
+            }
+        }
+        --inflight;
+        if (++slot == RING_D) slot = 0;
         // element reads go through scalars: __builtin_bit_cast applied directly to `vec.y` of an
         // ext-vector reads element 0 with this compiler
         if (c_fmt == kChainW16) {
@@ -1002,44 +1081,52 @@ __device__ void stream_waves(Shared& sh, const unsigned* xs, int nphases) {
                 }
             }
         }
-        if (++c_j == c_wpt) {
-            const int slot = ucount % NSLOT;
+        if (c_j + 1 < c_wpt && r_more) request();   // (the unit's last step: after the hand-over below)
+        }   // j-steps
+        {
+            const int hslot = ucount % NSLOT;
             const float v = reduce_unit(acc, lane);
 #pragma unroll
             for (int p = 0; p < TP; ++p)
 #pragma unroll
                 for (int c = 0; c < 4; ++c) acc[p][c] = 0.f;
-            unsigned spins = 0;
+            Patience pat(8 * budget);
             while (uni(lds_ld(&sh.consumed)) < ucount - NSLOT + 1) {
                 __builtin_amdgcn_s_sleep(1);
-                if (uni(lds_ld(&sh.abort)) || ++spins > (1u << 24)) return;
+                if (uni(lds_ld(&sh.abort)) || pat.spent()) { alive = false; break; }
             }
-            if ((lane & 15) < 3) sh.red[slot][wave][3 * (lane >> 4) + (lane & 15)] = v;
+            if (!alive) break;
+            if ((lane & 15) < 3) sh.red[hslot][wave][3 * (lane >> 4) + (lane & 15)] = v;
             GPTRS_LDS_RELEASE();
-            if (lane == 0) __hip_atomic_fetch_add(&sh.red_cnt[slot], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (lane == 0) __hip_atomic_fetch_add(&sh.red_cnt[hslot], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             ++ucount;
-            ++c_unit;
-            if (c_unit >= c_unit_end) alive = c_seek(); else { c_j = 0; c_sidx += TP * c_G; }
+            c_sidx += TP * c_G;
+            if (r_more) request();
         }
+      }   // units
     }
 }
 
 template <int FMT>
-__global__ __launch_bounds__(NT, 1) void chain_kernel(const ChainPhase* __restrict__ phases, int nphases, unsigned* bar, int* abort_flag) {
+__global__ __launch_bounds__(NT, 1) void chain_kernel(const ChainPhase* __restrict__ phases, int nphases, unsigned* bar, int* abort_flag,
+                                                        int xs_bytes, unsigned long long budget, int stall_phase) {
     extern __shared__ __align__(16) unsigned char smem[];
     Shared& sh = *reinterpret_cast<Shared*>(smem);
     unsigned* xs = reinterpret_cast<unsigned*>(smem + sizeof(Shared));
+    unsigned char* ring = smem + sizeof(Shared) + xs_bytes;
+    PhaseTable table = (PhaseTable)phases;
     {
-        const int* src = (const int*)phases;
-        int* dst = (int*)sh.ph;
-        const int nw = nphases * (int)(sizeof(ChainPhase) / 4);
-        for (int i = threadIdx.x; i < nw; i += NT) dst[i] = src[i];
         if (threadIdx.x < NSLOT) sh.red_cnt[threadIdx.x] = 0;
         if (threadIdx.x == 0) { sh.go = -1; sh.consumed = 0; sh.abort = 0; }
         __syncthreads();
     }
-    if (threadIdx.x >= NS) control_wave<FMT>(sh, xs, nphases, bar, abort_flag);
-    else stream_waves<FMT>(sh, xs, nphases);
+    const int wave = threadIdx.x >> 6;
+    if (wave < NWS) {
+        compute_waves<FMT>(sh, xs, table, nphases, ring, budget);
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): no load may land in LDS after the workgroup has gone
+    } else {
+        control_wave<FMT>(sh, xs, phases, nphases, bar, abort_flag, budget, stall_phase);
+    }
 }
 
 // ---------------------------------------------------------------------------- weight layout
@@ -1104,7 +1191,7 @@ __global__ void chain_pack_scales_kernel(const bf16_t* __restrict__ sc, const bf
 }
 
 static int g_grid = 0;
-static size_t g_smem_set[3] = {0, 0, 0};
+static int g_occupancy_ok[3] = {-1, -1, -1};   // per weight format: does a workgroup of the kernel fit a CU with the LDS it asks for
 
 }  // namespace
 
@@ -1215,21 +1302,38 @@ void chain_fill_attn(ChainPhase& partial, ChainPhase& combine, int64_t n_q, int6
     combine.lds_bytes = combine.lds_total = (int)(NW * 64 * sizeof(float4));
 }
 
-bool chain_launch(hipStream_t s, const ChainPhase* dev_table, int nphases, int lds_bytes, unsigned* bar, int* abort_flag, int wfmt) {
+bool chain_launch(hipStream_t s, const ChainPhase* dev_table, int nphases, int lds_bytes, unsigned* bar, int* abort_flag, int wfmt,
+                  int stall_phase) {
     const int grid = chain_grid();
     if (grid <= 0 || nphases <= 0 || nphases > kChainMaxPhases || lds_bytes > kChainMaxXsWords * 4) return false;
     if (wfmt < kChainW16 || wfmt > kChainW4) return false;
     const void* fn = wfmt == kChainW16 ? (const void*)chain_kernel<kChainW16>
                    : wfmt == kChainW8  ? (const void*)chain_kernel<kChainW8> : (const void*)chain_kernel<kChainW4>;
-    const size_t smem = sizeof(Shared) + (size_t)((lds_bytes + 15) / 16 * 16);
-    if (smem > g_smem_set[wfmt]) {
-        const size_t want = sizeof(Shared) + (size_t)kChainMaxXsWords * 4;
-        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)want) != hipSuccess) return false;
-        g_smem_set[wfmt] = want;
+    const int xs_bytes = (lds_bytes + 1023) / 1024 * 1024;
+    const size_t smem = sizeof(Shared) + (size_t)xs_bytes + (size_t)RING_D * SLOT_BYTES;
+    if (smem > (size_t)LDS_BYTES) return false;
+    if (g_occupancy_ok[wfmt] < 0) {
+        // The grid barrier needs every workgroup resident at once: one workgroup per CU, grid <= CUs (chain_grid), and the
+        // kernel with the most LDS it may ask for must fit a CU.  Checked once per weight format.
+        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess) { g_occupancy_ok[wfmt] = 0; return false; }
+        int per_cu = 0;
+        hipError_t e = wfmt == kChainW16 ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, chain_kernel<kChainW16>, NT, LDS_BYTES)
+                     : wfmt == kChainW8  ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, chain_kernel<kChainW8>, NT, LDS_BYTES)
+                                         : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, chain_kernel<kChainW4>, NT, LDS_BYTES);
+        g_occupancy_ok[wfmt] = (e == hipSuccess && per_cu >= 1) ? 1 : 0;
     }
-    if (wfmt == kChainW16) chain_kernel<kChainW16><<<grid, NT, smem, s>>>(dev_table, nphases, bar, abort_flag);
-    else if (wfmt == kChainW8) chain_kernel<kChainW8><<<grid, NT, smem, s>>>(dev_table, nphases, bar, abort_flag);
-    else chain_kernel<kChainW4><<<grid, NT, smem, s>>>(dev_table, nphases, bar, abort_flag);
+    if (!g_occupancy_ok[wfmt]) return false;
+    // wall-clock budget of a grid-barrier wait, in ticks of the 100 MHz counter (GPTRS_HIP_CHAIN_WAIT_MS, default 50 ms;
+    // a stalled test launch gets 2 ms)
+    static const unsigned long long budget = [] {
+        const char* e = getenv("GPTRS_HIP_CHAIN_WAIT_MS");
+        const long ms = e ? atol(e) : 50;
+        return (unsigned long long)std::max<long>(1, std::min<long>(ms, 10000)) * 100000ull;
+    }();
+    const unsigned long long ticks = stall_phase >= 0 ? 200000ull : budget;
+    if (wfmt == kChainW16) chain_kernel<kChainW16><<<grid, NT, smem, s>>>(dev_table, nphases, bar, abort_flag, xs_bytes, ticks, stall_phase);
+    else if (wfmt == kChainW8) chain_kernel<kChainW8><<<grid, NT, smem, s>>>(dev_table, nphases, bar, abort_flag, xs_bytes, ticks, stall_phase);
+    else chain_kernel<kChainW4><<<grid, NT, smem, s>>>(dev_table, nphases, bar, abort_flag, xs_bytes, ticks, stall_phase);
     return true;
 }
 

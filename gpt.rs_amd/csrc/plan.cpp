@@ -918,7 +918,8 @@ static bool run_chain(const Plan& plan, const Step& head, ExecCtx& cx) {
         GPTRS_HIP_CHECK(hipEventCreate(&e1));
         GPTRS_HIP_CHECK(hipEventRecord(e0, cx.stream));
     }
-    if (!k::chain_launch(cx.stream, table, (int)phases.size(), lds_bytes, cx.be->chain_barrier(), cx.be->chain_abort_flag(), wfmt)) {
+    const int stall = cx.be->chain_stall_phase >= 0 ? std::min(cx.be->chain_stall_phase, (int)phases.size() - 1) : -1;
+    if (!k::chain_launch(cx.stream, table, (int)phases.size(), lds_bytes, cx.be->chain_barrier(), cx.be->chain_abort_flag(), wfmt, stall)) {
         if (e0) { (void)hipEventDestroy(e0); (void)hipEventDestroy(e1); }
         cx.chain = false;
         return false;

@@ -195,6 +195,7 @@ class Backend {
     unsigned* skinny_tickets() const { return d_chain_bar_ + k::kChainBarrierBytes / sizeof(unsigned); }
     int* chain_abort_flag() const { return d_err_flag_ + 1; }
     bool opt_chain = true;
+    int chain_stall_phase = -1;   // tests of the give-up path: the next chain launch expects an arrival too many at this phase
     int64_t n_chain_launches = 0, n_chain_phases = 0;
     int64_t n_tiled_built = 0;
     void release_block(void* p, size_t cap) { pool_.release(p, cap); }

@@ -165,15 +165,19 @@ const char* gptrs_hip_last_error(void);
  * to_literal and sample_decode_token synchronise by themselves). */
 int gptrs_hip_synchronize(gptrs_hip_backend* b);
 
-/* Execution options: name in {"fusion", "profile"}; value 0/1.  "fusion" = rewrite matched
- * functional sequences to fused kernels (on by default; off = one generic kernel per
+/* Execution options: name in {"fusion", "profile", "graphs", "chain", "chain_stall_phase"}; value 0/1 unless stated.
+ * "fusion" = rewrite matched functional sequences to fused kernels (on by default; off = one generic kernel per
  * instruction, the reference harness's "optimizer off" leg,
  * crates/gpt-rs-backend-tests/src/torch_parity/harness.rs:494-511).  "profile" = bracket every
  * linear-layer launch with HIP events on the execution stream (the per-op ns/calls counters the
  * reference C backend exports, crates/gpt-rs-backend-c/src/lib.rs:587-671); setting it resets
  * the linear_* counters.  "graphs" (default 1) = replay a cached program that runs again over the
  * same buffer addresses as a recorded HIP graph, one launch per program instead of one per kernel
- * (no counterpart in the reference: its backends launch op by op). */
+ * (no counterpart in the reference: its backends launch op by op).
+ * "chain" (default 1) = run a decode step's linear layers and attention as one persistent launch (no counterpart either).
+ * "chain_stall_phase" (default -1; a test hook) = value >= 1: the next persistent launch expects, at that phase's grid
+ * barrier, one arrival more than its workgroups can deliver, so that its bounded wait gives up: the call that next
+ * synchronises reports an Execution error and the option returns to -1. */
 int gptrs_hip_set_option(gptrs_hip_backend* b, const char* name, int64_t value);
 
 /* Counters since creation (the reference's cache_event / WorkStats fields,

@@ -177,3 +177,31 @@ def test_decode_attention_in_chain(hip, hq, hkv, dh, rope):
             mask[pos] = False
             assert np.array_equal(g[:, mask], w[:, mask]), "cache rows other than the appended one must be untouched"
             assert_close(g[:, pos], w[:, pos], atol=2e-2, rtol=2e-2, what=f"appended row of cache {i} at pos {pos}")
+
+
+def test_grid_barrier_gives_up_and_the_backend_goes_on(hip):
+    """A grid barrier that cannot complete must end in an execution error, not in a hang: the host option
+    "chain_stall_phase" makes every workgroup of the next launch expect one arrival more than the grid can deliver at that
+    phase's barrier, so each control wave runs out of its (wall-clock) budget, raises the abort flag, and every wave leaves
+    the kernel.  The error is reported at the next synchronisation; the launch after it runs the chain again and is right."""
+    from gptrs_amd.backend import BackendError
+    k = 1024
+    x = rnd(60, (1, k))
+    ws = [rnd(61 + i, (k, k), 2.0 / np.sqrt(k)) for i in range(3)]
+
+    def build(fb, a, w0, w1, w2):
+        return a.matmul(w0).matmul(w1).matmul(w2)
+
+    specs = [[1, k]] + [[k, k]] * 3
+    p = prog(build, [("Bf16", d) for d in specs])
+    good = hip_run(hip, p, [x] + ws)[0]
+    hip.set_option("chain_stall_phase", 1)
+    launches = hip.counter("chain_launches")
+    with pytest.raises(BackendError, match="grid barrier timed out"):
+        hip_run(hip, p, [x] + ws)
+    assert hip.counter("chain_launches") == launches + 1, "the stalled program must have taken the chain path"
+    # the stall applies to one launch; the barrier counters were reset with the error
+    before = hip.counter("chain_launches")
+    again = hip_run(hip, p, [x] + ws)[0]
+    assert hip.counter("chain_launches") == before + 1, "the chain must still be in use after a requested stall"
+    assert np.array_equal(np.asarray(again), np.asarray(good))
