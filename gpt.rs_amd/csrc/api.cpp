@@ -56,14 +56,20 @@ Backend::Backend(int dev) : device(dev) {
         fail_exec("no HIP device is visible: the hip backend has no CPU fallback");
     if (dev < 0 || dev >= count) fail_exec("device index out of range");
     GPTRS_HIP_CHECK(hipSetDevice(dev));
-    // Graph replay is off when GPTRS_HIP_GRAPHS=0, and under a rocprofiler-sdk tool (rocprofv3): a
-    // replayed graph of this size under its kernel tracing was answered with "AQL packet is
-    // malformed" and a stalled queue, while the same steps launched one by one trace fine.
+    // Graph replay is off when GPTRS_HIP_GRAPHS=0, and under any tool that sits between the runtime and the queues
+    // (rocprofv3 and its relatives): a replayed graph under rocprofiler-sdk's kernel tracing was answered with "AQL
+    // packet is malformed" and a stalled queue, while the same steps launched one by one trace fine.  The cause is not
+    // established (every recorded node passes check_graph_nodes below), so replay stays off whenever a tool may be loaded.
     {
         const char* g = getenv("GPTRS_HIP_GRAPHS");
-        const char* tool = getenv("ROCP_TOOL_LIBRARIES");
+        bool tool = false;
+        for (const char* name : {"ROCP_TOOL_LIBRARIES", "HSA_TOOLS_LIB", "ROCPROFILER_LIBRARY", "ROCTRACER_DOMAIN", "ROCPROFILER_REGISTER_FORCE_LOAD"}) {
+            const char* v = getenv(name);
+            if (v && v[0]) tool = true;
+        }
         const char* pre = getenv("LD_PRELOAD");
-        if ((g && g[0] == '0') || (tool && tool[0]) || (pre && strstr(pre, "rocprofiler-sdk"))) opt_graphs = false;
+        if (pre && (strstr(pre, "rocprof") || strstr(pre, "roctracer") || strstr(pre, "rocprofiler"))) tool = true;
+        if ((g && g[0] == '0') || tool) opt_graphs = false;
     }
     GPTRS_HIP_CHECK(hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
     GPTRS_HIP_CHECK(hipMalloc((void**)&d_err_flag_, 256));
@@ -481,6 +487,37 @@ Plan::~Plan() {
 // recorded once by stream capture and replayed with one hipGraphLaunch.  An address set is recorded
 // the second time it is seen, after an eager run has built every derived weight copy, so nothing is
 // allocated while recording.  Returns false when the caller must run the steps eagerly.
+// Every node of a recorded graph against what a queue accepts: kernel nodes with a function, non-empty grids and blocks
+// within the device's limits and dynamic LDS within the opt-in maximum; copies and nothing else besides.  A graph that
+// fails is not instantiated (the step runs launch by launch).
+static bool check_graph_nodes(hipGraph_t graph, int device) {
+    size_t n = 0;
+    if (hipGraphGetNodes(graph, nullptr, &n) != hipSuccess) return false;
+    if (n == 0) return true;
+    std::vector<hipGraphNode_t> nodes(n);
+    if (hipGraphGetNodes(graph, nodes.data(), &n) != hipSuccess) return false;
+    int max_threads = 1024, max_lds = 64 * 1024, max_grid_x = INT32_MAX;
+    (void)hipDeviceGetAttribute(&max_threads, hipDeviceAttributeMaxThreadsPerBlock, device);
+    (void)hipDeviceGetAttribute(&max_lds, hipDeviceAttributeSharedMemPerBlockOptin, device);
+    (void)hipDeviceGetAttribute(&max_grid_x, hipDeviceAttributeMaxGridDimX, device);
+    for (size_t i = 0; i < n; ++i) {
+        hipGraphNodeType type;
+        if (hipGraphNodeGetType(nodes[i], &type) != hipSuccess) return false;
+        if (type == hipGraphNodeTypeKernel) {
+            hipKernelNodeParams kp{};
+            if (hipGraphKernelNodeGetParams(nodes[i], &kp) != hipSuccess) return false;
+            const uint64_t threads = (uint64_t)kp.blockDim.x * kp.blockDim.y * kp.blockDim.z;
+            if (!kp.func || threads == 0 || threads > (uint64_t)max_threads) return false;
+            if (kp.gridDim.x == 0 || kp.gridDim.y == 0 || kp.gridDim.z == 0 || kp.gridDim.x > (unsigned)max_grid_x) return false;
+            if ((uint64_t)kp.gridDim.x * kp.blockDim.x > 0xFFFFFFFFull) return false;   // an AQL packet holds the grid in work-items, 32 bits
+            if (kp.sharedMemBytes > (unsigned)max_lds) return false;
+        } else if (type != hipGraphNodeTypeMemcpy && type != hipGraphNodeTypeEmpty) {
+            return false;   // memset nodes in particular: cleared memory goes through fill kernels
+        }
+    }
+    return true;
+}
+
 bool Backend::run_graphed(Plan& plan, ExecCtx& cx, const std::vector<BufferP>& out_bufs) {
     constexpr size_t kMaxGraphs = 8, kSeenRing = 32;
     if (!opt_graphs || opt_profile || chain_stall_phase >= 0 || !plan.cacheable || plan.steps.size() < 4) return false;
@@ -525,6 +562,10 @@ bool Backend::run_graphed(Plan& plan, ExecCtx& cx, const std::vector<BufferP>& o
     }
     capturing = false;
     hipError_t ec = hipStreamEndCapture(stream, &pg.graph);
+    if (err.empty() && ec == hipSuccess && pg.graph && !check_graph_nodes(pg.graph, device)) {
+        err = "a recorded node is outside what a queue accepts";
+        ++n_graphs_refused;
+    }
     if (!err.empty() || ec != hipSuccess || !pg.graph) {
         if (pg.graph) (void)hipGraphDestroy(pg.graph);
         (void)hipGetLastError();
@@ -965,6 +1006,7 @@ int64_t gptrs_hip_counter(const gptrs_hip_backend* b, const char* name) {
     if (!strcmp(name, "last_program_launches")) return i.last_launches;
     if (!strcmp(name, "graph_launches")) return i.n_graph_launches;
     if (!strcmp(name, "graphs_built")) return i.n_graphs_built;
+    if (!strcmp(name, "graphs_refused")) return i.n_graphs_refused;
     if (!strcmp(name, "chain_launches")) return i.n_chain_launches;
     if (!strcmp(name, "chain_phases")) return i.n_chain_phases;
     return -1;

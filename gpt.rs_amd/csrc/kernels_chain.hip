@@ -9,7 +9,7 @@
 //     (global_load_lds_dwordx4: no registers), each wave into a ring of its own (3 KiB per j-step: one 16-byte
 //     word per lane and tile of the unit), in the order they are consumed: phase by phase, unit by unit (TP
 //     tiles of 4 output columns for the whole of K), j-step by j-step.  Weights do not depend on activations,
-//     so a wave's requests run RING_D j-steps ahead of its reads across unit AND phase boundaries: while the
+//     so a wave's requests run four or five j-steps ahead of its reads across unit AND phase boundaries: while the
 //     wave stands at the grid barrier, stages the next input or runs an attention phase, HBM keeps delivering
 //     the next phase's first words.  Loads of a wave return in order, so "j-step g has landed" is a wait on
 //     the count of loads in flight: a ring private to the wave needs no flags and no barrier.  The loop
@@ -64,7 +64,7 @@ constexpr int NC = kChainCounters;
 constexpr int EPI_MAX = 640;     // bias/residual values staged per workgroup and phase: N <= 160 * grid columns
 constexpr int MAXI = 8;          // 8-byte items per thread in the norm staging: K <= 4*MAXI*NT
 constexpr int SLOT_BYTES = TP * NS * 16;     // one j-step of a workgroup: a word per compute lane and tile
-constexpr int RING_D = 4;                    // j-steps a wave's ring holds: its requests run that far ahead of its reads
+constexpr int RING_MIN = 4, RING_MAX = 5;    // j-steps a wave's ring holds (its requests run that far ahead of its reads): 5 where the staged activations leave room
 constexpr int LDS_BYTES = 160 * 1024;        // per workgroup on gfx950
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
@@ -138,7 +138,7 @@ struct Shared {
 // compiler use scalar loads (uniform addresses), which do not queue behind a wave's vector memory traffic.
 #define GPTRS_CONST __attribute__((address_space(4)))
 typedef const GPTRS_CONST ChainPhase* PhaseTable;
-static_assert(sizeof(Shared) + (size_t)kChainMaxXsWords * 4 + (size_t)RING_D * SLOT_BYTES <= (size_t)LDS_BYTES, "the largest launch fits a CU's LDS");
+static_assert(sizeof(Shared) + (size_t)kChainMaxXsWords * 4 + (size_t)RING_MIN * SLOT_BYTES <= (size_t)LDS_BYTES, "the largest launch fits a CU's LDS");
 constexpr int kPhaseDwords = (int)(sizeof(ChainPhase) / 4);
 static_assert(kPhaseDwords <= 64, "one lane of the control wave per dword of a phase descriptor");
 
@@ -598,6 +598,9 @@ __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
         if (d == 0) { cstore4(rec, __float_as_uint(mn)); cstore4(rec + 1, __float_as_uint(Ls)); }
         cstore4(rec + 2 + d, __float_as_uint(O));
     }
+    // every lane's stores (record words, the appended cache row) have left the CU before the control wave, which passes
+    // this barrier last of all it executes here, reports the workgroup's arrival
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     wg_barrier();
     return true;
 }
@@ -656,6 +659,7 @@ __device__ bool attn_combine(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
             }
             cstore4(ctx + (long)hq * dh + 2 * d2, pack_bf16x2(a0 / Lt, a1 / Lt));
         }
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the context words are out before the arrival is reported
         wg_barrier();
     }
     return true;
@@ -885,16 +889,18 @@ __device__ __forceinline__ float reduce_unit(const float (&acc)[TP][4], int lane
 // s_waitcnt that waits until at most 3 * steps vector memory operations of the wave are in flight (and for nothing else);
 // the count is an immediate of the instruction
 template <int N> __device__ __forceinline__ void wait_vm_imm() { __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14)); }
-__device__ __forceinline__ void wait_vm_steps(int steps) {   // the last steps of a launch only: the ring runs empty
-    if (steps <= 0) wait_vm_imm<0>();
-    else if (steps == 1) wait_vm_imm<3>();
-    else if (steps == 2) wait_vm_imm<6>();
-    else if (steps == 3) wait_vm_imm<9>();
-    else wait_vm_imm<12>();
-    static_assert(RING_D - 1 <= 4, "cases above");
+__device__ __forceinline__ void wait_vm_count(int n) {   // steps without loads in flight (padding, tiles that do not exist): rare
+    switch (n) {
+#define GPTRS_VM(k) case k: wait_vm_imm<k>(); break;
+        GPTRS_VM(1) GPTRS_VM(2) GPTRS_VM(3) GPTRS_VM(4) GPTRS_VM(5) GPTRS_VM(6) GPTRS_VM(7) GPTRS_VM(8)
+        GPTRS_VM(9) GPTRS_VM(10) GPTRS_VM(11) GPTRS_VM(12)
+#undef GPTRS_VM
+        default: wait_vm_imm<0>(); break;   // 0, and anything unexpected: wait for everything
+    }
+    static_assert(3 * (RING_MAX - 1) <= 12, "cases above");
 }
 
-template <int FMT>
+template <int FMT, int RING_D>
 __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, int nphases, const unsigned char* ring, unsigned long long budget) {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int blk = blockIdx.x;
@@ -912,8 +918,14 @@ __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, 
     const unsigned ring_end = ring_lds + RING_D * SLOT_BYTES;
     unsigned r_dst = ring_lds;        // LDS address of lane 0's word of tile 0 in the next slot to fill
     int inflight = 0;                 // j-steps requested and not yet read
+    unsigned pend = 0u;               // bits 2i, 2i + 1: loads that the i-th oldest of them carries
+    int loads = 0;                    // loads in flight
+    int r_tiles = TP;                 // tiles of the unit that exist
+    bool r_plain = false;             // the unit has all its tiles and its streams end with a j-step
     auto r_unit_setup = [&]() {
-        // a group's last tiles may not exist: the last tile is re-read in their place, never stored
+        // a phase's last tiles may not exist: nothing is fetched for them
+        r_tiles = min(TP, r_ntiles - r_unit * TP);
+        r_plain = r_tiles == TP && r_last + 16u == (unsigned)r_wpt * STEP;
 #pragma unroll
         for (int p = 0; p < TP; ++p) r_base[p] = r_w + (unsigned long long)(unsigned)min(r_unit * TP + p, r_ntiles - 1) * r_tile_bytes;
         r_off = (unsigned)t * 16u;
@@ -939,13 +951,33 @@ __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, 
         }
     };
     bool r_more = r_seek();
-    // asks for one j-step: three loads, always three, so that the count of loads in flight tells which steps have landed.
-    // Lanes whose word is padding behind K re-read the stream's last weight word (the reader zeroes them).
+    // Asks for one j-step: one load per tile of the unit that exists (three but for a phase's last unit), none when all of
+    // the wave's words of the step are padding behind K (the reader counts such words as zeros, and sums of tiles that do
+    // not exist are never stored); `pend` records how many loads each step in flight carries, two bits per step, oldest
+    // first.  Every load that is issued fetches weights never fetched before, so all of them take the same way through
+    // the memory system and return in the order of issue: a load that re-read words already in a cache was seen to
+    // complete ahead of older ones, which a count of loads in flight cannot express.  Lanes behind K in a partly filled
+    // wave issue nothing.
     auto request = [&]() {
-        const unsigned off = min(r_off, r_last);
+        int cnt = TP;
+        if (__builtin_expect(r_plain, 1)) {   // three tiles, no padding: nothing to decide
 #pragma unroll
-        for (int p = 0; p < TP; ++p)   // M0: LDS address of lane 0's word
-            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(off), "s"((unsigned long long)uni_ptr((const char*)r_base[p])), "s"((unsigned)uni((int)(r_dst + (unsigned)(p * NS * 16)))) : "memory", "m0");
+            for (int p = 0; p < TP; ++p)   // M0: LDS address of lane 0's word
+                asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(r_off), "s"((unsigned long long)uni_ptr((const char*)r_base[p])), "s"((unsigned)uni((int)(r_dst + (unsigned)(p * NS * 16)))) : "memory", "m0");
+        } else {
+            const bool any = (unsigned)((r_j * NS + wave * 64) * 16) <= r_last;   // the wave's first word of the step holds weights
+            cnt = any ? r_tiles : 0;
+            if (any) {
+                if (r_off <= r_last) {
+#pragma unroll
+                    for (int p = 0; p < TP; ++p)
+                        if (p < r_tiles)
+                            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(r_off), "s"((unsigned long long)uni_ptr((const char*)r_base[p])), "s"((unsigned)uni((int)(r_dst + (unsigned)(p * NS * 16)))) : "memory", "m0");
+                }
+            }
+        }
+        pend |= (unsigned)cnt << (2 * inflight);
+        loads += cnt;
         r_off += STEP;
         r_dst += SLOT_BYTES;
         if (r_dst == ring_end) r_dst = ring_lds;
@@ -1008,8 +1040,15 @@ __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, 
         for (c_j = 0; c_j < c_wpt; ++c_j) {
         const GPTRS_LDS u32x4* wp = mine + slot * (SLOT_BYTES / 16);
         // the loads of this j-step are the oldest in flight: they have landed once no more than the younger ones remain
-        if (__builtin_expect(inflight == RING_D, 1)) wait_vm_imm<3 * (RING_D - 1)>();
-        else wait_vm_steps(inflight - 1);
+        {
+            const int oldest = (int)(pend & 3u), younger = loads - oldest;
+            if (oldest) {
+                if (__builtin_expect(younger == 3 * (RING_D - 1), 1)) wait_vm_imm<3 * (RING_D - 1)>();
+                else wait_vm_count(younger);
+            }
+            pend >>= 2;
+            loads = younger;
+        }
         asm volatile("" ::: "memory");
         u32x4 cur[TP];
 #pragma unroll
@@ -1107,7 +1146,7 @@ __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, 
     }
 }
 
-template <int FMT>
+template <int FMT, int RING_D>
 __global__ __launch_bounds__(NT, 1) void chain_kernel(const ChainPhase* __restrict__ phases, int nphases, unsigned* bar, int* abort_flag,
                                                         int xs_bytes, unsigned long long budget, int stall_phase) {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -1122,7 +1161,7 @@ __global__ __launch_bounds__(NT, 1) void chain_kernel(const ChainPhase* __restri
     }
     const int wave = threadIdx.x >> 6;
     if (wave < NWS) {
-        compute_waves<FMT>(sh, xs, table, nphases, ring, budget);
+        compute_waves<FMT, RING_D>(sh, xs, table, nphases, ring, budget);
         __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): no load may land in LDS after the workgroup has gone
     } else {
         control_wave<FMT>(sh, xs, phases, nphases, bar, abort_flag, budget, stall_phase);
@@ -1191,7 +1230,7 @@ __global__ void chain_pack_scales_kernel(const bf16_t* __restrict__ sc, const bf
 }
 
 static int g_grid = 0;
-static int g_occupancy_ok[3] = {-1, -1, -1};   // per weight format: does a workgroup of the kernel fit a CU with the LDS it asks for
+static int g_occupancy_ok[6] = {-1, -1, -1, -1, -1, -1};   // per kernel: does a workgroup fit a CU with the LDS it asks for
 
 }  // namespace
 
@@ -1307,22 +1346,27 @@ bool chain_launch(hipStream_t s, const ChainPhase* dev_table, int nphases, int l
     const int grid = chain_grid();
     if (grid <= 0 || nphases <= 0 || nphases > kChainMaxPhases || lds_bytes > kChainMaxXsWords * 4) return false;
     if (wfmt < kChainW16 || wfmt > kChainW4) return false;
-    const void* fn = wfmt == kChainW16 ? (const void*)chain_kernel<kChainW16>
-                   : wfmt == kChainW8  ? (const void*)chain_kernel<kChainW8> : (const void*)chain_kernel<kChainW4>;
     const int xs_bytes = (lds_bytes + 1023) / 1024 * 1024;
-    const size_t smem = sizeof(Shared) + (size_t)xs_bytes + (size_t)RING_D * SLOT_BYTES;
+    static const int max_depth = [] { const char* e = getenv("GPTRS_HIP_CHAIN_RING"); return e ? std::max(RING_MIN, std::min(RING_MAX, atoi(e))) : RING_MAX; }();
+    const int depth = sizeof(Shared) + (size_t)xs_bytes + (size_t)max_depth * SLOT_BYTES <= (size_t)LDS_BYTES ? max_depth : RING_MIN;
+    const size_t smem = sizeof(Shared) + (size_t)xs_bytes + (size_t)depth * SLOT_BYTES;
     if (smem > (size_t)LDS_BYTES) return false;
-    if (g_occupancy_ok[wfmt] < 0) {
+    static_assert(RING_MAX == RING_MIN + 1, "two kernels per weight format");
+    const int variant = wfmt * 2 + (depth - RING_MIN);
+    typedef void (*Kernel)(const ChainPhase*, int, unsigned*, int*, int, unsigned long long, int);
+    static const Kernel kernels[6] = {chain_kernel<kChainW16, RING_MIN>, chain_kernel<kChainW16, RING_MAX>, chain_kernel<kChainW8, RING_MIN>,
+                                      chain_kernel<kChainW8, RING_MAX>,  chain_kernel<kChainW4, RING_MIN>,  chain_kernel<kChainW4, RING_MAX>};
+    static_assert(kChainW16 == 0 && kChainW8 == 1 && kChainW4 == 2, "index of a kernel");
+    const Kernel fn = kernels[variant];
+    if (g_occupancy_ok[variant] < 0) {
         // The grid barrier needs every workgroup resident at once: one workgroup per CU, grid <= CUs (chain_grid), and the
-        // kernel with the most LDS it may ask for must fit a CU.  Checked once per weight format.
-        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess) { g_occupancy_ok[wfmt] = 0; return false; }
+        // kernel with the LDS it asks for must fit a CU.  Checked once per kernel.
         int per_cu = 0;
-        hipError_t e = wfmt == kChainW16 ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, chain_kernel<kChainW16>, NT, LDS_BYTES)
-                     : wfmt == kChainW8  ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, chain_kernel<kChainW8>, NT, LDS_BYTES)
-                                         : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, chain_kernel<kChainW4>, NT, LDS_BYTES);
-        g_occupancy_ok[wfmt] = (e == hipSuccess && per_cu >= 1) ? 1 : 0;
+        const bool ok = hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) == hipSuccess &&
+                        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void*)fn, NT, smem) == hipSuccess && per_cu >= 1;
+        g_occupancy_ok[variant] = ok ? 1 : 0;
     }
-    if (!g_occupancy_ok[wfmt]) return false;
+    if (!g_occupancy_ok[variant]) return false;
     // wall-clock budget of a grid-barrier wait, in ticks of the 100 MHz counter (GPTRS_HIP_CHAIN_WAIT_MS, default 50 ms;
     // a stalled test launch gets 2 ms)
     static const unsigned long long budget = [] {
@@ -1331,9 +1375,7 @@ bool chain_launch(hipStream_t s, const ChainPhase* dev_table, int nphases, int l
         return (unsigned long long)std::max<long>(1, std::min<long>(ms, 10000)) * 100000ull;
     }();
     const unsigned long long ticks = stall_phase >= 0 ? 200000ull : budget;
-    if (wfmt == kChainW16) chain_kernel<kChainW16><<<grid, NT, smem, s>>>(dev_table, nphases, bar, abort_flag, xs_bytes, ticks, stall_phase);
-    else if (wfmt == kChainW8) chain_kernel<kChainW8><<<grid, NT, smem, s>>>(dev_table, nphases, bar, abort_flag, xs_bytes, ticks, stall_phase);
-    else chain_kernel<kChainW4><<<grid, NT, smem, s>>>(dev_table, nphases, bar, abort_flag, xs_bytes, ticks, stall_phase);
+    fn<<<grid, NT, smem, s>>>(dev_table, nphases, bar, abort_flag, xs_bytes, ticks, stall_phase);
     return true;
 }
 

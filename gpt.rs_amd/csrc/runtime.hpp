@@ -207,7 +207,7 @@ class Backend {
     // replay steady-state programs (same plan, same buffer addresses) as captured HIP graphs
     bool opt_graphs = true;
     bool capturing = false;
-    int64_t n_graph_launches = 0, n_graphs_built = 0;
+    int64_t n_graph_launches = 0, n_graphs_built = 0, n_graphs_refused = 0;
     // opt-in timing of the linear-layer launches with HIP events on the execution stream
     bool opt_profile = false;
     std::vector<std::pair<hipEvent_t, hipEvent_t>> prof_events;

@@ -184,7 +184,8 @@ int gptrs_hip_set_option(gptrs_hip_backend* b, const char* name, int64_t value);
  * crates/gpt-rs/src/ops/graph/arena.rs:1201-1243): name in {"kernel_launches",
  * "programs_compiled", "program_cache_hits", "fused_ops", "bytes_allocated",
  * "inplace_updates", "last_program_launches", "derived_weights_built" (column-tiled weight copies
- * made for the decode GEMV), "graph_launches", "graphs_built", and with the "profile" option "linear_time_ns",
+ * made for the decode GEMV), "graph_launches", "graphs_built", "graphs_refused" (recorded graphs with a node outside
+ * what a queue accepts: such a step runs launch by launch), "chain_launches", "chain_phases", and with the "profile" option "linear_time_ns",
  * "linear_calls", "linear_bytes" (these three synchronise)}.  Unknown names return -1. */
 int64_t gptrs_hip_counter(const gptrs_hip_backend* b, const char* name);
 

@@ -205,3 +205,24 @@ def test_grid_barrier_gives_up_and_the_backend_goes_on(hip):
     again = hip_run(hip, p, [x] + ws)[0]
     assert hip.counter("chain_launches") == before + 1, "the chain must still be in use after a requested stall"
     assert np.array_equal(np.asarray(again), np.asarray(good))
+
+
+@pytest.mark.parametrize("k,n", [(2560, 32768), (1536, 32768), (3072, 32776), (200, 4100)])
+def test_padded_steps_and_missing_tiles_are_stable(hip, k, n):
+    """Shapes whose tile streams end inside a j-step (K = 2560, 1536: the last step's upper waves hold nothing but padding;
+    K = 200: a wave that is partly padding) or whose last unit lacks tiles (N = 32776 -> 8194 tiles = 2731 units + 1 tile;
+    N = 4100 -> 1025 tiles), run many times: a wave asks for weights several steps ahead and tells by the count of its loads
+    in flight which step has landed, which holds only while every load it issues returns in order.  (Loads that re-read
+    cached words in place of padding did not, and whole units came out wrong now and then.)"""
+    x, w = rnd(70, (1, k)), rnd(71, (k, n), 2.0 / np.sqrt(k))
+    p = prog(lambda fb, a, b: a.matmul(b), [("Bf16", [1, k]), ("Bf16", [k, n])])
+    hip.set_option("chain", 0)
+    try:
+        plain = np.asarray(hip_run(hip, p, [x, w])[0], np.float32)
+    finally:
+        hip.set_option("chain", 1)
+    before = hip.counter("chain_launches")
+    for rep in range(25):
+        got = np.asarray(hip_run(hip, p, [x, w])[0], np.float32)
+        assert_close(got, plain, atol=2e-5, rtol=ULP, what=f"run {rep} vs per-linear kernel")
+    assert hip.counter("chain_launches") == before + 25
