@@ -191,6 +191,26 @@ BufferP Backend::derived_weights(const BufferP& src, int kind, DType dtype, int6
     return t;
 }
 
+// Frees every derived weight layout (and with them the recorded graphs, which hold their addresses) and returns the
+// cached blocks to the driver.  Layouts are built at first use, per kernel family; a caller that is done with one
+// family (the prefill copies once a server only decodes) gets their memory back here, the layouts still in use are
+// rebuilt by the next call that needs them.
+void Backend::drop_derived_weights() {
+    GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
+    for (auto& kv : plan_lru_) {
+        Plan& p = *kv.second;
+        for (auto& g : p.graphs) {
+            if (g.exec) (void)hipGraphExecDestroy(g.exec);
+            if (g.graph) (void)hipGraphDestroy(g.graph);
+        }
+        p.graphs.clear();
+        p.seen_keys.clear();
+        p.graph_builds = p.graph_hits = 0;
+    }
+    tiled_cache_.clear();
+    pool_.trim();
+}
+
 const k::ChainPhase* Backend::chain_table(const std::vector<k::ChainPhase>& phases) {
     const size_t bytes = phases.size() * sizeof(k::ChainPhase);
     for (auto& t : chain_tables_)
@@ -482,11 +502,6 @@ Plan::~Plan() {
     }
 }
 
-// Steady-state decode runs the same plan over the same addresses every step (weights and KV caches
-// stay put, the pool hands the small per-step buffers back in the same order).  Such a step is
-// recorded once by stream capture and replayed with one hipGraphLaunch.  An address set is recorded
-// the second time it is seen, after an eager run has built every derived weight copy, so nothing is
-// allocated while recording.  Returns false when the caller must run the steps eagerly.
 // Every node of a recorded graph against what a queue accepts: kernel nodes with a function, non-empty grids and blocks
 // within the device's limits and dynamic LDS within the opt-in maximum; copies and nothing else besides.  A graph that
 // fails is not instantiated (the step runs launch by launch).
@@ -518,6 +533,11 @@ static bool check_graph_nodes(hipGraph_t graph, int device) {
     return true;
 }
 
+// Steady-state decode runs the same plan over the same addresses every step (weights and KV caches
+// stay put, the pool hands the small per-step buffers back in the same order).  Such a step is
+// recorded once by stream capture and replayed with one hipGraphLaunch.  An address set is recorded
+// the second time it is seen, after an eager run has built every derived weight copy, so nothing is
+// allocated while recording.  Returns false when the caller must run the steps eagerly.
 bool Backend::run_graphed(Plan& plan, ExecCtx& cx, const std::vector<BufferP>& out_bufs) {
     constexpr size_t kMaxGraphs = 8, kSeenRing = 32;
     if (!opt_graphs || opt_profile || chain_stall_phase >= 0 || !plan.cacheable || plan.steps.size() < 4) return false;
@@ -980,6 +1000,7 @@ int gptrs_hip_set_option(gptrs_hip_backend* b, const char* name, int64_t value) 
         else if (!strcmp(name, "chain")) b->impl.opt_chain = value != 0;
         else if (!strcmp(name, "chain_stall_phase")) b->impl.chain_stall_phase = value < 0 ? -1 : (int)std::min<int64_t>(value, 1 << 20);
         else if (!strcmp(name, "profile")) { b->impl.profile_reset(); b->impl.opt_profile = value != 0; }
+        else if (!strcmp(name, "drop_derived_weights")) { if (value) b->impl.drop_derived_weights(); }
         else gptrs::fail_spec(std::string("unknown option `") + name + "`");
     });
 }

@@ -188,6 +188,7 @@ class Backend {
     // codes for the MFMA GEMM, which applies the scales itself; kind 8: 16-column tiled k-grouped copy for batched decode
     // (kernels_skinny.hip); kind 9 / 10: int8 / int4 codes in that tile order.
     BufferP derived_weights(const BufferP& src, int kind, DType dtype, int64_t k, int64_t n, const BufferP& src2 = nullptr);
+    void drop_derived_weights();
     // Device copy of a chain's phase table, cached by content (steady-state decode repeats a few tables).
     const k::ChainPhase* chain_table(const std::vector<k::ChainPhase>& phases);
     unsigned* chain_barrier() const { return d_chain_bar_; }

@@ -165,7 +165,7 @@ const char* gptrs_hip_last_error(void);
  * to_literal and sample_decode_token synchronise by themselves). */
 int gptrs_hip_synchronize(gptrs_hip_backend* b);
 
-/* Execution options: name in {"fusion", "profile", "graphs", "chain", "chain_stall_phase"}; value 0/1 unless stated.
+/* Execution options: name in {"fusion", "profile", "graphs", "chain", "chain_stall_phase", "drop_derived_weights"}; value 0/1 unless stated.
  * "fusion" = rewrite matched functional sequences to fused kernels (on by default; off = one generic kernel per
  * instruction, the reference harness's "optimizer off" leg,
  * crates/gpt-rs-backend-tests/src/torch_parity/harness.rs:494-511).  "profile" = bracket every
@@ -177,7 +177,11 @@ int gptrs_hip_synchronize(gptrs_hip_backend* b);
  * "chain" (default 1) = run a decode step's linear layers and attention as one persistent launch (no counterpart either).
  * "chain_stall_phase" (default -1; a test hook) = value >= 1: the next persistent launch expects, at that phase's grid
  * barrier, one arrival more than its workgroups can deliver, so that its bounded wait gives up: the call that next
- * synchronises reports an Execution error and the option returns to -1. */
+ * synchronises reports an Execution error and the option returns to -1.
+ * "drop_derived_weights" = 1 (an action, not a state): frees the re-ordered weight copies that the kernels built at
+ * first use (and the recorded graphs that point at them) and returns cached device blocks to the driver; copies still
+ * needed are rebuilt by the next call that uses them.  For a caller that has finished with a kernel family, e.g. the
+ * prefill copies of a server that only decodes from then on ("bytes_allocated" shows the effect). */
 int gptrs_hip_set_option(gptrs_hip_backend* b, const char* name, int64_t value);
 
 /* Counters since creation (the reference's cache_event / WorkStats fields,
