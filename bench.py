@@ -361,6 +361,46 @@ def microbench(args, be):
 README_GPT2_TOKENS_PER_S = 74.71   # reference README.md:18-25: GPT-2 small f32, generate 64 tokens, C backend, 1 thread of a Ryzen 9 9950X3D
 
 
+def chain_floor_record(be, phases: int = 157, reps: int = 20):
+    """What a decode chain of `phases` phases costs when there is next to nothing to stream: a persistent launch over
+    dependent bf16 linears alternating [1, 64] x [64, 3072] (every workgroup takes part: staging, one j-step, epilogue,
+    barrier) and [1, 3072] x [3072, 64] (six workgroups work, all meet at the barrier), 393 KB of weights per phase.  The
+    launch time (HIP events of the library's "profile" option around the launch) over the number of phases is the
+    synchronisation cost per phase that a real chain pays on top of its streaming."""
+    from gptrs_amd.ptir import FunctionBuilder, Program, f32_to_bf16_bits
+
+    def build():
+        fb = FunctionBuilder("main")
+        h = fb.param("Bf16", [1, 64])
+        for i in range(phases):
+            h = h.matmul(fb.param("Bf16", [64, 3072] if i % 2 == 0 else [3072, 64]))
+        fb.set_results([h])
+        return Program(fb)
+
+    prog = build()
+    rng = np.random.default_rng(5)
+    handles = []
+    for spec in prog.param_specs:
+        a = (rng.standard_normal(spec.dims) * 0.02).astype(np.float32)
+        handles.append(be.materialize(spec, (f32_to_bf16_bits(a)).tobytes()))
+    for _ in range(3):
+        be.run_program(prog, handles, None)
+    be.synchronize()
+    c0, p0 = be.counter("chain_launches"), be.counter("chain_phases")
+    be.set_option("profile", 1)
+    for _ in range(reps):
+        be.run_program(prog, handles, None)
+    t_ns, calls = be.counter("linear_time_ns"), be.counter("linear_calls")
+    be.set_option("profile", 0)
+    chains, ph = be.counter("chain_launches") - c0, be.counter("chain_phases") - p0
+    if chains != reps or calls != reps or ph != reps * phases:
+        return {"error": "the probe program did not run as one chain launch per call", "chains": chains, "calls": calls, "phases": ph}
+    us = t_ns / calls / 1e3
+    return {"phases": phases, "us_per_launch": round(us, 1), "us_per_phase": round(us / phases, 2),
+            "what": "persistent launch over %d dependent bf16 linears with 393 KB of weights each (alternating 64 -> 3072 and 3072 -> 64): "
+                    "grid barrier, staging, one or three j-steps, epilogue and store acknowledgement per phase, nothing to stream" % phases}
+
+
 def gpt2_record(be, steps: int, warmup: int, cpu=None):
     """BASELINE configs[0]: GPT-2 small f32, weights N(0, 0.02) from seed 0, prompt of 16 ids (seed 1), greedy, 64 tokens
     with KV cache (capacity 128).  Timed like the reference's published figure (README.md:27-50,
@@ -507,6 +547,7 @@ def main():
                     help="f32 (default): bf16 weights and matmul operands with an f32 residual stream, f32 norms and f32 logits "
                          "(DotGeneral out_dtype); bf16: every tensor of the program is bf16")
     ap.add_argument("--no-gpt2", action="store_true", help="skip the GPT-2 small f32 sub-record of the default run")
+    ap.add_argument("--no-floor", action="store_true", help="skip the chain_floor sub-record (a chain with nothing to stream) of the default run")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain elementwise kernel of known traffic (x + 0 over 2^28 f32: 1 GiB read, 1 GiB written, "
                          "kernel binary_scalar_kernel) so FETCH_SIZE / WRITE_SIZE can be scaled to bytes")
@@ -639,6 +680,7 @@ def main():
                "what": "wall time of one 1024-token prefill call (median of three; head on the last row), all launches included"}
     bytes_allocated = be.counter("bytes_allocated")
     gpt2 = None
+    floor = chain_floor_record(be) if args.quant == "none" and not args.no_floor else None
     if not args.no_gpt2:
         del gen, model
         gpt2 = gpt2_record(be, 8, 2, cpu_gpt2)
@@ -659,6 +701,7 @@ def main():
         "roofline": roof,
         "cpu_baseline": cpu_main,
         "prefill": prefill,
+        "chain_floor": floor,
         "gpt2_f32": gpt2,
     }
     print(json.dumps(out))

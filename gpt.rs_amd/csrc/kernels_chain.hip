@@ -122,7 +122,7 @@ template <typename P> __device__ __forceinline__ void lds_st(P p, int v) { __hip
 #define GPTRS_LDS_RELEASE() __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local")
 #define GPTRS_LDS_ACQUIRE() __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local")
 
-struct Shared {
+struct alignas(16) Shared {
     float red[NSLOT][NWS][16];
     float epi_bias[EPI_MAX];
     float epi_res[EPI_MAX];
@@ -814,24 +814,44 @@ __device__ void control_wave(Shared& sh, unsigned* xs, const ChainPhase* phases,
                 const int tile = u * TP + lane;
                 if (lane < TP && tile < ntiles) {
                     const int e = min(((u - u0) * TP + lane) * cpt, EPI_MAX - 4);
+                    // the staged values of the tile's columns in one round of LDS reads, and only those the phase has
+                    float sc[4] = {1.f, 1.f, 1.f, 1.f}, bi[4] = {0.f, 0.f, 0.f, 0.f}, re[4] = {0.f, 0.f, 0.f, 0.f};
                     if (wfmt == kChainW8) {
-                        if (dual) { s[0] *= sh.epi_s[e]; s[1] *= sh.epi_s[EPI_MAX + e]; s[2] *= sh.epi_s[e + 1]; s[3] *= sh.epi_s[EPI_MAX + e + 1]; }
-                        else { s[0] *= sh.epi_s[e]; s[1] *= sh.epi_s[e + 1]; s[2] *= sh.epi_s[e + 2]; s[3] *= sh.epi_s[e + 3]; }
+                        if (dual) {
+                            const float2 a = *reinterpret_cast<const float2*>(&sh.epi_s[e]), b = *reinterpret_cast<const float2*>(&sh.epi_s[EPI_MAX + e]);
+                            sc[0] = a.x; sc[1] = b.x; sc[2] = a.y; sc[3] = b.y;
+                        } else {
+                            const float4 a = *reinterpret_cast<const float4*>(&sh.epi_s[e]);
+                            sc[0] = a.x; sc[1] = a.y; sc[2] = a.z; sc[3] = a.w;
+                        }
+                    }
+                    if (flags & (kChainBias | kChainResidual)) {   // both arrays are staged when either is present
+                        if (dual) {
+                            const float2 b = *reinterpret_cast<const float2*>(&sh.epi_bias[e]), r = *reinterpret_cast<const float2*>(&sh.epi_res[e]);
+                            bi[0] = b.x; bi[1] = b.y; re[0] = r.x; re[1] = r.y;
+                        } else {
+                            const float4 b = *reinterpret_cast<const float4*>(&sh.epi_bias[e]), r = *reinterpret_cast<const float4*>(&sh.epi_res[e]);
+                            bi[0] = b.x; bi[1] = b.y; bi[2] = b.z; bi[3] = b.w;
+                            re[0] = r.x; re[1] = r.y; re[2] = r.z; re[3] = r.w;
+                        }
+                    }
+                    if (wfmt == kChainW8) {
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) s[c] *= sc[c];
                     }
                     if (dual) {   // columns interleaved (gate, up, gate, up): activation.rs:141-162
-                        const float a0 = finish((s[0] / (1.0f + expf(s[0] * -1.0f))) * s[1], flags, sh.epi_bias[e], sh.epi_res[e]);
-                        const float a1 = finish((s[2] / (1.0f + expf(s[2] * -1.0f))) * s[3], flags, sh.epi_bias[e + 1], sh.epi_res[e + 1]);
-                        cstore4(out + 2 * (size_t)(tile * 2), pack_bf16x2(a0, a1));
+                        const float a0 = finish((s[0] / (1.0f + expf(s[0] * -1.0f))) * s[1], flags, bi[0], re[0]);
+                        const float a1 = finish((s[2] / (1.0f + expf(s[2] * -1.0f))) * s[3], flags, bi[1], re[1]);
+                        cstore4(out + 2 * (size_t)(tile * 2), pack_hw(a0, a1));
                     } else {
                         float o[4];
 #pragma unroll
-                        for (int c = 0; c < 4; ++c) o[c] = finish(s[c], flags, sh.epi_bias[e + c], sh.epi_res[e + c]);
+                        for (int c = 0; c < 4; ++c) o[c] = finish(s[c], flags, bi[c], re[c]);
                         if (out_f32) {
                             cstore8(out + 4 * (size_t)(tile * 4), (unsigned long long)__float_as_uint(o[0]) | ((unsigned long long)__float_as_uint(o[1]) << 32));
                             cstore8(out + 4 * (size_t)(tile * 4) + 8, (unsigned long long)__float_as_uint(o[2]) | ((unsigned long long)__float_as_uint(o[3]) << 32));
                         } else {
-                            cstore8(out + 2 * (size_t)(tile * 4),
-                                    (unsigned long long)pack_bf16x2(o[0], o[1]) | ((unsigned long long)pack_bf16x2(o[2], o[3]) << 32));
+                            cstore8(out + 2 * (size_t)(tile * 4), (unsigned long long)pack_hw(o[0], o[1]) | ((unsigned long long)pack_hw(o[2], o[3]) << 32));
                         }
                     }
                 }
@@ -991,6 +1011,7 @@ __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, 
 
     // ---- read side
     int c_phase = -1, c_unit = 0, c_unit_end = 0, c_j = 0, c_wpt = 1, c_sidx = 0, c_G = 0, c_soff = 0, c_Kv = 0, ucount = 0;
+    int c_consumed = 0;   // units the control wave has taken, as last read
     constexpr int c_fmt = FMT;
     // advance to this workgroup's next linear unit, taking part in attention phases on the way
     auto c_seek = [&]() -> bool {
@@ -1129,12 +1150,16 @@ __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, 
             for (int p = 0; p < TP; ++p)
 #pragma unroll
                 for (int c = 0; c < 4; ++c) acc[p][c] = 0.f;
-            Patience pat(8 * budget);
-            while (uni(lds_ld(&sh.consumed)) < ucount - NSLOT + 1) {
-                __builtin_amdgcn_s_sleep(1);
-                if (uni(lds_ld(&sh.abort)) || pat.spent()) { alive = false; break; }
+            // the hand-over slot is free once the control wave has taken the unit that used it last; its count only
+            // grows, so the LDS read is skipped while the last value seen says enough
+            if (c_consumed < ucount - NSLOT + 1) {
+                Patience pat(8 * budget);
+                while ((c_consumed = uni(lds_ld(&sh.consumed))) < ucount - NSLOT + 1) {
+                    __builtin_amdgcn_s_sleep(1);
+                    if (uni(lds_ld(&sh.abort)) || pat.spent()) { alive = false; break; }
+                }
+                if (!alive) break;
             }
-            if (!alive) break;
             if ((lane & 15) < 3) sh.red[hslot][wave][3 * (lane >> 4) + (lane & 15)] = v;
             GPTRS_LDS_RELEASE();
             if (lane == 0) __hip_atomic_fetch_add(&sh.red_cnt[hslot], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
