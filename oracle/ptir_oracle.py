@@ -24,9 +24,13 @@ tests/test_oracle.py):
   * bf16 execution: parity unpinned -- the reference executes no bf16
     (crates/gpt-rs-backend-ref-cpu/src/cpu.rs:21-25); semantics defined here as
     "compute each op in f32, round each op OUTPUT to bf16 (RNE)", per
-    docs/backend.md:99,104-115.
-  * gptrs.hip.* custom calls (weight-only int8/int4): parity unpinned -- the reference
-    has no quantization scheme (docs/backend.md:620-632); closed form defined here.
+    docs/backend.md:99,104-115; a DotGeneral whose out_dtype is F32 keeps its f32 sums over
+    bf16 operands (spec.rs:354-361).
+  * gptrs.hip.* custom calls (weight-only int8/int4): parity unpinned BY THE REFERENCE -- it
+    has no quantization scheme (docs/backend.md:620-632); closed form defined here.  The
+    closed form itself is pinned against hand-written vectors (ties of both signs, zero
+    columns and groups, clamping, the k = 127/128 group boundary, nibble order, one expected
+    byte string) and against a pure-Python per-element loop (tests/test_oracle.py).
 """
 from __future__ import annotations
 
