@@ -286,7 +286,7 @@ struct AttnDecodeArgs {
     void* k_caches[16]; void* v_caches[16];
 };
 size_t attn_decode_workspace_bytes(int64_t n_q, int64_t head_dim, int64_t capacity);
-void attn_decode(hipStream_t s, const AttnDecodeArgs& a);
+int attn_decode(hipStream_t s, const AttnDecodeArgs& a);   // returns the number of launches it made
 
 // Prefill causal attention (ops/functional/attention.rs:443-522): packed qkv [T, P] ->
 // ctx [T, n_q*head_dim], and K/V in cache layout [n_kv, T, head_dim].

@@ -1338,8 +1338,7 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
             a.ws = cx.ws + st.scratch_off;
             a.ws_bytes = st.scratch_bytes;
             if (in.rot_half > 0) { a.cos = src_ptr(st, cx, 5); a.sin = src_ptr(st, cx, 6); a.rot_half = in.rot_half; }
-            k::attn_decode(s, a);
-            cx.launches += 2;
+            cx.launches += k::attn_decode(s, a);
             break;
         }
         case OpKind::FAttnPrefill: {
