@@ -673,12 +673,24 @@ void Backend::execute(Plan& plan, gptrs_hip_tensor* const* inputs, const uint8_t
             case Storage::InPlace: break;
         }
     }
-    if (!run_graphed(plan, cx, out_bufs))
-        for (const Step& st : plan.steps) run_step(plan, st, cx);
-    ++plan.runs;
-    {
+    // From here on kernels that update donated inputs in place may be queued: whatever happens next, those handles no
+    // longer hold what the caller gave (an error below leaves them consumed rather than silently changed).
+    auto consume_donated = [&]() {
+        for (size_t ip = 0; ip < n_in; ++ip)
+            if (inplace_ok[ip] && !inputs[ip]->consumed) {
+                inputs[ip]->consumed = true;
+                inputs[ip]->buf->id = next_buffer_id_++;  // contents changed: derived copies are stale
+            }
+    };
+    try {
+        if (!run_graphed(plan, cx, out_bufs))
+            for (const Step& st : plan.steps) run_step(plan, st, cx);
+        ++plan.runs;
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) fail_exec(std::string("kernel launch failed: ") + hipGetErrorString(e));
+    } catch (...) {
+        consume_donated();
+        throw;
     }
     n_launches += cx.launches;
     last_launches = cx.launches;
@@ -690,11 +702,7 @@ void Backend::execute(Plan& plan, gptrs_hip_tensor* const* inputs, const uint8_t
         else t->buf = out_bufs[plan.out_buffer_of_result[i]];
         outputs[i] = t;
     }
-    for (size_t ip = 0; ip < n_in; ++ip)
-        if (inplace_ok[ip]) {
-            inputs[ip]->consumed = true;
-            inputs[ip]->buf->id = next_buffer_id_++;  // contents changed: derived copies are stale
-        }
+    consume_donated();
 }
 
 void Backend::run_program(const char* json, size_t len, uint64_t key, gptrs_hip_tensor* const* inputs,
