@@ -479,11 +479,27 @@ static int64_t mfma_tail_plan(int64_t tiles, int64_t k_tiles, int* splits) {
     *splits = sp;
     return tiles - tail;
 }
+// A launch of few 64 x 64 tiles (under a quarter of the CUs) splits EVERY tile over k between up to 16 workgroups, the
+// same way (partial sums through the workspace, a ticket per tile, the last ticket adds them in split order): twelve
+// tiles with 96 k-tiles each otherwise keep twelve CUs busy for 96 steps while 244 wait.  Returns the split (1: none).
+static int mfma_few_tiles_split(int64_t tiles64, int64_t k_tiles) {
+    static const bool allow = [] { const char* e = getenv("GPTRS_HIP_GEMM_TAILSPLIT"); return !(e && e[0] == '0'); }();
+    if (!allow || tiles64 > 64 || tiles64 > (int64_t)kSkinnyTickets) return 1;
+    int sp = 16;
+    while (sp > 1 && (tiles64 * sp > 256 || k_tiles < 4 * sp)) sp /= 2;
+    return sp;
+}
 size_t mfma_workspace_bytes(int dtype, int64_t m, int64_t k, int64_t n, bool dual, int quant) {
     if (!mfma_gemm_supported(dtype, m, k, n, quant)) return 0;
     const int64_t tiles = cdiv(m, 128) * cdiv(mfma_padded_n(n), dual ? 64 : 128);
+    const int64_t k_tiles = k / (kKb * kpc_of(dtype));
+    if (!dual && cdiv(m, 128) * cdiv(n, 128) < 128) {   // the 64 x 64 kernel runs (see mfma_gemm)
+        const int64_t t64 = cdiv(m, 64) * cdiv(mfma_padded_n(n), 64);
+        const int sp = mfma_few_tiles_split(t64, k_tiles);
+        return sp > 1 ? (size_t)t64 * sp * 64 * 64 * sizeof(float) : 0;
+    }
     int sp = 1;
-    const int64_t full = mfma_tail_plan(tiles, k / (kKb * kpc_of(dtype)), &sp);
+    const int64_t full = mfma_tail_plan(tiles, k_tiles, &sp);
     return sp > 1 ? (size_t)(tiles - full) * sp * 128 * 128 * sizeof(float) : 0;
 }
 
@@ -505,6 +521,10 @@ static void launch_mfma(hipStream_t s, const MfmaLinearArgs& a) {
         int sp = 1;
         const int64_t f = mfma_tail_plan(nt * mt, a.k / (kKb * Mma<T>::KPC), &sp);
         if (sp > 1 && a.part_bytes >= (size_t)(nt * mt - f) * sp * BM * BN * sizeof(float)) { full = f; splits = sp; }
+    }
+    if (KW == 1 && BM == 64 && BN == 64 && !DUAL && a.part && a.tickets) {
+        const int sp = mfma_few_tiles_split(nt * mt, a.k / (kKb * Mma<T>::KPC));
+        if (sp > 1 && a.part_bytes >= (size_t)(nt * mt) * sp * BM * BN * sizeof(float)) { full = 0; splits = sp; }
     }
     const unsigned grid = (unsigned)(cdiv(full, 8) * 8 + (nt * mt - full) * splits);
     kern<<<grid, 256 * KW, lds_bytes, s>>>((const T*)a.x, (const T*)a.wk, (const T*)a.wk2, (const T*)a.bias, (const T*)a.residual, (T*)a.y,

@@ -642,3 +642,29 @@ def test_drop_derived_weights_frees_memory_and_results_stay(hip):
     zm = hip.to_numpy(hip.run_program(pm, [hm, hw])[0])
     assert hip.counter("derived_weights_built") == built + 4
     assert np.array_equal(np.asarray(y1), np.asarray(z1)) and np.array_equal(np.asarray(ym), np.asarray(zm))
+
+
+@pytest.mark.parametrize("dtype", ["F32", "Bf16"])
+@pytest.mark.parametrize("m,k,n", [(64, 3072, 768), (48, 1024, 200), (100, 2048, 64)])
+def test_few_tile_gemm_splits_k_and_is_reproducible(hip, dtype, m, k, n):
+    """A prefill-shaped linear with few 64 x 64 tiles splits every tile over k between workgroups (partial sums through a
+    workspace, a ticket per tile, the last ticket adds them in split order): the result matches the oracle and two runs
+    give the same bits whichever workgroup drew the last ticket."""
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    w = (rng.standard_normal((k, n)) / np.sqrt(k)).astype(np.float32)
+    b = rng.standard_normal((n,)).astype(np.float32)
+    if dtype == "Bf16":
+        x, w, b = (bf16_bits_to_f32(f32_to_bf16_bits(a)) for a in (x, w, b))
+    fb = FunctionBuilder("main")
+    a, c, d = fb.param(dtype, [m, k]), fb.param(dtype, [k, n]), fb.param(dtype, [n])
+    fb.set_results([F.linear(a, c, d)])
+    p = Program(fb)
+    (want,) = oracle_run(p, [x, w, b])
+    (got,) = hip_run(hip, p, [x, w, b])
+    (again,) = hip_run(hip, p, [x, w, b])
+    assert np.array_equal(np.asarray(got), np.asarray(again)), "split-k sums must not depend on the arrival order"
+    if dtype == "F32":
+        assert_close(got, want, atol=2e-4, rtol=1e-4, what="few-tile f32 linear")
+    else:
+        assert_close(got, want, atol=1e-2, rtol=2.0 ** -7, what="few-tile bf16 linear")
