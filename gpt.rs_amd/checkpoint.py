@@ -181,7 +181,8 @@ def _index_bytes(items, data_start: int) -> bytes:
 
 
 def write_checkpoint(path: str, kind: str, config: Mapping[str, Any], tensors: Mapping[str, np.ndarray],
-                     dtypes: Optional[Mapping[str, str]] = None, flags: Optional[Mapping[str, bool]] = None) -> None:
+                     dtypes: Optional[Mapping[str, str]] = None, flags: Optional[Mapping[str, bool]] = None,
+                     runtime: Optional[Mapping[str, Any]] = None) -> None:
     """Write side, as the exporters do (scripts/gptrs_eval/checkpoint.py): tensors sorted by name, stored ids 0,
     compact JSON config.  float32 / int32 arrays store as they are; `dtypes[name] = "Bf16"` stores a float32
     array rounded to bf16 (tag 2), uint16 arrays given as "Bf16" / "F16" store their words."""
@@ -202,7 +203,10 @@ def write_checkpoint(path: str, kind: str, config: Mapping[str, Any], tensors: M
             raise CheckpointError(f"unsupported dtype for {name}: {arr.dtype} as {want}")
         items.append((name, tuple(int(d) for d in arr.shape), tag, 1 if (flags or {}).get(name) else 0, len(data)))
         payloads.append(data)
-    cfg = json.dumps({"kind": str(kind), "config": dict(config)}, separators=(",", ":")).encode("utf-8")
+    doc = {"kind": str(kind), "config": dict(config)}
+    if runtime:   # runtime-only knobs, e.g. {"weight_streaming": {...}} (docs/formats.md:32, model/config.rs:31-40)
+        doc["runtime"] = dict(runtime)
+    cfg = json.dumps(doc, separators=(",", ":")).encode("utf-8")
     index_len = len(_index_bytes(items, 0))
     data_start = len(MAGIC) + 4 + 4 + len(cfg) + 4 + index_len
     with open(path, "wb") as f:

@@ -46,7 +46,9 @@ void DevicePool::trim() {
 }
 
 Buffer::~Buffer() {
-    if (ptr && owner) owner->release_block(ptr, cap);
+    if (!owner) return;
+    if (has_derived) owner->note_dead_source();
+    if (ptr) owner->release_block(ptr, cap);
 }
 
 // ------------------------------------------------------------------------------ backend
@@ -154,7 +156,9 @@ BufferP Backend::derived_weights(const BufferP& src, int kind, DType dtype, int6
         tiled_cache_.erase(it);
     }
     if (capturing) fail_exec("derived weight copy missing while recording a graph");
-    if (tiled_cache_.size() >= 64 && (tiled_cache_.size() & 63) == 0) {  // drop entries whose source died
+    // A weight that was freed (a streamed parameter between two forwards) takes its layouts with it, before the next one
+    // is built: the memory a caller saves by streaming is not spent on copies of weights that are gone.
+    if (dead_sources_.exchange(0, std::memory_order_relaxed) > 0) {
         for (auto e = tiled_cache_.begin(); e != tiled_cache_.end();)
             e = (e->second.src.expired() || (e->first[1] && e->second.src2.expired())) ? tiled_cache_.erase(e) : std::next(e);
     }
@@ -184,7 +188,8 @@ BufferP Backend::derived_weights(const BufferP& src, int kind, DType dtype, int6
     }
     Derived d;
     d.src = src;
-    if (src2) d.src2 = src2;
+    src->has_derived = true;
+    if (src2) { d.src2 = src2; src2->has_derived = true; }
     d.tiled = t;
     tiled_cache_[ckey] = std::move(d);
     ++n_tiled_built;

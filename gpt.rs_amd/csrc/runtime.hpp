@@ -49,6 +49,7 @@ struct Buffer {
     size_t cap = 0;
     Backend* owner = nullptr;
     uint64_t id = 0;  // identity of the CONTENTS: fresh per allocation, bumped when updated in place
+    bool has_derived = false;  // some derived weight layout was built from this buffer
     ~Buffer();
 };
 using BufferP = std::shared_ptr<Buffer>;
@@ -200,6 +201,7 @@ class Backend {
     int64_t n_chain_launches = 0, n_chain_phases = 0;
     int64_t n_tiled_built = 0;
     void release_block(void* p, size_t cap) { pool_.release(p, cap); }
+    void note_dead_source() { dead_sources_.fetch_add(1, std::memory_order_relaxed); }
 
     std::mutex mu;
     hipStream_t stream = nullptr;
@@ -246,6 +248,7 @@ class Backend {
     void* h_pinned_ = nullptr;  // 64 bytes of pinned host memory for readbacks
     struct Derived { std::weak_ptr<Buffer> src, src2; BufferP tiled; };
     std::map<std::array<uint64_t, 3>, Derived> tiled_cache_;
+    std::atomic<int> dead_sources_{0};  // weights with derived layouts that were freed since the last sweep
     unsigned* d_chain_bar_ = nullptr;
     struct ChainTable { std::vector<k::ChainPhase> host; BufferP dev; uint64_t last_use = 0; };
     std::vector<ChainTable> chain_tables_;

@@ -77,8 +77,29 @@ class _ModelBase:
         self.param_specs: Dict[str, TensorSpec] = {}
         self._programs: Dict[tuple, Tuple[Program, dict]] = {}
         self._param_handles: Optional[list] = None
+        self._source = None                 # loader.CheckpointParamSource of a model opened by loader.load_model
+        self._base_ids: Dict[str, int] = {}
+        self._lazy = False                  # weight streaming: parameters are resolved through the source at every run
 
     # -- parameters ------------------------------------------------------------------
+    def param_dtype(self, name: str) -> str:
+        """Storage dtype of the parameter `name`."""
+        return self.dtype
+
+    def bind_param_source(self, source, base_ids: Dict[str, int], specs: Dict[str, TensorSpec], lazy: bool):
+        """runtime/loader.rs:264-297: parameters come from `source` by base id.  Not lazy: each is loaded once and
+        stored in the backend's memo under its stable id; lazy (`runtime.weight_streaming.enabled`): nothing is
+        loaded here, every run asks the memo and then the source (`DeviceTensor::lazy_param`)."""
+        self._source, self._lazy = source, bool(lazy)
+        for name, spec in specs.items():
+            if name not in self.param_specs:
+                self.param_names.append(name)
+            self.param_specs[name] = spec
+            self._base_ids[name] = base_ids[name]
+            if not lazy:
+                self.backend.param_resolver().set(param_id(self.namespace, name), source.load(base_ids[name]))
+        self._param_handles = None
+
     def set_param(self, name: str, array: np.ndarray, dtype: Optional[str] = None):
         """runtime/loader.rs:234-239: materialize once, store under the stable id."""
         dtype = dtype or self.dtype
@@ -152,7 +173,7 @@ class _ModelBase:
                 raise CheckpointError(f"tensor `{name}`: dtype {e.dtype} cannot feed a model parameter")
             self.set_param(name, host, dtype)
 
-    def save_checkpoint(self, path: str, kind: str, config: Dict[str, object]):
+    def save_checkpoint(self, path: str, kind: str, config: Dict[str, object], runtime: Optional[Dict[str, object]] = None):
         """Write the parameters back as a GPTRSCHK v2 file (checkpoint/saver.rs), in their storage dtype."""
         from .checkpoint import write_checkpoint
         tensors, dtypes = {}, {}
@@ -166,10 +187,12 @@ class _ModelBase:
             else:
                 tensors[name] = np.frombuffer(raw, "<u2").reshape(spec.dims)
                 dtypes[name] = "Bf16"
-        write_checkpoint(path, kind, config, tensors, dtypes)
+        write_checkpoint(path, kind, config, tensors, dtypes, runtime=runtime)
 
     def param_handle(self, name: str):
         h = self.backend.param_resolver().get(param_id(self.namespace, name))
+        if h is None and self._source is not None and name in self._base_ids:
+            h = self._source.load(self._base_ids[name])
         if h is None:
             raise KeyError(f"parameter {name} not materialized")
         return h
@@ -185,9 +208,12 @@ class _ModelBase:
         return self.backend.materialize(TensorSpec(self.dtype, dims), None)
 
     def _run(self, program: Program, args: list, donate: Optional[list] = None):
-        if self._param_handles is None:   # Param inputs are fed by stable id (arena.rs:1163-1168)
-            self._param_handles = [self.param_handle(n) for n in self.param_names]
-        params = self._param_handles
+        if self._lazy:                    # streamed weights: resolved anew for every run, kept only by the source's cache
+            params = [self.param_handle(n) for n in self.param_names]
+        else:
+            if self._param_handles is None:   # Param inputs are fed by stable id (arena.rs:1163-1168)
+                self._param_handles = [self.param_handle(n) for n in self.param_names]
+            params = self._param_handles
         don = None
         if donate is not None:
             don = list(donate) + [False] * len(params)
@@ -274,6 +300,12 @@ class Gpt(_ModelBase):
         out.update({"final_ln.gamma": (d,), "final_ln.beta": (d,), "lm_head": (d, c.vocab_size)})
         return out
 
+    @staticmethod
+    def config_from_json(c) -> GptConfig:
+        """GptConfig's serde form (model/gpt.rs)."""
+        return GptConfig(vocab_size=int(c["vocab_size"]), context_length=int(c["context_length"]), embed_dim=int(c["embed_dim"]),
+                         num_layers=int(c["num_layers"]), num_heads=int(c["num_heads"]), mlp_ratio=int(c.get("mlp_ratio", 4)))
+
     @classmethod
     def from_checkpoint(cls, path: str, backend, dtype: str = "F32") -> "Gpt":
         """runtime/loader.rs:19-241 for kind "gpt": config from the file, tensors streamed by name."""
@@ -281,10 +313,7 @@ class Gpt(_ModelBase):
         with Checkpoint(path) as ck:
             if ck.kind != "gpt":
                 raise CheckpointError(f"checkpoint holds a `{ck.kind}` model, not `gpt`")
-            c = ck.config
-            cfg = GptConfig(vocab_size=int(c["vocab_size"]), context_length=int(c["context_length"]), embed_dim=int(c["embed_dim"]),
-                            num_layers=int(c["num_layers"]), num_heads=int(c["num_heads"]), mlp_ratio=int(c.get("mlp_ratio", 4)))
-            m = cls(cfg, backend, dtype)
+            m = cls(cls.config_from_json(ck.config), backend, dtype)
             m._load_tensors(ck, m.expected_params())
         return m
 
@@ -596,6 +625,22 @@ class Ministral(_ModelBase):
         raise ValueError(f"unknown rope scaling kind {js['kind']!r}")
 
     @classmethod
+    def config_from_json(cls, c) -> MinistralConfig:
+        """MinistralConfig's serde form (model/ministral.rs:13-30)."""
+        from .checkpoint import CheckpointError
+        head_dim = int(c["head_dim"]) if c.get("head_dim") else int(c["embed_dim"]) // int(c["num_heads"])
+        if c.get("kv_head_dim") and int(c["kv_head_dim"]) != head_dim:
+            raise CheckpointError("kv_head_dim different from head_dim is not supported")
+        return MinistralConfig(vocab_size=int(c["vocab_size"]), context_length=int(c["context_length"]), embed_dim=int(c["embed_dim"]),
+                               num_layers=int(c["num_layers"]), num_heads=int(c["num_heads"]), num_kv_heads=int(c["num_kv_heads"]),
+                               head_dim=head_dim, ffn_dim=int(c["mlp_hidden_dim"]), rotary_dim=int(c["rotary_dim"]),
+                               rope_theta=float(c["rope_theta"]), eps=float(c["rms_norm_eps"]),
+                               rope_scaling=cls._scaling_from_json(c.get("rope_scaling")))
+
+    def param_dtype(self, name: str) -> str:
+        return self.norm_dtype if name.endswith(".gamma") else self.dtype
+
+    @classmethod
     def from_checkpoint(cls, path: str, backend, dtype: str = "Bf16", quant: Optional[str] = None,
                         residual_dtype: Optional[str] = None) -> "Ministral":
         """runtime/loader.rs:19-241 for kind "ministral" (MinistralConfig, model/ministral.rs:13-30)."""
@@ -603,16 +648,7 @@ class Ministral(_ModelBase):
         with Checkpoint(path) as ck:
             if ck.kind != "ministral":
                 raise CheckpointError(f"checkpoint holds a `{ck.kind}` model, not `ministral`")
-            c = ck.config
-            head_dim = int(c["head_dim"]) if c.get("head_dim") else int(c["embed_dim"]) // int(c["num_heads"])
-            if c.get("kv_head_dim") and int(c["kv_head_dim"]) != head_dim:
-                raise CheckpointError("kv_head_dim different from head_dim is not supported")
-            cfg = MinistralConfig(vocab_size=int(c["vocab_size"]), context_length=int(c["context_length"]), embed_dim=int(c["embed_dim"]),
-                                  num_layers=int(c["num_layers"]), num_heads=int(c["num_heads"]), num_kv_heads=int(c["num_kv_heads"]),
-                                  head_dim=head_dim, ffn_dim=int(c["mlp_hidden_dim"]), rotary_dim=int(c["rotary_dim"]),
-                                  rope_theta=float(c["rope_theta"]), eps=float(c["rms_norm_eps"]),
-                                  rope_scaling=cls._scaling_from_json(c.get("rope_scaling")))
-            m = cls(cfg, backend, dtype, residual_dtype)
+            m = cls(cls.config_from_json(ck.config), backend, dtype, residual_dtype)
             for name, dims in m.expected_params().items():
                 m._load_tensors(ck, {name: dims}, m.norm_dtype if name.endswith(".gamma") else None)
                 if quant and len(dims) == 2 and name != "tok_embeddings.weight":

@@ -143,6 +143,42 @@ def test_model_from_checkpoint_on_device(hip, tmp_path):
     assert len(models.Generator(m_q, PROMPT, kv_cache_capacity=32).generate(4)) == 4
 
 
+def test_streamed_weights_on_device(hip, tmp_path):
+    """runtime/loader.rs:163-236 on the device: a model whose parameters are read out of the checkpoint at every forward
+    (no budget; a budget that holds about half of them; everything prefetched) writes the tokens of the resident model,
+    and a weight that was streamed out takes its derived layouts with it."""
+    from gptrs_amd import loader
+    from gptrs_amd.loader import WeightStreamingConfig as WS
+    ref = models.Ministral.random(MID_MINISTRAL, OracleBackend(), seed=5, dtype="F32", std=0.05)
+    total = sum(int(np.prod(s.dims)) * 4 for s in ref.param_specs.values())
+    want = None
+    for i, ws in enumerate([WS(), WS(enabled=True), WS(enabled=True, device_budget_bytes=total // 2, small_param_persist_threshold=4096),
+                            WS(enabled=True, prefetch_layers=MID_MINISTRAL.num_layers)]):
+        path = str(tmp_path / f"s{i}.gptrs")
+        ref.save_checkpoint(path, "ministral", ref.checkpoint_config(), runtime={"weight_streaming": ws.to_json()} if ws.enabled else None)
+        m = loader.load_model(hip, path, dtype="Bf16")
+        assert m._lazy == ws.enabled
+        built0 = hip.counter("derived_weights_built")
+        gen = models.Generator(m, PROMPT, kv_cache_capacity=32)
+        toks = gen.generate(8)
+        if want is None:
+            want, resident_built = toks, hip.counter("derived_weights_built") - built0
+            assert m._source.loads == len(m.param_names)
+            continue
+        assert toks == want, ws
+        loads, n = m._source.loads, len(m.param_names)
+        if ws.device_budget_bytes is None and ws.prefetch_layers is None:
+            assert loads == 8 * n, "prefill and seven decode steps each load every parameter"
+            assert hip.counter("derived_weights_built") - built0 > 2 * resident_built, "layouts follow the weights"
+        elif ws.device_budget_bytes is not None:
+            assert n < loads < 8 * n
+            assert m._source.cache.cached_bytes <= total // 2
+        else:
+            blocks = sum(1 for x in m.param_names if x.startswith("blocks."))
+            assert loads == blocks + 8 * (n - blocks)
+        del gen, m
+
+
 def test_tiny_gpt_kv_cache_equals_full_context(hip):
     # smoke.rs:43-82: KV-cache greedy decode == full-context greedy decode for 16 steps
     m = models.Gpt.random(TINY_GPT, hip, seed=11, std=0.2)
