@@ -876,13 +876,85 @@ class BatchGenerator:
         return out
 
 
+# ================================================================================ host sampler
+class Sampler:
+    """The reference's host sampler (crates/gpt-rs/src/inference/sampler.rs:7-104): what a generation loop falls back to
+    when the backend answers `Ok(None)` to sample_decode_token, and the only path for top-k (sampler.rs:74-76: a request
+    with top_k is never offered to the backend).
+
+    `sample(row, rng)`: temperature <= 0 -> arg-max (the LAST of equal maxima, as `Iterator::max_by` returns it).  Otherwise
+    logits / temperature in f32; with top_k = k < len every value below the k-th largest becomes -inf (values equal to it
+    stay); softmax with the maximum taken out; a sum that is not finite or not positive falls back to arg-max; the token is
+    drawn from the cumulative f32 weights as `WeightedIndex` does (a uniform draw in [0, total), first cumulative weight
+    above it).  The reference draws from `thread_rng()`, which no one can replay: `rng` is a numpy Generator here, so the
+    distribution is the reference's and the stream is this implementation's own."""
+
+    def __init__(self, temperature: float, top_k: Optional[int] = None):
+        self.temperature = float(temperature)
+        self.top_k = None if top_k is None else max(int(top_k), 1)   # with_top_k: k.max(1)
+
+    @staticmethod
+    def argmax(values: np.ndarray) -> int:
+        v = np.asarray(values, np.float32).reshape(-1)
+        if v.size == 0:
+            return 0
+        return int(v.size - 1 - np.argmax(v[::-1]))
+
+    def adjusted(self, row: np.ndarray) -> np.ndarray:
+        """logits / temperature with everything below the k-th largest value at -inf (sampler.rs:34-50)."""
+        adj = (np.asarray(row, np.float32).reshape(-1) / np.float32(self.temperature)).astype(np.float32)
+        k = self.top_k
+        if k is not None and 0 < k < adj.size:
+            kth = np.partition(adj, adj.size - k)[adj.size - k]
+            adj = np.where(adj < kth, np.float32(-np.inf), adj).astype(np.float32)
+        return adj
+
+    def probabilities(self, row: np.ndarray) -> Optional[np.ndarray]:
+        """The f32 weights the draw is made from; None where the reference falls back to arg-max."""
+        adj = self.adjusted(row)
+        with np.errstate(over="ignore", invalid="ignore"):
+            probs = np.exp(adj - np.max(adj), dtype=np.float32)
+            total = np.cumsum(probs, dtype=np.float32)[-1]   # the f32 running sum, in order, of `iter().sum()`
+        if not np.isfinite(total) or total <= 0.0:
+            return None
+        return (probs * (np.float32(1.0) / total)).astype(np.float32)
+
+    def sample(self, row: np.ndarray, rng: np.random.Generator) -> int:
+        row = np.asarray(row, np.float32).reshape(-1)
+        if row.size == 0:
+            raise ValueError("cannot sample from empty logits")
+        if self.temperature <= 0.0:
+            return self.argmax(row)
+        probs = self.probabilities(row)
+        if probs is None or not np.all(np.isfinite(probs)):
+            return self.argmax(row)
+        cum = np.cumsum(probs, dtype=np.float32)
+        total = cum[-1]
+        if not total > 0.0:
+            return self.argmax(row)
+        x = np.float32(rng.uniform(0.0, float(total)))
+        return int(min(np.searchsorted(cum, x, side="right"), row.size - 1))
+
+    def supports_backend_decode_sampling(self) -> bool:
+        return self.top_k is None
+
+    def decode_sample_request(self, rng: np.random.Generator) -> Optional[dict]:
+        """sampler.rs:78-93: None with top-k; greedy; or the temperature with a uniform draw in [eps, 1 - eps)."""
+        if not self.supports_backend_decode_sampling():
+            return None
+        if self.temperature <= 0.0:
+            return {"temperature": 0.0, "top_k": None, "random_u": None}
+        eps = float(np.finfo(np.float32).eps)
+        return {"temperature": self.temperature, "top_k": None, "random_u": float(np.float32(rng.uniform(eps, 1.0 - eps)))}
+
+
 # ================================================================================ Generator
 class Generator:
     """Generation loop, greedy by default (crates/gpt-rs/src/inference/generate.rs:37-203).
 
     With `device_sampling` the token comes from backend.sample_decode_token (spec.rs:1333-1348)
-    and only 8 bytes cross PCIe per step; otherwise the last logits row is read back and
-    arg-maxed on the host (sampler.rs:96-103).
+    and only 8 bytes cross PCIe per step; otherwise, where the backend declines (`Ok(None)`), and always with `top_k`
+    (sampler.rs:74-76), the last logits row is read back and the host `Sampler` draws the token.
 
     `pipelined` (default: on when the backend offers sample_decode_token_begin / _wait and sampling is on the
     device): a step queues the sampling of token t, then the forward of step t + 1 fed by the device copy of that
@@ -892,9 +964,14 @@ class Generator:
 
     def __init__(self, model, prompt: Sequence[int], kv_cache_capacity: Optional[int] = None,
                  device_sampling: bool = True, temperature: float = 0.0, seed: int = 0,
-                 pipelined: Optional[bool] = None, last_logits_only: bool = True):
+                 pipelined: Optional[bool] = None, last_logits_only: bool = True, top_k: Optional[int] = None):
         if len(prompt) == 0:
             raise ValueError("prompt must be non-empty")
+        self.sampler = Sampler(temperature, top_k)
+        if not self.sampler.supports_backend_decode_sampling():
+            if pipelined:
+                raise ValueError("pipelined generation needs device sampling: top-k is sampled on the host")
+            device_sampling = False
         self.model = model
         self.tokens = list(prompt)
         self.capacity = kv_cache_capacity
@@ -919,17 +996,16 @@ class Generator:
 
     def _sample(self) -> int:
         be = self.model.backend
-        if self.temperature > 0.0:
-            tok = be.sample_decode_token(self.logits, temperature=self.temperature, random_u=self._draw_u())
-            if tok is None:
-                raise RuntimeError("backend declined temperature sampling")
-            return tok
         if self.device_sampling:
-            tok = be.sample_decode_token(self.logits, temperature=0.0)
-            if tok is not None:
-                return tok
-        row = be.to_numpy(self.logits)[-1]
-        return int(np.argmax(row))
+            req = self.sampler.decode_sample_request(self._rng)
+            if req is not None:
+                state = self._rng.bit_generator.state
+                tok = be.sample_decode_token(self.logits, temperature=req["temperature"], random_u=req["random_u"])
+                if tok is not None:
+                    return tok
+                self._rng.bit_generator.state = state   # Ok(None): the host sampler draws instead
+        row = be.to_numpy(self.logits)
+        return self.sampler.sample(row[-1] if row.ndim == 2 else row, self._rng)
 
     def _prefill(self, context):
         if self.last_logits_only:
