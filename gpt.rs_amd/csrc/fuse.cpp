@@ -529,6 +529,13 @@ struct Fuser {
             // mask: BroadcastTo chain down to the Select
             int mv = mk;
             for (int d = 0; d < 3; ++d) { int src; if (bcast(mv, src)) mv = src; else break; }
+            // a growing cache: the rows of the mask plane that belong to the new tokens, Slice([C, 0], [T, L])
+            int64_t mask_row0 = 0;
+            {
+                int msrc;
+                std::vector<int64_t> ms, mz;
+                if (slice(strip(mv), msrc, ms, mz) && ms.size() == 2 && ms[1] == 0 && mz[0] == T && mz[1] == L) { mask_row0 = ms[0]; mv = msrc; }
+            }
             int cl, cr;
             if (!m_mask_select(mv, cl, cr)) continue;
             int qkv, qkv2, qkv3;
@@ -568,8 +575,40 @@ struct Fuser {
                 kill(vout);
                 replace_root(in.out_ids[0], ni);
                 reindex();
+            } else if (L > T) {
+                // attention over a growing cache (attention.rs:359-437): K = Concat_1(cache_k, new K rows), same for V,
+                // causal mask rows C .. C + T - 1 of the [L, L] plane
+                const int64_t C = L - T;
+                if (mask_row0 != C || dh > 256 || hq % hkv) continue;
+                if (!is_iota(cl, 0) || !is_iota(cr, 1)) continue;
+                const Spec* i0 = spec_of(strip(cl));
+                if (!i0 || i0->dims != std::vector<int64_t>{L, L}) continue;
+                const Instr* kc = producer(strip(Ksrc));
+                const Instr* vc = producer(strip(Vsrc));
+                if (!kc || !vc || kc->op != OpKind::Concat || vc->op != OpKind::Concat || kc->axis != 1 || vc->axis != 1) continue;
+                if (kc->operands.size() != 2 || vc->operands.size() != 2) continue;
+                const int cache_k = kc->operands[0].value, cache_v = vc->operands[0].value;
+                if (cache_k < 0 || cache_v < 0 || kc->operands[1].value < 0 || vc->operands[1].value < 0) continue;
+                const Spec* cks = spec_of(cache_k);
+                const Spec* cvs = spec_of(cache_v);
+                if (!cks || !cvs || cks->dims != std::vector<int64_t>{hkv, C, dh} || cvs->dims != cks->dims) continue;
+                if (cks->dtype != out.dtype || cvs->dtype != out.dtype) continue;
+                if (!m_qkv_block(Q, true, qkv, col, width) || col != 0 || width != hq * dh) continue;
+                if (!m_qkv_block(kc->operands[1].value, true, qkv2, col, width) || qkv2 != qkv || col != hq * dh || width != hkv * dh) continue;
+                if (!m_qkv_block(vc->operands[1].value, true, qkv3, col, width) || qkv3 != qkv || col != (hq + hkv) * dh || width != hkv * dh) continue;
+                const Spec* qs = spec_of(qkv);
+                if (!qs || qs->dims != std::vector<int64_t>{T, (hq + 2 * hkv) * dh}) continue;
+                const int kout = kc->out_ids[0], vout = vc->out_ids[0];
+                Instr ni = make(OpKind::FAttnConcat, "fused.attention_concat_cache", {qkv, cache_k, cache_v}, in.out_ids[0], out);
+                ni.out_ids = {in.out_ids[0], kout, vout};
+                ni.out_specs = {out, kc->out_specs[0], vc->out_specs[0]};
+                ni.n_q = hq; ni.n_kv = hkv; ni.head_dim = dh; ni.scale = scale;
+                kill(kout);
+                kill(vout);
+                replace_root(in.out_ids[0], ni);
+                reindex();
             } else {
-                if (L != T || dh > 256) continue;
+                if (L != T || dh > 256 || mask_row0 != 0) continue;
                 if (!is_iota(cl, 0) || !is_iota(cr, 1)) continue;
                 const Spec* i0 = spec_of(strip(cl));
                 if (!i0 || i0->dims != std::vector<int64_t>{T, T}) continue;

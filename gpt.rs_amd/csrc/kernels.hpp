@@ -299,5 +299,17 @@ struct AttnPrefillArgs {
 };
 void attn_prefill(hipStream_t s, const AttnPrefillArgs& a);
 
+// Causal attention over a growing cache (ops/functional/attention.rs:359-437, the `cache = Some` branch): T new rows of
+// packed qkv [T, P] behind caches [n_kv, C, head_dim]: k_all / v_all [n_kv, C + T, head_dim] = the caches with the new
+// rows appended, ctx [T, n_q*head_dim] = row i attends keys 0 .. C + i.  Two launches.
+struct AttnConcatArgs {
+    int dtype;
+    const void* qkv; const void* k_cache; const void* v_cache;
+    void* ctx; void* k_all; void* v_all;
+    int64_t t, cache_len, n_q, n_kv, head_dim;
+    float scale;
+};
+void attn_concat(hipStream_t s, const AttnConcatArgs& a);
+
 }  // namespace k
 }  // namespace gptrs

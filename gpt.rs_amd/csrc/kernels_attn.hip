@@ -1066,5 +1066,97 @@ void attn_prefill(hipStream_t s, const AttnPrefillArgs& a) {
         attn_prefill_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)a.qkv, (bf16_t*)a.ctx, a.t, (int)a.n_q, (int)a.n_kv, (int)a.head_dim, a.scale);
 }
 
+// ------------------------------------------------------------------------------ attention over a growing cache
+// k_all / v_all [n_kv, L, dh], L = C + T: positions < C from the caches, the rest from the K / V blocks of packed qkv
+template <typename T>
+__global__ __launch_bounds__(256) void attn_concat_kv_kernel(const T* __restrict__ qkv, const T* __restrict__ kc, const T* __restrict__ vc,
+                                                             T* __restrict__ k_all, T* __restrict__ v_all, int64_t t, int64_t c,
+                                                             int n_q, int n_kv, int dh) {
+    const int64_t L = c + t, total = (int64_t)n_kv * L * dh;
+    const int64_t P = (int64_t)(n_q + 2 * n_kv) * dh;
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (int64_t)gridDim.x * 256) {
+        const int d = (int)(e % dh);
+        const int64_t pos = (e / dh) % L;
+        const int h = (int)(e / ((int64_t)dh * L));
+        if (pos < c) {
+            const int64_t src = ((int64_t)h * c + pos) * dh + d;
+            k_all[e] = kc[src];
+            v_all[e] = vc[src];
+        } else {
+            const int64_t row = (pos - c) * P + (int64_t)h * dh + d;
+            k_all[e] = qkv[row + (int64_t)n_q * dh];
+            v_all[e] = qkv[row + (int64_t)(n_q + n_kv) * dh];
+        }
+    }
+}
+// grid (ceil(T/4), n_q), 256 threads: one wave per query row, as attn_prefill_kernel, over keys 0 .. C + i of the
+// combined caches
+template <typename T>
+__global__ __launch_bounds__(256) void attn_concat_kernel(const T* __restrict__ qkv, const T* __restrict__ k_all, const T* __restrict__ v_all,
+                                                          T* __restrict__ ctx, int64_t t, int64_t c, int n_q, int n_kv, int dh, float scale) {
+    __shared__ float qsm[4][256];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t i = (int64_t)blockIdx.x * 4 + wave;
+    const int h = blockIdx.y;
+    const int kvh = h / (n_q / n_kv);
+    const int64_t P = (int64_t)(n_q + 2 * n_kv) * dh, L = c + t;
+    const T* kb = k_all + (int64_t)kvh * L * dh;
+    const T* vb = v_all + (int64_t)kvh * L * dh;
+    if (i < t)
+        for (int d = lane; d < dh; d += 64) qsm[wave][d] = ldf(qkv, i * P + (int64_t)h * dh + d);
+    __syncthreads();
+    if (i >= t) return;
+    const int64_t last = c + i;   // the row's own position
+    float m = -INFINITY, l = 0.f;
+    float o[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int64_t j0 = 0; j0 <= last; j0 += 64) {
+        const int64_t j = j0 + lane;
+        float s = -INFINITY;
+        if (j <= last) {
+            const T* kr = kb + j * dh;
+            float acc = 0.f;
+            for (int d = 0; d < dh; ++d) acc += qsm[wave][d] * ldf(kr, d);
+            s = acc * scale;
+        }
+        const float mn = fmaxf(m, wave_max(s));
+        const float corr = expf(m - mn);
+        const float pe = j <= last ? expf(s - mn) : 0.f;
+        l = l * corr + wave_sum(pe);
+#pragma unroll
+        for (int cc = 0; cc < 4; ++cc) o[cc] *= corr;
+        const int cnt = (int)((last - j0 + 1) < 64 ? (last - j0 + 1) : 64);
+        for (int jj = 0; jj < cnt; ++jj) {
+            const float pj = __shfl(pe, jj, 64);
+            const T* vr = vb + (j0 + jj) * dh;
+#pragma unroll
+            for (int cc = 0; cc < 4; ++cc) {
+                const int d = lane + 64 * cc;
+                if (d < dh) o[cc] += pj * ldf(vr, d);
+            }
+        }
+        m = mn;
+    }
+#pragma unroll
+    for (int cc = 0; cc < 4; ++cc) {
+        const int d = lane + 64 * cc;
+        if (d < dh) stf(ctx, i * (int64_t)n_q * dh + (int64_t)h * dh + d, o[cc] / l);
+    }
+}
+template <typename T>
+static void attn_concat_t(hipStream_t s, const AttnConcatArgs& a) {
+    const int64_t total = a.n_kv * (a.cache_len + a.t) * a.head_dim;
+    const unsigned g = (unsigned)std::min<int64_t>(cdiv(total, 256), 4096);
+    attn_concat_kv_kernel<T><<<g, 256, 0, s>>>((const T*)a.qkv, (const T*)a.k_cache, (const T*)a.v_cache, (T*)a.k_all, (T*)a.v_all, a.t,
+                                               a.cache_len, (int)a.n_q, (int)a.n_kv, (int)a.head_dim);
+    dim3 grid((unsigned)cdiv(a.t, 4), (unsigned)a.n_q);
+    attn_concat_kernel<T><<<grid, 256, 0, s>>>((const T*)a.qkv, (const T*)a.k_all, (const T*)a.v_all, (T*)a.ctx, a.t, a.cache_len,
+                                               (int)a.n_q, (int)a.n_kv, (int)a.head_dim, a.scale);
+}
+void attn_concat(hipStream_t s, const AttnConcatArgs& a) {
+    if (a.t <= 0) return;
+    if (a.dtype == 0) attn_concat_t<float>(s, a);
+    else attn_concat_t<bf16_t>(s, a);
+}
+
 }  // namespace k
 }  // namespace gptrs

@@ -1353,6 +1353,23 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
             ++cx.launches;
             break;
         }
+        case OpKind::FAttnConcat: {
+            const Spec& x = in_spec(0);
+            const Spec& ck = in_spec(1);
+            k::AttnConcatArgs a{};
+            a.dtype = (int)out.dtype;
+            a.qkv = src_ptr(st, cx, 0);
+            a.k_cache = src_ptr(st, cx, 1);
+            a.v_cache = src_ptr(st, cx, 2);
+            a.ctx = dst;
+            a.k_all = cx.ptr[st.dst[1]];
+            a.v_all = cx.ptr[st.dst[2]];
+            a.t = x.dims[0]; a.cache_len = ck.dims[1]; a.n_q = in.n_q; a.n_kv = in.n_kv; a.head_dim = in.head_dim;
+            a.scale = in.scale;
+            k::attn_concat(s, a);
+            cx.launches += 2;
+            break;
+        }
         default:
             fail_unimpl(in.op_name, "no kernel bound to this operation");
     }

@@ -70,7 +70,7 @@ enum class OpKind {
     Constant, Unary, Binary, Dot, Reduce, Compare, Select, Cast, StopGradient, Reshape, Transpose,
     BroadcastTo, Slice, Concat, Iota, Take, DynamicSlice, DynamicUpdateSlice, CustomCall,
     // fused forms produced by the executor's pattern pass (never present on the wire)
-    FLayerNorm, FRmsNorm, FSoftmax, FGelu, FSilu, FSwiglu, FLinear, FRope, FAttnDecode, FAttnPrefill,
+    FLayerNorm, FRmsNorm, FSoftmax, FGelu, FSilu, FSwiglu, FLinear, FRope, FAttnDecode, FAttnPrefill, FAttnConcat,
     FEmbed, FQuant,
     Unsupported
 };

@@ -381,7 +381,6 @@ def test_attention_prefill(hip, hq, hkv, dh, seq):
 def test_batched_decode_linear_on_matrix_cores(hip, m, k, n):
     """2..16 bf16 rows (batched decode): the 16x16x32 MFMA kernel over the 16-column tiled weight copy, plain and
     under bias + exact GELU + residual; reference = the f32 oracle on the same bf16-representable inputs."""
-    from gptrs_amd.ptir import f32_to_bf16_bits
     r16 = lambda a: (f32_to_bf16_bits(np.asarray(a, np.float32)).astype(np.uint32) << 16).view(np.float32)  # noqa: E731
     x, w = r16(rng_uniform(50, (m, k))), r16(rng_uniform(51, (k, n)) * (2.0 / np.sqrt(k)))
     b, r = r16(rng_uniform(52, (n,))), r16(rng_uniform(53, (m, n)))
@@ -412,7 +411,6 @@ def test_batched_decode_linear_f32_on_matrix_cores(hip, m, k, n):
 
 @pytest.mark.parametrize("m,k,n", [(8, 3072, 9216), (4, 256, 96), (16, 3072, 9216), (12, 512, 256)])
 def test_batched_decode_norm_swiglu_on_matrix_cores(hip, m, k, n):
-    from gptrs_amd.ptir import f32_to_bf16_bits
     r16 = lambda a: (f32_to_bf16_bits(np.asarray(a, np.float32)).astype(np.uint32) << 16).view(np.float32)  # noqa: E731
     x, g = r16(rng_uniform(54, (m, k)) * 3.0), r16(rng_uniform(55, (k,)) + 1.5)
     wg, wu = r16(rng_uniform(56, (k, n)) * (2.0 / np.sqrt(k))), r16(rng_uniform(57, (k, n)) * (2.0 / np.sqrt(k)))
@@ -433,7 +431,6 @@ def test_temperature_sampling_matches_oracle(hip, dtype):
     oracle restate the same Gumbel-max rule, so they must pick the same token whenever the two best scores are not
     within float noise of each other; the reference's own case (decode_sampling.rs:22-48) must land in range."""
     from parity import TensorSpec, po, to_bytes
-    from gptrs_amd.ptir import f32_to_bf16_bits
     h = hip.materialize(TensorSpec("F32", [1, 4]), np.array([[0.1, 0.2, 0.3, 0.4]], np.float32).tobytes())
     assert 0 <= hip.sample_decode_token(h, temperature=0.8, random_u=0.42) < 4
     assert hip.sample_decode_token(h, temperature=0.8) is None                # no draw supplied: host sampler's job
@@ -461,7 +458,6 @@ def test_attention_prefill_bf16_matrix_cores(hip, hq, hkv, dh, seq):
     """bf16 prefill attention on the MFMA kernel (head_dim 32/64/128; group sizes 1, 2, 4, 8; sequence lengths
     around the 32-row / 32-key tile edges) against the f32 oracle on the same bf16-representable input.  The kernel
     keeps f32 scores and sums and rounds the probabilities to bf16 for the P.V product; the result is stored as bf16."""
-    from gptrs_amd.ptir import f32_to_bf16_bits
     cfg = F.AttentionConfig(hq * dh, hq, hkv, dh)
     P = cfg.total_projection_dim
     qkv = rng_uniform(33, (seq, P))
@@ -473,13 +469,40 @@ def test_attention_prefill_bf16_matrix_cores(hip, hq, hkv, dh, seq):
         assert np.array_equal(np.asarray(got[i], np.float32), want[i])
 
 
-def test_attention_with_concat_cache(hip):
-    cfg = F.AttentionConfig(16, 4, 2, 4)
-    qkv = rng_uniform(27, (3, cfg.total_projection_dim))
-    ck, cv = rng_uniform(28, (2, 4, 4)), rng_uniform(29, (2, 4, 4))
-    p = prog(lambda fb, a, k, v: list(F.attention(cfg, a, (k, v))),
-             [("F32", [3, cfg.total_projection_dim]), ("F32", [2, 4, 4]), ("F32", [2, 4, 4])])
-    check_program(hip, p, [qkv, ck, cv])
+@pytest.mark.parametrize("dtype", ["F32", "Bf16"])
+@pytest.mark.parametrize("hq,hkv,dh,seq,clen", [(4, 2, 4, 3, 4), (3, 3, 2, 4, 1), (4, 4, 8, 1, 9), (4, 1, 4, 5, 70), (8, 2, 16, 33, 100),
+                                                (12, 12, 64, 2, 130), (32, 8, 128, 5, 64)])
+def test_attention_with_concat_cache(hip, dtype, hq, hkv, dh, seq, clen):
+    """attention.rs:359-437 (`cache = Some`): new rows behind a growing cache, in one fused step (two launches: the
+    combined caches, then the attention over them).  Context against the oracle's op-by-op evaluation; the combined caches
+    are copies and must be exact; the fused row i equals what the prefill of all clen + seq rows gives at row clen + i."""
+    cfg = F.AttentionConfig(hq * dh, hq, hkv, dh)
+    P = cfg.total_projection_dim
+    r16 = (lambda a: a) if dtype == "F32" else (lambda a: (f32_to_bf16_bits(np.asarray(a, np.float32)).astype(np.uint32) << 16).view(np.float32))
+    qkv_all = r16(rng_uniform(27, (clen + seq, P)))
+    # the cache holds the K / V rows of the first clen tokens
+    k_full = qkv_all[:, hq * dh:(hq + hkv) * dh].reshape(clen + seq, hkv, dh).transpose(1, 0, 2)
+    v_full = qkv_all[:, (hq + hkv) * dh:].reshape(clen + seq, hkv, dh).transpose(1, 0, 2)
+    ck, cv = np.ascontiguousarray(k_full[:, :clen]), np.ascontiguousarray(v_full[:, :clen])
+    qkv = np.ascontiguousarray(qkv_all[clen:])
+    build = lambda fb, a, k, v: list(F.attention(cfg, a, (k, v)))  # noqa: E731
+    specs = lambda dt: [(dt, [seq, P]), (dt, [hkv, clen, dh]), (dt, [hkv, clen, dh])]  # noqa: E731
+    fused0 = hip.counter("fused_ops")
+    got = hip_run(hip, prog(build, specs(dtype)), [qkv, ck, cv])
+    assert hip.counter("fused_ops") > fused0 and hip.counter("last_program_launches") == 2, "one fused step"
+    want = oracle_run(prog(build, specs("F32")), [qkv, ck, cv])
+    tol = dict() if dtype == "F32" else dict(atol=2e-2, rtol=2e-2)
+    assert_close(got[0], want[0], what="context", **tol)
+    assert np.array_equal(np.asarray(got[1], np.float32), k_full) and np.array_equal(np.asarray(got[2], np.float32), v_full)
+    whole = oracle_run(prog(lambda fb, a: list(F.attention(cfg, a, None)), [("F32", [clen + seq, P])]), [qkv_all])
+    assert_close(got[0], whole[0][clen:], what="rows of the whole prefill", **tol)
+    # fusion off: the same program op by op, same results to the same bar
+    hip.set_option("fusion", 0)
+    try:
+        plain = hip_run(hip, prog(build, specs(dtype)), [qkv, ck, cv])
+    finally:
+        hip.set_option("fusion", 1)
+    assert_close(plain[0], want[0], what="context, op by op", **tol)
 
 
 @pytest.mark.parametrize("dtype", ["F32", "Bf16"])
