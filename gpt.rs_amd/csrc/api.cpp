@@ -89,6 +89,7 @@ Backend::Backend(int dev) : device(dev) {
     {
         const char* c = getenv("GPTRS_HIP_CHAIN");
         if (c && c[0] == '0') opt_chain = false;
+        if (const char* m = getenv("GPTRS_HIP_CHAIN_F32_MIN_KB")) chain_f32_min_bytes = std::max<int64_t>(0, atoll(m)) << 10;
     }
     k::fill_zero(stream, d_err_flag_, 256);
     k::fill_zero(stream, d_counters_, k::kLinearCounters * sizeof(int));
@@ -169,8 +170,8 @@ BufferP Backend::derived_weights(const BufferP& src, int kind, DType dtype, int6
     } else if (kind == 1) {
         t = new_buffer(k::mfma_weight_bytes((int)dtype, k, n));
         k::mfma_pack_weights(stream, (int)dtype, src->ptr, t->ptr, k, n);
-    } else if (kind == 2 || kind == 3 || kind == 4) {   // decode chain: bf16 / int8 codes / int4 codes (src2: SwiGLU partner)
-        const int wfmt = kind - 2;
+    } else if (kind == 2 || kind == 3 || kind == 4 || kind == 11) {   // decode chain: bf16 / int8 codes / int4 codes (src2: SwiGLU partner) / f32
+        const int wfmt = kind == 11 ? k::kChainW32 : kind - 2;
         t = new_buffer(k::chain_weight_bytes(k, n, src2 != nullptr, wfmt));
         k::chain_pack_weights(stream, src->ptr, src2 ? src2->ptr : nullptr, t->ptr, k, n, wfmt);
     } else if (kind == 5) {                             // decode chain: int4 group scales (src2: the partner's)
@@ -552,6 +553,7 @@ bool Backend::run_graphed(Plan& plan, ExecCtx& cx, const std::vector<BufferP>& o
     for (const auto& b : cx.input_bufs) key.push_back((uint64_t)(uintptr_t)b->ptr);
     for (const auto& b : out_bufs) key.push_back((uint64_t)(uintptr_t)b->ptr);
     key.push_back(opt_chain ? 1 : 0);
+    key.push_back((uint64_t)chain_f32_min_bytes);
     for (const Step& st : plan.steps) {
         if (st.tiled_w_input >= 0) key.push_back(cx.input_bufs[st.tiled_w_input]->id);
         if (st.tiled_w2_input >= 0) key.push_back(cx.input_bufs[st.tiled_w2_input]->id);
@@ -1011,6 +1013,7 @@ int gptrs_hip_set_option(gptrs_hip_backend* b, const char* name, int64_t value) 
         if (!strcmp(name, "fusion")) b->impl.opt_fusion = value != 0;
         else if (!strcmp(name, "graphs")) b->impl.opt_graphs = value != 0;
         else if (!strcmp(name, "chain")) b->impl.opt_chain = value != 0;
+        else if (!strcmp(name, "chain_f32_min_kb")) b->impl.chain_f32_min_bytes = std::max<int64_t>(0, value) << 10;
         else if (!strcmp(name, "chain_stall_phase")) b->impl.chain_stall_phase = value < 0 ? -1 : (int)std::min<int64_t>(value, 1 << 20);
         else if (!strcmp(name, "profile")) { b->impl.profile_reset(); b->impl.opt_profile = value != 0; }
         else if (!strcmp(name, "drop_derived_weights")) { if (value) b->impl.drop_derived_weights(); }

@@ -181,8 +181,12 @@ constexpr int kChainMaxXsWords = 12288;   // staged activation words (48 KiB): K
 constexpr size_t kChainBarrierBytes = (kChainCounters * 64 + 64) * sizeof(unsigned);  // zero-initialised once
 // kChainOutF32: y and the residual are f32.  kChainXF32 (with kChainNorm): x and gamma are f32, the normalised row is
 // rounded to bf16 once as it is staged.
-enum : int { kChainNorm = 1, kChainDual = 2, kChainGelu = 4, kChainResidual = 8, kChainBias = 16, kChainOutF32 = 32, kChainXF32 = 64 };
-enum : int { kChainW16 = 0, kChainW8 = 1, kChainW4 = 2 };   // weight format of a linear phase
+// kChainLayerNorm (with kChainNorm, f32 phases only): LayerNorm with gains `gamma` and offsets `beta` instead of RMSNorm.
+enum : int { kChainNorm = 1, kChainDual = 2, kChainGelu = 4, kChainResidual = 8, kChainBias = 16, kChainOutF32 = 32, kChainXF32 = 64,
+             kChainLayerNorm = 128, kChainAttnFinal = 256 };
+// weight format of a linear phase; kChainW32: f32 weights (16-byte word = 4 columns x 1 k) with f32 activations,
+// bias, residual and output (the launch's attention phases then read f32 rows and caches as well)
+enum : int { kChainW16 = 0, kChainW8 = 1, kChainW4 = 2, kChainW32 = 3 };
 enum : int { kChainLinear = 0, kChainAttnPartial = 1, kChainAttnCombine = 2 };
 // One phase of a chain.  Linear: y = act(norm?(x) . W + bias) (+ residual).  Decode attention
 // (attention.rs:657-779, T = 1) takes two phases: "partial" appends this step's K/V row and leaves
@@ -208,12 +212,13 @@ struct ChainPhase {
     int n_q, n_kv, head_dim, capacity, rot_half, nch;
     float scale;
     int pad;
+    const void* beta;                          // LayerNorm offsets (kChainLayerNorm)
 };
 int chain_grid();  // workgroups per launch (one per CU), 0 when no device is current
 bool chain_supported(int dtype, int64_t m, int64_t k, int64_t n, bool dual, bool norm, int wfmt = kChainW16, bool x_f32 = false);
 size_t chain_weight_bytes(int64_t k, int64_t n, bool dual, int wfmt = kChainW16);
 // w2 != nullptr: SwiGLU pair, columns of w (gate) and w2 (up) interleaved.  wfmt 0: w is bf16 [k,n];
-// 1: si8 [k,n]; 2: packed int4, ui8 [k/2,n]
+// 1: si8 [k,n]; 2: packed int4, ui8 [k/2,n]; 3: f32 [k,n] (no pair)
 void chain_pack_weights(hipStream_t s, const void* w, const void* w2, void* out, int64_t k, int64_t n, int wfmt = kChainW16);
 // int4 only: derived scale copy sc[tile][group][4] (bf16) from s [k/128, n] (and the partner's s2)
 size_t chain_scale_bytes(int64_t k, int64_t n, bool dual);
@@ -225,6 +230,9 @@ bool chain_fill_phase(ChainPhase& p, int64_t k, int64_t n, bool dual, int wfmt =
 // two phases (shape fields filled; the caller sets the pointers of both).
 bool chain_attn_supported(int dtype, int64_t t, int64_t n_q, int64_t n_kv, int64_t head_dim, int64_t rot_half);
 size_t chain_attn_part_bytes(int64_t n_q, int64_t n_kv, int64_t head_dim);
+// phases a decode attention takes: 2, or 1 for a cache of at most 128 positions (one chunk per kv head; the "partial"
+// phase then writes the context row itself, kChainAttnFinal, and `combine` is left untouched)
+int chain_attn_phases(int64_t capacity);
 void chain_fill_attn(ChainPhase& partial, ChainPhase& combine, int64_t n_q, int64_t n_kv, int64_t head_dim, int64_t capacity,
                      int64_t rot_half, float scale);
 // bar: kChainBarrierBytes of device memory zeroed once; abort_flag: raised when a barrier wait

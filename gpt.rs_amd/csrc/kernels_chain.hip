@@ -46,6 +46,7 @@
 #include <climits>
 #include <cstddef>
 #include <cstdlib>
+#include <type_traits>
 
 #include "kernels.hpp"
 #include "device_utils.hpp"
@@ -129,7 +130,7 @@ struct alignas(16) Shared {
     // int8: [0, EPI_MAX) scale of each owned output column (gate of a SwiGLU pair), [EPI_MAX, 2 EPI_MAX) the pair's
     // up column.  (int4 group scales are staged behind the activations, see stage_block.)
     float epi_s[2 * EPI_MAX];
-    float ssq[16];
+    float ssq[32];   // per-wave sums of the norm statistics (LayerNorm takes two rounds: [0, 16) and [16, 32))
     int red_cnt[NSLOT];
     int go, consumed, abort, pad;
 };
@@ -155,14 +156,14 @@ __device__ __forceinline__ void wg_barrier() {
 struct PhaseRegs {
     int K, N, Kw, ntiles, upb, units, lds_bytes, flags, wfmt;
     float inv_n, eps;
-    const void *x, *gamma, *bias, *residual, *wscale, *wscale2;
+    const void *x, *gamma, *beta, *bias, *residual, *wscale, *wscale2;
     void* y;
 };
 __device__ __forceinline__ void regs_from_table(PhaseRegs& R, const GPTRS_CONST ChainPhase* D) {
     R.K = uni(D->K); R.N = uni(D->N); R.Kw = uni(D->Kw); R.ntiles = uni(D->ntiles); R.upb = uni(D->upb); R.units = uni(D->units);
     R.lds_bytes = uni(D->lds_bytes); R.flags = uni(D->flags); R.wfmt = uni(D->wfmt);
     R.inv_n = __int_as_float(uni(__float_as_int(D->inv_n))); R.eps = __int_as_float(uni(__float_as_int(D->eps)));
-    R.x = uni_ptr(D->x); R.gamma = uni_ptr(D->gamma); R.bias = uni_ptr(D->bias); R.residual = uni_ptr(D->residual);
+    R.x = uni_ptr(D->x); R.gamma = uni_ptr(D->gamma); R.beta = uni_ptr(D->beta); R.bias = uni_ptr(D->bias); R.residual = uni_ptr(D->residual);
     R.wscale = uni_ptr(D->wscale); R.wscale2 = uni_ptr(D->wscale2); R.y = uni_ptr(D->y);
 }
 #define GPTRS_PD_INT(field) __builtin_amdgcn_readlane(pd, (int)(offsetof(ChainPhase, field) / 4))
@@ -172,7 +173,7 @@ __device__ __forceinline__ void regs_from_lanes(PhaseRegs& R, int pd) {   // pd:
     R.K = GPTRS_PD_INT(K); R.N = GPTRS_PD_INT(N); R.Kw = GPTRS_PD_INT(Kw); R.ntiles = GPTRS_PD_INT(ntiles); R.upb = GPTRS_PD_INT(upb);
     R.units = GPTRS_PD_INT(units); R.lds_bytes = GPTRS_PD_INT(lds_bytes); R.flags = GPTRS_PD_INT(flags); R.wfmt = GPTRS_PD_INT(wfmt);
     R.inv_n = __int_as_float(GPTRS_PD_INT(inv_n)); R.eps = __int_as_float(GPTRS_PD_INT(eps));
-    R.x = GPTRS_PD_PTR(x); R.gamma = GPTRS_PD_PTR(gamma); R.bias = GPTRS_PD_PTR(bias); R.residual = GPTRS_PD_PTR(residual);
+    R.x = GPTRS_PD_PTR(x); R.gamma = GPTRS_PD_PTR(gamma); R.beta = GPTRS_PD_PTR(beta); R.bias = GPTRS_PD_PTR(bias); R.residual = GPTRS_PD_PTR(residual);
     R.wscale = GPTRS_PD_PTR(wscale); R.wscale2 = GPTRS_PD_PTR(wscale2); R.y = const_cast<void*>(GPTRS_PD_PTR(y));
 }
 
@@ -326,6 +327,78 @@ __device__ __forceinline__ void stage_block(const PhaseRegs& P, unsigned* xs, fl
 }
 
 
+// f32 phases (kChainW32): xs[j] = x[j] as f32, zero beyond K; with norm: LayerNorm as the stand-alone kernel computes it,
+// ((x - mean) * inv_std) * gamma + beta with the mean and the variance of the centred row taken in two rounds
+// (normalization.rs:36-120).
+__device__ __forceinline__ void stage_block_f32(const PhaseRegs& P, unsigned* xs, float* ssq) {
+    const int t = local_tid(), lane = t & 63, wave = uni(t >> 6);
+    const int n = P.K / 4;                // 16-byte items holding data (K % 4 == 0)
+    const int npad = P.lds_bytes >> 4;    // items the readers see
+    const char* x = (const char*)P.x;
+    constexpr int MF = MAXI / 2;          // items per thread: K <= 4 * MF * NT
+    const bool norm = P.flags & kChainNorm;
+    uint4 v[MF], gg[MF], bb[MF];
+#pragma unroll
+    for (int u = 0; u < MF; ++u) {
+        const int i = u * NT + t;
+        v[u] = make_uint4(0u, 0u, 0u, 0u);
+        gg[u] = make_uint4(0u, 0u, 0u, 0u);
+        bb[u] = make_uint4(0u, 0u, 0u, 0u);
+        if (u * NT < n && i < n) {
+            const unsigned long long a = cload8(x + 16 * (size_t)i), b = cload8(x + 16 * (size_t)i + 8);
+            v[u] = make_uint4((unsigned)a, (unsigned)(a >> 32), (unsigned)b, (unsigned)(b >> 32));
+            if (norm) {
+                gg[u] = gload4((const char*)P.gamma + 16 * (size_t)i);
+                bb[u] = gload4((const char*)P.beta + 16 * (size_t)i);
+            }
+        }
+    }
+    if (norm) {
+        float s = 0.f;
+#pragma unroll
+        for (int u = 0; u < MF; ++u)
+            if (u * NT < n) { s += __uint_as_float(v[u].x); s += __uint_as_float(v[u].y); s += __uint_as_float(v[u].z); s += __uint_as_float(v[u].w); }
+        const float ws = wave_sum(s);
+        if (lane == 0) ssq[wave] = ws;
+        wg_barrier();
+        float tot = 0.f;
+#pragma unroll
+        for (int w = 0; w < NT / 64; ++w) tot += ssq[w];
+        const float mean = tot * P.inv_n;
+        float c[MF][4];
+        float q = 0.f;
+#pragma unroll
+        for (int u = 0; u < MF; ++u) {
+            const bool in = u * NT < n && u * NT + t < n;
+            c[u][0] = in ? __uint_as_float(v[u].x) - mean : 0.f;
+            c[u][1] = in ? __uint_as_float(v[u].y) - mean : 0.f;
+            c[u][2] = in ? __uint_as_float(v[u].z) - mean : 0.f;
+            c[u][3] = in ? __uint_as_float(v[u].w) - mean : 0.f;
+            q += c[u][0] * c[u][0]; q += c[u][1] * c[u][1]; q += c[u][2] * c[u][2]; q += c[u][3] * c[u][3];
+        }
+        const float wq = wave_sum(q);
+        if (lane == 0) ssq[16 + wave] = wq;
+        wg_barrier();
+        float var = 0.f;
+#pragma unroll
+        for (int w = 0; w < NT / 64; ++w) var += ssq[16 + w];
+        const float inv_std = 1.0f / sqrtf(var * P.inv_n + P.eps);
+#pragma unroll
+        for (int u = 0; u < MF; ++u) {
+            v[u].x = __float_as_uint((c[u][0] * inv_std) * __uint_as_float(gg[u].x) + __uint_as_float(bb[u].x));
+            v[u].y = __float_as_uint((c[u][1] * inv_std) * __uint_as_float(gg[u].y) + __uint_as_float(bb[u].y));
+            v[u].z = __float_as_uint((c[u][2] * inv_std) * __uint_as_float(gg[u].z) + __uint_as_float(bb[u].z));
+            v[u].w = __float_as_uint((c[u][3] * inv_std) * __uint_as_float(gg[u].w) + __uint_as_float(bb[u].w));
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < MF; ++u) {
+        const int i = u * NT + t;
+        if (u * NT < npad && i < npad) *reinterpret_cast<uint4*>(&xs[4 * i]) = i < n ? v[u] : make_uint4(0u, 0u, 0u, 0u);
+    }
+    wg_barrier();
+}
+
 // ---------------------------------------------------------------------------- decode attention
 constexpr int NW = NT / 64;
 
@@ -431,9 +504,13 @@ __device__ __forceinline__ void lane_pair(float v, int off, float& a, float& b) 
 // the waves of different heads re-read the same rows out of the caches.  Cache rows older than
 // this launch are requested BEFORE the grid barrier is awaited (they do not depend on the
 // previous phase); only the query row and this step's K/V row are read after it.
+// F32: the query row, this step's K / V row and the caches are f32 (a lane's 8 values are two 16-byte words; no RoPE).
+template <bool F32>
 __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const ChainPhase& P, GPTRS_LDS float* lds, int unit, int phase,
                              unsigned long long budget) {
-    constexpr int PP = 4;   // positions per lane group requested ahead of the barrier
+    typedef typename std::conditional<F32, float, bf16_t>::type E;
+    constexpr int PP = F32 ? 2 : 4;   // positions per lane group requested ahead of the barrier
+    constexpr int RW = F32 ? 2 : 1;   // 16-byte words of a lane's 8 values
     const int t = local_tid(), lane = t & 63, wave = uni(t >> 6);
     const bool control = wave == NWS;
     const int dh = P.head_dim, n_q = P.n_q, n_kv = P.n_kv, nch = P.nch, half = P.rot_half;
@@ -443,33 +520,59 @@ __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
     const int g = wave % G, part = wave / G;
     const int stride = nparts * rpw, sid = part * rpw + sub;   // position slots of this head's waves
     const int kvh = unit / nch, c = unit - kvh * nch;
-    const bf16_t* qkv = (const bf16_t*)P.x;
-    bf16_t* kc = (bf16_t*)P.k_cache;
-    bf16_t* vc = (bf16_t*)P.v_cache;
-    const bf16_t* cs = (const bf16_t*)P.cos;
-    const bf16_t* sn = (const bf16_t*)P.sin;
+    const E* qkv = (const E*)P.x;
+    E* kc = (E*)P.k_cache;
+    E* vc = (E*)P.v_cache;
+    const bf16_t* cs = F32 ? nullptr : (const bf16_t*)P.cos;
+    const bf16_t* sn = F32 ? nullptr : (const bf16_t*)P.sin;
     const long qpos = clampl(uni(gload(P.query_start)), 0, cap - 1);       // DynamicSlice clamp (cpu.rs:804-820)
     const long upd = clampl(uni(gload(P.update_starts + 1)), 0, cap - 1);  // DynamicUpdateSlice clamp
     const float scale = P.scale;
     const long L = qpos + 1, CL = (L + nch - 1) / nch;
     const long p0 = c * CL, p1 = min(L, p0 + CL);
     const int owner = (int)min(upd / CL, (long)nch - 1);
-    const bf16_t* knew = qkv + (long)n_q * dh + (long)kvh * dh;
-    const bf16_t* vnew = qkv + (long)(n_q + n_kv) * dh + (long)kvh * dh;
+    const E* knew = qkv + (long)n_q * dh + (long)kvh * dh;
+    const E* vnew = qkv + (long)(n_q + n_kv) * dh + (long)kvh * dh;
     const int c0 = li * 8;
-    uint4 kraw[PP], vraw[PP];
+    uint4 kraw[PP][RW], vraw[PP][RW];
 #pragma unroll
     for (int j = 0; j < PP; ++j) {
         const long p = p0 + sid + (long)j * stride;
-        if (!control && p < p1 && p != upd) {
-            const long row = ((long)kvh * cap + p) * dh + c0;
-            kraw[j] = gload4(kc + row);
-            vraw[j] = gload4(vc + row);
-        } else {
-            kraw[j] = make_uint4(0, 0, 0, 0);
-            vraw[j] = make_uint4(0, 0, 0, 0);
+        const bool take = !control && p < p1 && p != upd;
+        const long row = ((long)kvh * cap + p) * dh + c0;
+#pragma unroll
+        for (int r = 0; r < RW; ++r) {
+            kraw[j][r] = take ? gload4(kc + row + 4 * r) : make_uint4(0, 0, 0, 0);
+            vraw[j][r] = take ? gload4(vc + row + 4 * r) : make_uint4(0, 0, 0, 0);
         }
     }
+    // a lane's 8 values of a row: unpacked from bf16 or taken as they are
+    auto row_values = [&](const uint4 (&raw)[RW], float (&f)[8]) {
+        if (F32) {
+            f[0] = __uint_as_float(raw[0].x); f[1] = __uint_as_float(raw[0].y); f[2] = __uint_as_float(raw[0].z); f[3] = __uint_as_float(raw[0].w);
+            f[4] = __uint_as_float(raw[RW - 1].x); f[5] = __uint_as_float(raw[RW - 1].y); f[6] = __uint_as_float(raw[RW - 1].z); f[7] = __uint_as_float(raw[RW - 1].w);
+        } else {
+            unpack_u4(raw[0], f);
+        }
+    };
+    auto load_row = [&](const E* p, float (&f)[8]) {   // plain loads (cache rows older than this launch)
+        uint4 raw[RW];
+#pragma unroll
+        for (int r = 0; r < RW; ++r) raw[r] = gload4(p + 4 * r);
+        row_values(raw, f);
+    };
+    auto cload_row = [&](const E* p, unsigned long long (&w)[2 * RW]) {   // agent-scope loads (rows written by the phase before)
+#pragma unroll
+        for (int r = 0; r < 2 * RW; ++r) w[r] = cload8(p + (F32 ? 2 : 4) * r);
+    };
+    auto words_values = [&](const unsigned long long (&w)[2 * RW], float (&f)[8]) {
+        if (F32) {
+#pragma unroll
+            for (int r = 0; r < 2 * RW; ++r) { f[(2 * r) & 7] = __uint_as_float((unsigned)w[r]); f[(2 * r + 1) & 7] = __uint_as_float((unsigned)(w[r] >> 32)); }
+        } else {
+            unpack8(w[0], w[1], f);
+        }
+    };
     if (!control && !wait_go(go, abort, phase, budget)) return false;
 
     float m = -INFINITY, l = 0.f, o[8];
@@ -484,26 +587,30 @@ __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
         const int j0 = first ? c0 : c0 - half, co = first ? c0 + half : c0 - half;
         float cosv[8], sinv[8];
         if (rot) { load_bf16x8(cs + j0, cosv); load_bf16x8(sn + j0, sinv); }
-        const bf16_t* head = qkv + (long)(kvh * G + g) * dh;
-        unsigned long long qa[2], qb[2] = {0ull, 0ull};
-        qa[0] = cload8(head + c0); qa[1] = cload8(head + c0 + 4);
-        if (rot) { qb[0] = cload8(head + co); qb[1] = cload8(head + co + 4); }
+        const E* head = qkv + (long)(kvh * G + g) * dh;
+        unsigned long long qa[2 * RW], qb[2 * RW];
+#pragma unroll
+        for (int r = 0; r < 2 * RW; ++r) qb[r] = 0ull;
+        cload_row(head + c0, qa);
+        if (rot) cload_row(head + co, qb);
         const bool fresh = c == owner && sid == 0;           // this lane group handles the new row
-        unsigned long long ka[2] = {0ull, 0ull}, kb[2] = {0ull, 0ull}, va[2] = {0ull, 0ull};
+        unsigned long long ka[2 * RW], kb[2 * RW], va[2 * RW];
+#pragma unroll
+        for (int r = 0; r < 2 * RW; ++r) { ka[r] = 0ull; kb[r] = 0ull; va[r] = 0ull; }
         if (fresh) {
-            ka[0] = cload8(knew + c0); ka[1] = cload8(knew + c0 + 4);
-            if (rot) { kb[0] = cload8(knew + co); kb[1] = cload8(knew + co + 4); }
-            va[0] = cload8(vnew + c0); va[1] = cload8(vnew + c0 + 4);
+            cload_row(knew + c0, ka);
+            if (rot) cload_row(knew + co, kb);
+            cload_row(vnew + c0, va);
         }
-        auto rope = [&](const unsigned long long (&own2)[2], const unsigned long long (&oth2)[2], float (&out)[8]) {
+        auto rope = [&](const unsigned long long (&own2)[2 * RW], const unsigned long long (&oth2)[2 * RW], float (&out)[8]) {
             float own[8], other[8];
-            unpack8(own2[0], own2[1], own);
+            words_values(own2, own);
             if (!rot) {
 #pragma unroll
                 for (int v = 0; v < 8; ++v) out[v] = own[v];
                 return;
             }
-            unpack8(oth2[0], oth2[1], other);
+            words_values(oth2, other);
 #pragma unroll
             for (int v = 0; v < 8; ++v)
                 out[v] = rbf(first ? own[v] * cosv[v] - other[v] * sinv[v] : own[v] * cosv[v] + other[v] * sinv[v]);
@@ -529,8 +636,8 @@ __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
             const long p = p0 + sid + (long)j * stride;
             if (p < p1 && p != upd) {
                 float kf[8], vf[8];
-                unpack_u4(kraw[j], kf);
-                unpack_u4(vraw[j], vf);
+                row_values(kraw[j], kf);
+                row_values(vraw[j], vf);
                 visit(kf, vf);
             }
         }
@@ -538,18 +645,26 @@ __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
             if (p == upd) continue;
             float kf[8], vf[8];
             const long row = ((long)kvh * cap + p) * dh + c0;
-            load_bf16x8(kc + row, kf);
-            load_bf16x8(vc + row, vf);
+            load_row(kc + row, kf);
+            load_row(vc + row, vf);
             visit(kf, vf);
         }
         if (fresh) {   // this step's row: attended to when in range; appended once (by head 0's wave)
             float kf[8], vf[8];
             rope(ka, kb, kf);
-            unpack8(va[0], va[1], vf);
+            words_values(va, vf);
             if (g == 0) {
                 const long row = ((long)kvh * cap + upd) * dh + c0;
-                gstore4(kc + row, make_uint4(pack_bf16x2(kf[0], kf[1]), pack_bf16x2(kf[2], kf[3]), pack_bf16x2(kf[4], kf[5]), pack_bf16x2(kf[6], kf[7])));
-                gstore4(vc + row, make_uint4((unsigned)va[0], (unsigned)(va[0] >> 32), (unsigned)va[1], (unsigned)(va[1] >> 32)));
+                if (F32) {
+#pragma unroll
+                    for (int r = 0; r < RW; ++r) {
+                        gstore4(kc + row + 4 * r, make_uint4((unsigned)ka[2 * r], (unsigned)(ka[2 * r] >> 32), (unsigned)ka[(2 * r + 1) % (2 * RW)], (unsigned)(ka[(2 * r + 1) % (2 * RW)] >> 32)));
+                        gstore4(vc + row + 4 * r, make_uint4((unsigned)va[2 * r], (unsigned)(va[2 * r] >> 32), (unsigned)va[(2 * r + 1) % (2 * RW)], (unsigned)(va[(2 * r + 1) % (2 * RW)] >> 32)));
+                    }
+                } else {
+                    gstore4(kc + row, make_uint4(pack_bf16x2(kf[0], kf[1]), pack_bf16x2(kf[2], kf[3]), pack_bf16x2(kf[4], kf[5]), pack_bf16x2(kf[6], kf[7])));
+                    gstore4(vc + row, make_uint4((unsigned)va[0], (unsigned)(va[0] >> 32), (unsigned)va[1], (unsigned)(va[1] >> 32)));
+                }
             }
             if (upd >= p0 && upd < p1) visit(kf, vf);
         }
@@ -582,6 +697,30 @@ __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
     }
     wg_barrier();
     float* partp = P.part;
+    if (P.flags & kChainAttnFinal) {
+        // one chunk per kv head: its record is the whole softmax, and the context row is written here (what the merge of a
+        // single record gives: O / L)
+        for (int idx = t; idx < G * dh / 2; idx += NT) {
+            const int gg = (2 * idx) / dh, d = 2 * idx - gg * dh;
+            float mn = -INFINITY;
+            for (int w = gg; w < NWS; w += G) mn = fmaxf(mn, sm[w]);
+            float Ls = 0.f, O0 = 0.f, O1 = 0.f;
+            if (mn != -INFINITY) {
+                for (int w = gg; w < NWS; w += G) {
+                    const float cw = fast_exp(sm[w] - mn);
+                    Ls += sl[w] * cw;
+                    O0 += so[w * dh + d] * cw;
+                    O1 += so[w * dh + d + 1] * cw;
+                }
+            }
+            const long at = (long)(kvh * G + gg) * dh + d;
+            if (F32) cstore8((float*)P.y + at, (unsigned long long)__float_as_uint(O0 / Ls) | ((unsigned long long)__float_as_uint(O1 / Ls) << 32));
+            else cstore4((bf16_t*)P.y + at, pack_bf16x2(O0 / Ls, O1 / Ls));
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        wg_barrier();
+        return true;
+    }
     for (int idx = t; idx < G * dh; idx += NT) {
         const int gg = idx / dh, d = idx - gg * dh;
         float mn = -INFINITY;
@@ -608,6 +747,7 @@ __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
 // unit = query head: softmax-merge of its nch chunk records into the context row.  Thread
 // (sg, d2) reads the records of the chunks s = sg, sg + NW, ... for the dims (2 d2, 2 d2 + 1) in
 // one round of loads and merges them locally; the NW subsets meet in LDS.
+template <bool F32>
 __device__ bool attn_combine(GPTRS_LDS int* go, GPTRS_LDS int* abort, const ChainPhase& P, GPTRS_LDS float* lds, int hq, int phase,
                              unsigned long long budget) {
     constexpr int MAXC = 8;   // chunks per thread: nch <= MAXC * NW
@@ -657,7 +797,8 @@ __device__ bool attn_combine(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
                 const float cw = r.x == -INFINITY ? 0.f : fast_exp(r.x - M);
                 Lt += r.y * cw; a0 += r.z * cw; a1 += r.w * cw;
             }
-            cstore4(ctx + (long)hq * dh + 2 * d2, pack_bf16x2(a0 / Lt, a1 / Lt));
+            if (F32) cstore8((float*)P.y + (long)hq * dh + 2 * d2, (unsigned long long)__float_as_uint(a0 / Lt) | ((unsigned long long)__float_as_uint(a1 / Lt) << 32));
+            else cstore4(ctx + (long)hq * dh + 2 * d2, pack_bf16x2(a0 / Lt, a1 / Lt));
         }
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the context words are out before the arrival is reported
         wg_barrier();
@@ -670,6 +811,7 @@ __device__ bool attn_combine(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
 // local-address-space pointers so their accesses stay ds_* instructions.
 // The descriptor comes straight from the table in memory (scalar loads): the compute waves enter an attention phase, and
 // request the cache rows it needs, before the control wave has seen the barrier and filled the LDS copy.
+template <bool F32>
 __device__ __forceinline__ bool run_attn_phase(const GPTRS_CONST ChainPhase* php, GPTRS_LDS float* lds, GPTRS_LDS int* go, GPTRS_LDS int* abort, int phase,
                                                unsigned long long budget) {
     ChainPhase P;
@@ -682,8 +824,8 @@ __device__ __forceinline__ bool run_attn_phase(const GPTRS_CONST ChainPhase* php
     const int kind = P.kind, units = P.units;
     for (int u = blockIdx.x; u < units; u += gridDim.x) {
         bool ok;
-        if (kind == kChainAttnCombine) ok = attn_combine(go, abort, P, lds, u, phase, budget);
-        else ok = attn_partial(go, abort, P, lds, u, phase, budget);
+        if (kind == kChainAttnCombine) ok = attn_combine<F32>(go, abort, P, lds, u, phase, budget);
+        else ok = attn_partial<F32>(go, abort, P, lds, u, phase, budget);
         if (!ok) return false;
     }
     return true;
@@ -735,7 +877,7 @@ __device__ void control_wave(Shared& sh, unsigned* xs, const ChainPhase* phases,
         if (kind != kChainLinear) {
             if (blk < units) {
                 if (lane == 0) lds_st(&sh.go, ph);
-                run_attn_phase(table + ph, (GPTRS_LDS float*)xs, (GPTRS_LDS int*)&sh.go, (GPTRS_LDS int*)&sh.abort, ph, budget);
+                run_attn_phase<FMT == kChainW32>(table + ph, (GPTRS_LDS float*)xs, (GPTRS_LDS int*)&sh.go, (GPTRS_LDS int*)&sh.abort, ph, budget);
             }
         } else if (u0 < u1) {
             if (lane == 0) lds_st(&sh.go, ph);
@@ -756,9 +898,15 @@ __device__ void control_wave(Shared& sh, unsigned* xs, const ChainPhase* phases,
             const unsigned* su = wfmt == kChainW8 ? (const unsigned*)P.wscale2 : nullptr;
             const bool out_f32 = flags & kChainOutF32;   // y and the residual are f32
             unsigned long long e_rf = 0ull;              // two f32 residual values
+            unsigned long long e_bf = 0ull;              // two f32 bias values (f32 phases)
             auto epi_load = [&](int i, unsigned& bw, unsigned& rw, unsigned& ga, unsigned& gb) {
                 const int col = col0 + i;
                 const bool in = i < ncols && col < N;
+                if (wfmt == kChainW32) {
+                    const u32x2 b2 = (bias && in) ? *(const GPTRS_GLOBAL u32x2*)((const char*)bias + 4 * (size_t)col) : u32x2{0u, 0u};
+                    e_bf = (unsigned long long)b2.x | ((unsigned long long)b2.y << 32);
+                    bw = 0u;
+                } else
                 bw = (bias && in) ? gload(bias + (col >> 1)) : 0u;
                 if (out_f32) e_rf = (resid && in) ? cload8(resid + 4 * (size_t)col) : 0ull;
                 rw = (resid && in && !out_f32) ? cload4(resid + 2 * (size_t)col) : 0u;
@@ -768,7 +916,8 @@ __device__ void control_wave(Shared& sh, unsigned* xs, const ChainPhase* phases,
             auto epi_store = [&](int i, unsigned bw, unsigned rw, unsigned ga, unsigned gb) {
                 if (i >= ncols) return;
                 if (bias || resid) {
-                    *reinterpret_cast<float2*>(&sh.epi_bias[i]) = make_float2(bf16lo(bw), bf16hi(bw));
+                    *reinterpret_cast<float2*>(&sh.epi_bias[i]) = wfmt == kChainW32 ? make_float2(__uint_as_float((unsigned)e_bf), __uint_as_float((unsigned)(e_bf >> 32)))
+                                                                                     : make_float2(bf16lo(bw), bf16hi(bw));
                     *reinterpret_cast<float2*>(&sh.epi_res[i]) = out_f32 ? make_float2(__uint_as_float((unsigned)e_rf), __uint_as_float((unsigned)(e_rf >> 32)))
                                                                           : make_float2(bf16lo(rw), bf16hi(rw));
                 }
@@ -780,7 +929,8 @@ __device__ void control_wave(Shared& sh, unsigned* xs, const ChainPhase* phases,
             const bool has_epi = bias || resid || sg;
             unsigned e_bw = 0u, e_rw = 0u, e_ga = 0u, e_gb = 0u;
             if (has_epi) epi_load(lane * 2, e_bw, e_rw, e_ga, e_gb);
-            stage_block(P, xs, sh.ssq);
+            if (wfmt == kChainW32) stage_block_f32(P, xs, sh.ssq);
+            else stage_block(P, xs, sh.ssq);
             if (has_epi) {
                 epi_store(lane * 2, e_bw, e_rw, e_ga, e_gb);
                 for (int i = lane * 2 + 128; i < ncols; i += 128) {
@@ -924,7 +1074,7 @@ template <int FMT, int RING_D>
 __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, int nphases, const unsigned char* ring, unsigned long long budget) {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int blk = blockIdx.x;
-    constexpr int kpw = FMT == kChainW16 ? 2 : (FMT == kChainW8 ? 4 : 8);
+    constexpr int kpw = FMT == kChainW32 ? 1 : (FMT == kChainW16 ? 2 : (FMT == kChainW8 ? 4 : 8));
     constexpr unsigned STEP = NS * 16;   // bytes of a tile stream per j-step
 
     // ---- request side: the wave's next j-step to ask for, in the order the steps are consumed.  Everything but r_off is
@@ -1022,7 +1172,7 @@ __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, 
             const int units = uni(D->units);
             if (uni(D->kind) != kChainLinear) {
                 if (blk >= units) continue;
-                if (!run_attn_phase(table + c_phase, (GPTRS_LDS float*)xs, (GPTRS_LDS int*)&sh.go, (GPTRS_LDS int*)&sh.abort, c_phase,
+                if (!run_attn_phase<FMT == kChainW32>(table + c_phase, (GPTRS_LDS float*)xs, (GPTRS_LDS int*)&sh.go, (GPTRS_LDS int*)&sh.abort, c_phase,
                                     budget)) return false;
                 continue;
             }
@@ -1038,7 +1188,8 @@ __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, 
             PhaseRegs R;
             regs_from_table(R, D);
             if (!wait_go(&sh.go, &sh.abort, c_phase, budget)) return false;
-            stage_block(R, const_cast<unsigned*>(xs), sh.ssq);
+            if (FMT == kChainW32) stage_block_f32(R, const_cast<unsigned*>(xs), sh.ssq);
+            else stage_block(R, const_cast<unsigned*>(xs), sh.ssq);
             return true;
         }
     };
@@ -1093,6 +1244,16 @@ __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, 
                 acc[p][1] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q1), xv, acc[p][1], false);
                 acc[p][2] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q2), xv, acc[p][2], false);
                 acc[p][3] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, q3), xv, acc[p][3], false);
+            }
+        } else if (c_fmt == kChainW32) {
+            const float xv = __uint_as_float(xs[c_j * NS + t]);
+#pragma unroll
+            for (int p = 0; p < TP; ++p) {
+                const unsigned q0 = cur[p].x, q1 = cur[p].y, q2 = cur[p].z, q3 = cur[p].w;
+                acc[p][0] = __builtin_fmaf(__uint_as_float(q0), xv, acc[p][0]);
+                acc[p][1] = __builtin_fmaf(__uint_as_float(q1), xv, acc[p][1]);
+                acc[p][2] = __builtin_fmaf(__uint_as_float(q2), xv, acc[p][2]);
+                acc[p][3] = __builtin_fmaf(__uint_as_float(q3), xv, acc[p][3]);
             }
         } else if (c_fmt == kChainW8) {
             const u32x2 xw = *reinterpret_cast<const u32x2*>(&xs[2 * (c_j * NS + t)]);
@@ -1220,6 +1381,17 @@ __global__ void chain_pack_kernel(const bf16_t* __restrict__ w, const bf16_t* __
 // 4j .. 4j+3 of its 4 columns.  int8: a code row is one k, bytes stored as q + 128 (flip = 0x80).  int4: a code
 // row is a packed byte (k = 2r low nibble, 2r + 1 high nibble), both nibbles stored as q + 8 (flip = 0x88).
 // Bytes outside the matrix hold the biased zero.
+// f32 weights: word (tile, k) = the 4 columns of the tile at row k
+__global__ void chain_pack_f32_kernel(const float* __restrict__ w, float* __restrict__ out, int64_t K, int64_t N, int64_t Kw, int64_t ntiles) {
+    const int64_t total = ntiles * Kw * 4;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int c = (int)(idx & 3);
+        const int64_t j = (idx >> 2) % Kw, tile = (idx >> 2) / Kw;
+        const int64_t col = tile * 4 + c;
+        out[idx] = (col < N && j < K) ? w[j * N + col] : 0.f;
+    }
+}
+
 __global__ void chain_pack_codes_kernel(const uint8_t* __restrict__ w, const uint8_t* __restrict__ w2, uint32_t* __restrict__ out,
                                         int64_t rows, int64_t N, int64_t Kw, int64_t ntiles, uint32_t flip) {
     const int64_t total = ntiles * Kw * 4;
@@ -1255,7 +1427,7 @@ __global__ void chain_pack_scales_kernel(const bf16_t* __restrict__ sc, const bf
 }
 
 static int g_grid = 0;
-static int g_occupancy_ok[6] = {-1, -1, -1, -1, -1, -1};   // per kernel: does a workgroup fit a CU with the LDS it asks for
+static int g_occupancy_ok[8] = {-1, -1, -1, -1, -1, -1, -1, -1};   // per kernel: does a workgroup fit a CU with the LDS it asks for
 
 }  // namespace
 
@@ -1271,17 +1443,24 @@ int chain_grid() {
 }
 
 static inline int64_t cdiv64(int64_t a, int64_t b) { return (a + b - 1) / b; }
-static inline int chain_kpw(int wfmt) { return wfmt == kChainW16 ? 2 : (wfmt == kChainW8 ? 4 : 8); }   // k per column of a word
+static inline int chain_kpw(int wfmt) { return wfmt == kChainW32 ? 1 : (wfmt == kChainW16 ? 2 : (wfmt == kChainW8 ? 4 : 8)); }   // k per column of a word
+// bytes of staged activations per weight word: kpw bf16 values, or one f32
+static inline int chain_xbytes(int wfmt) { return wfmt == kChainW32 ? 4 : chain_kpw(wfmt) * 2; }
 static inline int64_t chain_kw(int64_t k, int wfmt) { return cdiv64(cdiv64(k, chain_kpw(wfmt)), NS) * NS; }
 
 bool chain_supported(int dtype, int64_t m, int64_t k, int64_t n, bool dual, bool norm, int wfmt, bool x_f32) {
-    if (dtype != 2 || m != 1 || k < 4 || n < 4) return false;
+    if (m != 1 || k < 4 || n < 4) return false;
+    if (wfmt < kChainW16 || wfmt > kChainW32) return false;
+    if (wfmt == kChainW32) {   // f32 weights, activations and output; no SwiGLU pair
+        if (dtype != 0 || dual || k % 4 != 0 || n % 4 != 0 || k > 4 * (MAXI / 2) * NT) return false;
+        return chain_kw(k, wfmt) * chain_xbytes(wfmt) / 4 <= kChainMaxXsWords;
+    }
+    if (dtype != 2) return false;
     if (x_f32 && (!norm || k > 4 * (MAXI / 2) * NT)) return false;
-    if (wfmt < kChainW16 || wfmt > kChainW4) return false;
     if (k % 4 != 0 || n % (dual ? 2 : 4) != 0) return false;
     if (wfmt == kChainW4 && k % 128 != 0) return false;
     if (norm && k > 4 * MAXI * NT) return false;
-    if (chain_kw(k, wfmt) * (chain_kpw(wfmt) / 2) > kChainMaxXsWords) return false;
+    if (chain_kw(k, wfmt) * chain_xbytes(wfmt) / 4 > kChainMaxXsWords) return false;
     return true;
 }
 
@@ -1295,7 +1474,9 @@ void chain_pack_weights(hipStream_t s, const void* w, const void* w2, void* out,
     const int64_t total = ntiles * kw * 4;
     if (total <= 0) return;
     const unsigned g = (unsigned)std::min<int64_t>(cdiv64(total, 256), 65536);
-    if (wfmt == kChainW16)
+    if (wfmt == kChainW32)
+        chain_pack_f32_kernel<<<g, 256, 0, s>>>((const float*)w, (float*)out, k, n, kw, ntiles);
+    else if (wfmt == kChainW16)
         chain_pack_kernel<<<g, 256, 0, s>>>((const bf16_t*)w, (const bf16_t*)w2, (uint32_t*)out, k, n, kw, ntiles);
     else
         chain_pack_codes_kernel<<<g, 256, 0, s>>>((const uint8_t*)w, (const uint8_t*)w2, (uint32_t*)out, wfmt == kChainW8 ? k : k / 2, n, kw,
@@ -1326,7 +1507,7 @@ bool chain_fill_phase(ChainPhase& p, int64_t k, int64_t n, bool dual, int wfmt) 
     p.upb = grid > 0 ? (p.units + grid - 1) / grid : p.units;
     p.kind = kChainLinear;
     p.wfmt = wfmt;
-    p.lds_bytes = p.Kw * (chain_kpw(wfmt) / 2) * 4;
+    p.lds_bytes = p.Kw * chain_xbytes(wfmt);
     // int4: the workgroup's group scales (8 bytes per tile and group) are staged behind the activations
     const int64_t total = p.lds_bytes + (wfmt == kChainW4 ? (int64_t)p.upb * TP * (p.Kw / 16) * 8 : 0);
     p.lds_total = (int)std::min<int64_t>(total, INT32_MAX);
@@ -1337,7 +1518,8 @@ bool chain_fill_phase(ChainPhase& p, int64_t k, int64_t n, bool dual, int wfmt) 
 bool chain_attn_supported(int dtype, int64_t t, int64_t n_q, int64_t n_kv, int64_t head_dim, int64_t rot_half) {
     static const bool enabled = [] { const char* e = getenv("GPTRS_HIP_CHAIN_ATTN"); return !(e && e[0] == '0'); }();
     if (!enabled) return false;   // GPTRS_HIP_CHAIN_ATTN=0: decode attention keeps its stand-alone kernels
-    if (dtype != 2 || t != 1 || n_kv <= 0 || n_q % n_kv != 0) return false;
+    if ((dtype != 2 && dtype != 0) || t != 1 || n_kv <= 0 || n_q % n_kv != 0) return false;
+    if (dtype == 0 && rot_half != 0) return false;   // f32 rows: no RoPE inside the phase
     const int64_t g = n_q / n_kv;
     if (g != 1 && g != 2 && g != 4 && g != 8) return false;
     if (head_dim != 64 && head_dim != 128 && head_dim != 256) return false;
@@ -1351,9 +1533,12 @@ static int chain_attn_nch(int64_t n_kv) {
 size_t chain_attn_part_bytes(int64_t n_q, int64_t n_kv, int64_t head_dim) {
     return (size_t)n_q * (size_t)chain_attn_nch(n_kv) * (size_t)(head_dim + 2) * sizeof(float);
 }
+int chain_attn_phases(int64_t capacity) { return capacity <= 128 ? 1 : 2; }
 void chain_fill_attn(ChainPhase& partial, ChainPhase& combine, int64_t n_q, int64_t n_kv, int64_t head_dim, int64_t capacity,
                      int64_t rot_half, float scale) {
-    const int nch = chain_attn_nch(n_kv);
+    const bool single = chain_attn_phases(capacity) == 1;
+    const int nch = single ? 1 : chain_attn_nch(n_kv);
+    if (single) partial.flags |= kChainAttnFinal;
     for (ChainPhase* p : {&partial, &combine}) {
         p->n_q = (int)n_q; p->n_kv = (int)n_kv; p->head_dim = (int)head_dim; p->capacity = (int)capacity;
         p->rot_half = (int)rot_half; p->nch = nch; p->scale = scale;
@@ -1370,7 +1555,7 @@ bool chain_launch(hipStream_t s, const ChainPhase* dev_table, int nphases, int l
                   int stall_phase) {
     const int grid = chain_grid();
     if (grid <= 0 || nphases <= 0 || nphases > kChainMaxPhases || lds_bytes > kChainMaxXsWords * 4) return false;
-    if (wfmt < kChainW16 || wfmt > kChainW4) return false;
+    if (wfmt < kChainW16 || wfmt > kChainW32) return false;
     const int xs_bytes = (lds_bytes + 1023) / 1024 * 1024;
     static const int max_depth = [] { const char* e = getenv("GPTRS_HIP_CHAIN_RING"); return e ? std::max(RING_MIN, std::min(RING_MAX, atoi(e))) : RING_MAX; }();
     const int depth = sizeof(Shared) + (size_t)xs_bytes + (size_t)max_depth * SLOT_BYTES <= (size_t)LDS_BYTES ? max_depth : RING_MIN;
@@ -1379,9 +1564,10 @@ bool chain_launch(hipStream_t s, const ChainPhase* dev_table, int nphases, int l
     static_assert(RING_MAX == RING_MIN + 1, "two kernels per weight format");
     const int variant = wfmt * 2 + (depth - RING_MIN);
     typedef void (*Kernel)(const ChainPhase*, int, unsigned*, int*, int, unsigned long long, int);
-    static const Kernel kernels[6] = {chain_kernel<kChainW16, RING_MIN>, chain_kernel<kChainW16, RING_MAX>, chain_kernel<kChainW8, RING_MIN>,
-                                      chain_kernel<kChainW8, RING_MAX>,  chain_kernel<kChainW4, RING_MIN>,  chain_kernel<kChainW4, RING_MAX>};
-    static_assert(kChainW16 == 0 && kChainW8 == 1 && kChainW4 == 2, "index of a kernel");
+    static const Kernel kernels[8] = {chain_kernel<kChainW16, RING_MIN>, chain_kernel<kChainW16, RING_MAX>, chain_kernel<kChainW8, RING_MIN>,
+                                      chain_kernel<kChainW8, RING_MAX>,  chain_kernel<kChainW4, RING_MIN>,  chain_kernel<kChainW4, RING_MAX>,
+                                      chain_kernel<kChainW32, RING_MIN>, chain_kernel<kChainW32, RING_MAX>};
+    static_assert(kChainW16 == 0 && kChainW8 == 1 && kChainW4 == 2 && kChainW32 == 3, "index of a kernel");
     const Kernel fn = kernels[variant];
     if (g_occupancy_ok[variant] < 0) {
         // The grid barrier needs every workgroup resident at once: one workgroup per CU, grid <= CUs (chain_grid), and the

@@ -9,6 +9,10 @@
 
 namespace gptrs {
 
+// The weight format of a linear layer inside a decode chain: f32 weights have a format of their own, the others follow
+// the quantisation of the layer.
+static inline int chain_format(const Instr& in, DType ldt) { return ldt == DType::F32 ? k::kChainW32 : (int)in.quant; }
+
 static constexpr size_t kAlign = 256;
 static size_t align_up(size_t n) { return (n + kAlign - 1) / kAlign * kAlign; }
 
@@ -779,32 +783,47 @@ void Builder::build() {
         if (in.op == OpKind::FAttnDecode) {
             if (in.batch > 1) return 0;
             const Spec& x = plan.values[st.src[0]].spec;
-            return k::chain_attn_supported((int)x.dtype, x.dims[0], in.n_q, in.n_kv, in.head_dim, in.rot_half) ? 2 : 0;
+            if (!k::chain_attn_supported((int)x.dtype, x.dims[0], in.n_q, in.n_kv, in.head_dim, in.rot_half)) return 0;
+            return k::chain_attn_phases(plan.values[st.src[1]].spec.dims[1]);
         }
         if (in.op != OpKind::FLinear || !in.tiled || st.tiled_w_input < 0) return 0;
         const Spec& x = plan.values[st.src[0]].spec;
         const Spec& w = plan.values[st.src[1]].spec;
         if (x.rank() != 2 || w.rank() != 2) return 0;
         const bool dual = in.act == 2;
-        if (in.norm_ln) return 0;   // the chain stages RMSNorm only
         const DType ldt = linear_dtype(in, w, in.quant ? &plan.values[st.src[2]].spec : nullptr);
-        if (!k::chain_supported((int)ldt, x.dims[0], x.dims[1], w.dims[1], dual, in.norm, in.quant, in.x_f32)) return 0;
+        const int wfmt = chain_format(in, ldt);
+        if (in.norm_ln && wfmt != k::kChainW32) return 0;   // LayerNorm is staged for f32 phases only
+        if (wfmt == k::kChainW32 && (in.norm && !in.norm_ln)) return 0;   // ... and RMSNorm for the others
+        if (!k::chain_supported((int)ldt, x.dims[0], x.dims[1], w.dims[1], dual, in.norm, wfmt, in.x_f32)) return 0;
         k::ChainPhase p{};
-        return k::chain_fill_phase(p, x.dims[1], w.dims[1], dual, in.quant) ? 1 : 0;
+        return k::chain_fill_phase(p, x.dims[1], w.dims[1], dual, wfmt) ? 1 : 0;
+    };
+    auto step_format = [&](const Step& st) {
+        const Instr& in = st.in;
+        const Spec& w = plan.values[st.src[1]].spec;
+        return chain_format(in, linear_dtype(in, w, in.quant ? &plan.values[st.src[2]].spec : nullptr));
+    };
+    // f32 linears and f32 attentions go together (the launch's kernel reads f32 rows and caches), the others likewise
+    auto f32_class = [&](const Step& st) {
+        if (st.in.op == OpKind::FAttnDecode) return plan.values[st.src[0]].spec.dtype == DType::F32;
+        return step_format(st) == k::kChainW32;
     };
     for (int s = 0; s < n_steps;) {
         int np = chain_phases(plan.steps[s]);
         if (!np) { ++s; continue; }
         int e = s + 1;
         bool has_linear = plan.steps[s].in.op == OpKind::FLinear;
-        int fmt = has_linear ? plan.steps[s].in.quant : -1;   // one weight format per launch
+        int fmt = has_linear ? step_format(plan.steps[s]) : -1;   // one weight format per launch
+        const bool cls = f32_class(plan.steps[s]);
         while (e < n_steps) {
             const Step& nx = plan.steps[e];
             const int q = chain_phases(nx);
             if (!q || np + q > k::kChainMaxPhases) break;
+            if (f32_class(nx) != cls) break;
             if (nx.in.op == OpKind::FLinear) {
-                if (fmt >= 0 && nx.in.quant != fmt) break;
-                fmt = nx.in.quant;
+                if (fmt >= 0 && step_format(nx) != fmt) break;
+                fmt = step_format(nx);
                 has_linear = true;
             }
             np += q;
@@ -846,6 +865,19 @@ static bool run_chain(const Plan& plan, const Step& head, ExecCtx& cx) {
     auto aligned8 = [](std::initializer_list<const void*> ps) {
         for (const void* q : ps) if ((uintptr_t)q & 7) fail_exec("decode chain: operand buffers must be 8-byte aligned");
     };
+    {   // f32 phases pay off once they have something to stream (Backend::chain_f32_min_bytes)
+        int64_t f32_bytes = 0, f32_linears = 0;
+        for (int i = 0; i < head.chain_len; ++i) {
+            const Step& st = (&head)[i];
+            if (st.in.op != OpKind::FLinear) continue;
+            const Spec& x = plan.values[st.src[0]].spec;
+            const Spec& w = plan.values[st.src[1]].spec;
+            if (chain_format(st.in, linear_dtype(st.in, w, st.in.quant ? &plan.values[st.src[2]].spec : nullptr)) != k::kChainW32) continue;
+            f32_bytes += x.dims[1] * w.dims[1] * 4;
+            ++f32_linears;
+        }
+        if (f32_linears > 0 && f32_bytes < cx.be->chain_f32_min_bytes * f32_linears) { cx.chain = false; return false; }
+    }
     for (int i = 0; i < head.chain_len; ++i) {
         const Step& st = (&head)[i];
         const Instr& in = st.in;
@@ -868,22 +900,24 @@ static bool run_chain(const Plan& plan, const Step& head, ExecCtx& cx) {
             pa.part = (float*)(cx.ws + st.scratch_off);
             pc.part = pa.part;
             pc.y = cx.ptr[st.dst[0]];
+            pa.y = pc.y;   // (written by the first phase when it is the only one)
             aligned8({pa.x, pa.part, pc.y});
             if (((uintptr_t)kout | (uintptr_t)vout | (uintptr_t)pa.cos | (uintptr_t)pa.sin) & 15)
                 fail_exec("decode chain: cache and RoPE buffers must be 16-byte aligned");
-            lds_bytes = std::max(lds_bytes, std::max(pa.lds_total, pc.lds_total));
+            const bool two = k::chain_attn_phases(ck.dims[1]) == 2;
+            lds_bytes = std::max(lds_bytes, two ? std::max(pa.lds_total, pc.lds_total) : pa.lds_total);
             phases.push_back(pa);
-            phases.push_back(pc);
+            if (two) phases.push_back(pc);
             continue;
         }
         const Spec& x = plan.values[st.src[0]].spec;
         const Spec& w = plan.values[st.src[1]].spec;
         const bool dual = in.act == 2;
         k::ChainPhase p{};
-        if (!k::chain_fill_phase(p, x.dims[1], w.dims[1], dual, in.quant)) { cx.chain = false; return false; }
-        wfmt = in.quant;
         const DType ldt = linear_dtype(in, w, in.quant ? &plan.values[st.src[2]].spec : nullptr);
-        BufferP wc = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], in.quant == 0 ? 2 : (in.quant == 1 ? 3 : 4), ldt,
+        wfmt = chain_format(in, ldt);
+        if (!k::chain_fill_phase(p, x.dims[1], w.dims[1], dual, wfmt)) { cx.chain = false; return false; }
+        BufferP wc = cx.be->derived_weights(cx.input_bufs[st.tiled_w_input], wfmt == k::kChainW32 ? 11 : (in.quant == 0 ? 2 : (in.quant == 1 ? 3 : 4)), ldt,
                                             x.dims[1], w.dims[1], dual ? cx.input_bufs[st.tiled_w2_input] : nullptr);
         p.w = wc->ptr;
         p.x = src_ptr(st, cx, 0);
@@ -900,12 +934,14 @@ static bool run_chain(const Plan& plan, const Step& head, ExecCtx& cx) {
         if (in.has_bias) { p.bias = src_ptr(st, cx, oi++); p.flags |= k::kChainBias; }
         if (in.has_residual) { p.residual = src_ptr(st, cx, oi++); p.flags |= k::kChainResidual; }
         if (in.norm) { p.gamma = src_ptr(st, cx, oi++); p.inv_n = in.scale; p.eps = in.eps; p.flags |= k::kChainNorm; }
+        if (in.norm && in.norm_ln) { p.beta = src_ptr(st, cx, oi++); p.flags |= k::kChainLayerNorm; }
         if (in.act == 1) p.flags |= k::kChainGelu;
-        if (in.out_f32) p.flags |= k::kChainOutF32;
-        if (in.x_f32) p.flags |= k::kChainXF32;
+        if (in.out_f32 || wfmt == k::kChainW32) p.flags |= k::kChainOutF32;
+        if (in.x_f32 || wfmt == k::kChainW32) p.flags |= k::kChainXF32;
         p.y = cx.ptr[st.dst[0]];
-        aligned8({p.x, p.y, p.residual, p.bias, p.gamma});
-        if (in.x_f32 && ((uintptr_t)p.gamma & 15)) fail_exec("decode chain: f32 gains must be 16-byte aligned");
+        aligned8({p.x, p.y, p.residual, p.bias, p.gamma, p.beta});
+        if ((p.flags & k::kChainXF32) && (((uintptr_t)p.gamma | (uintptr_t)p.beta | (uintptr_t)p.x) & 15))
+            fail_exec("decode chain: f32 rows, gains and offsets must be 16-byte aligned");
         lds_bytes = std::max(lds_bytes, p.lds_total);
         bytes += (int64_t)dtype_size(x.dtype) * x.dims[1] + (int64_t)(in.out_f32 ? 4 : dtype_size(ldt)) * w.dims[1] + linear_weight_bytes(in, ldt, x, w);
         phases.push_back(p);

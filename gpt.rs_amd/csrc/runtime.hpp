@@ -187,7 +187,7 @@ class Backend {
     // Quantised weights: kind 3 / 4: chain copies of int8 / int4 codes (src2: the partner's codes); kind 5:
     // chain copy of int4 group scales (src2: the partner's); kind 6 / 7: k-grouped copy of the int8 / int4
     // codes for the MFMA GEMM, which applies the scales itself; kind 8: 16-column tiled k-grouped copy for batched decode
-    // (kernels_skinny.hip); kind 9 / 10: int8 / int4 codes in that tile order.
+    // (kernels_skinny.hip); kind 9 / 10: int8 / int4 codes in that tile order; kind 11: chain copy of f32 weights.
     BufferP derived_weights(const BufferP& src, int kind, DType dtype, int64_t k, int64_t n, const BufferP& src2 = nullptr);
     void drop_derived_weights();
     // Device copy of a chain's phase table, cached by content (steady-state decode repeats a few tables).
@@ -197,6 +197,9 @@ class Backend {
     unsigned* skinny_tickets() const { return d_chain_bar_ + k::kChainBarrierBytes / sizeof(unsigned); }
     int* chain_abort_flag() const { return d_err_flag_ + 1; }
     bool opt_chain = true;
+    // f32 chains run only when a linear phase streams at least this much on average (option "chain_f32_min_kb",
+    // GPTRS_HIP_CHAIN_F32_MIN_KB): below it a phase's fixed cost is what a stand-alone kernel costs
+    int64_t chain_f32_min_bytes = 8ll << 20;
     int chain_stall_phase = -1;   // tests of the give-up path: the next chain launch expects an arrival too many at this phase
     int64_t n_chain_launches = 0, n_chain_phases = 0;
     int64_t n_tiled_built = 0;

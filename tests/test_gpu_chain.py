@@ -134,14 +134,15 @@ def test_block_tail_chain(hip, d, f):
     assert hip.counter("chain_phases") - before >= 4
 
 
-@pytest.mark.parametrize("hq,hkv,dh,rope", [(8, 2, 128, True), (4, 4, 64, False), (8, 1, 128, True), (4, 2, 256, False)])
-def test_decode_attention_in_chain(hip, hq, hkv, dh, rope):
+@pytest.mark.parametrize("hq,hkv,dh,rope,cap", [(8, 2, 128, True, 2048), (4, 4, 64, False, 2048), (8, 1, 128, True, 2048), (4, 2, 256, False, 2048),
+                                                (8, 2, 128, True, 128), (4, 4, 64, False, 96)])
+def test_decode_attention_in_chain(hip, hq, hkv, dh, rope, cap):
     """projection -> (RoPE) -> attention_decode_cache -> out-projection as ONE launch: the attention takes
     two phases of the chain (per-chunk online softmax, then the merge).  Positions cover an empty cache,
     fewer positions than chunks, chunk boundaries, more positions per lane group than are requested
     ahead of the barrier, and the last slot; the updated caches must match as well (bit-exact when no
     RoPE touches the appended row)."""
-    d, cap = 256, 2048
+    d = 256
     cfg = F.AttentionConfig(embed_dim=d, num_query_heads=hq, num_key_value_heads=hkv, head_dim=dh)
     tp, qp = cfg.total_projection_dim, cfg.query_projection_dim
     rcfg = F.RopeConfig(rotary_dim=dh, theta=10000.0) if rope else None
@@ -157,7 +158,7 @@ def test_decode_attention_in_chain(hip, hq, hkv, dh, rope):
         return [c.matmul(w2), k2, v2]
 
     fspecs = [[1, d], [d, tp], [qp, d], [hkv, cap, dh], [hkv, cap, dh]]
-    for pos in (0, 5, 31, 32, 100, 1500, cap - 1):
+    for pos in sorted({0, 5, 31, 32, min(100, cap - 2), (3 * cap) // 4, cap - 1}):
         us, qs = np.array([0, pos, 0], np.int32), np.array([pos], np.int32)
         arrays, ispecs = [x, wqkv, wo, kc, vc], [("Si32", [3]), ("Si32", [1])]
         extra, especs = [], []
@@ -168,7 +169,8 @@ def test_decode_attention_in_chain(hip, hq, hkv, dh, rope):
         pf = prog(build, [("F32", s) for s in fspecs] + ispecs + [("F32", s) for s in especs])
         before = hip.counter("chain_phases")
         got = hip_run(hip, pb, arrays + [us, qs] + extra)
-        assert hip.counter("chain_phases") - before == 4, "projection, attention (2 phases) and out-projection must share one launch"
+        # (a cache of at most 128 positions is one chunk per kv head: the attention is then one phase)
+        assert hip.counter("chain_phases") - before == (3 if cap <= 128 else 4), "projection, attention and out-projection must share one launch"
         want = oracle_run(pf, [bf16_round(a) for a in arrays] + [us, qs] + [bf16_round(a) for a in extra])
         assert_close(got[0], want[0], atol=3e-2, rtol=2e-2, what=f"context projection at pos {pos}")
         for i in (1, 2):
@@ -226,3 +228,131 @@ def test_padded_steps_and_missing_tiles_are_stable(hip, k, n):
         got = np.asarray(hip_run(hip, p, [x, w])[0], np.float32)
         assert_close(got, plain, atol=2e-5, rtol=ULP, what=f"run {rep} vs per-linear kernel")
     assert hip.counter("chain_launches") == before + 25
+
+
+# ------------------------------------------------------------------------------ f32 phases (GPT-2)
+def run_both_f32(hip, build, specs, arrays, atol=5e-4, rtol=1e-4, phases=1):
+    """f32 program: chain on vs the oracle and vs chain off (the reference suite's f32 bar, 5e-4 + 1e-4 relative:
+    only the order of the f32 sums differs)."""
+    p = prog(build, [("F32", d) for d in specs])
+    hip.set_option("chain_f32_min_kb", 0)   # (by default f32 phases that stream little keep their stand-alone kernels)
+    try:
+        before, ph0 = hip.counter("chain_launches"), hip.counter("chain_phases")
+        got = hip_run(hip, p, arrays)
+        assert hip.counter("chain_launches") > before, "the program did not take the chain path"
+        assert hip.counter("chain_phases") - ph0 >= phases
+    finally:
+        hip.set_option("chain_f32_min_kb", 8192)
+    want = oracle_run(p, arrays)
+    hip.set_option("chain", 0)
+    try:
+        plain = hip_run(hip, p, arrays)
+    finally:
+        hip.set_option("chain", 1)
+    for i, (g, w, q) in enumerate(zip(got, want, plain)):
+        assert np.asarray(g).dtype == np.float32
+        assert_close(g, w, atol=atol, rtol=rtol, what=f"result {i} vs oracle")
+        assert_close(g, q, atol=atol, rtol=rtol, what=f"result {i} vs per-linear kernels")
+
+
+@pytest.mark.parametrize("k,n", [(768, 2304), (768, 3072), (3072, 768), (768, 768), (200, 52), (4608, 64), (64, 12)])
+def test_f32_single_linear(hip, k, n):
+    x, w = rnd(31, (1, k)), rnd(32, (k, n), 2.0 / np.sqrt(k))
+    run_both_f32(hip, lambda fb, a, b: a.matmul(b), [[1, k], [k, n]], [x, w])
+
+
+@pytest.mark.parametrize("k,n", [(768, 2304), (3072, 768), (100, 40)])
+def test_f32_layer_norm_linear_bias(hip, k, n):
+    x, g, bt = rnd(33, (1, k), 3.0) + 0.7, rnd(34, (k,)) + 1.5, rnd(35, (k,))
+    w, b = rnd(36, (k, n), 2.0 / np.sqrt(k)), rnd(37, (n,))
+    run_both_f32(hip, lambda fb, a, gm, be, c, d: F.linear(F.layer_norm(a, gm, be, 1e-5)[0], c, d),
+                 [[1, k], [k], [k], [k, n], [n]], [x, g, bt, w, b])
+
+
+@pytest.mark.parametrize("k,n", [(768, 3072), (3072, 768), (128, 64)])
+def test_f32_bias_gelu_residual(hip, k, n):
+    x, w, b, r = rnd(38, (1, k)), rnd(39, (k, n), 2.0 / np.sqrt(k)), rnd(40, (n,)), rnd(41, (1, n))
+    run_both_f32(hip, lambda fb, a, c, d, e: F.gelu(F.linear(a, c, d)) + e, [[1, k], [k, n], [n], [1, n]], [x, w, b, r])
+    run_both_f32(hip, lambda fb, a, c, d, e: F.linear(a, c, d) + e, [[1, k], [k, n], [n], [1, n]], [x, w, b, r])
+
+
+@pytest.mark.parametrize("d", [768, 96])
+def test_f32_block_tail_chain(hip, d):
+    """out-proj (+bias, +residual) -> LayerNorm -> fc (+bias, GELU) -> proj (+bias, +residual) -> LayerNorm -> next qkv
+    (+bias): the linears of a GPT-2 block behind its attention (model/gpt.rs:585-751), four dependent phases."""
+    f = 4 * d
+    ctx, x = rnd(50, (1, d)), rnd(51, (1, d))
+    wo, bo = rnd(52, (d, d), 2.0 / np.sqrt(d)), rnd(53, (d,))
+    wf, bf = rnd(54, (d, f), 2.0 / np.sqrt(d)), rnd(55, (f,))
+    wp, bp = rnd(56, (f, d), 2.0 / np.sqrt(f)), rnd(57, (d,))
+    wq, bq = rnd(58, (d, 3 * d), 2.0 / np.sqrt(d)), rnd(59, (3 * d,))
+    g1, b1, g2, b2 = rnd(60, (d,)) + 1.5, rnd(61, (d,)), rnd(62, (d,)) + 1.5, rnd(63, (d,))
+
+    def build(fb, c, xx, a_wo, a_bo, a_wf, a_bf, a_wp, a_bp, a_wq, a_bq, a_g1, a_b1, a_g2, a_b2):
+        h = F.linear(c, a_wo, a_bo) + xx
+        m = F.gelu(F.linear(F.layer_norm(h, a_g1, a_b1, 1e-5)[0], a_wf, a_bf))
+        out = F.linear(m, a_wp, a_bp) + h
+        return [F.linear(F.layer_norm(out, a_g2, a_b2, 1e-5)[0], a_wq, a_bq), out]
+
+    specs = [[1, d], [1, d], [d, d], [d], [d, f], [f], [f, d], [d], [d, 3 * d], [3 * d], [d], [d], [d], [d]]
+    run_both_f32(hip, build, specs, [ctx, x, wo, bo, wf, bf, wp, bp, wq, bq, g1, b1, g2, b2], atol=2e-3, rtol=1e-3, phases=4)
+
+
+def test_f32_phases_that_stream_little_keep_their_kernels(hip):
+    """The default policy: f32 linears join a persistent launch from 8 MiB of weights each on average."""
+    x = rnd(80, (1, 768))
+    small, big = rnd(81, (768, 768), 0.05), rnd(82, (768, 4096), 0.05)
+    p_small = prog(lambda fb, a, b: a.matmul(b), [("F32", [1, 768]), ("F32", [768, 768])])
+    p_big = prog(lambda fb, a, b: a.matmul(b), [("F32", [1, 768]), ("F32", [768, 4096])])
+    before = hip.counter("chain_launches")
+    hip_run(hip, p_small, [x, small])
+    assert hip.counter("chain_launches") == before, "2.4 MB of f32 weights: stand-alone kernel"
+    hip_run(hip, p_big, [x, big])
+    assert hip.counter("chain_launches") == before + 1, "12.6 MB of f32 weights: persistent launch"
+
+
+@pytest.mark.parametrize("hq,hkv,dh,cap", [(12, 12, 64, 128), (4, 4, 64, 1024), (8, 2, 128, 2048), (4, 1, 256, 256)])
+def test_f32_decode_attention_in_chain(hip, hq, hkv, dh, cap):
+    """f32 projection (+bias) -> attention_decode_cache over f32 caches -> out-projection (+bias) as ONE launch (the
+    attention of a GPT-2 block, model/gpt.rs:585-751): context to the f32 bar against the oracle and against the
+    stand-alone kernels, caches exact but for the appended row, which is a copy of the projection's output."""
+    d = 192
+    cfg = F.AttentionConfig(embed_dim=d, num_query_heads=hq, num_key_value_heads=hkv, head_dim=dh)
+    tp, qp = cfg.total_projection_dim, cfg.query_projection_dim
+    x = rnd(70, (1, d))
+    wqkv, bqkv = rnd(71, (d, tp), 2.0 / np.sqrt(d)), rnd(72, (tp,))
+    wo, bo = rnd(73, (qp, d), 2.0 / np.sqrt(qp)), rnd(74, (d,))
+    kc, vc = rnd(75, (hkv, cap, dh)), rnd(76, (hkv, cap, dh))
+
+    def build(fb, a, w1, b1, w2, b2, k, v, us, qs):
+        c, k2, v2 = F.attention_decode_cache(cfg, F.linear(a, w1, b1), k, v, us, qs)
+        return [F.linear(c, w2, b2), k2, v2]
+
+    specs = [("F32", s) for s in [[1, d], [d, tp], [tp], [qp, d], [d], [hkv, cap, dh], [hkv, cap, dh]]] + [("Si32", [3]), ("Si32", [1])]
+    p = prog(build, specs)
+    for pos in sorted({0, 5, 31, 32, 100, cap // 2, cap - 1}):
+        us, qs = np.array([0, pos, 0], np.int32), np.array([pos], np.int32)
+        arrays = [x, wqkv, bqkv, wo, bo, kc, vc, us, qs]
+        hip.set_option("chain_f32_min_kb", 0)
+        try:
+            before = hip.counter("chain_phases")
+            got = hip_run(hip, p, arrays)
+        finally:
+            hip.set_option("chain_f32_min_kb", 8192)
+        # a cache of at most 128 positions is one chunk per kv head: the attention is one phase
+        assert hip.counter("chain_phases") - before == (3 if cap <= 128 else 4), "projection, attention and out-projection must share one launch"
+        want = oracle_run(p, arrays)
+        hip.set_option("chain", 0)
+        try:
+            plain = hip_run(hip, p, arrays)
+        finally:
+            hip.set_option("chain", 1)
+        assert_close(got[0], want[0], atol=5e-4, rtol=1e-4, what=f"context projection at pos {pos}")
+        assert_close(got[0], plain[0], atol=5e-4, rtol=1e-4, what=f"context projection at pos {pos} vs stand-alone kernels")
+        for i in (1, 2):
+            g, w = np.asarray(got[i]), np.asarray(want[i])
+            mask = np.ones(cap, bool)
+            mask[pos] = False
+            assert np.array_equal(g[:, mask], w[:, mask]), "cache rows other than the appended one must be untouched"
+            assert_close(g[:, pos], w[:, pos], atol=5e-4, rtol=1e-4, what=f"appended row of cache {i} at pos {pos}")
+            assert np.array_equal(g[:, pos], np.asarray(plain[i])[:, pos]) or np.allclose(g[:, pos], np.asarray(plain[i])[:, pos], atol=5e-4)
