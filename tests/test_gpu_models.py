@@ -179,6 +179,37 @@ def test_streamed_weights_on_device(hip, tmp_path):
         del gen, m
 
 
+MID_GPT = models.GptConfig(vocab_size=512, context_length=256, embed_dim=256, num_layers=2, num_heads=4, mlp_ratio=4)
+
+
+@pytest.mark.parametrize("prompt_len", [4, 140])
+def test_gpt_f32_decode_on_the_chain(hip, prompt_len):
+    """A GPT-2-shaped f32 model (head_dim 64) decoding on the persistent launch (LayerNorm + linear + bias / GELU /
+    residual phases and the f32 attention: one phase while the cache holds at most 128 positions, two beyond) writes the
+    tokens of the stand-alone kernels and of the oracle, with logits to the f32 bar.  (The default keeps f32 layers this
+    narrow on their own kernels: the option forces the launch.)"""
+    prompt = [int(t) for t in np.random.default_rng(5).integers(0, MID_GPT.vocab_size, prompt_len)]
+    t_ref, l_ref = run_generate(OracleBackend(), models.Gpt, MID_GPT, 9, 10, "F32", std=0.08, prompt=prompt)
+    t_plain, l_plain = run_generate(hip, models.Gpt, MID_GPT, 9, 10, "F32", std=0.08, prompt=prompt)
+    hip.set_option("chain_f32_min_kb", 0)
+    hip.set_option("graphs", 0)   # (a replayed step does not pass the counters)
+    try:
+        ph0 = hip.counter("chain_phases")
+        t_chain, l_chain = run_generate(hip, models.Gpt, MID_GPT, 9, 10, "F32", std=0.08, prompt=prompt)
+        phases, last = hip.counter("chain_phases") - ph0, hip.counter("last_program_launches")
+    finally:
+        hip.set_option("chain_f32_min_kb", 8192)
+        hip.set_option("graphs", 1)
+    # per layer qkv, attention (1 phase, or 2 beyond 128 positions), out-projection, fc, projection; then the lm_head
+    per_step = 2 * (5 if prompt_len + 10 <= 128 else 6) + 1
+    assert last <= 4, "a decode step is two embedding gathers, their sum and ONE persistent launch"
+    assert phases >= 8 * per_step, f"{phases} phases in 10 decode steps"   # (steps that grow the caches run other programs too)
+    assert t_chain == t_plain == t_ref
+    for a, b, c in zip(l_chain, l_plain, l_ref):
+        scale = float(np.abs(c).max())
+        assert np.max(np.abs(a - c)) <= 1e-4 * scale + 5e-4 and np.max(np.abs(a - b)) <= 1e-4 * scale + 5e-4
+
+
 def test_tiny_gpt_kv_cache_equals_full_context(hip):
     # smoke.rs:43-82: KV-cache greedy decode == full-context greedy decode for 16 steps
     m = models.Gpt.random(TINY_GPT, hip, seed=11, std=0.2)
