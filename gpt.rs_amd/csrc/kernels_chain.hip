@@ -159,21 +159,24 @@ struct PhaseRegs {
     const void *x, *gamma, *beta, *bias, *residual, *wscale, *wscale2;
     void* y;
 };
+// (F32: the launch has f32 phases; only those read the LayerNorm offsets, and a register pair that nobody reads is not kept)
+template <bool F32>
 __device__ __forceinline__ void regs_from_table(PhaseRegs& R, const GPTRS_CONST ChainPhase* D) {
     R.K = uni(D->K); R.N = uni(D->N); R.Kw = uni(D->Kw); R.ntiles = uni(D->ntiles); R.upb = uni(D->upb); R.units = uni(D->units);
     R.lds_bytes = uni(D->lds_bytes); R.flags = uni(D->flags); R.wfmt = uni(D->wfmt);
     R.inv_n = __int_as_float(uni(__float_as_int(D->inv_n))); R.eps = __int_as_float(uni(__float_as_int(D->eps)));
-    R.x = uni_ptr(D->x); R.gamma = uni_ptr(D->gamma); R.beta = uni_ptr(D->beta); R.bias = uni_ptr(D->bias); R.residual = uni_ptr(D->residual);
+    R.x = uni_ptr(D->x); R.gamma = uni_ptr(D->gamma); R.beta = F32 ? uni_ptr(D->beta) : nullptr; R.bias = uni_ptr(D->bias); R.residual = uni_ptr(D->residual);
     R.wscale = uni_ptr(D->wscale); R.wscale2 = uni_ptr(D->wscale2); R.y = uni_ptr(D->y);
 }
 #define GPTRS_PD_INT(field) __builtin_amdgcn_readlane(pd, (int)(offsetof(ChainPhase, field) / 4))
 #define GPTRS_PD_PTR(field) ((const void*)(((unsigned long long)(unsigned)__builtin_amdgcn_readlane(pd, (int)(offsetof(ChainPhase, field) / 4) + 1) << 32) | \
                                           (unsigned)__builtin_amdgcn_readlane(pd, (int)(offsetof(ChainPhase, field) / 4))))
+template <bool F32>
 __device__ __forceinline__ void regs_from_lanes(PhaseRegs& R, int pd) {   // pd: dword `lane` of the descriptor
     R.K = GPTRS_PD_INT(K); R.N = GPTRS_PD_INT(N); R.Kw = GPTRS_PD_INT(Kw); R.ntiles = GPTRS_PD_INT(ntiles); R.upb = GPTRS_PD_INT(upb);
     R.units = GPTRS_PD_INT(units); R.lds_bytes = GPTRS_PD_INT(lds_bytes); R.flags = GPTRS_PD_INT(flags); R.wfmt = GPTRS_PD_INT(wfmt);
     R.inv_n = __int_as_float(GPTRS_PD_INT(inv_n)); R.eps = __int_as_float(GPTRS_PD_INT(eps));
-    R.x = GPTRS_PD_PTR(x); R.gamma = GPTRS_PD_PTR(gamma); R.beta = GPTRS_PD_PTR(beta); R.bias = GPTRS_PD_PTR(bias); R.residual = GPTRS_PD_PTR(residual);
+    R.x = GPTRS_PD_PTR(x); R.gamma = GPTRS_PD_PTR(gamma); R.beta = F32 ? GPTRS_PD_PTR(beta) : nullptr; R.bias = GPTRS_PD_PTR(bias); R.residual = GPTRS_PD_PTR(residual);
     R.wscale = GPTRS_PD_PTR(wscale); R.wscale2 = GPTRS_PD_PTR(wscale2); R.y = const_cast<void*>(GPTRS_PD_PTR(y));
 }
 
@@ -697,30 +700,7 @@ __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
     }
     wg_barrier();
     float* partp = P.part;
-    if (P.flags & kChainAttnFinal) {
-        // one chunk per kv head: its record is the whole softmax, and the context row is written here (what the merge of a
-        // single record gives: O / L)
-        for (int idx = t; idx < G * dh / 2; idx += NT) {
-            const int gg = (2 * idx) / dh, d = 2 * idx - gg * dh;
-            float mn = -INFINITY;
-            for (int w = gg; w < NWS; w += G) mn = fmaxf(mn, sm[w]);
-            float Ls = 0.f, O0 = 0.f, O1 = 0.f;
-            if (mn != -INFINITY) {
-                for (int w = gg; w < NWS; w += G) {
-                    const float cw = fast_exp(sm[w] - mn);
-                    Ls += sl[w] * cw;
-                    O0 += so[w * dh + d] * cw;
-                    O1 += so[w * dh + d + 1] * cw;
-                }
-            }
-            const long at = (long)(kvh * G + gg) * dh + d;
-            if (F32) cstore8((float*)P.y + at, (unsigned long long)__float_as_uint(O0 / Ls) | ((unsigned long long)__float_as_uint(O1 / Ls) << 32));
-            else cstore4((bf16_t*)P.y + at, pack_bf16x2(O0 / Ls, O1 / Ls));
-        }
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-        wg_barrier();
-        return true;
-    }
+    const bool final = P.flags & kChainAttnFinal;
     for (int idx = t; idx < G * dh; idx += NT) {
         const int gg = idx / dh, d = idx - gg * dh;
         float mn = -INFINITY;
@@ -732,6 +712,14 @@ __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
                 Ls += sl[w] * cw;
                 O += so[w * dh + d] * cw;
             }
+        }
+        if (final) {
+            // one chunk per kv head: its record is the whole softmax, and the context row is written here (what the merge of
+            // a single record gives: O / L)
+            const long at = (long)(kvh * G + gg) * dh + d;
+            if (F32) cstore4((float*)P.y + at, __float_as_uint(O / Ls));
+            else __hip_atomic_store(as_global((unsigned short*)P.y + at), (unsigned short)pack_bf16x2(O / Ls, 0.f), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            continue;
         }
         float* rec = partp + ((long)(kvh * G + gg) * nch + c) * (dh + 2);
         if (d == 0) { cstore4(rec, __float_as_uint(mn)); cstore4(rec + 1, __float_as_uint(Ls)); }
@@ -882,7 +870,7 @@ __device__ void control_wave(Shared& sh, unsigned* xs, const ChainPhase* phases,
         } else if (u0 < u1) {
             if (lane == 0) lds_st(&sh.go, ph);
             PhaseRegs P;
-            regs_from_lanes(P, pd);
+            regs_from_lanes<FMT == kChainW32>(P, pd);
             const int flags = P.flags, ntiles = P.ntiles, N = P.N;
             const bool dual = flags & kChainDual;
             const int cpt = dual ? 2 : 4;              // output columns per tile
@@ -1186,7 +1174,7 @@ __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, 
             c_sidx = 0;   // int4: entry of the unit's first tile and group in the staged scales ...
             c_soff = uni(D->lds_bytes) >> 2;   // ... which sit behind the activations
             PhaseRegs R;
-            regs_from_table(R, D);
+            regs_from_table<FMT == kChainW32>(R, D);
             if (!wait_go(&sh.go, &sh.abort, c_phase, budget)) return false;
             if (FMT == kChainW32) stage_block_f32(R, const_cast<unsigned*>(xs), sh.ssq);
             else stage_block(R, const_cast<unsigned*>(xs), sh.ssq);
