@@ -507,9 +507,253 @@ __device__ __forceinline__ void lane_pair(float v, int off, float& a, float& b) 
 // the waves of different heads re-read the same rows out of the caches.  Cache rows older than
 // this launch are requested BEFORE the grid barrier is awaited (they do not depend on the
 // previous phase); only the query row and this step's K/V row are read after it.
-// F32: the query row, this step's K / V row and the caches are f32 (a lane's 8 values are two 16-byte words; no RoPE).
-template <bool F32>
 __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const ChainPhase& P, GPTRS_LDS float* lds, int unit, int phase,
+                             unsigned long long budget) {
+    constexpr int PP = 4;   // positions per lane group requested ahead of the barrier
+    const int t = local_tid(), lane = t & 63, wave = uni(t >> 6);
+    const bool control = wave == NWS;
+    const int dh = P.head_dim, n_q = P.n_q, n_kv = P.n_kv, nch = P.nch, half = P.rot_half;
+    const int G = n_q / n_kv, nparts = NWS / G;
+    const long cap = P.capacity;
+    const int lpr = dh >> 3, rpw = 64 / lpr, sub = lane / lpr, li = lane % lpr;
+    const int g = wave % G, part = wave / G;
+    const int stride = nparts * rpw, sid = part * rpw + sub;   // position slots of this head's waves
+    const int kvh = unit / nch, c = unit - kvh * nch;
+    const bf16_t* qkv = (const bf16_t*)P.x;
+    bf16_t* kc = (bf16_t*)P.k_cache;
+    bf16_t* vc = (bf16_t*)P.v_cache;
+    const bf16_t* cs = (const bf16_t*)P.cos;
+    const bf16_t* sn = (const bf16_t*)P.sin;
+    const long qpos = clampl(uni(gload(P.query_start)), 0, cap - 1);       // DynamicSlice clamp (cpu.rs:804-820)
+    const long upd = clampl(uni(gload(P.update_starts + 1)), 0, cap - 1);  // DynamicUpdateSlice clamp
+    const float scale = P.scale;
+    const long L = qpos + 1, CL = (L + nch - 1) / nch;
+    const long p0 = c * CL, p1 = min(L, p0 + CL);
+    const int owner = (int)min(upd / CL, (long)nch - 1);
+    const bf16_t* knew = qkv + (long)n_q * dh + (long)kvh * dh;
+    const bf16_t* vnew = qkv + (long)(n_q + n_kv) * dh + (long)kvh * dh;
+    const int c0 = li * 8;
+    uint4 kraw[PP], vraw[PP];
+#pragma unroll
+    for (int j = 0; j < PP; ++j) {
+        const long p = p0 + sid + (long)j * stride;
+        if (!control && p < p1 && p != upd) {
+            const long row = ((long)kvh * cap + p) * dh + c0;
+            kraw[j] = gload4(kc + row);
+            vraw[j] = gload4(vc + row);
+        } else {
+            kraw[j] = make_uint4(0, 0, 0, 0);
+            vraw[j] = make_uint4(0, 0, 0, 0);
+        }
+    }
+    if (!control && !wait_go(go, abort, phase, budget)) return false;
+
+    float m = -INFINITY, l = 0.f, o[8];
+#pragma unroll
+    for (int v = 0; v < 8; ++v) o[v] = 0.f;
+    if (!control) {
+        // the wave's query head (RoPE applied on the fly) and, in the first lane group of each head's
+        // first wave of the workgroup that owns position `upd`, this step's K/V row: all requested
+        // before any is consumed
+        const bool rot = cs != nullptr && c0 < 2 * half;
+        const bool first = c0 < half;
+        const int j0 = first ? c0 : c0 - half, co = first ? c0 + half : c0 - half;
+        float cosv[8], sinv[8];
+        if (rot) { load_bf16x8(cs + j0, cosv); load_bf16x8(sn + j0, sinv); }
+        const bf16_t* head = qkv + (long)(kvh * G + g) * dh;
+        unsigned long long qa[2], qb[2] = {0ull, 0ull};
+        qa[0] = cload8(head + c0); qa[1] = cload8(head + c0 + 4);
+        if (rot) { qb[0] = cload8(head + co); qb[1] = cload8(head + co + 4); }
+        const bool fresh = c == owner && sid == 0;           // this lane group handles the new row
+        unsigned long long ka[2] = {0ull, 0ull}, kb[2] = {0ull, 0ull}, va[2] = {0ull, 0ull};
+        if (fresh) {
+            ka[0] = cload8(knew + c0); ka[1] = cload8(knew + c0 + 4);
+            if (rot) { kb[0] = cload8(knew + co); kb[1] = cload8(knew + co + 4); }
+            va[0] = cload8(vnew + c0); va[1] = cload8(vnew + c0 + 4);
+        }
+        auto rope = [&](const unsigned long long (&own2)[2], const unsigned long long (&oth2)[2], float (&out)[8]) {
+            float own[8], other[8];
+            unpack8(own2[0], own2[1], own);
+            if (!rot) {
+#pragma unroll
+                for (int v = 0; v < 8; ++v) out[v] = own[v];
+                return;
+            }
+            unpack8(oth2[0], oth2[1], other);
+#pragma unroll
+            for (int v = 0; v < 8; ++v)
+                out[v] = rbf(first ? own[v] * cosv[v] - other[v] * sinv[v] : own[v] * cosv[v] + other[v] * sinv[v]);
+        };
+        float qf[8];
+        rope(qa, qb, qf);
+
+        auto visit = [&](const float (&kf)[8], const float (&vf)[8]) {
+            float sc = 0.f;
+#pragma unroll
+            for (int v = 0; v < 8; ++v) sc += qf[v] * kf[v];
+            sc = group_sum(sc, lpr) * scale;
+            const float mn = fmaxf(m, sc);
+            const float corr = fast_exp(m - mn);
+            const float pe = fast_exp(sc - mn);
+            l = l * corr + pe;
+#pragma unroll
+            for (int v = 0; v < 8; ++v) o[v] = o[v] * corr + pe * vf[v];
+            m = mn;
+        };
+#pragma unroll
+        for (int j = 0; j < PP; ++j) {
+            const long p = p0 + sid + (long)j * stride;
+            if (p < p1 && p != upd) {
+                float kf[8], vf[8];
+                unpack_u4(kraw[j], kf);
+                unpack_u4(vraw[j], vf);
+                visit(kf, vf);
+            }
+        }
+        for (long p = p0 + sid + (long)PP * stride; p < p1; p += stride) {
+            if (p == upd) continue;
+            float kf[8], vf[8];
+            const long row = ((long)kvh * cap + p) * dh + c0;
+            load_bf16x8(kc + row, kf);
+            load_bf16x8(vc + row, vf);
+            visit(kf, vf);
+        }
+        if (fresh) {   // this step's row: attended to when in range; appended once (by head 0's wave)
+            float kf[8], vf[8];
+            rope(ka, kb, kf);
+            unpack8(va[0], va[1], vf);
+            if (g == 0) {
+                const long row = ((long)kvh * cap + upd) * dh + c0;
+                gstore4(kc + row, make_uint4(pack_bf16x2(kf[0], kf[1]), pack_bf16x2(kf[2], kf[3]), pack_bf16x2(kf[4], kf[5]), pack_bf16x2(kf[6], kf[7])));
+                gstore4(vc + row, make_uint4((unsigned)va[0], (unsigned)(va[0] >> 32), (unsigned)va[1], (unsigned)(va[1] >> 32)));
+            }
+            if (upd >= p0 && upd < p1) visit(kf, vf);
+        }
+        // merge the lane groups of this wave
+        for (int off = lpr; off < 64; off <<= 1) {
+            float ma, mb, la, lb;
+            lane_pair(m, off, ma, mb);
+            lane_pair(l, off, la, lb);
+            const float mn = fmaxf(ma, mb);
+            const float ca = mn == -INFINITY ? 0.f : fast_exp(ma - mn);
+            const float cb = mn == -INFINITY ? 0.f : fast_exp(mb - mn);
+            l = la * ca + lb * cb;
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                float oa, ob;
+                lane_pair(o[v], off, oa, ob);
+                o[v] = oa * ca + ob * cb;
+            }
+            m = mn;
+        }
+    }
+    // merge the waves of each head through LDS and leave one record per query head
+    GPTRS_LDS float* sm = lds;
+    GPTRS_LDS float* sl = lds + NWS;
+    GPTRS_LDS float* so = lds + 2 * NWS;
+    if (!control && sub == 0) {
+        if (li == 0) { sm[wave] = m; sl[wave] = l; }
+#pragma unroll
+        for (int v = 0; v < 8; ++v) so[wave * dh + c0 + v] = o[v];
+    }
+    wg_barrier();
+    float* partp = P.part;
+    const bool final = P.flags & kChainAttnFinal;
+    for (int idx = t; idx < G * dh; idx += NT) {
+        const int gg = idx / dh, d = idx - gg * dh;
+        float mn = -INFINITY;
+        for (int w = gg; w < NWS; w += G) mn = fmaxf(mn, sm[w]);
+        float Ls = 0.f, O = 0.f;
+        if (mn != -INFINITY) {
+            for (int w = gg; w < NWS; w += G) {
+                const float cw = fast_exp(sm[w] - mn);
+                Ls += sl[w] * cw;
+                O += so[w * dh + d] * cw;
+            }
+        }
+        if (final) {
+            // one chunk per kv head: its record is the whole softmax, and the context row is written here (what the merge of
+            // a single record gives: O / L)
+            __hip_atomic_store(as_global((unsigned short*)P.y + (long)(kvh * G + gg) * dh + d), (unsigned short)pack_bf16x2(O / Ls, 0.f),
+                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            continue;
+        }
+        float* rec = partp + ((long)(kvh * G + gg) * nch + c) * (dh + 2);
+        if (d == 0) { cstore4(rec, __float_as_uint(mn)); cstore4(rec + 1, __float_as_uint(Ls)); }
+        cstore4(rec + 2 + d, __float_as_uint(O));
+    }
+    // every lane's stores (record words, the appended cache row) have left the CU before the control wave, which passes
+    // this barrier last of all it executes here, reports the workgroup's arrival
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    wg_barrier();
+    return true;
+}
+
+// unit = query head: softmax-merge of its nch chunk records into the context row.  Thread
+// (sg, d2) reads the records of the chunks s = sg, sg + NW, ... for the dims (2 d2, 2 d2 + 1) in
+// one round of loads and merges them locally; the NW subsets meet in LDS.
+__device__ bool attn_combine(GPTRS_LDS int* go, GPTRS_LDS int* abort, const ChainPhase& P, GPTRS_LDS float* lds, int hq, int phase,
+                             unsigned long long budget) {
+    constexpr int MAXC = 8;   // chunks per thread: nch <= MAXC * NW
+    const int t = local_tid(), wave = uni(t >> 6);
+    const int dh = P.head_dim, nch = P.nch;
+    if (wave != NWS && !wait_go(go, abort, phase, budget)) return false;
+    const float* base = P.part + (long)hq * nch * (dh + 2);
+    bf16_t* ctx = (bf16_t*)P.y;
+    const int h2 = dh / 2;
+    for (int d0 = 0; d0 < h2; d0 += 64) {
+        const int d2 = d0 + (t & 63);
+        const bool act = d2 < h2;
+        unsigned long long ml[MAXC], ov[MAXC];
+#pragma unroll
+        for (int u = 0; u < MAXC; ++u) {
+            const int s = wave + u * NW;
+            const bool ok = act && s < nch;
+            ml[u] = ok ? cload8(base + (long)s * (dh + 2)) : 0ull;
+            ov[u] = ok ? cload8(base + (long)s * (dh + 2) + 2 + 2 * d2) : 0ull;
+        }
+        float mn = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < MAXC; ++u)
+            if (wave + u * NW < nch) mn = fmaxf(mn, __uint_as_float((unsigned)ml[u]));
+        float Ls = 0.f, o0 = 0.f, o1 = 0.f;
+#pragma unroll
+        for (int u = 0; u < MAXC; ++u) {
+            if (wave + u * NW < nch) {
+                const float ms = __uint_as_float((unsigned)ml[u]);
+                const float cw = ms == -INFINITY ? 0.f : fast_exp(ms - mn);
+                Ls += __uint_as_float((unsigned)(ml[u] >> 32)) * cw;
+                o0 += __uint_as_float((unsigned)ov[u]) * cw;
+                o1 += __uint_as_float((unsigned)(ov[u] >> 32)) * cw;
+            }
+        }
+        GPTRS_LDS f32x4* rec = (GPTRS_LDS f32x4*)lds;
+        { f32x4 r4; r4.x = mn; r4.y = Ls; r4.z = o0; r4.w = o1; rec[wave * 64 + (t & 63)] = r4; }
+        wg_barrier();
+        if (wave == 0 && act) {
+            float M = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) M = fmaxf(M, rec[w * 64 + t].x);
+            float Lt = 0.f, a0 = 0.f, a1 = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) {
+                const f32x4 r = rec[w * 64 + t];
+                const float cw = r.x == -INFINITY ? 0.f : fast_exp(r.x - M);
+                Lt += r.y * cw; a0 += r.z * cw; a1 += r.w * cw;
+            }
+            cstore4(ctx + (long)hq * dh + 2 * d2, pack_bf16x2(a0 / Lt, a1 / Lt));
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the context words are out before the arrival is reported
+        wg_barrier();
+    }
+    return true;
+}
+
+// The two attention phases once more with the element type as a parameter, instantiated for f32 rows and caches only (a
+// lane's 8 values are then two 16-byte words; no RoPE): written this way the bf16 phases above lost a microsecond each
+// to the compiler, so they keep their own text.
+template <bool F32>
+__device__ bool attn_partial_t(GPTRS_LDS int* go, GPTRS_LDS int* abort, const ChainPhase& P, GPTRS_LDS float* lds, int unit, int phase,
                              unsigned long long budget) {
     typedef typename std::conditional<F32, float, bf16_t>::type E;
     constexpr int PP = F32 ? 2 : 4;   // positions per lane group requested ahead of the barrier
@@ -736,7 +980,7 @@ __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const Chai
 // (sg, d2) reads the records of the chunks s = sg, sg + NW, ... for the dims (2 d2, 2 d2 + 1) in
 // one round of loads and merges them locally; the NW subsets meet in LDS.
 template <bool F32>
-__device__ bool attn_combine(GPTRS_LDS int* go, GPTRS_LDS int* abort, const ChainPhase& P, GPTRS_LDS float* lds, int hq, int phase,
+__device__ bool attn_combine_t(GPTRS_LDS int* go, GPTRS_LDS int* abort, const ChainPhase& P, GPTRS_LDS float* lds, int hq, int phase,
                              unsigned long long budget) {
     constexpr int MAXC = 8;   // chunks per thread: nch <= MAXC * NW
     const int t = local_tid(), wave = uni(t >> 6);
@@ -812,8 +1056,13 @@ __device__ __forceinline__ bool run_attn_phase(const GPTRS_CONST ChainPhase* php
     const int kind = P.kind, units = P.units;
     for (int u = blockIdx.x; u < units; u += gridDim.x) {
         bool ok;
-        if (kind == kChainAttnCombine) ok = attn_combine<F32>(go, abort, P, lds, u, phase, budget);
-        else ok = attn_partial<F32>(go, abort, P, lds, u, phase, budget);
+        if (F32) {
+            if (kind == kChainAttnCombine) ok = attn_combine_t<true>(go, abort, P, lds, u, phase, budget);
+            else ok = attn_partial_t<true>(go, abort, P, lds, u, phase, budget);
+        } else {
+            if (kind == kChainAttnCombine) ok = attn_combine(go, abort, P, lds, u, phase, budget);
+            else ok = attn_partial(go, abort, P, lds, u, phase, budget);
+        }
         if (!ok) return false;
     }
     return true;
