@@ -41,7 +41,7 @@ MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 # rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a copy kernel of known size (commands and raw figures: `profile`).  The
 # figure belongs to ONE version of the kernel: `source_sha256` is the hash of gpt.rs_amd/csrc/kernels_chain.hip it was
 # measured on, and `roofline.traffic` is null whenever the file in the tree hashes differently.
-CHAIN_TRAFFIC = {"bytes": 7.0184e9 + 0.0279e9, "source_sha256": "e107eb98b5752852873a5b978693f11538dd7b4d3bc726cc72cc106131a91278",
+CHAIN_TRAFFIC = {"bytes": 7.0184e9 + 0.0279e9, "source_sha256": "253fbf93e863204bcf87bf713c9dbdc4213318f03409c700052e1ba5df94fbc0",
                  "profile": "profiles/chain_kernel_ministral3b_bf16_b1_decode.md"}
 
 
