@@ -222,12 +222,22 @@ const k::ChainPhase* Backend::chain_table(const std::vector<k::ChainPhase>& phas
     for (auto& t : chain_tables_)
         if (t.host.size() == phases.size() && !memcmp(t.host.data(), phases.data(), bytes)) {
             t.last_use = ++chain_clock_;
+            if (capturing) t.recorded = true;
             return (const k::ChainPhase*)t.dev->ptr;
         }
     if (capturing) fail_exec("chain table missing while recording a graph");
-    // Recorded graphs keep table addresses, so a table is never freed while the backend lives;
-    // past the cap the caller runs the linears one by one instead.
-    if (chain_tables_.size() >= 4096) return nullptr;
+    // A recorded graph keeps the address of its table, so such a table lives as long as the backend.  The others (a
+    // launch whose buffer addresses never come back: streamed weights, growing caches) go, least recently used first,
+    // once there are 64 of them; the stream orders the reuse of their memory behind the launch that read them.
+    size_t loose = 0;
+    for (auto& t : chain_tables_) loose += t.recorded ? 0 : 1;
+    if (loose >= 64) {
+        size_t victim = chain_tables_.size();
+        for (size_t i = 0; i < chain_tables_.size(); ++i)
+            if (!chain_tables_[i].recorded && (victim == chain_tables_.size() || chain_tables_[i].last_use < chain_tables_[victim].last_use)) victim = i;
+        chain_tables_.erase(chain_tables_.begin() + (std::ptrdiff_t)victim);
+    }
+    if (chain_tables_.size() >= 4096) return nullptr;   // (all recorded: the caller runs the linears one by one instead)
     ChainTable t;
     t.host = phases;
     t.dev = new_buffer(bytes);

@@ -253,7 +253,7 @@ class Backend {
     std::map<std::array<uint64_t, 3>, Derived> tiled_cache_;
     std::atomic<int> dead_sources_{0};  // weights with derived layouts that were freed since the last sweep
     unsigned* d_chain_bar_ = nullptr;
-    struct ChainTable { std::vector<k::ChainPhase> host; BufferP dev; uint64_t last_use = 0; };
+    struct ChainTable { std::vector<k::ChainPhase> host; BufferP dev; uint64_t last_use = 0; bool recorded = false; };
     std::vector<ChainTable> chain_tables_;
     uint64_t chain_clock_ = 0;
     uint64_t next_buffer_id_ = 1;

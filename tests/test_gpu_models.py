@@ -179,6 +179,26 @@ def test_streamed_weights_on_device(hip, tmp_path):
         del gen, m
 
 
+def test_streamed_decode_keeps_its_launches_and_its_memory(hip, tmp_path):
+    """Streamed weights give every decode step new buffer addresses, hence a new table of phases for the persistent
+    launch: tables that no recorded graph refers to are dropped least recently used first, so step 120 still runs as one
+    launch and the memory in use has stopped growing long before."""
+    from gptrs_amd import loader
+    from gptrs_amd.loader import WeightStreamingConfig as WS
+    ref = models.Ministral.random(MID_MINISTRAL, OracleBackend(), seed=6, dtype="F32", std=0.05)
+    path = str(tmp_path / "s.gptrs")
+    ref.save_checkpoint(path, "ministral", ref.checkpoint_config(), runtime={"weight_streaming": WS(enabled=True).to_json()})
+    m = loader.load_model(hip, path, dtype="Bf16")
+    gen = models.Generator(m, PROMPT, kv_cache_capacity=128)
+    gen.generate(80)
+    hip.synchronize()
+    mem, launches = hip.counter("bytes_allocated"), hip.counter("chain_launches")
+    gen.generate(40)
+    hip.synchronize()
+    assert hip.counter("chain_launches") - launches >= 39, "every streamed step still runs its linears as one launch"
+    assert hip.counter("bytes_allocated") <= mem + (16 << 10), "tables of phases and weight layouts of steps gone by are given back"
+
+
 MID_GPT = models.GptConfig(vocab_size=512, context_length=256, embed_dim=256, num_layers=2, num_heads=4, mlp_ratio=4)
 
 
