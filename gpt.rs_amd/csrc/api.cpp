@@ -208,6 +208,7 @@ void Backend::drop_derived_weights() {
         for (auto& g : p.graphs) {
             if (g.exec) (void)hipGraphExecDestroy(g.exec);
             if (g.graph) (void)hipGraphDestroy(g.graph);
+            release_graph_tables(g);
         }
         p.graphs.clear();
         p.seen_keys.clear();
@@ -217,27 +218,33 @@ void Backend::drop_derived_weights() {
     pool_.trim();
 }
 
+void Backend::release_graph_tables(const PlanGraph& g) {
+    for (const void* p : g.tables)
+        for (auto& t : chain_tables_)
+            if (t.dev->ptr == p) { if (t.refs > 0) --t.refs; break; }
+}
+
 const k::ChainPhase* Backend::chain_table(const std::vector<k::ChainPhase>& phases) {
     const size_t bytes = phases.size() * sizeof(k::ChainPhase);
     for (auto& t : chain_tables_)
         if (t.host.size() == phases.size() && !memcmp(t.host.data(), phases.data(), bytes)) {
             t.last_use = ++chain_clock_;
-            if (capturing) t.recorded = true;
+            if (capturing) capture_tables_.push_back(t.dev->ptr);
             return (const k::ChainPhase*)t.dev->ptr;
         }
     if (capturing) fail_exec("chain table missing while recording a graph");
-    // A recorded graph keeps the address of its table, so such a table lives as long as the backend.  The others (a
+    // A recorded graph keeps the address of its table, so such a table lives as long as the graph.  The others (a
     // launch whose buffer addresses never come back: streamed weights, growing caches) go, least recently used first,
     // once there are 64 of them; the stream orders the reuse of their memory behind the launch that read them.
     size_t loose = 0;
-    for (auto& t : chain_tables_) loose += t.recorded ? 0 : 1;
+    for (auto& t : chain_tables_) loose += t.refs > 0 ? 0 : 1;
     if (loose >= 64) {
         size_t victim = chain_tables_.size();
         for (size_t i = 0; i < chain_tables_.size(); ++i)
-            if (!chain_tables_[i].recorded && (victim == chain_tables_.size() || chain_tables_[i].last_use < chain_tables_[victim].last_use)) victim = i;
+            if (chain_tables_[i].refs == 0 && (victim == chain_tables_.size() || chain_tables_[i].last_use < chain_tables_[victim].last_use)) victim = i;
         chain_tables_.erase(chain_tables_.begin() + (std::ptrdiff_t)victim);
     }
-    if (chain_tables_.size() >= 4096) return nullptr;   // (all recorded: the caller runs the linears one by one instead)
+    if (chain_tables_.size() >= 4096) return nullptr;   // (all held by graphs: the caller runs the linears one by one instead)
     ChainTable t;
     t.host = phases;
     t.dev = new_buffer(bytes);
@@ -504,6 +511,7 @@ std::shared_ptr<Plan> Backend::get_plan(const char* json, size_t len, uint64_t k
         plan_lru_.emplace_front(k2, plan);
         plan_index_[k2] = plan_lru_.begin();
         while (plan_lru_.size() > 64) {  // program LRU of 64, as the reference arena keeps (plan.rs:20-29)
+            for (auto& g : plan_lru_.back().second->graphs) release_graph_tables(g);
             plan_index_.erase(plan_lru_.back().first);
             plan_lru_.pop_back();
         }
@@ -590,6 +598,7 @@ bool Backend::run_graphed(Plan& plan, ExecCtx& cx, const std::vector<BufferP>& o
     PlanGraph pg;
     pg.key = std::move(key);
     GPTRS_HIP_CHECK(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+    capture_tables_.clear();
     capturing = true;
     std::string err;
     try {
@@ -619,6 +628,10 @@ bool Backend::run_graphed(Plan& plan, ExecCtx& cx, const std::vector<BufferP>& o
         return false;
     }
     pg.launches = cx.launches;
+    pg.tables = capture_tables_;
+    for (const void* p : pg.tables)
+        for (auto& t : chain_tables_)
+            if (t.dev->ptr == p) { ++t.refs; break; }
     pg.last_use = ++plan.graph_clock;
     ++plan.graph_builds;
     ++n_graphs_built;
@@ -627,6 +640,7 @@ bool Backend::run_graphed(Plan& plan, ExecCtx& cx, const std::vector<BufferP>& o
                                     [](const PlanGraph& a, const PlanGraph& b) { return a.last_use < b.last_use; });
         (void)hipGraphExecDestroy(lru->exec);
         (void)hipGraphDestroy(lru->graph);
+        release_graph_tables(*lru);
         plan.graphs.erase(lru);
     }
     GPTRS_HIP_CHECK(hipGraphLaunch(pg.exec, stream));
@@ -1056,6 +1070,7 @@ int64_t gptrs_hip_counter(const gptrs_hip_backend* b, const char* name) {
     if (!strcmp(name, "graphs_refused")) return i.n_graphs_refused;
     if (!strcmp(name, "chain_launches")) return i.n_chain_launches;
     if (!strcmp(name, "chain_phases")) return i.n_chain_phases;
+    if (!strcmp(name, "chain_tables")) return i.chain_table_count();
     return -1;
 }
 

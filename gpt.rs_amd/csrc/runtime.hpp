@@ -115,6 +115,7 @@ struct PlanGraph {
     hipGraphExec_t exec = nullptr;
     uint64_t last_use = 0;
     int64_t launches = 0;
+    std::vector<const void*> tables;  // device tables of phases that its persistent launches read
 };
 
 struct Plan {
@@ -253,7 +254,12 @@ class Backend {
     std::map<std::array<uint64_t, 3>, Derived> tiled_cache_;
     std::atomic<int> dead_sources_{0};  // weights with derived layouts that were freed since the last sweep
     unsigned* d_chain_bar_ = nullptr;
-    struct ChainTable { std::vector<k::ChainPhase> host; BufferP dev; uint64_t last_use = 0; bool recorded = false; };
+    struct ChainTable { std::vector<k::ChainPhase> host; BufferP dev; uint64_t last_use = 0; int refs = 0; };   // refs: recorded graphs that hold its address
+    std::vector<const void*> capture_tables_;   // tables looked up while a graph is being recorded
+    void release_graph_tables(const PlanGraph& g);
+  public:
+    int64_t chain_table_count() const { return (int64_t)chain_tables_.size(); }
+  private:
     std::vector<ChainTable> chain_tables_;
     uint64_t chain_clock_ = 0;
     uint64_t next_buffer_id_ = 1;

@@ -199,6 +199,27 @@ def test_streamed_decode_keeps_its_launches_and_its_memory(hip, tmp_path):
     assert hip.counter("bytes_allocated") <= mem + (16 << 10), "tables of phases and weight layouts of steps gone by are given back"
 
 
+def test_many_sequences_do_not_pile_up_tables_of_phases(hip):
+    """Each live sequence has its own caches, hence its own buffer addresses, recorded graph and table of phases for the
+    persistent launch; a program keeps 8 graphs, and a table goes when the last graph that holds its address has gone
+    (64 loose tables are kept for launches that are not recorded)."""
+    m = models.Ministral.random(MID_MINISTRAL, hip, seed=4, dtype="Bf16", std=0.05)
+    held = hip.counter("chain_tables")    # the graphs of programs that ran before this test keep theirs
+    first = models.Generator(m, PROMPT, kv_cache_capacity=64)
+    want = first.generate(6)
+    gens, seen = [], []
+    for i in range(160):
+        g = models.Generator(m, PROMPT, kv_cache_capacity=64)
+        assert g.generate(6) == want
+        gens.append(g)
+        if i in (99, 159):
+            hip.synchronize()
+            seen.append(hip.counter("chain_tables"))
+    # this model's two programs (prefill, decode step) hold at most 8 graphs each
+    assert seen[0] <= held + 64 + 2 * 8 and seen[1] <= seen[0], (held, seen)
+    assert first.generate(4) == gens[0].generate(4)   # an early sequence goes on (its graph is recorded again)
+
+
 MID_GPT = models.GptConfig(vocab_size=512, context_length=256, embed_dim=256, num_layers=2, num_heads=4, mlp_ratio=4)
 
 
