@@ -457,6 +457,299 @@ __global__ __launch_bounds__(256 * KW) void gemm_mfma_kernel(const T* __restrict
         }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// bf16 GEMM whose tiles go memory -> LDS without passing through registers (global_load_lds_dwordx4), for unquantised
+// bf16 operands.  Against the kernel above: no staging registers and no LDS store instructions, a ring of NST staged
+// tiles (loads run NST - 1 tiles ahead), and tile shapes chosen per launch so that the tiles fill the 256 CUs in whole
+// rounds (128 x 192 and 128 x 96 as well as 128 x 128).
+//
+// Workgroup: KW groups of WM x WN waves.  A wave owns 64 x (32 TN) outputs as 2 x TN fragments of 32 x 32; the tile is
+// (64 WM) x (32 TN WN).  All groups share the staged tiles; group g multiplies k-steps [g KSW, (g + 1) KSW) of every
+// tile (KSW = 4 / KW k-steps of 16) and the groups' sums meet through LDS before the epilogue, so a launch of one tile
+// per CU still has 8 waves per CU.
+//
+// LDS, per stage: A as rows of 128 bytes (64 k), B k-group-major ([k-group][column][8 k]).  One load instruction moves
+// 64 x 16 bytes to 1 KiB of consecutive LDS, lane l to byte 16 l, so the layout is fixed by WHICH 16 bytes of memory a
+// lane asks for: in A, position p of row r holds k-group p ^ ((r >> 1) & 7); eight lanes still read one row's 128
+// contiguous bytes, and a fragment read (32 rows x 2 k-groups) touches every bank once per 16 lanes.  B fragments are
+// contiguous as they are.
+//
+// Order of issue, fixed by hand with scheduling barriers: the fragments of the next k-step are requested before the
+// MFMAs of this one; in a tile's last k-step half the MFMAs are issued, then the wave waits for its own loads of the
+// next tile (vmcnt, which counts only LDS-direct loads here), passes the barrier that makes that tile complete and this
+// one free, requests the tile NST ahead into the freed stage and the next tile's first fragments, and issues the other
+// half.  Loads past the last tile repeat it into a stage nobody reads, so the count the wait relies on never changes.
+// DUAL (SwiGLU pair): the tile's first BN / 2 columns are columns of W, the others the same columns of W2.
+__device__ __forceinline__ void gemm_lds_load16(const void* gptr, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(lds_addr) : "memory", "m0");
+}
+template <int N> __device__ __forceinline__ void gemm_wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory"); }
+
+template <int NST, int WM, int WN, int TN, int KW, bool DUAL>
+__global__ __launch_bounds__(64 * WM * WN * KW) void gemm_dma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wk,
+                                                                   const bf16_t* __restrict__ wk2, const bf16_t* __restrict__ bias,
+                                                                   const bf16_t* __restrict__ residual, bf16_t* __restrict__ y,
+                                                                   int M, int K, int N, int Npad, int act, int NT, int MT, int out_f32) {
+    constexpr int BK = 64, KG = 8, ROWB = 128;
+    constexpr int BM = 64 * WM, BN = 32 * TN * WN, NW = WM * WN * KW;
+    constexpr int NREAL = DUAL ? BN / 2 : BN;                          // output columns per tile
+    constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
+    constexpr int LAI = A_BYTES / 1024, LBI = B_BYTES / 1024;          // load instructions per tile
+    constexpr int LA = (LAI + NW - 1) / NW, LB = (LBI + NW - 1) / NW;  // per wave (a wave past the end repeats an earlier one)
+    constexpr int LPT = LA + LB;
+    constexpr int KSW = 4 / KW;
+    static_assert(KSW == 2 || KSW == 4, "an even number of k-steps per wave and tile: the last one's fragments sit in slot 1");
+    static_assert(!DUAL || WN == 2, "pair tiles: wave column 0 multiplies W, wave column 1 the same columns of W2");
+    static_assert((NST - 2) * LPT < 64, "vmcnt is a 6-bit counter");
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wg = wave / (WM * WN), wq = wave % (WM * WN);
+    const int wm = wq / WN, wn = wq % WN;
+    int bx, by;
+    {
+        // XCD c takes a contiguous range of a grouped tile order (see gemm_mfma_kernel)
+        const int total = NT * MT, per = (total + 7) / 8;
+        const int v = (int)(blockIdx.x % 8) * per + (int)(blockIdx.x / 8);
+        if (v >= total) return;
+        const int gsz = 8 * NT, g = v / gsz, first = g * 8;
+        const int gm = MT - first < 8 ? MT - first : 8;
+        by = first + (v % gsz) % gm;
+        bx = (v % gsz) / gm;
+    }
+    const int m0 = by * BM, n0 = bx * NREAL;
+    // what each of this wave's load instructions fetches (per lane) and where its KiB goes
+    const unsigned char* a_src[LA];
+    const unsigned char* b_src[LB];
+    unsigned a_dst[LA], b_dst[LB];
+#pragma unroll
+    for (int j = 0; j < LA; ++j) {
+        const int q = (wave * LA + j) % LAI;
+        const int sl = q * 64 + lane, row = sl / KG, pos = sl % KG;
+        int m = m0 + row;
+        if (m > M - 1) m = M - 1;
+        a_src[j] = reinterpret_cast<const unsigned char*>(x + (int64_t)m * K) + ((pos ^ ((row >> 1) & 7)) * 16);
+        a_dst[j] = q * 1024;
+    }
+#pragma unroll
+    for (int j = 0; j < LB; ++j) {
+        const int q = (wave * LB + j) % LBI;
+        const int sl = q * 64 + lane, kg = sl / BN, bc = sl % BN;
+        int col = n0 + bc;
+        const bf16_t* src = wk;
+        if (DUAL) {
+            col = n0 + bc % NREAL;
+            src = bc >= NREAL ? wk2 : wk;
+        }
+        if (col > Npad - 1) col = Npad - 1;
+        b_src[j] = reinterpret_cast<const unsigned char*>(src) + ((int64_t)kg * Npad + col) * 16;
+        b_dst[j] = A_BYTES + q * 1024;
+    }
+    const int64_t b_tile_step = (int64_t)KG * Npad * 16;
+    const unsigned lds0 = (unsigned)(uintptr_t)lds;
+    const int nt = K / BK;
+    auto issue = [&](int t, int st) {
+        if (t > nt - 1) t = nt - 1;
+        const unsigned sbase = lds0 + st * STAGE;
+#pragma unroll
+        for (int j = 0; j < LA; ++j)
+            gemm_lds_load16(a_src[j] + (int64_t)t * (BK * 2), (unsigned)__builtin_amdgcn_readfirstlane((int)(sbase + a_dst[j])));
+#pragma unroll
+        for (int j = 0; j < LB; ++j)
+            gemm_lds_load16(b_src[j] + (int64_t)t * b_tile_step, (unsigned)__builtin_amdgcn_readfirstlane((int)(sbase + b_dst[j])));
+    };
+    f32x16_t acc[2][TN];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    const int fsel = lane >> 5;
+    const int b_rd = A_BYTES + (wn * 32 * TN + (lane & 31)) * 16;
+    bf16x8_t af[2][2], bfr[2][TN];
+    auto fread = [&](int st, int kk, int slot) {   // kk: k-step of the tile
+        const unsigned char* base = lds + st * STAGE;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int row = wm * 64 + i * 32 + (lane & 31), kg = 2 * kk + fsel;
+            af[slot][i] = *reinterpret_cast<const bf16x8_t*>(base + row * ROWB + ((kg ^ ((row >> 1) & 7)) * 16));
+        }
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bfr[slot][j] = *reinterpret_cast<const bf16x8_t*>(base + b_rd + (2 * kk + fsel) * (BN * 16) + j * 512);
+    };
+    for (int st = 0; st < NST - 1; ++st) issue(st, st);
+    gemm_wait_loads<(NST - 2) * LPT>();
+    __syncthreads();
+    issue(NST - 1, NST - 1);
+    fread(0, wg * KSW, 0);
+    int st = 0;
+    for (int t = 0; t < nt; ++t) {
+        const int st1 = st + 1 == NST ? 0 : st + 1;
+#pragma unroll
+        for (int kk = 0; kk < KSW; ++kk) {
+            if (kk + 1 < KSW) fread(st, wg * KSW + kk + 1, (kk + 1) & 1);
+            __builtin_amdgcn_sched_barrier(0);
+            if (kk + 1 < KSW) {
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], bfr[kk & 1][j], acc[i][j], 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][0], bfr[kk & 1][j], acc[0][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                gemm_wait_loads<(NST - 2) * LPT>();
+                __syncthreads();
+                issue(t + NST, st);
+                fread(st1, wg * KSW, 0);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[1][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][1], bfr[kk & 1][j], acc[1][j], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        st = st1;
+    }
+    gemm_wait_loads<0>();   // the repeated loads of the last tile have landed before LDS is used for anything else
+    // The two k-groups swap halves through LDS (the staged tiles are dead behind the barrier): group g gives the sums of
+    // fragment row 1 - g and keeps row g, so all 8 waves take part in the epilogue, 32 rows each.
+    static_assert(KW == 2, "two k-groups");
+    f32x16_t mine[TN];
+    {
+        float* give = reinterpret_cast<float*>(lds) + (wg * (WM * WN) + wq) * (TN * 16 * 64) + lane;
+        const float* take = reinterpret_cast<const float*>(lds) + ((1 - wg) * (WM * WN) + wq) * (TN * 16 * 64) + lane;
+        __syncthreads();
+        if (wg == 0) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) give[(j * 16 + v) * 64] = acc[1][j][v];
+        } else {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) give[(j * 16 + v) * 64] = acc[0][j][v];
+        }
+        __syncthreads();
+        if (wg == 0) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) mine[j][v] = acc[0][j][v] + take[(j * 16 + v) * 64];
+        } else {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) mine[j][v] = acc[1][j][v] + take[(j * 16 + v) * 64];
+        }
+        __syncthreads();   // every wave has taken its half before the area is written again
+    }
+    // Rows of 8 outputs: a wave's 32 x (32 TN) sums go through an LDS area of its own (a lane holds one column of
+    // four-row groups, memory wants runs along a row); then bias, GELU and the residual are applied to 8 neighbours at a
+    // time and leave in one 16-byte store (two for f32 results; element by element when N is not a multiple of 8).
+    // DUAL: the wave columns are the two matrices (wn = 0: x.W, wn = 1: x.W2, same output columns), so the pair of
+    // waves meets here: each takes half of the pair's chunks and reads both areas.
+    constexpr int RSF = 32 * TN + 4;     // floats per row of an area
+    constexpr int CH = 32 * TN / 8;      // chunks of 8 per row
+    constexpr int PASSES = 32 * CH / 64 / (DUAL ? 2 : 1);
+    static_assert((32 * CH) % (DUAL ? 128 : 64) == 0, "whole passes of the wave");
+    {
+        float* tr = reinterpret_cast<float*>(lds) + wave * (32 * RSF);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) tr[(8 * (v >> 2) + 4 * (lane >> 5) + (v & 3)) * RSF + j * 32 + (lane & 31)] = mine[j][v];
+    }
+    if (DUAL) __syncthreads();
+    const float* area = reinterpret_cast<const float*>(lds) + (DUAL ? wave - wn : wave) * (32 * RSF);
+    const int mrow0 = m0 + wm * 64 + wg * 32, ncol0 = DUAL ? n0 : n0 + wn * 32 * TN;
+    const bool vec = (N & 7) == 0;
+#pragma unroll
+    for (int it = 0; it < PASSES; ++it) {
+        const int c = (DUAL ? wn * PASSES + it : it) * 64 + lane, r = c / CH, cc = c % CH;
+        const int m = mrow0 + r, n = ncol0 + cc * 8;
+        if (m >= M || n >= N) continue;
+        float o[8];
+        *reinterpret_cast<f32x4_t*>(o) = *reinterpret_cast<const f32x4_t*>(area + r * RSF + cc * 8);
+        *reinterpret_cast<f32x4_t*>(o + 4) = *reinterpret_cast<const f32x4_t*>(area + r * RSF + cc * 8 + 4);
+        if (DUAL) {
+            float u[8];
+            *reinterpret_cast<f32x4_t*>(u) = *reinterpret_cast<const f32x4_t*>(area + 32 * RSF + r * RSF + cc * 8);
+            *reinterpret_cast<f32x4_t*>(u + 4) = *reinterpret_cast<const f32x4_t*>(area + 32 * RSF + r * RSF + cc * 8 + 4);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[e] = (o[e] / (1.0f + expf(o[e] * -1.0f))) * u[e];   // activation.rs:141-162
+        }
+        const int64_t at = (int64_t)m * N + n;
+        if (vec) {
+            if (bias) {
+                const u32x4_t bw = *reinterpret_cast<const u32x4_t*>(bias + n);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    o[2 * e] += __uint_as_float(bw[e] << 16);            // tensor_ops.rs:42-56
+                    o[2 * e + 1] += __uint_as_float(bw[e] & 0xFFFF0000u);
+                }
+            }
+            if (act == 1) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[e] = (o[e] * 0.5f) * (erff(o[e] / 1.41421354f) + 1.0f);   // activation.rs:96-113
+            }
+            if (residual) {
+                if (out_f32) {
+                    const f32x4_t r0 = *reinterpret_cast<const f32x4_t*>(reinterpret_cast<const float*>(residual) + at);
+                    const f32x4_t r1 = *reinterpret_cast<const f32x4_t*>(reinterpret_cast<const float*>(residual) + at + 4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) { o[e] += r0[e]; o[4 + e] += r1[e]; }
+                } else {
+                    const u32x4_t rw = *reinterpret_cast<const u32x4_t*>(residual + at);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        o[2 * e] += __uint_as_float(rw[e] << 16);
+                        o[2 * e + 1] += __uint_as_float(rw[e] & 0xFFFF0000u);
+                    }
+                }
+            }
+            if (out_f32) {
+                *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(y) + at) = *reinterpret_cast<const f32x4_t*>(o);
+                *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(y) + at + 4) = *reinterpret_cast<const f32x4_t*>(o + 4);
+            } else {
+                u32x4_t w;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) w[e] = (uint32_t)f32_to_bf16(o[2 * e]) | ((uint32_t)f32_to_bf16(o[2 * e + 1]) << 16);
+                *reinterpret_cast<u32x4_t*>(y + at) = w;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                if (n + e >= N) break;
+                const float bv = bias ? bf16_to_f32(bias[n + e]) : 0.f;
+                const float rv = residual ? (out_f32 ? reinterpret_cast<const float*>(residual)[at + e] : bf16_to_f32(residual[at + e])) : 0.f;
+                const float f = mfma_finish(o[e], 0.f, false, act, bv, residual != nullptr, rv);
+                if (out_f32) reinterpret_cast<float*>(y)[at + e] = f;
+                else y[at + e] = f32_to_bf16(f);
+            }
+        }
+    }
+}
+
+template <int NST, int WM, int WN, int TN, int KW, bool DUAL>
+static void launch_dma(hipStream_t s, const MfmaLinearArgs& a) {
+    constexpr int BM = 64 * WM, BN = 32 * TN * WN, NREAL = DUAL ? BN / 2 : BN;
+    constexpr int stage = (BM + BN) * 128, xch = WM * WN * KW * TN * 16 * 64 * 4, rows = WM * WN * KW * 32 * (32 * TN + 4) * 4;
+    constexpr int lds_bytes = NST * stage > (xch > rows ? xch : rows) ? NST * stage : (xch > rows ? xch : rows);
+    static_assert(lds_bytes <= 160 * 1024, "LDS of one CU");
+    auto kern = gemm_dma_kernel<NST, WM, WN, TN, KW, DUAL>;
+    static bool configured = false;
+    if (!configured) {
+        (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        configured = true;
+    }
+    const int64_t nt = cdiv(a.n, NREAL), mt = cdiv(a.m, BM);
+    const unsigned grid = (unsigned)(cdiv(nt * mt, 8) * 8);
+    kern<<<grid, 64 * WM * WN * KW, lds_bytes, s>>>((const bf16_t*)a.x, (const bf16_t*)a.wk, (const bf16_t*)a.wk2, (const bf16_t*)a.bias,
+                                                   (const bf16_t*)a.residual, (bf16_t*)a.y, (int)a.m, (int)a.k, (int)a.n,
+                                                   (int)mfma_padded_n(a.n), a.act, (int)nt, (int)mt, a.out_f32);
+}
+
 bool mfma_gemm_supported(int dtype, int64_t m, int64_t k, int64_t n, int quant) {
     if (dtype != 0 && dtype != 2) return false;
     if (quant != 0 && (dtype != 2 || (quant == 2 && k % 128 != 0))) return false;
@@ -556,6 +849,17 @@ void mfma_gemm(hipStream_t s, const MfmaLinearArgs& a) {
         else if (split) launch_mfma<float, 128, 128, false, 0, 2>(s, a);
         else launch_mfma<float, 128, 128, false>(s, a);
     } else {
+        // unquantised bf16: the LDS-direct kernel, on the tile shape that fills the CUs in the fewest rounds (the cost
+        // of a round grows with the tile's width; narrow tiles pay 12 % more per column).  M = 1024: N = 6144 is 256
+        // tiles of 128 x 192, N = 3072 is 256 tiles of 128 x 96, a 9216-wide pair 768 tiles of 128 x 96 outputs
+        static const bool allow_dma = [] { const char* e = getenv("GPTRS_HIP_GEMM_DMA"); return !(e && e[0] == '0'); }();
+        if (allow_dma && !small && a.wk2) return launch_dma<3, 2, 2, 3, 2, true>(s, a);
+        if (allow_dma && !small) {
+            const int64_t mt = cdiv(a.m, 128);
+            const double wide = (double)cdiv(mt * cdiv(a.n, 192), 256) * 192.0;
+            const double narrow = (double)cdiv(mt * cdiv(a.n, 96), 256) * 96.0 * 1.12;
+            return wide <= narrow ? launch_dma<3, 2, 2, 3, 2, false>(s, a) : launch_dma<3, 2, 1, 3, 2, false>(s, a);
+        }
         if (a.wk2) launch_mfma<bf16_t, 128, 128, true>(s, a);
         else if (small) launch_mfma<bf16_t, 64, 64, false>(s, a);
         else if (split) launch_mfma<bf16_t, 128, 128, false, 0, 2>(s, a);
