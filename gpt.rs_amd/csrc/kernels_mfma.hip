@@ -477,11 +477,18 @@ __global__ __launch_bounds__(256 * KW) void gemm_mfma_kernel(const T* __restrict
 // Order of issue, fixed by hand with scheduling barriers: the fragments of the next k-step are requested before the
 // MFMAs of this one; in a tile's last k-step half the MFMAs are issued, then the wave waits for its own loads of the
 // next tile (vmcnt, which counts only LDS-direct loads here), passes the barrier that makes that tile complete and this
-// one free, requests the tile NST ahead into the freed stage and the next tile's first fragments, and issues the other
-// half.  Loads past the last tile repeat it into a stage nobody reads, so the count the wait relies on never changes.
+// one free, requests the next tile's first fragments, issues the other half and, behind it, requests the tile NST
+// ahead into the freed stage.  Loads past the last tile repeat it into a stage nobody reads, so the count the wait relies on never changes.
 // DUAL (SwiGLU pair): the tile's first BN / 2 columns are columns of W, the others the same columns of W2.
-__device__ __forceinline__ void gemm_lds_load16(const void* gptr, unsigned lds_addr) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(lds_addr) : "memory", "m0");
+// One load instruction: lane l asks for the 16 bytes at base + offset(l) (a scalar base and a 32-bit offset per lane, so
+// stepping to the next k tile is scalar arithmetic; vector instructions in the step loop cost the matrix pipe issue
+// slots: per-lane 64-bit addresses were 5-10 % slower) and they land at LDS byte lds_addr + 16 l.
+__device__ __forceinline__ void gemm_lds_load16(unsigned voff, unsigned long long sbase, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(sbase), "s"(lds_addr) : "memory", "m0");
+}
+__device__ __forceinline__ unsigned long long gemm_uniform64(unsigned long long p) {
+    return ((unsigned long long)(unsigned)__builtin_amdgcn_readfirstlane((int)(p >> 32)) << 32) |
+           (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)p);
 }
 template <int N> __device__ __forceinline__ void gemm_wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory"); }
 
@@ -518,8 +525,7 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_dma_kernel(const bf16_
     }
     const int m0 = by * BM, n0 = bx * NREAL;
     // what each of this wave's load instructions fetches (per lane) and where its KiB goes
-    const unsigned char* a_src[LA];
-    const unsigned char* b_src[LB];
+    unsigned a_off[LA], b_off[LB];
     unsigned a_dst[LA], b_dst[LB];
 #pragma unroll
     for (int j = 0; j < LA; ++j) {
@@ -527,35 +533,39 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_dma_kernel(const bf16_
         const int sl = q * 64 + lane, row = sl / KG, pos = sl % KG;
         int m = m0 + row;
         if (m > M - 1) m = M - 1;
-        a_src[j] = reinterpret_cast<const unsigned char*>(x + (int64_t)m * K) + ((pos ^ ((row >> 1) & 7)) * 16);
+        a_off[j] = (unsigned)((m - m0) * K * 2 + ((pos ^ ((row >> 1) & 7)) * 16));   // under 128 rows of K bf16: fits 32 bits (K < 2^23)
         a_dst[j] = q * 1024;
     }
+    // DUAL: both matrices are addressed from the lower of the two pointers (the launcher has checked that the other
+    // lies less than 2^32 bytes above it, a k tile included)
+    const unsigned long long w_lo = DUAL && (unsigned long long)wk2 < (unsigned long long)wk ? (unsigned long long)wk2 : (unsigned long long)wk;
 #pragma unroll
     for (int j = 0; j < LB; ++j) {
         const int q = (wave * LB + j) % LBI;
         const int sl = q * 64 + lane, kg = sl / BN, bc = sl % BN;
         int col = n0 + bc;
-        const bf16_t* src = wk;
+        unsigned long long src = (unsigned long long)wk;
         if (DUAL) {
             col = n0 + bc % NREAL;
-            src = bc >= NREAL ? wk2 : wk;
+            src = bc >= NREAL ? (unsigned long long)wk2 : (unsigned long long)wk;
         }
         if (col > Npad - 1) col = Npad - 1;
-        b_src[j] = reinterpret_cast<const unsigned char*>(src) + ((int64_t)kg * Npad + col) * 16;
+        b_off[j] = (unsigned)(src - w_lo) + (unsigned)(((unsigned long long)kg * Npad + col) * 16);
         b_dst[j] = A_BYTES + q * 1024;
     }
+    const unsigned long long a_base = (unsigned long long)(x + (int64_t)m0 * K);
     const int64_t b_tile_step = (int64_t)KG * Npad * 16;
     const unsigned lds0 = (unsigned)(uintptr_t)lds;
     const int nt = K / BK;
     auto issue = [&](int t, int st) {
         if (t > nt - 1) t = nt - 1;
+        const unsigned long long ab = gemm_uniform64(a_base + (unsigned long long)t * (BK * 2));
+        const unsigned long long bb = gemm_uniform64(w_lo + (unsigned long long)(t * b_tile_step));
         const unsigned sbase = lds0 + st * STAGE;
 #pragma unroll
-        for (int j = 0; j < LA; ++j)
-            gemm_lds_load16(a_src[j] + (int64_t)t * (BK * 2), (unsigned)__builtin_amdgcn_readfirstlane((int)(sbase + a_dst[j])));
+        for (int j = 0; j < LA; ++j) gemm_lds_load16(a_off[j], ab, (unsigned)__builtin_amdgcn_readfirstlane((int)(sbase + a_dst[j])));
 #pragma unroll
-        for (int j = 0; j < LB; ++j)
-            gemm_lds_load16(b_src[j] + (int64_t)t * b_tile_step, (unsigned)__builtin_amdgcn_readfirstlane((int)(sbase + b_dst[j])));
+        for (int j = 0; j < LB; ++j) gemm_lds_load16(b_off[j], bb, (unsigned)__builtin_amdgcn_readfirstlane((int)(sbase + b_dst[j])));
     };
     f32x16_t acc[2][TN];
 #pragma unroll
@@ -600,11 +610,12 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_dma_kernel(const bf16_
                 __builtin_amdgcn_sched_barrier(0);
                 gemm_wait_loads<(NST - 2) * LPT>();
                 __syncthreads();
-                issue(t + NST, st);
                 fread(st1, wg * KSW, 0);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int j = 0; j < TN; ++j) acc[1][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][1], bfr[kk & 1][j], acc[1][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                issue(t + NST, st);   // behind the MFMAs: the address arithmetic and the requests run under them (6 % faster than ahead of them)
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -853,8 +864,13 @@ void mfma_gemm(hipStream_t s, const MfmaLinearArgs& a) {
         // of a round grows with the tile's width; narrow tiles pay 12 % more per column).  M = 1024: N = 6144 is 256
         // tiles of 128 x 192, N = 3072 is 256 tiles of 128 x 96, a 9216-wide pair 768 tiles of 128 x 96 outputs
         static const bool allow_dma = [] { const char* e = getenv("GPTRS_HIP_GEMM_DMA"); return !(e && e[0] == '0'); }();
-        if (allow_dma && !small && a.wk2) return launch_dma<3, 2, 2, 3, 2, true>(s, a);
-        if (allow_dma && !small) {
+        // its loads address a k tile with 32-bit offsets from one scalar base: 128 rows of x, 8 k-groups of the padded
+        // weights, and for a pair the distance between the two matrices
+        const uint64_t w_span = (uint64_t)mfma_padded_n(a.n) * 128;
+        const uint64_t w_dist = !a.wk2 ? 0 : (a.wk2 > a.wk ? (uint64_t)((const char*)a.wk2 - (const char*)a.wk) : (uint64_t)((const char*)a.wk - (const char*)a.wk2));
+        const bool reach = a.k <= (1 << 22) && w_span < (1ull << 31) && w_dist + w_span < (1ull << 32);
+        if (allow_dma && reach && !small && a.wk2) return launch_dma<3, 2, 2, 3, 2, true>(s, a);
+        if (allow_dma && reach && !small) {
             const int64_t mt = cdiv(a.m, 128);
             const double wide = (double)cdiv(mt * cdiv(a.n, 192), 256) * 192.0;
             const double narrow = (double)cdiv(mt * cdiv(a.n, 96), 256) * 96.0 * 1.12;
