@@ -89,6 +89,8 @@ Backend::Backend(int dev) : device(dev) {
     {
         const char* c = getenv("GPTRS_HIP_CHAIN");
         if (c && c[0] == '0') opt_chain = false;
+        const char* d = getenv("GPTRS_HIP_GEMM_DMA");
+        if (d && d[0] == '0') opt_gemm_lds_direct = false;
         if (const char* m = getenv("GPTRS_HIP_CHAIN_F32_MIN_KB")) chain_f32_min_bytes = std::max<int64_t>(0, atoll(m)) << 10;
     }
     k::fill_zero(stream, d_err_flag_, 256);
@@ -572,6 +574,7 @@ bool Backend::run_graphed(Plan& plan, ExecCtx& cx, const std::vector<BufferP>& o
     for (const auto& b : out_bufs) key.push_back((uint64_t)(uintptr_t)b->ptr);
     key.push_back(opt_chain ? 1 : 0);
     key.push_back((uint64_t)chain_f32_min_bytes);
+    key.push_back(opt_gemm_lds_direct ? 1 : 0);
     for (const Step& st : plan.steps) {
         if (st.tiled_w_input >= 0) key.push_back(cx.input_bufs[st.tiled_w_input]->id);
         if (st.tiled_w2_input >= 0) key.push_back(cx.input_bufs[st.tiled_w2_input]->id);
@@ -1037,6 +1040,7 @@ int gptrs_hip_set_option(gptrs_hip_backend* b, const char* name, int64_t value) 
         if (!strcmp(name, "fusion")) b->impl.opt_fusion = value != 0;
         else if (!strcmp(name, "graphs")) b->impl.opt_graphs = value != 0;
         else if (!strcmp(name, "chain")) b->impl.opt_chain = value != 0;
+        else if (!strcmp(name, "gemm_lds_direct")) b->impl.opt_gemm_lds_direct = value != 0;
         else if (!strcmp(name, "chain_f32_min_kb")) b->impl.chain_f32_min_bytes = std::max<int64_t>(0, value) << 10;
         else if (!strcmp(name, "chain_stall_phase")) b->impl.chain_stall_phase = value < 0 ? -1 : (int)std::min<int64_t>(value, 1 << 20);
         else if (!strcmp(name, "profile")) { b->impl.profile_reset(); b->impl.opt_profile = value != 0; }

@@ -258,6 +258,7 @@ struct MfmaLinearArgs {
     // counters, zero before and after every launch); without them every tile runs whole
     void* part = nullptr; size_t part_bytes = 0; unsigned* tickets = nullptr;
     int out_f32 = 0;   // bf16 only: y and residual are f32
+    int lds_direct = 1;   // unquantised bf16: the LDS-direct kernel where it applies (0: the register-staged one)
 };
 size_t mfma_workspace_bytes(int dtype, int64_t m, int64_t k, int64_t n, bool dual, int quant);
 size_t mfma_weight_bytes(int dtype, int64_t k, int64_t n);

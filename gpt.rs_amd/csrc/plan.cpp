@@ -1114,6 +1114,7 @@ void run_step(const Plan& plan, const Step& st, ExecCtx& cx) {
                 k::MfmaLinearArgs ma{};
                 ma.dtype = (int)ldt;
                 ma.out_f32 = in.out_f32;
+                ma.lds_direct = cx.be->opt_gemm_lds_direct ? 1 : 0;
                 ma.x = src_ptr(st, cx, 0);
                 ma.m = x.dims[0]; ma.k = x.dims[1]; ma.n = w.dims[1];
                 // quantised weights: the k-grouped copy holds the codes; the kernel applies the scales on the way into LDS

@@ -198,6 +198,9 @@ class Backend {
     unsigned* skinny_tickets() const { return d_chain_bar_ + k::kChainBarrierBytes / sizeof(unsigned); }
     int* chain_abort_flag() const { return d_err_flag_ + 1; }
     bool opt_chain = true;
+    // unquantised bf16 prefill linears on the LDS-direct GEMM (option "gemm_lds_direct", GPTRS_HIP_GEMM_DMA); off: the
+    // register-staged kernel that also serves f32 and quantised weights
+    bool opt_gemm_lds_direct = true;
     // f32 chains run only when a linear phase streams at least this much on average (option "chain_f32_min_kb",
     // GPTRS_HIP_CHAIN_F32_MIN_KB): below it a phase's fixed cost is what a stand-alone kernel costs
     int64_t chain_f32_min_bytes = 8ll << 20;

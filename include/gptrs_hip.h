@@ -165,7 +165,8 @@ const char* gptrs_hip_last_error(void);
  * to_literal and sample_decode_token synchronise by themselves). */
 int gptrs_hip_synchronize(gptrs_hip_backend* b);
 
-/* Execution options: name in {"fusion", "profile", "graphs", "chain", "chain_f32_min_kb", "chain_stall_phase", "drop_derived_weights"};
+/* Execution options: name in {"fusion", "profile", "graphs", "chain", "chain_f32_min_kb", "chain_stall_phase", "gemm_lds_direct",
+ * "drop_derived_weights"};
  * value 0/1 unless stated.
  * "fusion" = rewrite matched functional sequences to fused kernels (on by default; off = one generic kernel per
  * instruction, the reference harness's "optimizer off" leg,
@@ -179,6 +180,9 @@ int gptrs_hip_synchronize(gptrs_hip_backend* b);
  * "chain_f32_min_kb" (default 8192) = f32 linear layers (with LayerNorm, bias, GELU, residual and f32 decode attention) join a
  * persistent launch only when they stream at least this many KiB of weights each on average: a phase of the launch costs
  * what a small stand-alone kernel costs, so a narrow f32 model (GPT-2 small: 7 MB per layer) gains nothing; 0 = always.
+ * "gemm_lds_direct" (default 1) = unquantised bf16 linear layers of more than 16 rows run on the GEMM whose tiles go from
+ * memory to LDS without passing through registers; 0 = on the register-staged GEMM that serves f32 and quantised weights
+ * (the two sum in different orders: results agree to bf16 rounding, not bit for bit).
  * "chain_stall_phase" (default -1; a test hook) = value >= 1: the next persistent launch expects, at that phase's grid
  * barrier, one arrival more than its workgroups can deliver, so that its bounded wait gives up: the call that next
  * synchronises reports an Execution error and the option returns to -1.

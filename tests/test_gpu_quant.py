@@ -189,8 +189,15 @@ def test_prefill_codes_equal_dequantised_weights(hip, scheme, m, k, n):
     built = hip.counter("derived_weights_built")
     (got,) = hip_run(hip, prog(lambda fb, a, b, c: F.linear_quantized(a, b, c), [("Bf16", [m, k]), cs_, ss_]), [x, q, s])
     assert hip.counter("derived_weights_built") == built + 1     # one copy: the codes (no dequantised matrix)
-    (want,) = hip_run(hip, prog(lambda fb, a, b: a.matmul(b), [("Bf16", [m, k]), ("Bf16", [k, n])]), [x, dequantize_host(q, s, scheme)])
+    # "same kernel": plain bf16 weights otherwise run on the LDS-direct GEMM, which sums in another order
+    hip.set_option("gemm_lds_direct", 0)
+    try:
+        (want,) = hip_run(hip, prog(lambda fb, a, b: a.matmul(b), [("Bf16", [m, k]), ("Bf16", [k, n])]), [x, dequantize_host(q, s, scheme)])
+    finally:
+        hip.set_option("gemm_lds_direct", 1)
     assert np.array_equal(got, want), f"max diff {np.max(np.abs(got - want))}"
+    (direct,) = hip_run(hip, prog(lambda fb, a, b: a.matmul(b), [("Bf16", [m, k]), ("Bf16", [k, n])]), [x, dequantize_host(q, s, scheme)])
+    assert_close(direct, want, atol=1e-4 * np.sqrt(k), rtol=2.0 ** -7, what="LDS-direct GEMM vs register-staged GEMM")
     pq = prog(lambda fb, a, b, c: F.linear_quantized(a, b, c), [("Bf16", [m, k]), cs_, ss_])
     (again,) = hip_run(hip, pq, [x, q, s])
     assert np.array_equal(again, got), "a second launch of the same GEMM differs (tickets not returned to zero?)"
@@ -203,10 +210,17 @@ def test_prefill_codes_equal_dequantised_weights(hip, scheme, m, k, n):
     assert_close(got, ref, atol=1e-4 * np.sqrt(k), rtol=2.0 ** -7, what="quantised GEMM vs oracle")
     (gotp,) = hip_run(hip, prog(lambda fb, a, b, bs, c, cs: F.swiglu(F.linear_quantized(a, b, bs), F.linear_quantized(a, c, cs)),
                                 [("Bf16", [m, k]), cs_, ss_, cs_, ss_]), [x, q, s, q2, s2])
-    (wantp,) = hip_run(hip, prog(lambda fb, a, b, c: F.swiglu(a.matmul(b), a.matmul(c)),
-                                 [("Bf16", [m, k]), ("Bf16", [k, n]), ("Bf16", [k, n])]),
-                       [x, dequantize_host(q, s, scheme), dequantize_host(q2, s2, scheme)])
+    pair = prog(lambda fb, a, b, c: F.swiglu(a.matmul(b), a.matmul(c)), [("Bf16", [m, k]), ("Bf16", [k, n]), ("Bf16", [k, n])])
+    pair_args = [x, dequantize_host(q, s, scheme), dequantize_host(q2, s2, scheme)]
+    hip.set_option("gemm_lds_direct", 0)
+    try:
+        (wantp,) = hip_run(hip, pair, pair_args)
+    finally:
+        hip.set_option("gemm_lds_direct", 1)
     assert np.array_equal(gotp, wantp), f"pair: max diff {np.max(np.abs(gotp - wantp))}"
+    (directp,) = hip_run(hip, pair, pair_args)
+    # silu(g) * u of two sums that each differ by a rounding of the f32 accumulation order, then one bf16 rounding
+    assert_close(directp, wantp, atol=2e-4 * np.sqrt(k), rtol=2.0 ** -6, what="LDS-direct pair vs register-staged pair")
 
 
 @pytest.mark.parametrize("scheme", ["w8", "w4g128"])
