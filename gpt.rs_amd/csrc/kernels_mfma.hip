@@ -7,6 +7,8 @@
 // column that fill 16 bytes (8 bf16 or 4 f32) are adjacent (Npad = N rounded up to the 128-column block tile, zero
 // filled); the backend builds it once per weight and keeps it beside the original.  With it a block's B tile is, per
 // 16-byte k-group, one contiguous 2 KiB run, and every data movement below is in 16-byte chunks whatever the type.
+#include <algorithm>
+
 #include "kernels.hpp"
 #include "device_utils.hpp"
 
@@ -498,7 +500,8 @@ template <int NST, int WM, int WN, int TN, int KW, bool DUAL>
 __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_dma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wk,
                                                                    const bf16_t* __restrict__ wk2, const bf16_t* __restrict__ bias,
                                                                    const bf16_t* __restrict__ residual, bf16_t* __restrict__ y,
-                                                                   int M, int K, int N, int Npad, int act, int NT, int MT, int out_f32) {
+                                                                   int M, int K, int N, int Npad, int act, int NT, int MT, int out_f32,
+                                                                   int splits, float* __restrict__ part, unsigned* __restrict__ tickets) {
     constexpr int BK = 64, KG = 8, ROWB = 128;
     constexpr int BM = 64 * WM, BN = 32 * TN * WN, NW = WM * WN * KW;
     constexpr int NREAL = DUAL ? BN / 2 : BN;                          // output columns per tile
@@ -514,12 +517,16 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_dma_kernel(const bf16_
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wg = wave / (WM * WN), wq = wave % (WM * WN);
     const int wm = wq / WN, wn = wq % WN;
-    int bx, by;
+    int bx, by, tile, sidx;
     {
         // XCD c takes a contiguous range of a grouped tile order (see gemm_mfma_kernel)
-        const int total = NT * MT, per = (total + 7) / 8;
-        const int v = (int)(blockIdx.x % 8) * per + (int)(blockIdx.x / 8);
-        if (v >= total) return;
+        // splits > 1: `splits` neighbours of that order share a tile and take a contiguous range of its k tiles each
+        const int total = NT * MT * splits, per = (total + 7) / 8;
+        const int u = (int)(blockIdx.x % 8) * per + (int)(blockIdx.x / 8);
+        if (u >= total) return;
+        tile = u / splits;
+        sidx = u % splits;
+        const int v = tile;
         const int gsz = 8 * NT, g = v / gsz, first = g * 8;
         const int gm = MT - first < 8 ? MT - first : 8;
         by = first + (v % gsz) % gm;
@@ -558,9 +565,11 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_dma_kernel(const bf16_
     const unsigned long long a_base = (unsigned long long)(x + (int64_t)m0 * K);
     const int64_t b_tile_step = (int64_t)KG * Npad * 16;
     const unsigned lds0 = (unsigned)(uintptr_t)lds;
-    const int nt = K / BK;
+    const int kt_all = K / BK, kt0 = (int)((int64_t)sidx * kt_all / splits);
+    const int nt = (int)((int64_t)(sidx + 1) * kt_all / splits) - kt0;   // this workgroup's k tiles: [kt0, kt0 + nt)
     auto issue = [&](int t, int st) {
         if (t > nt - 1) t = nt - 1;
+        t += kt0;
         const unsigned long long ab = gemm_uniform64(a_base + (unsigned long long)t * (BK * 2));
         const unsigned long long bb = gemm_uniform64(w_lo + (unsigned long long)(t * b_tile_step));
         const unsigned sbase = lds0 + st * STAGE;
@@ -657,6 +666,40 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_dma_kernel(const bf16_
         }
         __syncthreads();   // every wave has taken its half before the area is written again
     }
+    if (!DUAL && splits > 1) {
+        // Split over k: the workgroups of a tile leave their sums in the workspace, [tile][split][wave][value][lane],
+        // through device-scope stores (coherent across the XCDs' L2s without cache maintenance); once they are
+        // acknowledged the workgroup draws the tile's ticket.  The one that draws the last ticket adds all partial sums
+        // in split order, its own included, so the result does not depend on which workgroup that is, leaves the ticket
+        // at zero and runs the epilogue.
+        float* mine_at = part + ((int64_t)(tile * splits + sidx) * NW + wave) * (TN * 16 * 64) + lane;
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) __hip_atomic_store(mine_at + (j * 16 + v) * 64, mine[j][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_s_waitcnt(0x0F70);                         // vmcnt(0)
+        asm volatile("" ::: "memory");
+        unsigned* flag = reinterpret_cast<unsigned*>(lds);
+        __syncthreads();
+        if (tid == 0) *flag = __hip_atomic_fetch_add(&tickets[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        const unsigned drawn = *flag;
+        __syncthreads();                                            // the flag has been read before its bytes are used again
+        if (drawn != (unsigned)(splits - 1)) return;
+        asm volatile("" ::: "memory");                              // the partial sums are read after the ticket is known
+        if (tid == 0) __hip_atomic_store(&tickets[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) mine[j][v] = 0.f;
+        for (int q = 0; q < splits; ++q) {
+            const float* src = part + ((int64_t)(tile * splits + q) * NW + wave) * (TN * 16 * 64) + lane;
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) mine[j][v] += __hip_atomic_load(src + (j * 16 + v) * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
     // Rows of 8 outputs: a wave's 32 x (32 TN) sums go through an LDS area of its own (a lane holds one column of
     // four-row groups, memory wants runs along a row); then bias, GELU and the residual are applied to 8 neighbours at a
     // time and leave in one 16-byte store (two for f32 results; element by element when N is not a multiple of 8).
@@ -745,7 +788,7 @@ __global__ __launch_bounds__(64 * WM * WN * KW) void gemm_dma_kernel(const bf16_
 }
 
 template <int NST, int WM, int WN, int TN, int KW, bool DUAL>
-static void launch_dma(hipStream_t s, const MfmaLinearArgs& a) {
+static void launch_dma(hipStream_t s, const MfmaLinearArgs& a, int splits = 1) {
     constexpr int BM = 64 * WM, BN = 32 * TN * WN, NREAL = DUAL ? BN / 2 : BN;
     constexpr int stage = (BM + BN) * 128, xch = WM * WN * KW * TN * 16 * 64 * 4, rows = WM * WN * KW * 32 * (32 * TN + 4) * 4;
     constexpr int lds_bytes = NST * stage > (xch > rows ? xch : rows) ? NST * stage : (xch > rows ? xch : rows);
@@ -757,10 +800,33 @@ static void launch_dma(hipStream_t s, const MfmaLinearArgs& a) {
         configured = true;
     }
     const int64_t nt = cdiv(a.n, NREAL), mt = cdiv(a.m, BM);
-    const unsigned grid = (unsigned)(cdiv(nt * mt, 8) * 8);
+    if (splits > 1 && (DUAL || !a.part || !a.tickets || nt * mt > (int64_t)kSkinnyTickets ||
+                       a.part_bytes < (size_t)(nt * mt) * splits * BM * BN * sizeof(float)))
+        splits = 1;
+    const unsigned grid = (unsigned)(cdiv(nt * mt * splits, 8) * 8);
     kern<<<grid, 64 * WM * WN * KW, lds_bytes, s>>>((const bf16_t*)a.x, (const bf16_t*)a.wk, (const bf16_t*)a.wk2, (const bf16_t*)a.bias,
                                                    (const bf16_t*)a.residual, (bf16_t*)a.y, (int)a.m, (int)a.k, (int)a.n,
-                                                   (int)mfma_padded_n(a.n), a.act, (int)nt, (int)mt, a.out_f32);
+                                                   (int)mfma_padded_n(a.n), a.act, (int)nt, (int)mt, a.out_f32, splits, (float*)a.part,
+                                                   a.tickets);
+}
+
+// Which tiles an unquantised bf16 launch of the LDS-direct kernel takes: 128 x 192 (`wide`), 128 x 96, or 128 x 192 with
+// every tile split two ways over k.  Estimated from what the kernels measure at M = 1024 (us): a round of wide tiles
+// 8 + 0.72 per k tile, of narrow ones 7 + 0.45 (28 KB per k tile against 40 KB, for half the flops), of split wide ones
+// 15 + 0.36 (half the k tiles; 7 us for 25 MB of partial sums out and in again).  N = 6144: 256 wide tiles; N = 3072:
+// 256 narrow tiles at K = 4096 (36.7 us; split 38.5), 128 wide tiles split in two at K = 9216 (66.7 us; narrow 72.8);
+// the 9216-wide pair: 768 tiles of 128 x 96 outputs.
+struct DmaPlan { bool wide; int splits; };
+static DmaPlan dma_plan(int64_t m, int64_t k, int64_t n) {
+    const int64_t mt = cdiv(m, 128), kt = k / 64;
+    const int64_t tw = mt * cdiv(n, 192), tn = mt * cdiv(n, 96);
+    const double wide = (double)cdiv(tw, 256) * (8.0 + 0.72 * kt);
+    const double narrow = (double)cdiv(tn, 256) * (7.0 + 0.45 * kt);
+    static const bool allow_split = [] { const char* e = getenv("GPTRS_HIP_GEMM_TAILSPLIT"); return !(e && e[0] == '0'); }();
+    const bool can_split = allow_split && kt >= 32 && tw <= (int64_t)kSkinnyTickets;
+    const double split = can_split ? (double)cdiv(2 * tw, 256) * (15.0 + 0.36 * kt) : 1e30;
+    if (split < wide && split < narrow) return {true, 2};
+    return {wide <= narrow, 1};
 }
 
 bool mfma_gemm_supported(int dtype, int64_t m, int64_t k, int64_t n, int quant) {
@@ -806,7 +872,12 @@ size_t mfma_workspace_bytes(int dtype, int64_t m, int64_t k, int64_t n, bool dua
     }
     int sp = 1;
     const int64_t full = mfma_tail_plan(tiles, k_tiles, &sp);
-    return sp > 1 ? (size_t)(tiles - full) * sp * 128 * 128 * sizeof(float) : 0;
+    size_t bytes = sp > 1 ? (size_t)(tiles - full) * sp * 128 * 128 * sizeof(float) : 0;
+    if (dtype == 2 && quant == 0 && !dual) {   // the LDS-direct kernel may split its 128 x 192 tiles over k
+        const DmaPlan p = dma_plan(m, k, n);
+        if (p.wide && p.splits > 1) bytes = std::max(bytes, (size_t)(cdiv(m, 128) * cdiv(n, 192)) * p.splits * 128 * 192 * sizeof(float));
+    }
+    return bytes;
 }
 
 template <typename T, int BM, int BN, bool DUAL, int QF = 0, int KW = 1>
@@ -862,9 +933,7 @@ void mfma_gemm(hipStream_t s, const MfmaLinearArgs& a) {
         else if (split) launch_mfma<float, 128, 128, false, 0, 2>(s, a);
         else launch_mfma<float, 128, 128, false>(s, a);
     } else {
-        // unquantised bf16: the LDS-direct kernel, on the tile shape that fills the CUs in the fewest rounds (the cost
-        // of a round grows with the tile's width; narrow tiles pay 12 % more per column).  M = 1024: N = 6144 is 256
-        // tiles of 128 x 192, N = 3072 is 256 tiles of 128 x 96, a 9216-wide pair 768 tiles of 128 x 96 outputs
+        // unquantised bf16: the LDS-direct kernel, on the tiles dma_plan() picks
         const bool allow_dma = a.lds_direct != 0;
         // its loads address a k tile with 32-bit offsets from one scalar base: 128 rows of x, 8 k-groups of the padded
         // weights, and for a pair the distance between the two matrices
@@ -873,10 +942,8 @@ void mfma_gemm(hipStream_t s, const MfmaLinearArgs& a) {
         const bool reach = a.k <= (1 << 22) && w_span < (1ull << 31) && w_dist + w_span < (1ull << 32);
         if (allow_dma && reach && !small && a.wk2) return launch_dma<3, 2, 2, 3, 2, true>(s, a);
         if (allow_dma && reach && !small) {
-            const int64_t mt = cdiv(a.m, 128);
-            const double wide = (double)cdiv(mt * cdiv(a.n, 192), 256) * 192.0;
-            const double narrow = (double)cdiv(mt * cdiv(a.n, 96), 256) * 96.0 * 1.12;
-            return wide <= narrow ? launch_dma<3, 2, 2, 3, 2, false>(s, a) : launch_dma<3, 2, 1, 3, 2, false>(s, a);
+            const DmaPlan p = dma_plan(a.m, a.k, a.n);
+            return p.wide ? launch_dma<3, 2, 2, 3, 2, false>(s, a, p.splits) : launch_dma<3, 2, 1, 3, 2, false>(s, a);
         }
         if (a.wk2) launch_mfma<bf16_t, 128, 128, true>(s, a);
         else if (small) launch_mfma<bf16_t, 64, 64, false>(s, a);

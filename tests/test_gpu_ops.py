@@ -223,15 +223,17 @@ def test_prefill_linear_on_matrix_cores(hip, m, k, n):
 @pytest.mark.parametrize("dtype", ["Bf16", "F32"])
 @pytest.mark.parametrize("m,k,n,pair", [(1024, 1024, 4860, False), (1100, 512, 5120, False), (1024, 1024, 2430, True), (1024, 256, 4864, False),
                                         (1024, 768, 4860, False), (1024, 1536, 2430, True), (1030, 960, 8192, False),
-                                        (1000, 512, 3072, False), (1000, 512, 3060, False), (1024, 512, 2432, True), (520, 64, 6144, False)])
+                                        (1000, 512, 3072, False), (1000, 512, 3060, False), (1024, 512, 2432, True), (520, 64, 6144, False),
+                                        (1000, 6144, 3072, False), (900, 6208, 3000, False)])
 def test_prefill_linear_tail_tiles_split_over_k(hip, m, k, n, pair, dtype):
     """Launches of more than 256 tiles whose last round holds at most 128: those tiles are split 4 or 2 ways over k
     between workgroups that meet through a workspace and a ticket (304 tiles -> 48 x 4, 360 -> 104 x 2, the SwiGLU pair
     with 64 real columns per tile, and K = 256 with too few k tiles to split;
     further K and tile counts with and without a tail).  Unquantised bf16 runs on the LDS-direct kernel instead: these
     shapes take its 128 x 192 tiles, its 128 x 96 tiles (N = 3072 / 3060 at M = 1000), the pair whose two matrices are
-    wave columns, ragged M, N that is and is not a multiple of 8 (16-byte and element-wise epilogues), and K = 64 (fewer
-    k tiles than the ring of staged tiles is deep).  Checked against the oracle, and a second
+    wave columns, ragged M, N that is and is not a multiple of 8 (16-byte and element-wise epilogues), K = 64 (fewer
+    k tiles than the ring of staged tiles is deep), and 128 tiles of 128 x 192 split two ways over k with partial sums
+    and tickets (K = 6144 / 6208 at N = 3072 / 3000; 97 k tiles split 48 + 49).  Checked against the oracle, and a second
     run (tickets must have returned to zero) must reproduce the first bit for bit."""
     x = rng_uniform(50, (m, k))
     w, w2 = rng_uniform(51, (k, n)) / np.sqrt(k) * 2, rng_uniform(52, (k, n)) / np.sqrt(k) * 2
