@@ -685,8 +685,13 @@ __global__ __launch_bounds__(256 * KG, 2 / KG) void attn_prefill_mfma_kernel(con
     // d-chunks (16 lanes, 8 rows apart, same position) would hit a single bank whatever the stride (8 rows are a
     // multiple of 128 bytes apart), which the skew spreads over 8 groups of 4 banks.  Measured at 1024 tokens: no skew
     // 88 us per layer, skew with 128-byte rows (reads 8-way conflicting) 68 us.
-    constexpr int VS = KG == 1 ? 104 : 72;   // two groups: 72 (rows 4 banks apart, 4 skews) keeps both sets of buffers in LDS
-    constexpr int SKEW = KG == 1 ? 7 : 3;
+    // Two key groups: rows of 88 elements (176 bytes: consecutive rows 44 banks apart, so the 8 rows of one d-chunk fall
+    // into 8 different groups of 4 banks, and a chunk's first row starts 32 banks from its neighbour's) and a skew of
+    // 16 bytes x (chunk / 2): the 16 chunks of one key then scatter into 16 different groups of 4 banks (with 72-element
+    // rows and 4 skews they shared 4, an 8-way conflict on every 2-byte store: 2.7 M conflict cycles per launch).
+    constexpr int VS = KG == 1 ? 104 : 88;
+    constexpr int SKEW = 7;
+    constexpr int SKSH = KG == 1 ? 0 : 1;     // the skew index is (chunk >> SKSH) & SKEW
     constexpr int ND = DH / 32;       // 32-row blocks of d in O^T
     constexpr int NK = DH / 16;       // k-steps of the score product
     constexpr int CH = KT * DH / 8;   // 16-byte chunks of a K (or V) tile
@@ -755,7 +760,7 @@ __global__ __launch_bounds__(256 * KG, 2 / KG) void attn_prefill_mfma_kernel(con
                 const uint32_t w[4] = {w0, w1, w2, w3};
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
-                    vsm[buf][(ch * 8 + e) * VS + 8 * (ch & SKEW) + pos] = (bf16_t)((w[e >> 1] >> ((e & 1) * 16)) & 0xFFFFu);
+                    vsm[buf][(ch * 8 + e) * VS + 8 * ((ch >> SKSH) & SKEW) + pos] = (bf16_t)((w[e >> 1] >> ((e & 1) * 16)) & 0xFFFFu);
             }
         }
     };
@@ -828,7 +833,7 @@ __global__ __launch_bounds__(256 * KG, 2 / KG) void attn_prefill_mfma_kernel(con
             for (int db = 0; db < ND; ++db) {
 #pragma unroll
                 for (int i = 0; i < 2; ++i) {
-                    const bf16x8_v vf = *reinterpret_cast<const bf16x8_v*>(&vsm[buf][(db * 32 + col) * VS + 8 * ((((db & 1) << 2) | (col >> 3)) & SKEW) + 16 * i + 8 * half]);
+                    const bf16x8_v vf = *reinterpret_cast<const bf16x8_v*>(&vsm[buf][(db * 32 + col) * VS + 8 * (((db * 4 + (col >> 3)) >> SKSH) & SKEW) + 16 * i + 8 * half]);
                     acc_o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[i], acc_o[db], 0, 0, 0);
                 }
             }
