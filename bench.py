@@ -210,7 +210,7 @@ class _HostParams:
 
 
 def cpu_gpt2_baseline(prompt, new_tokens: int, capacity: int = 128):
-    """BASELINE.md's CPU workload (ii): GPT-2 small f32 greedy decode with a KV cache on the reference C kernels
+    """The CPU baseline workload: GPT-2 small f32 greedy decode with a KV cache on the reference C kernels
     (oracle/ref_harness.c: every matrix product through gpt_rs_c_matmul_f32_cached_b with a warm packed-B cache, the
     other ops as plain C loops), same seeded weights and prompt as the device run.  The prompt goes through token by
     token (the harness has no batched prefill); timed: the last `new_tokens` steps, steady decode.  One core, then one
