@@ -354,9 +354,14 @@ __global__ __launch_bounds__(256 * KW) void gemm_mfma_kernel(const T* __restrict
     lwrite(0, 0, 1);
     gload(t_begin + 1 < nt ? t_begin + 1 : t_begin, 0, 1);
     __syncthreads();
+    fread(0, wg * KSTEPS, 0);
+    // The order of issue inside a k-step is fixed by hand (the scheduling barriers): the fragments of the NEXT k-step
+    // are requested before the MFMAs of this one, so their LDS latency runs under the matrix work; left to itself the
+    // compiler sinks the reads below the MFMAs into the same registers and the matrix pipe waits for every fragment.
+    // The tile's barrier sits between the two halves of the last k-step's MFMAs, and the first fragments of the next
+    // tile are requested right behind it.
     for (int t = t_begin; t < nt; ++t) {
         const int cur = (t - t_begin) & 1;
-        fread(cur, wg * KSTEPS, 0);
 #pragma unroll
         for (int kk = 0; kk < KSTEPS; ++kk) {
             if (kk + 1 < KSTEPS) fread(cur, wg * KSTEPS + kk + 1, (kk + 1) & 1);
@@ -365,13 +370,32 @@ __global__ __launch_bounds__(256 * KW) void gemm_mfma_kernel(const T* __restrict
             if (QF == 2 && kk == 0) q_scale = q_scale_next;   // the scale that came with tile t+1
             lwrite(cur ^ 1, kk, KSTEPS);
             gload(t + 2 < nt ? t + 2 : nt - 1, kk, KSTEPS);
+            __builtin_amdgcn_sched_barrier(0);
+            if (kk + 1 < KSTEPS) {
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+                for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = Mma<T>::mma(af[kk & 1][i], bfr[kk & 1][j], acc[i][j]);
+                    for (int j = 0; j < TN; ++j)
+                        acc[i][j] = Mma<T>::mma(af[kk & 1][i], bfr[kk & 1][j], acc[i][j]);
+            } else {
+                static_assert(((KSTEPS - 1) & 1) == 1, "the last k-step's fragments are in slot 1, the next tile's first in slot 0");
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN / 2; ++j)
+                        acc[i][j] = Mma<T>::mma(af[kk & 1][i], bfr[kk & 1][j], acc[i][j]);
+                __builtin_amdgcn_sched_barrier(0);
+                __syncthreads();
+                fread(cur ^ 1, wg * KSTEPS, 0);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = TN / 2; j < TN; ++j)
+                        acc[i][j] = Mma<T>::mma(af[kk & 1][i], bfr[kk & 1][j], acc[i][j]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __syncthreads();
     }
 
     if (KW == 2) {
