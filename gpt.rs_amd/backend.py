@@ -28,7 +28,7 @@ EXPORTS = [
     "gptrs_hip_param_get", "gptrs_hip_param_set", "gptrs_hip_supports_decode_sampling",
     "gptrs_hip_sample_decode_token", "gptrs_hip_sample_decode_token_begin", "gptrs_hip_sample_decode_token_wait",
     "gptrs_hip_decode_token_tensor", "gptrs_hip_sample_decode_rows_begin", "gptrs_hip_sample_decode_rows_wait",
-    "gptrs_hip_decode_rows_tensor", "gptrs_hip_sample_decode_rows_into", "gptrs_hip_last_error", "gptrs_hip_synchronize", "gptrs_hip_set_option",
+    "gptrs_hip_decode_rows_tensor", "gptrs_hip_sample_decode_rows_into", "gptrs_hip_fusion_report", "gptrs_hip_last_error", "gptrs_hip_synchronize", "gptrs_hip_set_option",
     "gptrs_hip_counter",
 ]
 
@@ -87,6 +87,7 @@ def load_library(path: str = LIB_PATH):
     lib.gptrs_hip_sample_decode_rows_wait.argtypes = [vp, ctypes.c_int64, ctypes.POINTER(ctypes.c_int32), sz]
     lib.gptrs_hip_decode_rows_tensor.argtypes = [vp, ctypes.c_int64, pvp]
     lib.gptrs_hip_sample_decode_rows_into.argtypes = [vp, vp, vp]
+    lib.gptrs_hip_fusion_report.argtypes = [cp, sz, ctypes.POINTER(ctypes.c_int64), sz, ctypes.c_char_p, sz, ctypes.POINTER(sz)]
     lib.gptrs_hip_last_error.argtypes = []
     lib.gptrs_hip_last_error.restype = cp
     lib.gptrs_hip_synchronize.argtypes = [vp]
@@ -95,6 +96,24 @@ def load_library(path: str = LIB_PATH):
     lib.gptrs_hip_counter.restype = ctypes.c_int64
     _lib = lib
     return lib
+
+
+def fusion_report(program: Program, bcast_len: Optional[Sequence[int]] = None) -> List[str]:
+    """gptrs_hip_fusion_report: the instructions that remain of `program` after the backend's fusion pass, one string
+    each (no device needed).  `bcast_len[i]` > 0 marks input i as a handle the backend made by broadcasting a vector of
+    that many values (a derived parameter of the reference's parameter-only fold)."""
+    lib = load_library()
+    js = program.json_bytes
+    n_in = len(program.param_specs)
+    lens = (ctypes.c_int64 * max(n_in, 1))(*([int(v) for v in bcast_len] if bcast_len is not None else [0] * n_in))
+    needed = ctypes.c_size_t(0)
+    code = lib.gptrs_hip_fusion_report(js, len(js), lens, n_in, None, 0, ctypes.byref(needed))
+    if code == 0:
+        buf = ctypes.create_string_buffer(needed.value)
+        code = lib.gptrs_hip_fusion_report(js, len(js), lens, n_in, buf, needed.value, ctypes.byref(needed))
+    if code != 0:
+        raise BackendError(code, lib.gptrs_hip_last_error().decode("utf-8", "replace"))
+    return buf.value.decode().splitlines()
 
 
 class TensorHandle:

@@ -52,6 +52,18 @@ Buffer::~Buffer() {
 }
 
 // ------------------------------------------------------------------------------ backend
+// Drops one reference; the last one frees the handle and lets go of the handles it holds.  The caller holds the owning
+// backend's mutex (returning a block to the pool touches backend state).
+void release_handle_locked(gptrs_hip_tensor* t) {
+    while (t && t->refs.fetch_sub(1) == 1) {
+        gptrs_hip_tensor* src = t->bcast_src;
+        gptrs_hip_tensor* lazy = t->lazy_input;
+        delete t;
+        if (lazy) release_handle_locked(lazy);
+        t = src;
+    }
+}
+
 Backend::Backend(int dev) : device(dev) {
     int count = 0;
     if (hipGetDeviceCount(&count) != hipSuccess || count <= 0)
@@ -102,9 +114,7 @@ Backend::~Backend() {
     (void)hipSetDevice(device);
     if (stream) (void)hipStreamSynchronize(stream);
     try { profile_collect(); } catch (...) {}
-    for (auto& kv : params_) {
-        if (kv.second->refs.fetch_sub(1) == 1) delete kv.second;
-    }
+    for (auto& kv : params_) release_handle_locked(kv.second);
     params_.clear();
     plan_index_.clear();
     plan_lru_.clear();
@@ -311,6 +321,7 @@ void Backend::check_device_errors() {
 }
 
 void Backend::to_literal(const gptrs_hip_tensor* t, void* dst, size_t cap) {
+    realize(t);
     GPTRS_HIP_CHECK(hipSetDevice(device));
     if (t->consumed) fail_exec("tensor handle was donated to run_program and can no longer be read");
     const size_t n = t->spec.bytes();
@@ -336,7 +347,7 @@ void Backend::param_set(const std::array<uint8_t, 16>& id, gptrs_hip_tensor* t) 
     t->refs.fetch_add(1);
     auto it = params_.find(id);
     if (it != params_.end()) {
-        if (it->second->refs.fetch_sub(1) == 1) delete it->second;
+        release_handle_locked(it->second);
         it->second = t;
     } else {
         params_[id] = t;
@@ -346,6 +357,7 @@ void Backend::param_set(const std::array<uint8_t, 16>& id, gptrs_hip_tensor* t) 
 bool Backend::queue_sampling(const gptrs_hip_tensor* logits, float temperature, bool has_top_k, bool has_u, float u) {
     GPTRS_HIP_CHECK(hipSetDevice(device));
     if (logits->consumed) fail_exec("tensor handle was donated to run_program and can no longer be read");
+    realize(logits);
     const Spec& s = logits->spec;
     if (!dtype_is_float(s.dtype) || s.rank() < 1 || s.rank() > 2 || s.count() == 0)
         fail_exec("sample_decode_token expects non-empty f32/bf16 logits of rank 1 or 2");
@@ -386,6 +398,7 @@ int64_t Backend::sample_begin(const gptrs_hip_tensor* logits, float temperature,
 int64_t Backend::sample_rows_begin(const gptrs_hip_tensor* logits) {
     GPTRS_HIP_CHECK(hipSetDevice(device));
     if (logits->consumed) fail_exec("tensor handle was donated to run_program and can no longer be read");
+    realize(logits);
     const Spec& s = logits->spec;
     if (!dtype_is_float(s.dtype) || s.rank() != 2 || s.count() == 0 || s.dims[0] > kMaxTokenRows)
         fail_exec("sample_decode_rows expects non-empty f32/bf16 logits [rows <= 64, vocab]");
@@ -406,6 +419,8 @@ int64_t Backend::sample_rows_begin(const gptrs_hip_tensor* logits) {
 void Backend::sample_rows_into(const gptrs_hip_tensor* logits, gptrs_hip_tensor* tokens_out) {
     GPTRS_HIP_CHECK(hipSetDevice(device));
     if (logits->consumed || tokens_out->consumed) fail_exec("tensor handle was donated to run_program and can no longer be used");
+    realize(logits);
+    realize(tokens_out);
     const Spec& s = logits->spec;
     const int max_rows = k::argmax_noalloc_max_rows();
     if (!dtype_is_float(s.dtype) || s.rank() != 2 || s.count() == 0)
@@ -467,12 +482,21 @@ gptrs_hip_tensor* Backend::token_tensor() {
     return t;
 }
 
-std::shared_ptr<Plan> Backend::get_plan(const char* json, size_t len, uint64_t key, const uint8_t* donate, size_t n_in) {
+std::shared_ptr<Plan> Backend::get_plan(const char* json, size_t len, uint64_t key, gptrs_hip_tensor* const* inputs, const uint8_t* donate, size_t n_in) {
     uint64_t k2 = key;
+    // inputs this backend produced as broadcasts of a vector are planned as BroadcastTo(vector): part of the compiled form
+    std::vector<const Spec*> bsrc(n_in, nullptr);
+    bool any_bsrc = false;
+    if (opt_fusion)
+        for (size_t i = 0; i < n_in; ++i)
+            if (inputs && inputs[i] && inputs[i]->bcast_src) { bsrc[i] = &inputs[i]->bcast_src->spec; any_bsrc = true; }
     if (key) {
         // donation pattern and fusion switch are part of the compiled form
         k2 = key * 1099511628211ull + (opt_fusion ? 0x9e3779b97f4a7c15ull : 0);
-        for (size_t i = 0; i < n_in; ++i) k2 = (k2 ^ (donate && donate[i] ? 0xA5 : 0x11)) * 1099511628211ull;
+        for (size_t i = 0; i < n_in; ++i) {
+            k2 = (k2 ^ (donate && donate[i] ? 0xA5 : 0x11)) * 1099511628211ull;
+            if (bsrc[i]) k2 = (k2 ^ (0xB7 + (uint64_t)bsrc[i]->rank())) * 1099511628211ull;
+        }
         if (!k2) k2 = 1;
         auto it = plan_index_.find(k2);
         if (it != plan_index_.end()) {
@@ -492,8 +516,31 @@ std::shared_ptr<Plan> Backend::get_plan(const char* json, size_t len, uint64_t k
         check.fn = plan->fn;
         build_plan(check, don);
     }
-    if (opt_fusion) plan->fused_ops = fuse_function(plan->fn);
+    plan->n_user_inputs = n_in;
+    plan->result_bcast_input.assign(plan->fn.result_ids.size(), -1);
+    for (size_t r = 0; r < plan->fn.result_ids.size(); ++r) plan->result_bcast_input[r] = result_broadcast_source(plan->fn, r);
+    if (opt_fusion) {
+        std::vector<BroadcastInput> expanded;
+        if (any_bsrc) expanded = expand_broadcast_inputs(plan->fn, bsrc);
+        for (const BroadcastInput& b : expanded) plan->ext_inputs.push_back(b.input);
+        plan->fused_ops = fuse_function(plan->fn);
+        collapse_broadcast_inputs(plan->fn, expanded);
+        don.resize(plan->fn.param_ids.size(), false);
+    }
     build_plan(*plan, don);
+    {
+        const Function& f = plan->fn;
+        plan->input_read.assign(f.param_ids.size(), false);
+        auto mark = [&](int v) {
+            for (size_t i = 0; i < f.param_ids.size(); ++i)
+                if (f.param_ids[i] == v) plan->input_read[i] = true;
+        };
+        for (const Instr& in : f.body)
+            if (!in.dead)
+                for (const Operand& o : in.operands)
+                    if (o.value >= 0) mark(o.value);
+        for (int r : f.result_ids) mark(r);
+    }
     plan->cacheable = key != 0;
     if (plan->workspace_bytes) plan->workspace = new_buffer(plan->workspace_bytes);
     if (!plan->const_host.empty()) {
@@ -570,7 +617,7 @@ bool Backend::run_graphed(Plan& plan, ExecCtx& cx, const std::vector<BufferP>& o
     if (plan.graph_builds >= 16 && plan.graph_hits < 4 * plan.graph_builds) return false;  // addresses never settle
     std::vector<uint64_t> key;
     key.reserve(cx.input_bufs.size() + out_bufs.size() + 8);
-    for (const auto& b : cx.input_bufs) key.push_back((uint64_t)(uintptr_t)b->ptr);
+    for (const auto& b : cx.input_bufs) key.push_back(b ? (uint64_t)(uintptr_t)b->ptr : 0);
     for (const auto& b : out_bufs) key.push_back((uint64_t)(uintptr_t)b->ptr);
     key.push_back(opt_chain ? 1 : 0);
     key.push_back((uint64_t)chain_f32_min_bytes);
@@ -652,14 +699,47 @@ bool Backend::run_graphed(Plan& plan, ExecCtx& cx, const std::vector<BufferP>& o
     return true;
 }
 
-void Backend::execute(Plan& plan, gptrs_hip_tensor* const* inputs, const uint8_t* donate, gptrs_hip_tensor** outputs) {
+void Backend::realize(const gptrs_hip_tensor* t) {
+    if (!t || t->buf || !t->lazy_plan) return;
+    std::shared_ptr<Plan> plan = std::move(t->lazy_plan);
+    gptrs_hip_tensor* in = t->lazy_input;
+    t->lazy_input = nullptr;
+    gptrs_hip_tensor* out = nullptr;
+    try {
+        execute(*plan, &in, nullptr, &out);
+    } catch (...) {
+        t->lazy_plan = plan;
+        t->lazy_input = in;
+        throw;
+    }
+    t->buf = out->buf;
+    delete out;
+    release_handle_locked(in);   // (the caller holds the backend's mutex)
+}
+
+void Backend::execute(Plan& plan, gptrs_hip_tensor* const* user_inputs, const uint8_t* user_donate, gptrs_hip_tensor** outputs) {
     const Function& fn = plan.fn;
     const size_t n_in = fn.param_ids.size();
+    // the caller's inputs, then the source vectors of the inputs that were planned as broadcasts
+    std::vector<gptrs_hip_tensor*> ext(n_in, nullptr);
+    std::vector<uint8_t> ext_don(n_in, 0);
+    for (size_t i = 0; i < plan.n_user_inputs; ++i) {
+        ext[i] = user_inputs[i];
+        ext_don[i] = user_donate && user_donate[i];
+    }
+    for (size_t j = 0; j < plan.ext_inputs.size(); ++j) {
+        gptrs_hip_tensor* t = user_inputs[plan.ext_inputs[j]];
+        if (!t || !t->bcast_src) fail_exec("input " + std::to_string(plan.ext_inputs[j]) + " lost its broadcast source between planning and execution");
+        ext[plan.n_user_inputs + j] = t->bcast_src;
+    }
+    gptrs_hip_tensor* const* inputs = ext.data();
+    const uint8_t* donate = user_donate ? ext_don.data() : nullptr;
     for (size_t i = 0; i < n_in; ++i) {
         if (!inputs[i]) fail_exec("null input handle");
         if (inputs[i]->consumed) fail_exec("input " + std::to_string(i) + " was donated to an earlier run_program call");
         if (inputs[i]->spec != fn.param_specs[i])
             fail_exec("entry input " + std::to_string(i) + " is " + inputs[i]->spec.str() + " but the program expects " + fn.param_specs[i].str());
+        if (plan.input_read[i]) realize(inputs[i]);
     }
     // a buffer donated for in-place update must not be reachable through another input or handle
     std::vector<bool> inplace_ok(n_in, false);
@@ -668,7 +748,7 @@ void Backend::execute(Plan& plan, gptrs_hip_tensor* const* inputs, const uint8_t
         if (ip < 0) continue;
         bool ok = donate && donate[ip] && inputs[ip]->refs.load() == 1 && inputs[ip]->buf.use_count() == 1;
         for (size_t j = 0; j < n_in && ok; ++j)
-            if ((int)j != ip && inputs[j]->buf == inputs[ip]->buf) ok = false;
+            if ((int)j != ip && inputs[j]->buf && inputs[j]->buf == inputs[ip]->buf) ok = false;
         inplace_ok[ip] = ok;
     }
     // output buffers
@@ -734,17 +814,42 @@ void Backend::execute(Plan& plan, gptrs_hip_tensor* const* inputs, const uint8_t
         t->spec = fn.result_specs[i];
         if (plan.result_input_alias[i] >= 0) t->buf = inputs[plan.result_input_alias[i]]->buf;
         else t->buf = out_bufs[plan.out_buffer_of_result[i]];
+        tag_broadcast_result(plan, i, user_inputs, t);
         outputs[i] = t;
     }
     consume_donated();
 }
 
+// A result that is a pure broadcast of input p along leading axes remembers the vector it came from.
+static gptrs_hip_tensor* broadcast_root(gptrs_hip_tensor* in) { return in->bcast_src ? in->bcast_src : in; }
+void Backend::tag_broadcast_result(const Plan& plan, size_t r, gptrs_hip_tensor* const* user_inputs, gptrs_hip_tensor* t) {
+    const int p = r < plan.result_bcast_input.size() ? plan.result_bcast_input[r] : -1;
+    if (p < 0 || !user_inputs[p]) return;
+    t->bcast_src = broadcast_root(user_inputs[p]);
+    t->bcast_src->refs.fetch_add(1);
+}
+
 void Backend::run_program(const char* json, size_t len, uint64_t key, gptrs_hip_tensor* const* inputs,
                           const uint8_t* donate, size_t n_in, gptrs_hip_tensor** outputs, size_t n_out) {
     GPTRS_HIP_CHECK(hipSetDevice(device));
-    auto plan = get_plan(json, len, key, donate, n_in);
+    auto plan = get_plan(json, len, key, inputs, donate, n_in);
     if (plan->fn.result_ids.size() != n_out)
         fail_exec("program produces " + std::to_string(plan->fn.result_ids.size()) + " results but " + std::to_string(n_out) + " were requested");
+    // One input, one result, the result a broadcast of the input (the subgraph the reference's parameter-only fold runs
+    // for a norm gain or a bias): nothing is computed until something reads the broadcast data itself.
+    if (opt_fusion && n_in == 1 && n_out == 1 && plan->result_bcast_input[0] == 0 && inputs[0] && !inputs[0]->consumed &&
+        inputs[0]->spec == plan->fn.param_specs[0] && !(donate && donate[0])) {
+        auto* t = new gptrs_hip_tensor();
+        t->spec = plan->fn.result_specs[0];
+        t->backend = this;
+        t->lazy_plan = plan;
+        t->lazy_input = inputs[0];
+        inputs[0]->refs.fetch_add(1);
+        tag_broadcast_result(*plan, 0, inputs, t);
+        outputs[0] = t;
+        last_launches = 0;
+        return;
+    }
     execute(*plan, inputs, donate, outputs);
 }
 
@@ -832,15 +937,12 @@ void gptrs_hip_tensor_retain(gptrs_hip_tensor* t) {
 
 void gptrs_hip_tensor_release(gptrs_hip_tensor* t) {
     if (!t) return;
-    if (t->refs.fetch_sub(1) == 1) {
-        // returning the block to the pool touches backend state
-        gptrs::Backend* owner = t->buf ? t->buf->owner : nullptr;
-        if (owner) {
-            std::lock_guard<std::mutex> g(owner->mu);
-            delete t;
-        } else {
-            delete t;
-        }
+    gptrs::Backend* owner = t->buf ? t->buf->owner : t->backend;
+    if (owner) {
+        std::lock_guard<std::mutex> g(owner->mu);
+        gptrs::release_handle_locked(t);
+    } else {
+        gptrs::release_handle_locked(t);
     }
 }
 
@@ -1024,6 +1126,47 @@ int gptrs_hip_decode_token_tensor(gptrs_hip_backend* b, gptrs_hip_tensor** out) 
 }
 
 const char* gptrs_hip_last_error(void) { return g_last_error.c_str(); }
+
+int gptrs_hip_fusion_report(const char* program_json, size_t json_len, const int64_t* bcast_len, size_t n_in, char* out, size_t cap,
+                            size_t* needed) {
+    return guarded([&] {
+        if (!program_json || !needed) gptrs::fail_exec("null argument");
+        gptrs::Function fn = gptrs::parse_program(program_json, json_len);
+        if (fn.param_ids.size() != n_in) gptrs::fail_exec("entry input arity mismatch");
+        std::vector<gptrs::Spec> vec(n_in);
+        std::vector<const gptrs::Spec*> src(n_in, nullptr);
+        for (size_t i = 0; i < n_in; ++i)
+            if (bcast_len && bcast_len[i] > 0) {
+                vec[i].dtype = fn.param_specs[i].dtype;
+                vec[i].dims = {bcast_len[i]};
+                src[i] = &vec[i];
+            }
+        const std::vector<gptrs::BroadcastInput> expanded = gptrs::expand_broadcast_inputs(fn, src);
+        gptrs::fuse_function(fn);
+        gptrs::collapse_broadcast_inputs(fn, expanded);
+        std::string text;
+        for (const gptrs::Instr& in : fn.body) {
+            if (in.dead) continue;
+            text += in.op_name;
+            if (in.op == gptrs::OpKind::FLinear) {
+                if (in.norm) text += in.norm_ln ? "+layer_norm" : "+rms_norm";
+                if (in.has_bias) text += "+bias";
+                if (in.act == 1) text += "+gelu";
+                if (in.act == 2) text += "+swiglu";
+                if (in.has_residual) text += "+residual";
+                text += in.mfma ? " [gemm]" : in.tiled ? " [stream]" : " [generic]";
+            }
+            if (in.op == gptrs::OpKind::FAttnDecode && in.rot_half > 0) text += "+rope";
+            text += '\n';
+        }
+        *needed = text.size() + 1;
+        if (out && cap) {
+            const size_t n = std::min(cap - 1, text.size());
+            memcpy(out, text.data(), n);
+            out[n] = 0;
+        }
+    });
+}
 
 int gptrs_hip_synchronize(gptrs_hip_backend* b) {
     return guarded([&] {

@@ -10,7 +10,9 @@
 // caller also asked for (e.g. layer_norm's mean) is still produced by the generic path.
 #include <algorithm>
 #include <cmath>
+#include <array>
 #include <cstring>
+#include <map>
 
 #include "kernels.hpp"
 #include "runtime.hpp"
@@ -135,11 +137,29 @@ struct Fuser {
         if (is_second(a)) { first = b; second = a; return true; }
         return false;
     }
-    bool vector_bcast_last(int v, int64_t n, int& vec) const {  // BroadcastTo(x[n]) along the last axis
+    // BroadcastTo(x) along leading axes of a vector x of n values (shape [n] or [1, .., 1, n]).  A program INPUT of n
+    // values and last extent n counts as the vector itself: that is what `BroadcastTo([1, n])(gamma)` has become when
+    // the reference's optimizer has folded it into a derived parameter ahead of a one-row program
+    // (crates/gpt-rs/src/backend/passes/param_only_fold_to_param.rs:24-160).
+    bool vector_bcast_last(int v, int64_t n, int& vec) const {
+        auto is_vector = [&](int q) {
+            const Spec* s = spec_of(q);
+            return s && s->rank() >= 1 && s->dims.back() == n && s->count() == n;
+        };
+        const int cur = strip(v);
+        if (!producer(cur)) {   // a program input
+            if (!is_vector(cur)) return false;
+            vec = cur;
+            return true;
+        }
         int src;
-        if (!bcast(v, src)) return false;
-        const Spec* s = spec_of(src);
-        if (!s || s->rank() != 1 || s->dims[0] != n) return false;
+        if (!bcast(cur, src)) return false;
+        for (int depth = 0; depth < 4 && !is_vector(src); ++depth) {   // broadcasts of broadcasts (the canonicaliser collapses them)
+            int inner;
+            if (!bcast(src, inner)) return false;
+            src = inner;
+        }
+        if (!is_vector(src)) return false;
         vec = src;
         return true;
     }
@@ -173,6 +193,45 @@ struct Fuser {
     }
     void kill(int v) {  // mark the (non-root) producer of a secondary output dead
         if (def[v] >= 0) fn.body[def[v]].dead = true;
+    }
+
+    // The front end's canonicaliser collapses Slice(Slice(x)) (crates/gpt-rs/src/backend/passes/slice_canonicalization.rs:
+    // 83-124): the rows of one sequence cut out of a stacked [B * T, P] projection and then its Q / K / V column blocks
+    // arrive as single slices of the stacked tensor.  The patterns below are written over "a packed [T, P] tensor and
+    // its column blocks", so such a slice is taken apart again: a row block (shared by the column blocks cut from it)
+    // and a column block of it.  Row blocks nothing else reads cost nothing: the fused ops read through them.
+    void pass_split_slices() {
+        std::map<std::array<int64_t, 3>, int> row_block;   // (source, first row, rows) -> value
+        std::vector<Instr> body;
+        body.reserve(fn.body.size() + 16);
+        bool changed = false;
+        for (const Instr& in : fn.body) {
+            if (!in.dead && in.op == OpKind::Slice && in.operands[0].value >= 0 && in.a.size() == 2) {
+                const Spec* xs = spec_of(in.operands[0].value);
+                if (xs && xs->rank() == 2 && in.b[0] < xs->dims[0] && in.b[1] < xs->dims[1]) {
+                    const std::array<int64_t, 3> key{in.operands[0].value, in.a[0], in.b[0]};
+                    auto it = row_block.find(key);
+                    if (it == row_block.end()) {
+                        Instr rb = make(OpKind::Slice, "Slice", {in.operands[0].value}, ++fn.max_value_id, Spec{xs->dtype, {in.b[0], xs->dims[1]}});
+                        rb.a = {in.a[0], 0};
+                        rb.b = {in.b[0], xs->dims[1]};
+                        it = row_block.emplace(key, rb.out_ids[0]).first;
+                        body.push_back(std::move(rb));
+                    }
+                    Instr cut = in;
+                    cut.operands[0].value = it->second;
+                    cut.a[0] = 0;
+                    body.push_back(std::move(cut));
+                    changed = true;
+                    continue;
+                }
+            }
+            body.push_back(in);   // (a copy: fn.body stays readable through spec_of while this loop runs)
+        }
+        if (changed) {
+            fn.body = std::move(body);
+            reindex();
+        }
     }
 
     // ---------------------------------------------------------------- elementwise sequences
@@ -1070,9 +1129,81 @@ struct Fuser {
 
 }  // namespace
 
+std::vector<BroadcastInput> expand_broadcast_inputs(Function& fn, const std::vector<const Spec*>& src) {
+    std::vector<BroadcastInput> out;
+    std::vector<Instr> front;
+    const size_t n_in = fn.param_ids.size();
+    for (size_t i = 0; i < n_in && i < src.size(); ++i) {
+        if (!src[i]) continue;
+        const Spec full = fn.param_specs[i];
+        const Spec& vec = *src[i];
+        if (vec.dtype != full.dtype || vec.rank() < 1 || full.rank() < 1 || vec.rank() > full.rank()) continue;
+        if (vec.dims.back() != full.dims.back() || vec.count() != vec.dims.back()) continue;
+        BroadcastInput b;
+        b.input = (int)i;
+        b.param_value = ++fn.max_value_id;
+        b.bcast_value = ++fn.max_value_id;
+        const int v = fn.param_ids[i];
+        bool read = false;
+        for (auto& in : fn.body)
+            for (auto& o : in.operands)
+                if (o.value == v) { o.value = b.bcast_value; read = true; }
+        if (!read) { fn.max_value_id -= 2; continue; }
+        fn.param_ids.push_back(b.param_value);
+        fn.param_specs.push_back(vec);
+        Instr bc;
+        bc.op = OpKind::BroadcastTo;
+        bc.op_name = "BroadcastTo";
+        Operand o; o.value = b.param_value;
+        bc.operands = {o};
+        bc.out_ids = {b.bcast_value};
+        bc.out_specs = {full};
+        front.push_back(std::move(bc));
+        out.push_back(b);
+    }
+    fn.body.insert(fn.body.begin(), front.begin(), front.end());
+    return out;
+}
+
+void collapse_broadcast_inputs(Function& fn, const std::vector<BroadcastInput>& expanded) {
+    for (const BroadcastInput& b : expanded) {
+        const int v = fn.param_ids[b.input];
+        for (auto& in : fn.body) {
+            if (in.dead) continue;
+            if (in.op == OpKind::BroadcastTo && in.out_ids[0] == b.bcast_value) { in.dead = true; continue; }
+            for (auto& o : in.operands)
+                if (o.value == b.bcast_value) o.value = v;
+        }
+    }
+}
+
+int result_broadcast_source(const Function& fn, size_t r) {
+    if (r >= fn.result_ids.size() || fn.result_specs[r].rank() < 1) return -1;
+    const int64_t n = fn.result_specs[r].dims.back();
+    int v = fn.result_ids[r];
+    bool widened = false;
+    for (int depth = 0; depth < 8; ++depth) {
+        for (size_t i = 0; i < fn.param_ids.size(); ++i)
+            if (fn.param_ids[i] == v) {
+                const Spec& s = fn.param_specs[i];
+                return (widened && s.rank() >= 1 && s.dims.back() == n && s.count() == n) ? (int)i : -1;
+            }
+        const Instr* p = nullptr;
+        for (const Instr& in : fn.body)
+            if (!in.dead && in.out_ids[0] == v) { p = &in; break; }
+        if (!p || (p->op != OpKind::BroadcastTo && p->op != OpKind::Reshape)) return -1;
+        if (p->operands.size() != 1 || p->operands[0].value < 0) return -1;
+        if (p->out_specs[0].rank() < 1 || p->out_specs[0].dims.back() != n) return -1;
+        widened = widened || p->op == OpKind::BroadcastTo;
+        v = p->operands[0].value;
+    }
+    return -1;
+}
+
 int fuse_function(Function& fn) {
     Fuser f(fn);
     f.dce();
+    f.pass_split_slices();
     f.pass_elementwise();
     f.dce();
     f.pass_norm_cast();

@@ -53,6 +53,7 @@ struct Buffer {
     ~Buffer();
 };
 using BufferP = std::shared_ptr<Buffer>;
+struct Plan;
 
 }  // namespace gptrs
 
@@ -60,8 +61,18 @@ using BufferP = std::shared_ptr<Buffer>;
 struct gptrs_hip_tensor {
     std::atomic<int> refs{1};
     gptrs::Spec spec;
-    gptrs::BufferP buf;
+    mutable gptrs::BufferP buf;
     bool consumed = false;  // donated to a run_program call
+    // A tensor this backend produced as a pure broadcast of a vector x[n] along leading axes (what the reference's
+    // ParamOnlyFoldToParamPass makes of `BroadcastTo(in)(gamma)` and of a bias broadcast,
+    // crates/gpt-rs/src/backend/passes/param_only_fold_to_param.rs:24-160): `bcast_src` is that vector (retained).  A
+    // program that takes such a tensor as an input is planned as if it held the BroadcastTo instruction itself, so the
+    // norm / bias patterns match and their kernels read the n values.  Until something reads the broadcast data
+    // itself, the handle has no buffer: `lazy_plan` run on `lazy_input` produces it (Backend::realize).
+    gptrs_hip_tensor* bcast_src = nullptr;
+    mutable std::shared_ptr<gptrs::Plan> lazy_plan;
+    mutable gptrs_hip_tensor* lazy_input = nullptr;
+    gptrs::Backend* backend = nullptr;   // set on handles without a buffer (the owner of a buffer is found through it)
     void* data() const { return buf ? buf->ptr : nullptr; }
 };
 
@@ -133,6 +144,14 @@ struct Plan {
     std::vector<int> result_input_alias;    // result position -> input position it aliases, or -1
     std::vector<size_t> out_buffer_bytes;
     std::vector<int> out_buffer_inplace_input;  // output buffer index -> donated input position or -1
+    // Inputs that arrived tagged as broadcasts of a vector: `ext_inputs[j]` is the position of the caller's input whose
+    // source vector is fed as input n_user_inputs + j (the function was rewritten to read BroadcastTo(vector) in place
+    // of that input before the fusion pass ran).
+    size_t n_user_inputs = 0;
+    std::vector<int> ext_inputs;
+    std::vector<bool> input_read;           // per (extended) input: some step or result reads its storage
+    // result position -> the caller's input it is a pure broadcast of along leading axes (or -1)
+    std::vector<int> result_bcast_input;
     size_t workspace_bytes = 0;
     BufferP workspace;
     BufferP consts;
@@ -230,8 +249,12 @@ class Backend {
     int64_t bytes_allocated() const { return (int64_t)pool_.bytes_allocated; }
 
   private:
-    std::shared_ptr<Plan> get_plan(const char* json, size_t len, uint64_t key, const uint8_t* donate, size_t n_in);
+    std::shared_ptr<Plan> get_plan(const char* json, size_t len, uint64_t key, gptrs_hip_tensor* const* inputs, const uint8_t* donate, size_t n_in);
     void execute(Plan& plan, gptrs_hip_tensor* const* inputs, const uint8_t* donate, gptrs_hip_tensor** outputs);
+    void tag_broadcast_result(const Plan& plan, size_t r, gptrs_hip_tensor* const* user_inputs, gptrs_hip_tensor* t);
+  public:
+    void realize(const gptrs_hip_tensor* t);   // gives a lazily broadcast handle its buffer
+  private:
     bool run_graphed(Plan& plan, ExecCtx& cx, const std::vector<BufferP>& out_bufs);
 
     DevicePool pool_;
@@ -268,8 +291,20 @@ class Backend {
     uint64_t next_buffer_id_ = 1;
 };
 
+void release_handle_locked(gptrs_hip_tensor* t);   // api.cpp
+
 // fuse.cpp: canonicalise + pattern-fuse the entry function in place.  Returns the number of fused ops.
 int fuse_function(Function& fn);
+// fuse.cpp: inputs that are known broadcasts of a vector.  `src[i]` is the vector's spec for input i (nullptr: an ordinary
+// input).  expand: appends one vector parameter per tagged input and makes the body read BroadcastTo(vector) instead of
+// the input; returns the positions of the tagged inputs, in the order of the appended parameters.  collapse (after the
+// fusion pass): whatever still reads a BroadcastTo that expand inserted reads the input itself again.
+struct BroadcastInput { int input = -1; int param_value = -1, bcast_value = -1; };
+std::vector<BroadcastInput> expand_broadcast_inputs(Function& fn, const std::vector<const Spec*>& src);
+void collapse_broadcast_inputs(Function& fn, const std::vector<BroadcastInput>& expanded);
+// fuse.cpp: the input position whose contents, broadcast along leading axes, are result `r` of the function as written
+// (a chain of BroadcastTo / Reshape instructions that keep the last axis), or -1.
+int result_broadcast_source(const Function& fn, size_t r);
 // plan.cpp: validate every instruction, assign storage and build launch descriptors.
 void build_plan(Plan& plan, const std::vector<bool>& donated);
 // plan.cpp: run one step with resolved pointers.

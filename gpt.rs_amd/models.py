@@ -80,6 +80,10 @@ class _ModelBase:
         self._source = None                 # loader.CheckpointParamSource of a model opened by loader.load_model
         self._base_ids: Dict[str, int] = {}
         self._lazy = False                  # weight streaming: parameters are resolved through the source at every run
+        # programs go through the reference's optimizer pipeline (front_end.py) before the backend sees them; False hands
+        # the backend the emitters' instruction stream as it is captured
+        self.front_end = True
+        self._optimized: Dict[int, tuple] = {}
 
     # -- parameters ------------------------------------------------------------------
     def param_dtype(self, name: str) -> str:
@@ -99,6 +103,7 @@ class _ModelBase:
             if not lazy:
                 self.backend.param_resolver().set(param_id(self.namespace, name), source.load(base_ids[name]))
         self._param_handles = None
+        self._optimized.clear()
 
     def set_param(self, name: str, array: np.ndarray, dtype: Optional[str] = None):
         """runtime/loader.rs:234-239: materialize once, store under the stable id."""
@@ -110,6 +115,7 @@ class _ModelBase:
             self.param_names.append(name)
         self.param_specs[name] = spec
         self._param_handles = None
+        self._optimized.clear()
 
     def set_param_bytes(self, name: str, spec: TensorSpec, data: bytes):
         handle = self.backend.materialize(spec, data)
@@ -118,6 +124,7 @@ class _ModelBase:
             self.param_names.append(name)
         self.param_specs[name] = spec
         self._param_handles = None
+        self._optimized.clear()
 
     def set_param_handle(self, name: str, handle):
         """Register a tensor that already lives on the device."""
@@ -126,6 +133,7 @@ class _ModelBase:
             self.param_names.append(name)
         self.param_specs[name] = handle.spec
         self._param_handles = None
+        self._optimized.clear()
         self._programs.clear()
 
     def drop_param(self, name: str):
@@ -135,6 +143,7 @@ class _ModelBase:
         stub = self.backend.materialize(TensorSpec(spec.dtype, [1]), None)
         self.backend.param_resolver().set(param_id(self.namespace, name), stub)
         self._param_handles = None
+        self._optimized.clear()
         self._programs.clear()
 
     _quant_programs: Dict[tuple, Program] = {}
@@ -208,6 +217,8 @@ class _ModelBase:
         return self.backend.materialize(TensorSpec(self.dtype, dims), None)
 
     def _run(self, program: Program, args: list, donate: Optional[list] = None):
+        if self.front_end:
+            return self._run_optimized(program, args, donate)
         if self._lazy:                    # streamed weights: resolved anew for every run, kept only by the source's cache
             params = [self.param_handle(n) for n in self.param_names]
         else:
@@ -218,6 +229,40 @@ class _ModelBase:
         if donate is not None:
             don = list(donate) + [False] * len(params)
         return self.backend.run_program(program, list(args) + params, don)
+
+    def _run_optimized(self, program: Program, args: list, donate: Optional[list] = None):
+        """The reference's path from a captured graph to the backend: the program goes through the optimizer once
+        (front_end.optimize: canonicalisers, parameter-only folds executed through the backend and stored in its memo
+        under derived ids, CSE, DCE; ops/graph/arena.rs:744-922), the optimised program and its input roles are kept
+        with the plan, and every run feeds Args positionally and Params by stable id (arena.rs:1116-1170)."""
+        from . import front_end as FE
+        n_args, names = len(args), self.param_names
+        entry = self._optimized.get(program.key)
+        if entry is None or entry[2] != tuple(names):
+            roles = [FE.ARG] * n_args + [FE.PARAM] * len(names)
+            stable = [None] * n_args + [int.from_bytes(param_id(self.namespace, n), "little") for n in names]
+            opt = FE.optimize(program, roles, stable, self.backend, self.backend.param_resolver())
+            entry = self._optimized[program.key] = (opt, {}, tuple(names))
+        opt, held, _ = entry
+        inputs, don = [], []
+        resolver = self.backend.param_resolver()
+        for pos, (p, src) in enumerate(zip(opt.inputs, opt.source_index)):
+            if p.role == FE.ARG:
+                inputs.append(args[src])
+                don.append(bool(donate[src]) if donate is not None else False)
+                continue
+            h = None if self._lazy and src is not None else held.get(pos)
+            if h is None:
+                if src is not None:
+                    h = self.param_handle(names[src - n_args])
+                else:
+                    h = resolver.get(FE.stable_id_bytes(p.stable_id))
+                    if h is None:
+                        raise KeyError(f"derived parameter {p.stable_id:#x} is not in the backend's memo")
+                held[pos] = h
+            inputs.append(h)
+            don.append(False)
+        return self.backend.run_program(opt.program, inputs, don if donate is not None else None)
 
 
 def _last_rows(hidden: Tensor, seq: int, batch: int) -> Tensor:

@@ -158,6 +158,19 @@ int gptrs_hip_decode_rows_tensor(gptrs_hip_backend* b, int64_t rows, gptrs_hip_t
  * one device) race.  Read the tokens with gptrs_hip_to_literal or feed tokens_out to the next program. */
 int gptrs_hip_sample_decode_rows_into(gptrs_hip_backend* b, const gptrs_hip_tensor* logits, gptrs_hip_tensor* tokens_out);
 
+/* No counterpart in the reference (a diagnostic; it touches no device and needs no backend).  Parses a program, runs the
+ * backend's fusion pass on it as gptrs_hip_run_program would, and writes one line per instruction that remains, its name
+ * followed for a fused linear layer by what it absorbed ("+rms_norm", "+layer_norm", "+bias", "+gelu", "+swiglu",
+ * "+residual") and the kernel family it was assigned ("[stream]" the weight-streaming decode kernels, "[gemm]" the
+ * matrix-core GEMM, "[generic]").  bcast_len (n_in entries, or NULL) says which inputs would arrive as handles this
+ * backend produced by broadcasting a vector of that many values along leading axes (0: an ordinary input): the
+ * reference's optimizer folds `BroadcastTo(shape)(gamma)` and bias broadcasts into such derived parameters before
+ * run_program (crates/gpt-rs/src/backend/passes/param_only_fold_to_param.rs:24-160), and the planner reads them as the
+ * broadcast they came from.  The text is truncated to cap - 1 bytes and terminated; *needed receives the size of the
+ * whole text with its terminator. */
+int gptrs_hip_fusion_report(const char* program_json, size_t json_len, const int64_t* bcast_len, size_t n_in, char* out, size_t cap,
+                            size_t* needed);
+
 /* Message of the calling thread's most recent non-zero return (BackendError Display). */
 const char* gptrs_hip_last_error(void);
 

@@ -141,6 +141,8 @@ def test_model_program_shapes_and_result_order():
         """RecordingBackend (crates/gpt-rs-backend-tests/src/recording_backend.rs:9-76): records, executes nothing."""
         def __init__(self):
             self.params, self.program, self.inputs, self.donate = {}, None, None, None
+        def backend_name(self):
+            return "recording"
         def param_resolver(self):
             return self
         def get(self, sid):
