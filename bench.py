@@ -546,6 +546,9 @@ def main():
     ap.add_argument("--residual", choices=["f32", "bf16"], default="f32",
                     help="f32 (default): bf16 weights and matmul operands with an f32 residual stream, f32 norms and f32 logits "
                          "(DotGeneral out_dtype); bf16: every tensor of the program is bf16")
+    ap.add_argument("--no-front-end", action="store_true",
+                    help="hand the backend the emitters' instruction stream; default: every model program goes through the "
+                         "reference's optimizer pipeline first (gpt.rs_amd/front_end.py), as the reference's arena does")
     ap.add_argument("--no-gpt2", action="store_true", help="skip the GPT-2 small f32 sub-record of the default run")
     ap.add_argument("--no-floor", action="store_true", help="skip the chain_floor sub-record (a chain with nothing to stream) of the default run")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -602,6 +605,7 @@ def main():
     model = models.Ministral.random(cfg, be, seed=5, dtype="Bf16", quant=None if args.quant == "none" else args.quant,
                                     residual_dtype="F32" if f32_stream else None)
     t_init = time.perf_counter() - t0
+    model.front_end = not args.no_front_end
     prompt = np.random.default_rng(6).integers(0, cfg.vocab_size, args.prompt).tolist()
     if args.batch > 1:
         return batched_decode(args, be, cfg, model, capacity)
@@ -691,7 +695,8 @@ def main():
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "ministral-3b-shape %s decode, batch 1, prompt %d, greedy, KV capacity %d" % (wname, args.prompt, capacity),
                    "layers": cfg.num_layers, "d_model": cfg.embed_dim, "heads": cfg.num_heads, "kv_heads": cfg.num_kv_heads,
-                   "head_dim": cfg.head_dim, "ffn": cfg.ffn_dim, "vocab": cfg.vocab_size, "cache_len_mid": mid_len},
+                   "head_dim": cfg.head_dim, "ffn": cfg.ffn_dim, "vocab": cfg.vocab_size, "cache_len_mid": mid_len,
+                   "program_stream": "emitters" if args.no_front_end else "optimizer pipeline (canonicalise, parameter-only fold, CSE, DCE) ahead of run_program"},
         "hbm_gbps": round(step_bytes / (elapsed / args.steps) / 1e9, 1),
         "hbm_frac": round(step_bytes / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS, 4),
         "algorithmic_bytes_per_step": step_bytes,
