@@ -1,9 +1,23 @@
 //! `PortableBackend` over the C ABI of `libgptrs_hip.so` (`include/gptrs_hip.h`), registered as backend "hip".
 //!
-//! Not compiled in this repository's build image (no Rust toolchain there).  One FFI symbol per trait method
-//! (crates/gpt-rs/src/backend/spec.rs:1288-1330); error codes map onto `BackendError` as the header states.
+//! Not compiled in this repository's build image (no Rust toolchain there): written against the reference's sources
+//! by reading, never type-checked.  One FFI symbol per trait method (crates/gpt-rs/src/backend/spec.rs:1288-1330);
+//! error codes map onto `BackendError` as the header states.
+//!
+//! `pipeline()` is not overridden (the default is `None`, spec.rs:1297): the library does its own pattern matching on
+//! the program `run_program` receives, after the front end's optimizer, and it plans a derived parameter that the
+//! parameter-only fold made of `BroadcastTo(shape)(gamma)` or of a bias broadcast as the broadcast it came from (the
+//! handle remembers its source vector), so the norm and bias patterns survive the fold without a
+//! `BackendPipeline::populate_pre` pass of the kind the Triton backend needs
+//! (crates/gpt-rs-backend-triton/src/optimizer/pipeline.rs:15-21).
+use gpt_rs::backend::param_resolver::ParamResolver;
 use gpt_rs::backend::spec::*;
-use std::{ffi::CStr, os::raw::c_char, sync::Arc};
+use std::{
+    collections::HashMap,
+    ffi::CStr,
+    os::raw::c_char,
+    sync::{Arc, Mutex},
+};
 
 #[repr(C)]
 pub struct RawBackend {
@@ -27,6 +41,7 @@ extern "C" {
     fn gptrs_hip_to_literal(b: *mut RawBackend, t: *const RawTensor, dst: *mut u8, cap: usize) -> i32;
     fn gptrs_hip_tensor_retain(t: *mut RawTensor);
     fn gptrs_hip_tensor_release(t: *mut RawTensor);
+    fn gptrs_hip_tensor_spec(t: *const RawTensor, dtype: *mut u32, dims: *mut i64, cap: usize) -> i32;
     fn gptrs_hip_run_program_donate(
         b: *mut RawBackend, json: *const c_char, len: usize, key: u64, inputs: *const *mut RawTensor, donate: *const u8,
         n_in: usize, outputs: *mut *mut RawTensor, n_out: usize,
@@ -88,6 +103,31 @@ fn dtype_tag(d: DType) -> BackendResult<u32> {
     })
 }
 
+fn dtype_of_tag(tag: u32) -> BackendResult<DType> {
+    Ok(match tag {
+        0 => DType::F32,
+        1 => DType::F16,
+        2 => DType::Bf16,
+        3 => DType::Si32,
+        4 => DType::I1,
+        5 => DType::Si8,
+        6 => DType::Ui8,
+        other => return Err(BackendError::execution(format!("unknown dtype tag {other}"))),
+    })
+}
+
+/// dtype and dims of a handle, as the library holds them (`gptrs_hip_tensor_spec`).
+fn spec_of_raw(raw: *const RawTensor) -> BackendResult<TensorSpec> {
+    let mut tag = 0u32;
+    let mut dims = [0i64; 8];
+    let rank = unsafe { gptrs_hip_tensor_spec(raw, &mut tag, dims.as_mut_ptr(), dims.len()) };
+    if rank < 0 || rank as usize > dims.len() {
+        return Err(BackendError::execution("tensor handle without a spec"));
+    }
+    let dims: Vec<Dimension> = dims[..rank as usize].iter().map(|&d| Dimension::Static(d as usize)).collect();
+    Ok(TensorSpec::new(dtype_of_tag(tag)?, Shape::new(dims)))
+}
+
 /// The parameter memo of the library, keyed by the 16 little-endian bytes of the reference's stable id (u128).
 pub struct HipParams {
     raw: *mut RawBackend,
@@ -102,8 +142,13 @@ impl ParamResolver for HipParams {
         if unsafe { gptrs_hip_param_get(self.raw, id.as_ptr(), &mut out) } != 0 || out.is_null() {
             return None;
         }
-        // the library hands back the spec through gptrs_hip_tensor_spec; elided here: the caller's ParamSource knows it
-        Some(HipTensor { raw: out, spec: TensorSpec::default() })
+        match spec_of_raw(out) {
+            Ok(spec) => Some(HipTensor { raw: out, spec }),
+            Err(_) => {
+                unsafe { gptrs_hip_tensor_release(out) };
+                None
+            }
+        }
     }
     fn set(&self, stable_id: u128, handle: HipTensor) {
         let id = stable_id.to_le_bytes();
@@ -111,9 +156,20 @@ impl ParamResolver for HipParams {
     }
 }
 
+/// The wire form of a program and the key the library caches its plan under.
+struct WireProgram {
+    json: String,
+    key: u64,
+}
+
 pub struct HipBackend {
     raw: *mut RawBackend,
     params: Arc<HipParams>,
+    /// serde-JSON text per program, found again by the FNV-1a hash of the program's bincode bytes.  `run_program`
+    /// receives `&Program` and nothing else (the arena's `PlanKey.hash`, ops/graph/arena.rs:993, does not cross the
+    /// trait), and a decode step's program is a few thousand instructions: serialising it to JSON and hashing a
+    /// megabyte of text on every step would cost more than the step.  bincode is several times cheaper and exact.
+    wire: Mutex<HashMap<u64, Arc<WireProgram>>>,
 }
 unsafe impl Send for HipBackend {}
 unsafe impl Sync for HipBackend {}
@@ -122,7 +178,23 @@ impl HipBackend {
     pub fn new(device: i32) -> BackendResult<Self> {
         let mut raw = std::ptr::null_mut();
         check(unsafe { gptrs_hip_create(device, &mut raw) })?;
-        Ok(Self { raw, params: Arc::new(HipParams { raw }) })
+        Ok(Self { raw, params: Arc::new(HipParams { raw }), wire: Mutex::new(HashMap::new()) })
+    }
+
+    fn wire_form(&self, program: &Program) -> BackendResult<Arc<WireProgram>> {
+        let bytes = program.to_bincode_bytes().map_err(|e| BackendError::execution(e.to_string()))?; // spec.rs:808-810
+        let key = bytes.iter().fold(0xcbf29ce484222325u64, |h, b| (h ^ *b as u64).wrapping_mul(0x100000001b3)) | 1;
+        let mut cache = self.wire.lock().expect("wire cache poisoned");
+        if let Some(hit) = cache.get(&key) {
+            return Ok(hit.clone());
+        }
+        if cache.len() >= 64 {
+            cache.clear(); // the arena keeps 64 programs (ops/graph/plan.rs:20-29); the library's plans have their own LRU
+        }
+        let json = program.to_json_string().map_err(|e| BackendError::execution(e.to_string()))?; // spec.rs:799-801
+        let entry = Arc::new(WireProgram { json, key });
+        cache.insert(key, entry.clone());
+        Ok(entry)
     }
 }
 impl Drop for HipBackend {
@@ -168,19 +240,27 @@ impl PortableBackend for HipBackend {
     }
 
     fn run_program(&self, program: &Program, inputs: &[HipTensor]) -> BackendResult<Vec<HipTensor>> {
-        let json = program.to_json_string().map_err(|e| BackendError::execution(e.to_string()))?; // spec.rs:799-801
-        // any stable 64-bit key of the program text; 0 would tell the library to hash the text itself
-        let key = json.bytes().fold(0xcbf29ce484222325u64, |h, b| (h ^ b as u64).wrapping_mul(0x100000001b3)) | 1;
-        let f = program.functions.iter().find(|f| f.name == program.entry).unwrap();
+        let wire = self.wire_form(program)?;
+        let f = program
+            .functions
+            .iter()
+            .find(|f| f.name == program.entry)
+            .ok_or_else(|| BackendError::execution("entry function not found"))?;
         let raw: Vec<*mut RawTensor> = inputs.iter().map(|t| t.raw).collect();
         let mut outs = vec![std::ptr::null_mut(); f.result_ids.len()];
         // donate = NULL: the arena still holds clones of every input, so nothing may be consumed here
         check(unsafe {
             gptrs_hip_run_program_donate(
-                self.raw, json.as_ptr() as _, json.len(), key, raw.as_ptr(), std::ptr::null(), raw.len(), outs.as_mut_ptr(), outs.len(),
+                self.raw, wire.json.as_ptr() as _, wire.json.len(), wire.key, raw.as_ptr(), std::ptr::null(), raw.len(),
+                outs.as_mut_ptr(), outs.len(),
             )
         })?;
-        Ok(outs.into_iter().zip(&f.results).map(|(raw, ty)| HipTensor { raw, spec: tensor_spec_of(ty) }).collect())
+        let mut handles = Vec::with_capacity(outs.len());
+        for (raw, ty) in outs.into_iter().zip(&f.results) {
+            // (a handle is owned from here on: an error below releases the ones already wrapped through Drop)
+            handles.push(HipTensor { raw, spec: tensor_spec_of(ty).or_else(|_| spec_of_raw(raw))? });
+        }
+        Ok(handles)
     }
 
     fn execute_instruction(&self, instruction: &Instruction, inputs: &[HipTensor]) -> BackendResult<Vec<HipTensor>> {
@@ -188,7 +268,7 @@ impl PortableBackend for HipBackend {
         let raw: Vec<*mut RawTensor> = inputs.iter().map(|t| t.raw).collect();
         let mut out = std::ptr::null_mut();
         check(unsafe { gptrs_hip_execute_instruction(self.raw, json.as_ptr() as _, json.len(), raw.as_ptr(), raw.len(), &mut out) })?;
-        Ok(vec![HipTensor { raw: out, spec: tensor_spec_of(&instruction.output) }])
+        Ok(vec![HipTensor { raw: out, spec: spec_of_raw(out)? }])
     }
 
     fn supports_decode_sampling(&self, r: DecodeSampleRequest) -> bool {
@@ -206,15 +286,18 @@ impl PortableBackend for HipBackend {
     }
 }
 
-fn tensor_spec_of(ty: &ValueType) -> TensorSpec {
+fn tensor_spec_of(ty: &ValueType) -> BackendResult<TensorSpec> {
     match ty {
-        ValueType::Tensor(spec) => spec.clone(),
-        _ => TensorSpec::default(),
+        ValueType::Tensor(spec) => Ok(spec.clone()),
+        _ => Err(BackendError::execution("the hip backend produces tensor values only")),
     }
 }
 
-// registration, as crates/gpt-rs-backend-ref-cpu/src/lib.rs:13-23 does
-#[linkme::distributed_slice(gpt_rs::backend::registry::BACKEND_REGISTRARS)]
-static REGISTER_HIP: fn() = || {
+/// Registers the backend under "hip" (crates/gpt-rs-backend-ref-cpu/src/lib.rs:13-23 does the same for "cpu").
+pub fn register_hip_backend() {
     gpt_rs::backend::registry::register_portable_backend("hip", || HipBackend::new(0).expect("no HIP device"));
-};
+}
+
+// Auto-register on library load, through the re-export as the reference's backends do
+#[gpt_rs::linkme::distributed_slice(gpt_rs::backend::registry::BACKEND_REGISTRARS)]
+static REGISTER_HIP_BACKEND: fn() = register_hip_backend;

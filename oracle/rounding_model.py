@@ -52,8 +52,11 @@ class MinistralRoundingModel:
     same tables); `cfg` carries embed_dim, num_heads, num_kv_heads, head_dim, ffn_dim, rotary_dim, eps, num_layers."""
 
     def __init__(self, cfg, params: Dict[str, np.ndarray], rope: Callable[[int, int], Tuple[np.ndarray, np.ndarray]],
-                 rounding: bool = True, bf16_scale: Optional[bool] = None):
+                 rounding: bool = True, bf16_scale: Optional[bool] = None, sites: Optional[Sequence[str]] = None):
         self.cfg, self.p, self.rope, self.rounding = cfg, params, rope, rounding
+        # `sites`: round only at the named places ("norm", "qkv", "rope", "p", "ctx", "act"; None: all of them), to
+        # see what each rounding point contributes
+        self.sites = None if sites is None else set(sites)
         # the attention scale 1 / sqrt(head_dim) reaches a program as a scalar literal of the tensor's dtype
         # (crates/gpt-rs/src/ops/ptir/graph.rs:2278-2298): a bf16 value in a bf16 attention (default with rounding on)
         self.bf16_scale = rounding if bf16_scale is None else bf16_scale
@@ -64,25 +67,26 @@ class MinistralRoundingModel:
             self.trace[name] = value
         return value
 
-    def _r(self, x):
-        return bf16_round(x) if self.rounding else np.asarray(x, np.float32)
+    def _r(self, x, site: Optional[str] = None):
+        on = self.rounding and (self.sites is None or site is None or site in self.sites)
+        return bf16_round(x) if on else np.asarray(x, np.float32)
 
     def _norm(self, x: np.ndarray, gamma: np.ndarray) -> np.ndarray:
         n = x.shape[-1]
         ms = (x * x).sum(axis=-1, keepdims=True, dtype=np.float32) * np.float32(1.0 / n)
         inv = (np.float32(1.0) / np.sqrt(ms + np.float32(self.cfg.eps), dtype=np.float32)).astype(np.float32)
-        return self._r((x * inv) * gamma.astype(np.float32))
+        return self._r((x * inv) * gamma.astype(np.float32), "norm")
 
     def _rope_rows(self, x: np.ndarray, heads: int, cos: np.ndarray, sin: np.ndarray) -> np.ndarray:
         """x [T, heads * Dh] -> rotate-half on the first rotary_dim of every head."""
         c = self.cfg
         T, dh, half = x.shape[0], c.head_dim, c.rotary_dim // 2
         xh = x.reshape(T, heads, dh).astype(np.float32)
-        cs, sn = self._r(cos)[:, None, :], self._r(sin)[:, None, :]
+        cs, sn = self._r(cos, "rope")[:, None, :], self._r(sin, "rope")[:, None, :]
         a, b = xh[:, :, :half], xh[:, :, half:2 * half]
         out = xh.copy()
-        out[:, :, :half] = self._r(a * cs - b * sn)
-        out[:, :, half:2 * half] = self._r(b * cs + a * sn)
+        out[:, :, :half] = self._r(a * cs - b * sn, "rope")
+        out[:, :, half:2 * half] = self._r(b * cs + a * sn, "rope")
         return out.reshape(T, heads * dh)
 
     def _attend(self, q: np.ndarray, K: np.ndarray, V: np.ndarray, first_pos: int, round_p: bool) -> np.ndarray:
@@ -104,14 +108,14 @@ class MinistralRoundingModel:
             s = np.where(visible, s, np.float32(-np.inf))
             e = np.exp(s - s.max(axis=1, keepdims=True), dtype=np.float32)
             l = e.sum(axis=1, keepdims=True, dtype=np.float32)
-            pe = self._r(e) if round_p else e
+            pe = self._r(e, "p") if round_p else e
             ctx[:, h, :] = (pe @ V[h // g]).astype(np.float32) / l
             if mass is not None:
                 mass[:, h, :] = (e @ np.abs(V[h // g])).astype(np.float32) / l
         if mass is not None:
             # sum_j p_j |v_j| per output: what a relative error of the probabilities is relative TO (the sum itself may cancel)
             self.trace["attention_mass"] = mass.reshape(T, hq * dh)
-        return self._r(ctx.reshape(T, hq * dh))
+        return self._r(ctx.reshape(T, hq * dh), "ctx")
 
     def _block(self, i: int, x: np.ndarray, pos0: int, cache: Optional[Tuple[np.ndarray, np.ndarray]]):
         c, p = self.cfg, self.p
@@ -120,7 +124,7 @@ class MinistralRoundingModel:
         hq, hkv, dh = c.num_heads, c.num_kv_heads, c.head_dim
         qp, kp = hq * dh, hkv * dh
         n1 = self._t(pre + "n1", self._norm(x, p[pre + "norm_1.gamma"]))
-        qkv = self._t(pre + "qkv", self._r(n1 @ p[pre + "attention.w_qkv"]))
+        qkv = self._t(pre + "qkv", self._r(n1 @ p[pre + "attention.w_qkv"], "qkv"))
         cos, sin = self.rope(pos0, T)
         q = self._rope_rows(qkv[:, :qp], hq, cos, sin)
         k = self._rope_rows(qkv[:, qp:qp + kp], hkv, cos, sin)
@@ -138,7 +142,7 @@ class MinistralRoundingModel:
         n2 = self._t(pre + "n2", self._norm(h, p[pre + "norm_2.gamma"]))
         gate = (n2 @ p[pre + "feed_forward.w_gate"]).astype(np.float32)
         up = (n2 @ p[pre + "feed_forward.w_up"]).astype(np.float32)
-        act = self._t(pre + "act", self._r((gate / (np.float32(1.0) + np.exp(gate * np.float32(-1.0), dtype=np.float32))) * up))
+        act = self._t(pre + "act", self._r((gate / (np.float32(1.0) + np.exp(gate * np.float32(-1.0), dtype=np.float32))) * up, "act"))
         out = self._t(pre + "out", (act @ p[pre + "feed_forward.w_down"]).astype(np.float32) + h)
         return out, (np.ascontiguousarray(K), np.ascontiguousarray(V))
 
