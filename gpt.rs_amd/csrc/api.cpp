@@ -306,8 +306,8 @@ void Backend::check_device_errors() {
         k::fill_zero(stream, d_err_flag_, 256);
         k::fill_zero(stream, d_chain_bar_, k::kChainBarrierBytes);
         GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
-        if (chain_stall_phase >= 0) {   // the stall was asked for (set_option "chain_stall_phase"): one launch, then back to normal
-            chain_stall_phase = -1;
+        if (chain_stall_fired) {   // the stall was asked for (set_option "chain_stall_phase"): one launch, then back to normal
+            chain_stall_fired = false;
             fail_exec("decode chain: grid barrier timed out (a stall was requested for this launch); the outputs of the program are invalid");
         }
         opt_chain = false;              // whatever kept the workgroups from meeting would do so again: one kernel per layer from here on
@@ -431,8 +431,13 @@ void Backend::sample_rows_into(const gptrs_hip_tensor* logits, gptrs_hip_tensor*
     const Spec& o = tokens_out->spec;
     if (o.dtype != DType::SI32 || o.count() != s.dims[0] || !tokens_out->data())
         fail_exec("sample_decode_rows_into: tokens_out must be si32[rows]");
+    if (tokens_out->buf == logits->buf) fail_exec("sample_decode_rows_into: tokens_out and logits are the same buffer");
     if (!k::argmax_rows_noalloc(stream, device, (int)s.dtype, logits->data(), s.dims[0], s.dims[1], (int32_t*)tokens_out->data()))
         fail_exec("sample_decode_rows_into: the scratch of this device is not initialised");
+    {
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) fail_exec(std::string("sample_decode_rows_into: kernel launch failed: ") + hipGetErrorString(e));
+    }
     if (tokens_out->buf) tokens_out->buf->id = next_buffer_id_++;   // the contents changed
     n_launches += 2;
 }
@@ -613,7 +618,7 @@ static bool check_graph_nodes(hipGraph_t graph, int device) {
 // allocated while recording.  Returns false when the caller must run the steps eagerly.
 bool Backend::run_graphed(Plan& plan, ExecCtx& cx, const std::vector<BufferP>& out_bufs) {
     constexpr size_t kMaxGraphs = 8, kSeenRing = 32;
-    if (!opt_graphs || opt_profile || chain_stall_phase >= 0 || !plan.cacheable || plan.steps.size() < 4) return false;
+    if (!opt_graphs || opt_profile || chain_stall_phase >= 0 || chain_stall_fired || !plan.cacheable || plan.steps.size() < 4) return false;
     if (plan.graph_builds >= 16 && plan.graph_hits < 4 * plan.graph_builds) return false;  // addresses never settle
     std::vector<uint64_t> key;
     key.reserve(cx.input_bufs.size() + out_bufs.size() + 8);
@@ -1185,7 +1190,11 @@ int gptrs_hip_set_option(gptrs_hip_backend* b, const char* name, int64_t value) 
         else if (!strcmp(name, "chain")) b->impl.opt_chain = value != 0;
         else if (!strcmp(name, "gemm_lds_direct")) b->impl.opt_gemm_lds_direct = value != 0;
         else if (!strcmp(name, "chain_f32_min_kb")) b->impl.chain_f32_min_bytes = std::max<int64_t>(0, value) << 10;
-        else if (!strcmp(name, "chain_stall_phase")) b->impl.chain_stall_phase = value < 0 ? -1 : (int)std::min<int64_t>(value, 1 << 20);
+        else if (!strcmp(name, "chain_stall_phase")) {
+            // phase 0 has no barrier in front of it: a stall there would never fire and the option would stay armed
+            if (value == 0) gptrs::fail_spec("chain_stall_phase must be >= 1 (or negative to disarm)");
+            b->impl.chain_stall_phase = value < 0 ? -1 : (int)std::min<int64_t>(value, 1 << 20);
+        }
         else if (!strcmp(name, "profile")) { b->impl.profile_reset(); b->impl.opt_profile = value != 0; }
         else if (!strcmp(name, "drop_derived_weights")) { if (value) b->impl.drop_derived_weights(); }
         else gptrs::fail_spec(std::string("unknown option `") + name + "`");

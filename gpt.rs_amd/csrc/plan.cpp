@@ -954,7 +954,13 @@ static bool run_chain(const Plan& plan, const Step& head, ExecCtx& cx) {
         GPTRS_HIP_CHECK(hipEventCreate(&e1));
         GPTRS_HIP_CHECK(hipEventRecord(e0, cx.stream));
     }
-    const int stall = cx.be->chain_stall_phase >= 0 ? std::min(cx.be->chain_stall_phase, (int)phases.size() - 1) : -1;
+    // a requested stall (a test hook) is consumed by the first launch that has a barrier to stall at
+    int stall = -1;
+    if (cx.be->chain_stall_phase >= 1 && phases.size() >= 2) {
+        stall = std::min(cx.be->chain_stall_phase, (int)phases.size() - 1);
+        cx.be->chain_stall_phase = -1;
+        cx.be->chain_stall_fired = true;
+    }
     if (!k::chain_launch(cx.stream, table, (int)phases.size(), lds_bytes, cx.be->chain_barrier(), cx.be->chain_abort_flag(), wfmt, stall)) {
         if (e0) { (void)hipEventDestroy(e0); (void)hipEventDestroy(e1); }
         cx.chain = false;

@@ -977,7 +977,9 @@ class Sampler:
         total = cum[-1]
         if not total > 0.0:
             return self.argmax(row)
-        x = np.float32(rng.uniform(0.0, float(total)))
+        # WeightedIndex draws in [0, total): the f32 rounding of the draw must not reach `total`, or the last index would
+        # be picked even where its weight is zero (a token that top-k masked)
+        x = min(np.float32(rng.uniform(0.0, float(total))), np.nextafter(total, np.float32(0.0)))
         return int(min(np.searchsorted(cum, x, side="right"), row.size - 1))
 
     def supports_backend_decode_sampling(self) -> bool:

@@ -207,6 +207,18 @@ def test_grid_barrier_gives_up_and_the_backend_goes_on(hip):
     again = hip_run(hip, p, [x] + ws)[0]
     assert hip.counter("chain_launches") == before + 1, "the chain must still be in use after a requested stall"
     assert np.array_equal(np.asarray(again), np.asarray(good))
+    # phase 0 has no barrier to stall at: the value is refused instead of staying armed for ever
+    with pytest.raises(BackendError):
+        hip.set_option("chain_stall_phase", 0)
+    # a stall that is armed while only one-phase launches run is consumed by the first launch that has a barrier, and
+    # a launch without one runs normally meanwhile
+    one = prog(lambda fb, a, w0: a.matmul(w0), [("Bf16", [1, k]), ("Bf16", [k, k])])
+    want_one = hip_run(hip, one, [x, ws[0]])[0]
+    hip.set_option("chain_stall_phase", 2)
+    assert np.array_equal(np.asarray(hip_run(hip, one, [x, ws[0]])[0]), np.asarray(want_one))
+    with pytest.raises(BackendError, match="a stall was requested"):
+        hip_run(hip, p, [x] + ws)
+    assert np.array_equal(np.asarray(hip_run(hip, p, [x] + ws)[0]), np.asarray(good))
 
 
 @pytest.mark.parametrize("k,n", [(2560, 32768), (1536, 32768), (3072, 32776), (200, 4100)])

@@ -136,3 +136,18 @@ def test_generator_falls_back_to_the_host_sampler_when_the_backend_declines():
     m_ref = models.Gpt.random(TINY, OracleBackend(), seed=2, std=0.3)
     assert models.Generator(m, [3, 9, 4]).generate(8) == models.Generator(m_ref, [3, 9, 4]).generate(8)
     assert len(models.Generator(m, [3, 9, 4], temperature=0.9, seed=1).generate(8)) == 8
+
+
+def test_a_draw_that_rounds_up_to_the_total_never_picks_a_zero_weight_token():
+    """WeightedIndex samples in [0, total) (sampler.rs:52-72): a uniform draw whose f32 rounding reaches `total` must not
+    fall behind the last cumulative weight, where the clamp would pick the last index whatever its weight."""
+    class Top:
+        """A generator whose uniform draw is the largest double below `high`."""
+        def uniform(self, low, high):
+            return float(np.nextafter(high, low))
+
+    s = Sampler(1.0, top_k=2)
+    row = np.array([3.0, 2.5, -1.0, -2.0, -3.0], np.float32)   # top-2 masks the last three: their weight is exactly 0
+    probs = s.probabilities(row)
+    assert probs[-1] == 0.0 and probs[2] == 0.0
+    assert s.sample(row, Top()) in (0, 1)
