@@ -401,6 +401,49 @@ def chain_floor_record(be, phases: int = 157, reps: int = 20):
                     "grid barrier, staging, one or three j-steps, epilogue and store acknowledgement per phase, nothing to stream" % phases}
 
 
+def quant_record(be, cfg, quant: str, prompt, capacity: int, steps: int = 64, warmup: int = 8, prof_steps: int = 16):
+    """The headline workload with weight-only quantised linears (BASELINE configs[4]; every linear incl. lm_head as int8
+    per output channel or int4 groups of 128, activations / KV cache / embeddings bf16, f32 residual stream): steady
+    decode rate, and the persistent launch priced with the step's algorithmic bytes (codes + scales once, valid KV
+    once), timed with HIP events on the backend's stream."""
+    from gptrs_amd import models
+    t0 = time.perf_counter()
+    model = models.Ministral.random(cfg, be, seed=5, dtype="Bf16", quant=quant, residual_dtype="F32")
+    t_init = time.perf_counter() - t0
+    gen = models.Generator(model, prompt, kv_cache_capacity=capacity)
+    for _ in range(warmup):
+        gen.step()
+    be.synchronize()
+    start = gen.processed_len
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        gen.step()
+    be.synchronize()
+    t_step = (time.perf_counter() - t0) / steps
+    launches = be.counter("last_program_launches")
+    step_bytes = algorithmic_bytes_per_step(cfg, 2, start + steps // 2, quant, True)
+    prof_start = gen.processed_len
+    c0, p0 = be.counter("chain_launches"), be.counter("chain_phases")
+    be.set_option("profile", 1)
+    for _ in range(prof_steps):
+        gen.step()
+    t_ns, calls = be.counter("linear_time_ns"), be.counter("linear_calls")
+    be.set_option("profile", 0)
+    chains, phases = be.counter("chain_launches") - c0, be.counter("chain_phases") - p0
+    roof = None
+    if t_ns > 0 and chains == calls and calls > 0:
+        nbytes = sum(algorithmic_bytes_per_step(cfg, 2, prof_start + i, quant, True) for i in range(prof_steps))
+        achieved = nbytes / (t_ns * 1e-9) / 1e9
+        roof = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                "traffic": None, "kernel": "chain_kernel over %s code words, %d phases per launch" % (quant, phases // max(chains, 1)),
+                "launches": calls, "avg_launch_us": round(t_ns / calls / 1e3, 2), "bytes_per_launch": round(nbytes / calls)}
+    return {"metric": "decode tokens/s, Ministral-3B-shape %s weight-only linears (lm_head included), batch 1" % quant,
+            "value": round(1.0 / t_step, 2), "unit": "tokens/s", "steps": steps, "warmup": warmup, "ms_per_step": round(t_step * 1e3, 4),
+            "dtype": "bf16 activations, %s weights" % ("int8" if quant == "w8" else "int4"), "data": "synthetic",
+            "hbm_gbps": round(step_bytes / t_step / 1e9, 1), "hbm_frac": round(step_bytes / t_step / 1e9 / HBM_PEAK_GBPS, 4),
+            "algorithmic_bytes_per_step": step_bytes, "launches_per_step": launches, "weight_init_s": round(t_init, 1), "roofline": roof}
+
+
 def gpt2_record(be, steps: int, warmup: int, cpu=None):
     """BASELINE configs[0]: GPT-2 small f32, weights N(0, 0.02) from seed 0, prompt of 16 ids (seed 1), greedy, 64 tokens
     with KV cache (capacity 128).  Timed like the reference's published figure (README.md:27-50,
@@ -550,6 +593,7 @@ def main():
                     help="hand the backend the emitters' instruction stream; default: every model program goes through the "
                          "reference's optimizer pipeline first (gpt.rs_amd/front_end.py), as the reference's arena does")
     ap.add_argument("--no-gpt2", action="store_true", help="skip the GPT-2 small f32 sub-record of the default run")
+    ap.add_argument("--no-int8", action="store_true", help="skip the int8 weight-only sub-record (BASELINE configs[4]) of the default run")
     ap.add_argument("--no-floor", action="store_true", help="skip the chain_floor sub-record (a chain with nothing to stream) of the default run")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain elementwise kernel of known traffic (x + 0 over 2^28 f32: 1 GiB read, 1 GiB written, "
@@ -683,8 +727,15 @@ def main():
                "mfma_frac": round(prefill_flops / t_prefill / 1e12 / MFMA_PEAK_TFLOPS, 4), "peak_tflop_per_s": MFMA_PEAK_TFLOPS,
                "what": "wall time of one 1024-token prefill call (median of three; head on the last row), all launches included"}
     bytes_allocated = be.counter("bytes_allocated")
-    gpt2 = None
+    gpt2 = int8 = None
     floor = chain_floor_record(be) if args.quant == "none" and not args.no_floor else None
+    default_line = args.quant == "none" and args.layers == 26
+    if default_line and not args.no_int8:
+        del gen, model
+        gen = model = None
+        be.set_option("drop_derived_weights", 1)
+        int8 = quant_record(be, cfg, "w8", prompt, capacity)
+        be.set_option("drop_derived_weights", 1)
     if not args.no_gpt2:
         del gen, model
         gpt2 = gpt2_record(be, 8, 2, cpu_gpt2)
@@ -707,6 +758,7 @@ def main():
         "cpu_baseline": cpu_main,
         "prefill": prefill,
         "chain_floor": floor,
+        "int8": int8,
         "gpt2_f32": gpt2,
     }
     print(json.dumps(out))

@@ -4,12 +4,14 @@
 //! by reading, never type-checked.  One FFI symbol per trait method (crates/gpt-rs/src/backend/spec.rs:1288-1330);
 //! error codes map onto `BackendError` as the header states.
 //!
-//! `pipeline()` is not overridden (the default is `None`, spec.rs:1297): the library does its own pattern matching on
-//! the program `run_program` receives, after the front end's optimizer, and it plans a derived parameter that the
-//! parameter-only fold made of `BroadcastTo(shape)(gamma)` or of a bias broadcast as the broadcast it came from (the
-//! handle remembers its source vector), so the norm and bias patterns survive the fold without a
-//! `BackendPipeline::populate_pre` pass of the kind the Triton backend needs
-//! (crates/gpt-rs-backend-triton/src/optimizer/pipeline.rs:15-21).
+//! `pipeline()` returns the backend's own optimizer hooks (`pipeline.rs`): one pass ahead of the parameter-only fold
+//! that hands the norms over as CustomCalls.  The library does its own pattern matching on the program `run_program`
+//! receives, after the front end's optimizer, and it also plans a derived parameter that the fold made of
+//! `BroadcastTo(shape)(gamma)` or of a bias broadcast as the broadcast it came from (the handle remembers its source
+//! vector), so bias epilogues survive the fold without a pass of their own.
+pub mod pipeline;
+
+use gpt_rs::backend::pipeline::BackendPipeline;
 use gpt_rs::backend::param_resolver::ParamResolver;
 use gpt_rs::backend::spec::*;
 use std::{
@@ -208,6 +210,10 @@ impl PortableBackend for HipBackend {
 
     fn backend_name(&self) -> &str {
         "hip"
+    }
+
+    fn pipeline(&self) -> Option<Arc<dyn BackendPipeline<Self>>> {
+        Some(Arc::new(pipeline::HipPipeline))
     }
 
     fn param_resolver(&self) -> Option<Arc<dyn ParamResolver<Handle = HipTensor>>> {

@@ -515,6 +515,7 @@ std::shared_ptr<Plan> Backend::get_plan(const char* json, size_t len, uint64_t k
     auto plan = std::make_shared<Plan>();
     plan->fn = parse_program(json, len);
     if (plan->fn.param_ids.size() != n_in) fail_exec("entry input arity mismatch");
+    lower_norm_calls(plan->fn);
     {
         // validate the program as written before any rewrite touches it
         Plan check;
@@ -1138,6 +1139,7 @@ int gptrs_hip_fusion_report(const char* program_json, size_t json_len, const int
         if (!program_json || !needed) gptrs::fail_exec("null argument");
         gptrs::Function fn = gptrs::parse_program(program_json, json_len);
         if (fn.param_ids.size() != n_in) gptrs::fail_exec("entry input arity mismatch");
+        gptrs::lower_norm_calls(fn);
         std::vector<gptrs::Spec> vec(n_in);
         std::vector<const gptrs::Spec*> src(n_in, nullptr);
         for (size_t i = 0; i < n_in; ++i)

@@ -1129,6 +1129,45 @@ struct Fuser {
 
 }  // namespace
 
+void lower_norm_calls(Function& fn) {
+    auto spec_of = [&](int v) -> const Spec* {
+        for (size_t i = 0; i < fn.param_ids.size(); ++i)
+            if (fn.param_ids[i] == v) return &fn.param_specs[i];
+        for (const Instr& in : fn.body)
+            for (size_t o = 0; o < in.out_ids.size(); ++o)
+                if (in.out_ids[o] == v) return &in.out_specs[o];
+        return nullptr;
+    };
+    for (Instr& in : fn.body) {
+        if (in.op != OpKind::CustomCall) continue;
+        const int kind = norm_call_target(in.target);
+        if (!kind) continue;
+        const size_t want = kind == 1 ? 3 : 2;
+        if (in.operands.size() != want) fail_spec(in.target + ": expects " + std::string(kind == 1 ? "(x, gamma, beta)" : "(x, gamma)"));
+        const Spec* xs = in.operands[0].value >= 0 ? spec_of(in.operands[0].value) : nullptr;
+        if (!xs || !dtype_is_float(xs->dtype) || xs->rank() < 1) fail_spec(in.target + ": x must be a float tensor of rank >= 1");
+        const int64_t n = xs->dims.back();
+        for (size_t o = 1; o < want; ++o) {
+            const Spec* vs = in.operands[o].value >= 0 ? spec_of(in.operands[o].value) : nullptr;
+            if (!vs || vs->dtype != xs->dtype || vs->dims != std::vector<int64_t>{n})
+                fail_spec(in.target + ": gamma / beta must be [" + std::to_string(n) + "] of x's dtype");
+        }
+        if (in.out_specs[0] != *xs) fail_spec(in.target + ": the output has x's type");
+        auto it = in.attrs.find("eps");
+        const Json* val = it == in.attrs.end() ? nullptr : it->second.find("value");
+        if (!val) fail_spec(in.target + ": attribute `eps` (F64) is missing");
+        try {
+            in.eps = (float)val->as_double();
+        } catch (const JsonError&) {
+            fail_spec(in.target + ": attribute `eps` must be a number");
+        }
+        if (!(in.eps > 0.0f) || !std::isfinite(in.eps)) fail_spec(in.target + ": eps must be positive and finite");
+        in.scale = 1.0f / (float)n;   // the functional's own literal (normalization.rs:123-217: 1.0 / n as f32)
+        in.op = kind == 1 ? OpKind::FLayerNorm : OpKind::FRmsNorm;
+        in.op_name = kind == 1 ? "fused.layer_norm" : "fused.rms_norm";
+    }
+}
+
 std::vector<BroadcastInput> expand_broadcast_inputs(Function& fn, const std::vector<const Spec*>& src) {
     std::vector<BroadcastInput> out;
     std::vector<Instr> front;

@@ -150,6 +150,15 @@ inline int quant_dot_target(const std::string& t) {
     if (t == "gpt_rs.hip.dot_w4g128.v1") return 2;
     return 0;
 }
+// CustomCall targets a front-end pass emits in place of a matched functional sequence (what a BackendPipeline's
+// populate_pre pass does ahead of the parameter-only fold, crates/gpt-rs/src/backend/pipeline.rs:60-65, 89-92; the
+// Triton backend's is crates/gpt-rs-backend-triton/src/optimizer/layer_norm_fusion.rs:30-97): 1 layer_norm(x, gamma,
+// beta), 2 rms_norm(x, gamma); attribute "eps" (F64), reduction over the last axis
+inline int norm_call_target(const std::string& t) {
+    if (t == "gpt_rs.hip.layer_norm.v1") return 1;
+    if (t == "gpt_rs.hip.rms_norm.v1") return 2;
+    return 0;
+}
 inline int quant_op_target(const std::string& t) {
     if (t == "gpt_rs.hip.quantize_w8_scales.v1") return 1;
     if (t == "gpt_rs.hip.quantize_w8.v1") return 2;

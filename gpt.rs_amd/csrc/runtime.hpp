@@ -303,6 +303,10 @@ int fuse_function(Function& fn);
 struct BroadcastInput { int input = -1; int param_value = -1, bcast_value = -1; };
 std::vector<BroadcastInput> expand_broadcast_inputs(Function& fn, const std::vector<const Spec*>& src);
 void collapse_broadcast_inputs(Function& fn, const std::vector<BroadcastInput>& expanded);
+// fuse.cpp: CustomCall norm targets (norm_call_target) become the FLayerNorm / FRmsNorm instructions the pattern pass
+// would have formed from the functional's own sequence; their operands are validated here.  Runs on every program,
+// fusion on or off: the targets are part of what the backend executes.
+void lower_norm_calls(Function& fn);
 // fuse.cpp: the input position whose contents, broadcast along leading axes, are result `r` of the function as written
 // (a chain of BroadcastTo / Reshape instructions that keep the last axis), or -1.
 int result_broadcast_source(const Function& fn, size_t r);

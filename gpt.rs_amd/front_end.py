@@ -828,3 +828,187 @@ def optimize(program: Program, roles: Sequence[str], stable_ids: Sequence[Option
     out = program_from_function(fn, program.obj.get("entry"))
     return OptimizedProgram(out, list(cx.entry), [original.index(p.id) if p.id in original else None for p in cx.entry],
                             cx.folds_run, cx.folds_reused)
+
+
+# ------------------------------------------------------------------------------------------ the hip backend's pipeline
+NORM_TARGETS = {"layer_norm": "gpt_rs.hip.layer_norm.v1", "rms_norm": "gpt_rs.hip.rms_norm.v1"}
+
+
+class HipNormFusionPass:
+    """What `gpt-rs-backend-hip`'s BackendPipeline puts into `populate_pre` (crates/gpt-rs/src/backend/pipeline.rs:60-65,
+    89-92), the route the reference's Triton backend takes for the same problem
+    (crates/gpt-rs-backend-triton/src/optimizer/layer_norm_fusion.rs:30-97, pipeline.rs:15-21): ahead of the
+    parameter-only fold, the instruction sequences of `functional::layer_norm` and `functional::rms_norm`
+    (ops/functional/normalization.rs:123-217) are replaced by ONE CustomCall each, with gamma and beta themselves as
+    operands, so the fold finds no broadcast of them to turn into a derived parameter.  The sequence's interior
+    instructions go only where nothing else reads them (a program that also asks for the mean keeps it).
+
+    The library does not need this pass: it plans a derived broadcast parameter as the broadcast it came from.  The pass
+    is the second, explicit route, for a front end whose derived parameters lose that provenance (handles copied through
+    the host, a resolver outside the library)."""
+
+    name = "hip-norm-fusion"
+
+    def run(self, fn: dict, cx: "OptimizeContext") -> bool:
+        rw = Rewriter(fn)
+        changed = False
+        # roots last to first: a layer norm ends in an rms-norm-shaped tail over the centred row, and the larger sequence
+        # has to claim its instructions first
+        for vid in reversed(rw.order()):
+            if not rw.contains(vid):
+                continue
+            ins = rw.inst[vid]
+            if op_name(ins["op"]) != "ElementwiseBinary":
+                continue
+            m = self._layer_norm(rw, ins) if op_attrs(ins["op"]) == "Add" else (self._rms_norm(rw, ins) if op_attrs(ins["op"]) == "Mul" else None)
+            if m is None:
+                continue
+            kind, operands, eps, interior = m
+            call = {"CustomCall": {"target": NORM_TARGETS[kind], "attrs": {"eps": {"kind": "F64", "value": float(eps)},
+                                                                             "axis": {"kind": "I64", "value": len(_static_dims(ins["output"])) - 1}}}}
+            new = rw.insert_before(vid, call, [{"Value": v} for v in operands], copy.deepcopy(ins["output"]))
+            rw.replace_value(vid, new)
+            for dead in interior:   # last to first: an instruction goes once its readers have gone
+                if rw.contains(dead) and not rw.users_of(dead) and dead not in fn["result_ids"]:
+                    rw.erase(dead)
+            changed = True
+        return changed
+
+    # -- matchers: every helper returns None when the shape of the graph is not the functional's
+    @staticmethod
+    def _def(rw, v, name, attr=None):
+        ins = rw.inst.get(v)
+        if ins is None or op_name(ins["op"]) != name:
+            return None
+        if attr is not None and op_attrs(ins["op"]) != attr:
+            return None
+        return ins
+
+    @classmethod
+    def _binary(cls, rw, v, kind):
+        ins = cls._def(rw, v, "ElementwiseBinary", kind)
+        if ins is None or len(ins["operands"]) != 2 or any("Value" not in o for o in ins["operands"]):
+            return None
+        return ins["operands"][0]["Value"], ins["operands"][1]["Value"]
+
+    @classmethod
+    def _bcast(cls, rw, v):
+        ins = cls._def(rw, v, "BroadcastTo")
+        return _single_value(ins) if ins is not None else None
+
+    @classmethod
+    def _scalar(cls, rw, v):
+        """BroadcastTo(shape)(BroadcastTo([])(Literal)) (ops/ptir/mod.rs:16-22): the literal's value as float."""
+        for _ in range(3):
+            ins = cls._def(rw, v, "BroadcastTo")
+            if ins is None or len(ins["operands"]) != 1:
+                return None
+            o = ins["operands"][0]
+            if "Literal" in o:
+                lit = o["Literal"]
+                data = bytes(lit["bytes"])
+                if lit["spec"]["dtype"] == "F32" and len(data) == 4:
+                    return float(struct.unpack("<f", data)[0])
+                if lit["spec"]["dtype"] == "Bf16" and len(data) == 2:
+                    return float(struct.unpack("<f", b"\x00\x00" + data)[0])
+                return None
+            v = o["Value"]
+        return None
+
+    @classmethod
+    def _reduce_sum_last(cls, rw, v):
+        ins = cls._def(rw, v, "Reduce")
+        if ins is None:
+            return None
+        a = op_attrs(ins["op"])
+        src = _single_value(ins)
+        if src is None or a["kind"] != "Sum" or not a["keepdims"] or list(a["axes"]) != [len(_static_dims(rw.types[src])) - 1]:
+            return None
+        return src
+
+    @classmethod
+    def _vector(cls, rw, v, n):
+        src = cls._bcast(rw, v)
+        if src is None or _static_dims(rw.types[src]) != (n,):
+            return None
+        return src
+
+    def _rms_norm(self, rw, root):
+        n = _static_dims(root["output"])[-1]
+        ops = self._binary(rw, root["id"], "Mul")
+        if ops is None:
+            return None
+        nrm, gb = ops
+        gamma = self._vector(rw, gb, n)
+        o2 = self._binary(rw, nrm, "Mul") if gamma is not None else None
+        if o2 is None:
+            return None
+        x, irb = o2
+        ir = self._bcast(rw, irb)
+        t = self._def(rw, ir, "ElementwiseUnary", "Rsqrt") if ir is not None else None
+        o3 = self._binary(rw, _single_value(t), "Add") if t is not None else None
+        if o3 is None:
+            return None
+        ms, eb = o3
+        eps = self._scalar(rw, eb)
+        o4 = self._binary(rw, ms, "Mul")
+        if eps is None or o4 is None:
+            return None
+        s, ic = o4
+        inv_n = self._scalar(rw, ic)
+        sq = self._reduce_sum_last(rw, s)
+        o5 = self._binary(rw, sq, "Mul") if sq is not None else None
+        if inv_n is None or o5 is None or o5 != (x, x) or rw.types[x] != root["output"]:
+            return None
+        if abs(inv_n * n - 1.0) > 1e-2:
+            return None
+        return "rms_norm", [x, gamma], eps, [nrm, gb, irb, ir, _single_value(t), eb, ms, ic, s, sq]
+
+    def _layer_norm(self, rw, root):
+        n = _static_dims(root["output"])[-1]
+        ops = self._binary(rw, root["id"], "Add")
+        if ops is None:
+            return None
+        t, bb = ops
+        beta = self._vector(rw, bb, n)
+        o1 = self._binary(rw, t, "Mul") if beta is not None else None
+        if o1 is None:
+            return None
+        nrm, gb = o1
+        gamma = self._vector(rw, gb, n)
+        o2 = self._binary(rw, nrm, "Mul") if gamma is not None else None
+        if o2 is None:
+            return None
+        cen, isb = o2
+        istd = self._bcast(rw, isb)
+        rs = self._def(rw, istd, "ElementwiseUnary", "Rsqrt") if istd is not None else None
+        o3 = self._binary(rw, _single_value(rs), "Add") if rs is not None else None
+        if o3 is None:
+            return None
+        vm, eb = o3
+        eps = self._scalar(rw, eb)
+        o4 = self._binary(rw, vm, "Mul")
+        if eps is None or o4 is None:
+            return None
+        vs, ic = o4
+        sq = self._reduce_sum_last(rw, vs)
+        o5 = self._binary(rw, sq, "Mul") if sq is not None else None
+        if self._scalar(rw, ic) is None or o5 is None or o5 != (cen, cen):
+            return None
+        o6 = self._binary(rw, cen, "Sub")
+        if o6 is None:
+            return None
+        x, mb = o6
+        mean = self._bcast(rw, mb)
+        o7 = self._binary(rw, mean, "Mul") if mean is not None else None
+        if o7 is None or self._scalar(rw, o7[1]) != self._scalar(rw, ic):
+            return None
+        s = o7[0]
+        if self._reduce_sum_last(rw, s) != x or rw.types[x] != root["output"]:
+            return None
+        return "layer_norm", [x, gamma, beta], eps, [t, bb, gb, nrm, isb, istd, _single_value(rs), eb, vm, vs, sq, cen, mb, mean, o7[1], ic, s]
+
+
+def hip_backend_pipeline() -> dict:
+    """The passes of the hip backend's BackendPipeline by hook, as keyword arguments of `optimize`."""
+    return {"pre": [HipNormFusionPass()]}

@@ -83,6 +83,9 @@ class _ModelBase:
         # programs go through the reference's optimizer pipeline (front_end.py) before the backend sees them; False hands
         # the backend the emitters' instruction stream as it is captured
         self.front_end = True
+        # with the front end on: also run the hip backend's own pipeline passes (front_end.hip_backend_pipeline: norms
+        # become CustomCalls ahead of the parameter-only fold), the second route through the reference's optimizer
+        self.backend_pipeline = False
         self._optimized: Dict[int, tuple] = {}
 
     # -- parameters ------------------------------------------------------------------
@@ -238,12 +241,13 @@ class _ModelBase:
         from . import front_end as FE
         n_args, names = len(args), self.param_names
         entry = self._optimized.get(program.key)
-        if entry is None or entry[2] != tuple(names):
+        if entry is None or entry[2] != tuple(names) or entry[3] != self.backend_pipeline:
             roles = [FE.ARG] * n_args + [FE.PARAM] * len(names)
             stable = [None] * n_args + [int.from_bytes(param_id(self.namespace, n), "little") for n in names]
-            opt = FE.optimize(program, roles, stable, self.backend, self.backend.param_resolver())
-            entry = self._optimized[program.key] = (opt, {}, tuple(names))
-        opt, held, _ = entry
+            hooks = FE.hip_backend_pipeline() if self.backend_pipeline else {}
+            opt = FE.optimize(program, roles, stable, self.backend, self.backend.param_resolver(), **hooks)
+            entry = self._optimized[program.key] = (opt, {}, tuple(names), self.backend_pipeline)
+        opt, held = entry[0], entry[1]
         inputs, don = [], []
         resolver = self.backend.param_resolver()
         for pos, (p, src) in enumerate(zip(opt.inputs, opt.source_index)):

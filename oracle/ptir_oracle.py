@@ -435,7 +435,50 @@ def dequantize_int4_g128(packed: np.ndarray, s: np.ndarray, group: int = 128) ->
     return (q.astype(np.float32) * sk).astype(np.float32)
 
 
+def _norm_call(target: str, attrs, ins: List[OTensor], out_dtype: str) -> OTensor:
+    """gpt_rs.hip.layer_norm.v1 (x, gamma, beta) / gpt_rs.hip.rms_norm.v1 (x, gamma), attribute eps: what a front-end
+    pass puts in place of the functional's instruction sequence (crates/gpt-rs/src/ops/functional/normalization.rs:
+    123-217).  Defined as that sequence: the same operations in the same order through the same op_* functions, every
+    intermediate in the tensor's dtype, so a program with the call computes bit for bit what the program with the
+    sequence computes."""
+    eps_attr = (attrs or {}).get("eps")
+    if not isinstance(eps_attr, dict) or "value" not in eps_attr:
+        raise OracleError("spec", f"{target}: attribute `eps` (F64) is missing")
+    x = ins[0]
+    dt, dims = x.dtype, tuple(x.a.shape)
+    n = dims[-1]
+    red = dims[:-1] + (1,)
+    axis = len(dims) - 1
+
+    def lit(v):   # scalar(v) broadcast to the reduced shape: a literal of the tensor's dtype (ops/ptir/graph.rs:2278-2298)
+        a = np.full(red, np.float32(v), dtype=np.float32)
+        return _finish(dt, a)
+
+    inv_count = lit(np.float32(1.0) / np.float32(n))
+    eps = lit(float(eps_attr["value"]))
+    if target == "gpt_rs.hip.layer_norm.v1":
+        if len(ins) != 3:
+            raise OracleError("spec", f"{target}: expects (x, gamma, beta)")
+        mean = op_binary(op_reduce(x, "Sum", [axis], True), inv_count, "Mul")
+        centered = op_binary(x, op_broadcast_to(mean, dims), "Sub")
+        var_mean = op_binary(op_reduce(op_binary(centered, centered, "Mul"), "Sum", [axis], True), inv_count, "Mul")
+        inv_std = op_unary(op_binary(var_mean, eps, "Add"), "Rsqrt")
+        normalized = op_binary(centered, op_broadcast_to(inv_std, dims), "Mul")
+        out = op_binary(op_binary(normalized, op_broadcast_to(ins[1], dims), "Mul"), op_broadcast_to(ins[2], dims), "Add")
+    else:
+        if len(ins) != 2:
+            raise OracleError("spec", f"{target}: expects (x, gamma)")
+        mean_square = op_binary(op_reduce(op_binary(x, x, "Mul"), "Sum", [axis], True), inv_count, "Mul")
+        inv_rms = op_unary(op_binary(mean_square, eps, "Add"), "Rsqrt")
+        out = op_binary(op_binary(x, op_broadcast_to(inv_rms, dims), "Mul"), op_broadcast_to(ins[1], dims), "Mul")
+    if out.dtype != out_dtype:
+        raise OracleError("spec", f"{target}: the output has x's type")
+    return out
+
+
 def _custom_call(target: str, attrs, ins: List[OTensor], out_dtype: str, out_dims) -> OTensor:
+    if target in ("gpt_rs.hip.layer_norm.v1", "gpt_rs.hip.rms_norm.v1"):
+        return _norm_call(target, attrs, ins, out_dtype)
     if target == "gpt_rs.hip.dot_w8.v1":
         x, q, s = ins
         w = dequantize_int8(q.a, s.a)

@@ -198,3 +198,56 @@ def test_backend_fusion_is_the_same_on_the_optimised_stream(kind, seq, decode, b
     assert not [line for line in emitted if line.split()[0] in ("ElementwiseBinary", "Reduce", "BroadcastTo", "Transpose", "Concat") and kind != "gpt"]
     if seq == 1 and batch == 1:
         assert B.fusion_report(opt.program, None) == emitted
+
+
+@pytest.mark.parametrize("kind", ["gpt", "ministral", "ministral-f32-stream"])
+@pytest.mark.parametrize("seq,decode,batch", [(1, True, 1), (64, False, 1), (1, True, 4)])
+def test_backend_pipeline_route(kind, seq, decode, batch):
+    """The second route through the optimizer: the hip backend's pre-pass turns every norm into a CustomCall ahead of the
+    parameter-only fold, so no gain or shift is folded into a derived parameter (only bias broadcasts are), and the
+    library's fusion of the result is what it makes of the emitted program -- without any provenance on the inputs but
+    for the biases."""
+    from gptrs_amd import backend as B
+    from gptrs_amd import models
+    m = _model(kind)
+    prog, layout = m._build(seq, 64, decode, batch, True)
+    n_args, be = layout["n_args"], m.backend
+    roles = [FE.ARG] * n_args + [FE.PARAM] * len(m.param_names)
+    stable = [None] * n_args + [int.from_bytes(models.param_id(m.namespace, n), "little") for n in m.param_names]
+    opt = FE.optimize(prog, roles, stable, be, be, **FE.hip_backend_pipeline())
+    body = opt.program.obj["functions"][0]["body"]
+    calls = [FE.op_attrs(i["op"])["target"] for i in body if FE.op_name(i["op"]) == "CustomCall"]
+    norms = 2 * 2 + 1
+    assert len([t for t in calls if t in FE.NORM_TARGETS.values()]) == norms
+    assert opt.folds_run == (0 if kind != "gpt" else 4 * 2)   # GPT-2: the four bias broadcasts of each block; Ministral has none
+    lens = [0 if src is not None else spec.dims[-1] for src, spec in zip(opt.source_index, opt.program.param_specs)]
+    assert B.fusion_report(opt.program, lens) == B.fusion_report(prog)
+    if kind != "gpt":
+        assert B.fusion_report(opt.program, None) == B.fusion_report(prog)
+
+
+def test_norm_calls_compute_what_the_sequences_compute():
+    """On the oracle the CustomCall is DEFINED as the functional's sequence: the program with the calls returns, bit for
+    bit, what the emitted program returns (f32 and bf16); a program that also returns the mean keeps the instructions
+    that produce it."""
+    from gptrs_amd import functional as F
+    from gptrs_amd.ptir import FunctionBuilder, Program
+    for dtype in ("F32", "Bf16"):
+        fb = FunctionBuilder("main", dtype)
+        x, g, b, g2 = fb.param(dtype, [5, 24]), fb.param(dtype, [24]), fb.param(dtype, [24]), fb.param(dtype, [24])
+        out, _, mean, _ = F.layer_norm(x, g, b, 1e-5)
+        out2, *_ = F.rms_norm(out, g2, 1e-6)
+        fb.set_results([out2, mean])
+        prog = Program(fb)
+        be = OracleBackend()
+        fn = __import__("copy").deepcopy(prog.obj["functions"][0])
+        cx = FE.OptimizeContext(be, be.param_resolver(), [FE.EntryParam(i, t, FE.ARG, None) for i, t in zip(fn["parameter_ids"], fn["parameters"])])
+        assert FE.HipNormFusionPass().run(fn, cx)
+        names = [FE.op_name(i["op"]) for i in fn["body"]]
+        assert names.count("CustomCall") == 2 and "Reduce" in names, "the mean is a result: its reduction stays"
+        opt = FE.program_from_function(fn, "main")
+        rng = np.random.default_rng(3)
+        arrays = [rng.standard_normal(s.dims).astype(np.float32) for s in prog.param_specs]
+        from parity import oracle_run
+        for got, want in zip(oracle_run(opt, arrays), oracle_run(prog, arrays)):
+            assert np.array_equal(got, want)

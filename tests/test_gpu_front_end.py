@@ -19,11 +19,12 @@ MID_MINISTRAL = models.MinistralConfig(vocab_size=512, context_length=128, embed
 PROMPT = [3, 17, 42, 5, 99, 311, 8, 250, 1]
 
 
-def _generate(be, make, front_end, n_new=8, counters=False):
+def _generate(be, make, front_end, n_new=8, counters=False, pipeline=False):
     """Tokens and per-step logits; with `counters` also (launches of the prefill, launches of a decode step, phases of
     the persistent launches of the decode steps, fused ops), with graph replay off so that every step counts."""
     m = make(be)
     m.front_end = front_end
+    m.backend_pipeline = pipeline
     if counters:
         be.set_option("graphs", 0)
     try:
@@ -61,6 +62,11 @@ def test_decode_through_the_optimizer_is_the_same_computation(hip, kind):
     assert t_opt == t_raw
     for a, b in zip(l_opt, l_raw):
         assert np.array_equal(a, b), "the optimised stream runs the same kernels on the same data"
+    # the second route: the backend's own pre-pass hands the norms over as CustomCalls
+    t_pipe, l_pipe, s_pipe = _generate(hip, make, True, counters=True, pipeline=True)
+    assert s_pipe[:3] == s_raw[:3] and t_pipe == t_raw, (s_raw, s_pipe)
+    for a, b in zip(l_pipe, l_raw):
+        assert np.array_equal(a, b)
     if kind.endswith("f32") and "stream" not in kind:
         t_ref, l_ref, _ = _generate(OracleBackend(), make, True)
         assert t_opt == t_ref
@@ -70,11 +76,37 @@ def test_decode_through_the_optimizer_is_the_same_computation(hip, kind):
 
 def test_oracle_runs_the_optimised_stream_to_the_same_values():
     """The optimizer must not change what a program computes: the oracle, which executes instruction by instruction,
-    returns the same logits for the emitted and for the optimised program (bit for bit: the same operations remain)."""
-    (t_a, l_a, _), (t_b, l_b, _) = (_generate(OracleBackend(), MAKERS["ministral-f32"], fe, n_new=3) for fe in (False, True))
-    assert t_a == t_b
-    for a, b in zip(l_a, l_b):
-        assert np.array_equal(a, b)
+    returns the same logits for the emitted program, for the optimised one and for the one whose norms the backend's
+    pre-pass made CustomCalls (bit for bit: the same operations remain)."""
+    runs = [_generate(OracleBackend(), MAKERS["ministral-f32"], fe, n_new=3, pipeline=pl) for fe, pl in ((False, False), (True, False), (True, True))]
+    for t_b, l_b, _ in runs[1:]:
+        assert runs[0][0] == t_b
+        for a, b in zip(runs[0][1], l_b):
+            assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", ["F32", "Bf16"])
+def test_norm_custom_calls_on_the_device(hip, dtype):
+    """gpt_rs.hip.layer_norm.v1 / rms_norm.v1 as instructions of a program: fusion on and off against the oracle, whose
+    definition of the calls is the functional's own sequence; a malformed call is a spec violation, not a crash."""
+    from gptrs_amd.backend import BackendError
+    from parity import check_program
+    fb = FunctionBuilder("main", dtype)
+    x, g, b, g2 = fb.param(dtype, [7, 96]), fb.param(dtype, [96]), fb.param(dtype, [96]), fb.param(dtype, [96])
+    attrs = {"eps": {"kind": "F64", "value": 1e-5}, "axis": {"kind": "I64", "value": 1}}
+    ln = fb.custom_call(FE.NORM_TARGETS["layer_norm"], [x, g, b], x.spec, attrs)
+    out = fb.custom_call(FE.NORM_TARGETS["rms_norm"], [ln, g2], x.spec, attrs)
+    fb.set_results([out, ln])
+    rng = np.random.default_rng(5)
+    arrays = [rng.standard_normal(s.dims).astype(np.float32) for s in Program(fb).param_specs]
+    tol = dict(atol=5e-4, rtol=1e-4) if dtype == "F32" else dict(atol=4e-2, rtol=2e-2)
+    check_program(hip, Program(fb), arrays, what="norm custom calls", **tol)
+    bad = FunctionBuilder("main", dtype)
+    x, g = bad.param(dtype, [7, 96]), bad.param(dtype, [95])
+    bad.set_results([bad.custom_call(FE.NORM_TARGETS["rms_norm"], [x, g], x.spec, attrs)])
+    with pytest.raises(BackendError) as err:
+        hip.run_program(Program(bad), [hip.materialize(TensorSpec(dtype, (7, 96)), None), hip.materialize(TensorSpec(dtype, (95,)), None)])
+    assert err.value.kind == "spec"
 
 
 @pytest.mark.parametrize("dtype", ["F32", "Bf16"])
