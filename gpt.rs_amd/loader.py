@@ -19,7 +19,6 @@ well: streaming trades time for memory, as in the reference.
 """
 from __future__ import annotations
 
-import hashlib
 from dataclasses import dataclass, field
 from typing import Callable, Dict, Iterable, List, Optional, Set
 
@@ -98,11 +97,12 @@ def block_layer_index(name: str) -> Optional[int]:
 
 
 def base_id_of(entry: Entry) -> int:
-    """The stored base id, or (stored 0 = "derive from the name", docs/formats.md) a 128-bit hash of the name.  The
-    reference hashes with blake3 (params.rs:29-48); blake2b-128 stands in for it here, as in models.param_id."""
+    """The stored base id, or (stored 0 = "derive from the name", docs/formats.md) the reference's `base_param_id` of the
+    name: the first 16 bytes of blake3(name), little endian (params.rs:29-37)."""
     if entry.base_id:
         return entry.base_id
-    return int.from_bytes(hashlib.blake2b(entry.name.encode(), digest_size=16).digest(), "little")
+    from .models import base_param_id
+    return base_param_id(entry.name)
 
 
 def prefetch_block_base_ids(entries: Iterable[Entry], prefetch_layers: Optional[int]) -> Set[int]:

@@ -13,7 +13,6 @@ materialize / to_literal / run_program / param_resolver / sample_decode_token.
 """
 from __future__ import annotations
 
-import hashlib
 import itertools
 import os
 from dataclasses import dataclass, field
@@ -22,6 +21,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import numpy as np
 
 from . import functional as F
+from .blake3 import blake3
 from .ptir import FunctionBuilder, Program, Tensor, TensorSpec, bf16_bits_to_f32, f32_to_bf16_bits
 
 
@@ -53,12 +53,26 @@ def _np_to_bytes(arr: np.ndarray, dtype: str) -> bytes:
     raise ValueError(dtype)
 
 
+def base_param_id(name: str) -> int:
+    """crates/gpt-rs/src/params.rs:29-37: the first 16 bytes of blake3(name) as a little-endian u128."""
+    if not name.isascii():
+        raise ValueError(f"param name must be ASCII, got '{name}'")
+    return int.from_bytes(blake3(name.encode("ascii"))[:16], "little")
+
+
+def namespace_id(namespace: str) -> int:
+    """The u128 a model instance is bound under.  The reference takes it from the model handle that `load_model` hands
+    out (runtime/loader.rs: a counter per loaded model); here it is derived from the instance's label the same way a
+    base id is derived from a name."""
+    return int.from_bytes(blake3(b"gpt-rs:model-namespace:" + namespace.encode())[:16], "little")
+
+
 def param_id(namespace: str, name: str) -> bytes:
-    """Stable 16-byte parameter key.  The reference derives it with blake3
-    (crates/gpt-rs/src/params.rs:29-48); only stability and uniqueness matter to a
-    backend's memo, so this build uses blake2b-128 over the same inputs."""
-    base = hashlib.blake2b(name.encode(), digest_size=16).digest()
-    return hashlib.blake2b(b"gpt-rs:param-key:v1" + namespace.encode() + base, digest_size=16).digest()
+    """Stable 16-byte parameter key, the reference's derivation (crates/gpt-rs/src/params.rs:39-48): the first 16 bytes of
+    blake3("gpt-rs:param-key:v1" || namespace u128 LE || base id u128 LE), which read as a little-endian u128 are
+    `ParamKey`; the memo of the C ABI is keyed by those 16 bytes."""
+    msg = b"gpt-rs:param-key:v1" + namespace_id(namespace).to_bytes(16, "little") + base_param_id(name).to_bytes(16, "little")
+    return blake3(msg)[:16]
 
 
 class _ModelBase:
