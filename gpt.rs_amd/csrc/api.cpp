@@ -166,15 +166,25 @@ BufferP Backend::derived_weights(const BufferP& src, int kind, DType dtype, int6
     auto it = tiled_cache_.find(ckey);
     if (it != tiled_cache_.end()) {
         if (it->second.src.lock() == src && it->second.src2.lock() == src2) return it->second.tiled;
+        forget_chain_copy(it->first, it->second);
         tiled_cache_.erase(it);
     }
     if (capturing) fail_exec("derived weight copy missing while recording a graph");
     // A weight that was freed (a streamed parameter between two forwards) takes its layouts with it, before the next one
     // is built: the memory a caller saves by streaming is not spent on copies of weights that are gone.
     if (dead_sources_.exchange(0, std::memory_order_relaxed) > 0) {
-        for (auto e = tiled_cache_.begin(); e != tiled_cache_.end();)
-            e = (e->second.src.expired() || (e->first[1] && e->second.src2.expired())) ? tiled_cache_.erase(e) : std::next(e);
+        for (auto e = tiled_cache_.begin(); e != tiled_cache_.end();) {
+            if (e->second.src.expired() || (e->first[1] && e->second.src2.expired())) {
+                forget_chain_copy(e->first, e->second);   // the surviving half of a pair gets its row-major form back first
+                e = tiled_cache_.erase(e);
+            } else {
+                ++e;
+            }
+        }
     }
+    // every layout is built from the row-major form
+    ensure_resident(src);
+    ensure_resident(src2);
     BufferP t;
     if (kind == 0) {
         t = new_buffer(k::tiled_weight_bytes((int)dtype, k, n));
@@ -204,9 +214,72 @@ BufferP Backend::derived_weights(const BufferP& src, int kind, DType dtype, int6
     src->has_derived = true;
     if (src2) { d.src2 = src2; src2->has_derived = true; }
     d.tiled = t;
+    d.k = k;
+    d.n = n;
+    if (kind == 2) {   // the bf16 chain copy is a permutation of the matrix: enough to rebuild it from
+        src->chain_key = ckey;
+        if (src2) src2->chain_key = ckey;
+    }
     tiled_cache_[ckey] = std::move(d);
     ++n_tiled_built;
     return t;
+}
+
+// Called before a chain copy leaves the cache: sources that were evicted in its favour are rebuilt from it first.
+void Backend::forget_chain_copy(const std::array<uint64_t, 3>& key, const Derived& d) {
+    if (key[2] != 2) return;
+    for (BufferP b : {d.src.lock(), d.src2.lock()}) {
+        if (!b || b->chain_key != key) continue;
+        ensure_resident(b);
+        b->chain_key = {{0, 0, 0}};
+    }
+}
+
+void Backend::ensure_resident(const BufferP& b) {
+    if (!b || !b->evicted) return;
+    if (capturing) fail_exec("a weight that was evicted in favour of its decode-chain copy is needed while recording a graph");
+    auto it = tiled_cache_.find(b->chain_key);
+    if (it == tiled_cache_.end() || it->first[2] != 2) fail_exec("an evicted weight has no packed copy left to rebuild it from");
+    const BufferP s1 = it->second.src.lock(), s2 = it->second.src2.lock();
+    const bool dual = it->first[1] != 0;
+    if (s1 != b && !(dual && s2 == b)) fail_exec("an evicted weight is not a source of the packed copy it names");
+    size_t cap = 0;
+    void* p = pool_.alloc(b->cap, &cap);
+    k::chain_unpack_weights(stream, it->second.tiled->ptr, s1 == b ? p : nullptr, dual && s2 == b ? p : nullptr, it->second.k, it->second.n, dual);
+    b->ptr = p;
+    b->cap = cap;
+    b->evicted = false;
+    ++n_weights_restored;
+}
+
+// After a program ran: inputs that this plan only ever uses through derived layouts, and whose values the bf16 chain
+// copy holds as well, give their row-major storage back.  The copy kernels that read them are queued on the one
+// stream, ahead of whatever is allocated from the freed blocks later.
+void Backend::evict_packed_sources(const Plan& plan, gptrs_hip_tensor* const* inputs, size_t n_in) {
+    if (!opt_evict_weights || capturing) return;
+    int n = 0;
+    for (size_t i = 0; i < n_in && i < plan.input_weight_only.size(); ++i) {
+        if (!plan.input_weight_only[i] || !inputs[i]) continue;
+        const BufferP& b = inputs[i]->buf;
+        if (!b || b->evicted || !b->ptr || b->chain_key[2] != 2) continue;
+        auto it = tiled_cache_.find(b->chain_key);
+        if (it == tiled_cache_.end()) { b->chain_key = {{0, 0, 0}}; continue; }
+        if (it->second.src.lock() != b && it->second.src2.lock() != b) continue;
+        if (it->first[0] != b->id && it->first[1] != b->id) { b->chain_key = {{0, 0, 0}}; continue; }   // updated in place since: the copy is stale
+        pool_.release(b->ptr, b->cap);
+        evicted_since_trim_ += b->cap;
+        b->ptr = nullptr;
+        b->evicted = true;
+        ++n;
+    }
+    n_weights_evicted += n;
+    // Back to the driver once it adds up (the point is the process's footprint, not the pool's free list); small
+    // amounts stay in the pool, where the next allocation of that size takes them.
+    if (n && evicted_since_trim_ >= (size_t)256 << 20) {
+        evicted_since_trim_ = 0;
+        GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
+        pool_.trim();
+    }
 }
 
 // Frees every derived weight layout (and with them the recorded graphs, which hold their addresses) and returns the
@@ -226,6 +299,8 @@ void Backend::drop_derived_weights() {
         p.seen_keys.clear();
         p.graph_builds = p.graph_hits = 0;
     }
+    for (auto& kv : tiled_cache_) forget_chain_copy(kv.first, kv.second);
+    GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
     tiled_cache_.clear();
     pool_.trim();
 }
@@ -326,6 +401,7 @@ void Backend::to_literal(const gptrs_hip_tensor* t, void* dst, size_t cap) {
     if (t->consumed) fail_exec("tensor handle was donated to run_program and can no longer be read");
     const size_t n = t->spec.bytes();
     if (cap < n) fail_exec("to_literal destination too small");
+    ensure_resident(t->buf);
     if (n) GPTRS_HIP_CHECK(hipMemcpyAsync(dst, t->data(), n, hipMemcpyDeviceToHost, stream));
     GPTRS_HIP_CHECK(hipStreamSynchronize(stream));
     check_device_errors();
@@ -546,6 +622,25 @@ std::shared_ptr<Plan> Backend::get_plan(const char* json, size_t len, uint64_t k
                 for (const Operand& o : in.operands)
                     if (o.value >= 0) mark(o.value);
         for (int r : f.result_ids) mark(r);
+        // inputs that only ever serve as the weight of an unquantised linear on a derived layout
+        std::vector<int> pos_of(plan->values.size(), -1);
+        for (size_t i = 0; i < f.param_ids.size(); ++i)
+            if (f.param_ids[i] >= 0 && f.param_ids[i] < (int)pos_of.size()) pos_of[f.param_ids[i]] = (int)i;
+        std::vector<int> good(f.param_ids.size(), 0), bad(f.param_ids.size(), 0);
+        for (const Instr& in : f.body) {
+            if (in.dead) continue;
+            const bool lin = in.op == OpKind::FLinear && (in.tiled || in.mfma) && !in.quant;
+            for (size_t o = 0; o < in.operands.size(); ++o) {
+                const int v = in.operands[o].value;
+                if (v < 0 || v >= (int)pos_of.size() || pos_of[v] < 0) continue;
+                const bool weight = lin && (o == 1 || (in.act == 2 && o == linear_w2_pos(in)));
+                ++(weight ? good : bad)[pos_of[v]];
+            }
+        }
+        for (int r : f.result_ids)
+            if (r >= 0 && r < (int)pos_of.size() && pos_of[r] >= 0) ++bad[pos_of[r]];
+        plan->input_weight_only.assign(f.param_ids.size(), false);
+        for (size_t i = 0; i < f.param_ids.size(); ++i) plan->input_weight_only[i] = good[i] > 0 && bad[i] == 0;
     }
     plan->cacheable = key != 0;
     if (plan->workspace_bytes) plan->workspace = new_buffer(plan->workspace_bytes);
@@ -746,6 +841,7 @@ void Backend::execute(Plan& plan, gptrs_hip_tensor* const* user_inputs, const ui
         if (inputs[i]->spec != fn.param_specs[i])
             fail_exec("entry input " + std::to_string(i) + " is " + inputs[i]->spec.str() + " but the program expects " + fn.param_specs[i].str());
         if (plan.input_read[i]) realize(inputs[i]);
+        if (!plan.input_weight_only[i]) ensure_resident(inputs[i]->buf);   // some kernel reads the row-major storage
     }
     // a buffer donated for in-place update must not be reachable through another input or handle
     std::vector<bool> inplace_ok(n_in, false);
@@ -824,6 +920,7 @@ void Backend::execute(Plan& plan, gptrs_hip_tensor* const* user_inputs, const ui
         outputs[i] = t;
     }
     consume_donated();
+    evict_packed_sources(plan, inputs, n_in);
 }
 
 // A result that is a pure broadcast of input p along leading axes remembers the vector it came from.
@@ -1199,6 +1296,7 @@ int gptrs_hip_set_option(gptrs_hip_backend* b, const char* name, int64_t value) 
         }
         else if (!strcmp(name, "profile")) { b->impl.profile_reset(); b->impl.opt_profile = value != 0; }
         else if (!strcmp(name, "drop_derived_weights")) { if (value) b->impl.drop_derived_weights(); }
+        else if (!strcmp(name, "evict_packed_weights")) b->impl.opt_evict_weights = value != 0;
         else gptrs::fail_spec(std::string("unknown option `") + name + "`");
     });
 }
@@ -1222,6 +1320,8 @@ int64_t gptrs_hip_counter(const gptrs_hip_backend* b, const char* name) {
     if (!strcmp(name, "bytes_allocated")) return i.bytes_allocated();
     if (!strcmp(name, "inplace_updates")) return i.n_inplace;
     if (!strcmp(name, "derived_weights_built")) return i.n_tiled_built;
+    if (!strcmp(name, "weights_evicted")) return i.n_weights_evicted;
+    if (!strcmp(name, "weights_restored")) return i.n_weights_restored;
     if (!strcmp(name, "last_program_launches")) return i.last_launches;
     if (!strcmp(name, "graph_launches")) return i.n_graph_launches;
     if (!strcmp(name, "graphs_built")) return i.n_graphs_built;

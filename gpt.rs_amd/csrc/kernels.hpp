@@ -220,6 +220,8 @@ size_t chain_weight_bytes(int64_t k, int64_t n, bool dual, int wfmt = kChainW16)
 // w2 != nullptr: SwiGLU pair, columns of w (gate) and w2 (up) interleaved.  wfmt 0: w is bf16 [k,n];
 // 1: si8 [k,n]; 2: packed int4, ui8 [k/2,n]; 3: f32 [k,n] (no pair)
 void chain_pack_weights(hipStream_t s, const void* w, const void* w2, void* out, int64_t k, int64_t n, int wfmt = kChainW16);
+// bf16 copies only: the row-major matrix (of a pair: whichever of w / w2 is non-null) back out of the packed copy, exactly
+void chain_unpack_weights(hipStream_t s, const void* packed, void* w, void* w2, int64_t k, int64_t n, bool dual);
 // int4 only: derived scale copy sc[tile][group][4] (bf16) from s [k/128, n] (and the partner's s2)
 size_t chain_scale_bytes(int64_t k, int64_t n, bool dual);
 void chain_pack_scales_w4(hipStream_t s, int dtype, const void* sc, const void* sc2, void* out, int64_t k, int64_t n);

@@ -297,5 +297,46 @@ void gemv_tiled(hipStream_t s, const TiledLinearArgs& a) {
     else gemv_tiled_t<bf16_t>(s, a);
 }
 
+// The inverse of the decode chain's bf16 weight copy (kernels_chain.hip: 4-column tiles, word j of a column holds rows
+// 2j and 2j + 1; a pair of matrices interleaves its columns gate, up, gate, up inside a tile): the row-major [K, N]
+// matrix back, exactly -- the copy is a permutation plus zero padding.  A matrix whose packed copy exists need not stay
+// resident in its row-major form; this brings it back when some other kernel family asks for it.
+__global__ void chain_unpack_kernel(const uint32_t* __restrict__ packed, bf16_t* __restrict__ w, bf16_t* __restrict__ w2,
+                                    int64_t K, int64_t N, int64_t Kw, int dual) {
+    const int64_t total = Kw * N;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t col = idx % N, j = idx / N;
+        if (2 * j >= K) continue;
+        const bool two = 2 * j + 1 < K;
+        if (!dual) {
+            const uint32_t v = packed[((col >> 2) * Kw + j) * 4 + (col & 3)];
+            w[(2 * j) * N + col] = (bf16_t)(v & 0xFFFFu);
+            if (two) w[(2 * j + 1) * N + col] = (bf16_t)(v >> 16);
+        } else {
+            const int64_t base = ((col >> 1) * Kw + j) * 4 + ((col & 1) << 1);
+            if (w) {
+                const uint32_t v = packed[base];
+                w[(2 * j) * N + col] = (bf16_t)(v & 0xFFFFu);
+                if (two) w[(2 * j + 1) * N + col] = (bf16_t)(v >> 16);
+            }
+            if (w2) {
+                const uint32_t v = packed[base + 1];
+                w2[(2 * j) * N + col] = (bf16_t)(v & 0xFFFFu);
+                if (two) w2[(2 * j + 1) * N + col] = (bf16_t)(v >> 16);
+            }
+        }
+    }
+}
+
+void chain_unpack_weights(hipStream_t s, const void* packed, void* w, void* w2, int64_t k, int64_t n, bool dual) {
+    const int64_t ntiles = ((dual ? 2 * n : n) + 3) / 4;
+    if (ntiles <= 0 || k <= 0 || (!w && !w2)) return;
+    const int64_t kw = (int64_t)(chain_weight_bytes(k, n, dual, kChainW16) / (size_t)(16 * ntiles));   // words per column
+    const int64_t total = kw * n;
+    const unsigned g = (unsigned)std::min<int64_t>((total + 255) / 256, 65536);
+    chain_unpack_kernel<<<g, 256, 0, s>>>((const uint32_t*)packed, (bf16_t*)w, (bf16_t*)w2, k, n, kw, dual ? 1 : 0);
+}
+
+
 }  // namespace k
 }  // namespace gptrs

@@ -50,6 +50,11 @@ struct Buffer {
     Backend* owner = nullptr;
     uint64_t id = 0;  // identity of the CONTENTS: fresh per allocation, bumped when updated in place
     bool has_derived = false;  // some derived weight layout was built from this buffer
+    // A bf16 weight whose decode-chain copy exists holds the same values twice.  Once no kernel of the programs that
+    // use it reads the row-major form, that form is given back (`evicted`: ptr is null, `cap` still says how much to
+    // allocate) and Backend::ensure_resident rebuilds it from the copy named by `chain_key` when something asks.
+    bool evicted = false;
+    std::array<uint64_t, 3> chain_key{{0, 0, 0}};   // key of the chain copy built from this buffer ({0,0,0}: none)
     ~Buffer();
 };
 using BufferP = std::shared_ptr<Buffer>;
@@ -150,6 +155,9 @@ struct Plan {
     size_t n_user_inputs = 0;
     std::vector<int> ext_inputs;
     std::vector<bool> input_read;           // per (extended) input: some step or result reads its storage
+    // per (extended) input: every use is the weight of an unquantised linear that runs on a derived layout, so no
+    // kernel of this plan reads the input's own storage
+    std::vector<bool> input_weight_only;
     // result position -> the caller's input it is a pure broadcast of along leading axes (or -1)
     std::vector<int> result_bcast_input;
     size_t workspace_bytes = 0;
@@ -210,6 +218,12 @@ class Backend {
     // (kernels_skinny.hip); kind 9 / 10: int8 / int4 codes in that tile order; kind 11: chain copy of f32 weights.
     BufferP derived_weights(const BufferP& src, int kind, DType dtype, int64_t k, int64_t n, const BufferP& src2 = nullptr);
     void drop_derived_weights();
+    // Row-major weights that a chain copy duplicates: evict_packed_sources frees those among `inputs` that `plan`
+    // never reads directly (option "evict_packed_weights", on by default); ensure_resident brings one back, exactly.
+    void ensure_resident(const BufferP& b);
+    void evict_packed_sources(const Plan& plan, gptrs_hip_tensor* const* inputs, size_t n_in);
+    bool opt_evict_weights = true;
+    int64_t n_weights_evicted = 0, n_weights_restored = 0;
     // Device copy of a chain's phase table, cached by content (steady-state decode repeats a few tables).
     const k::ChainPhase* chain_table(const std::vector<k::ChainPhase>& phases);
     unsigned* chain_barrier() const { return d_chain_bar_; }
@@ -277,8 +291,10 @@ class Backend {
     int64_t next_ticket_ = 0;
     bool queue_sampling(const gptrs_hip_tensor* logits, float temperature, bool has_top_k, bool has_u, float u);
     void* h_pinned_ = nullptr;  // 64 bytes of pinned host memory for readbacks
-    struct Derived { std::weak_ptr<Buffer> src, src2; BufferP tiled; };
+    struct Derived { std::weak_ptr<Buffer> src, src2; BufferP tiled; int64_t k = 0, n = 0; };
     std::map<std::array<uint64_t, 3>, Derived> tiled_cache_;
+    void forget_chain_copy(const std::array<uint64_t, 3>& key, const Derived& d);
+    size_t evicted_since_trim_ = 0;
     std::atomic<int> dead_sources_{0};  // weights with derived layouts that were freed since the last sweep
     unsigned* d_chain_bar_ = nullptr;
     struct ChainTable { std::vector<k::ChainPhase> host; BufferP dev; uint64_t last_use = 0; int refs = 0; };   // refs: recorded graphs that hold its address

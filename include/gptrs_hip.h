@@ -179,7 +179,7 @@ const char* gptrs_hip_last_error(void);
 int gptrs_hip_synchronize(gptrs_hip_backend* b);
 
 /* Execution options: name in {"fusion", "profile", "graphs", "chain", "chain_f32_min_kb", "chain_stall_phase", "gemm_lds_direct",
- * "drop_derived_weights"};
+ * "drop_derived_weights", "evict_packed_weights"};
  * value 0/1 unless stated.
  * "fusion" = rewrite matched functional sequences to fused kernels (on by default; off = one generic kernel per
  * instruction, the reference harness's "optimizer off" leg,
@@ -202,7 +202,14 @@ int gptrs_hip_synchronize(gptrs_hip_backend* b);
  * "drop_derived_weights" = 1 (an action, not a state): frees the re-ordered weight copies that the kernels built at
  * first use (and the recorded graphs that point at them) and returns cached device blocks to the driver; copies still
  * needed are rebuilt by the next call that uses them.  For a caller that has finished with a kernel family, e.g. the
- * prefill copies of a server that only decodes from then on ("bytes_allocated" shows the effect). */
+ * prefill copies of a server that only decodes from then on ("bytes_allocated" shows the effect).
+ * "evict_packed_weights" (default 1; no counterpart in the reference, whose backends read a weight where it was
+ * materialised): an unquantised bf16 matrix that a program only ever uses as the weight of linear layers, and of which
+ * the persistent decode launch has built its copy, frees its row-major storage after that program ran (the copy is a
+ * permutation of the matrix).  It is rebuilt from the copy, bit for bit, whenever something reads the tensor itself:
+ * to_literal, a program that uses it in any other way, a kernel family that has no copy of it yet, or
+ * "drop_derived_weights".  With prefill and decode copies both built, a model then holds its linear weights twice instead
+ * of three times. */
 int gptrs_hip_set_option(gptrs_hip_backend* b, const char* name, int64_t value);
 
 /* Counters since creation (the reference's cache_event / WorkStats fields,
@@ -210,7 +217,8 @@ int gptrs_hip_set_option(gptrs_hip_backend* b, const char* name, int64_t value);
  * "programs_compiled", "program_cache_hits", "fused_ops", "bytes_allocated",
  * "inplace_updates", "last_program_launches", "derived_weights_built" (column-tiled weight copies
  * made for the decode GEMV), "graph_launches", "graphs_built", "graphs_refused" (recorded graphs with a node outside
- * what a queue accepts: such a step runs launch by launch), "chain_launches", "chain_phases", and with the "profile" option "linear_time_ns",
+ * what a queue accepts: such a step runs launch by launch), "chain_launches", "chain_phases", "weights_evicted" / "weights_restored"
+ * (row-major weight storage freed in favour of the decode copy / rebuilt from it), and with the "profile" option "linear_time_ns",
  * "linear_calls", "linear_bytes" (these three synchronise)}.  Unknown names return -1. */
 int64_t gptrs_hip_counter(const gptrs_hip_backend* b, const char* name);
 
