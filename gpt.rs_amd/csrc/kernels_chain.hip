@@ -65,6 +65,7 @@ constexpr int NC = kChainCounters;
 constexpr int EPI_MAX = 640;     // bias/residual values staged per workgroup and phase: N <= 160 * grid columns
 constexpr int MAXI = 8;          // 8-byte items per thread in the norm staging: K <= 4*MAXI*NT
 constexpr int SLOT_BYTES = TP * NS * 16;     // one j-step of a workgroup: a word per compute lane and tile
+constexpr int PARK = 3;             // j-steps a compute wave can hold in registers while it waits for a phase to open
 constexpr int RING_MIN = 4, RING_MAX = 5;    // j-steps a wave's ring holds (its requests run that far ahead of its reads): 5 where the staged activations leave room
 constexpr int LDS_BYTES = 160 * 1024;        // per workgroup on gfx950
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -183,6 +184,7 @@ __device__ __forceinline__ void regs_from_lanes(PhaseRegs& R, int pd) {   // pd:
 // ---------------------------------------------------------------------------- staging (all waves)
 // xs[j] = (x[2j], x[2j+1]) as a bf16 pair, zero beyond K; with norm: the value the stand-alone
 // RMSNorm kernels store, ((x * inv_rms) * gamma) -> bf16 (normalization.rs:183-217).
+template <int FMT>
 __device__ __forceinline__ void stage_block(const PhaseRegs& P, unsigned* xs, float* ssq) {
     const int t = local_tid(), lane = t & 63, wave = uni(t >> 6);
     const int K = P.K;
@@ -197,7 +199,7 @@ __device__ __forceinline__ void stage_block(const PhaseRegs& P, unsigned* xs, fl
     const uint2* sc_src = nullptr;
     uint2* sc_dst = reinterpret_cast<uint2*>(xs + 2 * npad);
     uint2 sv[SB];
-    if (P.wfmt == kChainW4) {
+    if (FMT == kChainW4) {   // (every linear phase of a launch has the kernel's weight format)
         const int G = P.Kw >> 4, upb = P.upb;
         const int t0 = (int)blockIdx.x * upb * TP, t1 = min(min(t0 + upb * TP, P.units * TP), P.ntiles);
         sc_n = max(t1 - t0, 0) * G;
@@ -307,7 +309,7 @@ __device__ __forceinline__ void stage_block(const PhaseRegs& P, unsigned* xs, fl
             }
         }
     }
-    if (sc_n > 0) {
+    if (FMT == kChainW4 && sc_n > 0) {
 #pragma unroll
         for (int u = 0; u < SB; ++u) {
             const int i = u * NT + t;
@@ -1167,7 +1169,7 @@ __device__ void control_wave(Shared& sh, unsigned* xs, const ChainPhase* phases,
             unsigned e_bw = 0u, e_rw = 0u, e_ga = 0u, e_gb = 0u;
             if (has_epi) epi_load(lane * 2, e_bw, e_rw, e_ga, e_gb);
             if (wfmt == kChainW32) stage_block_f32(P, xs, sh.ssq);
-            else stage_block(P, xs, sh.ssq);
+            else stage_block<FMT>(P, xs, sh.ssq);
             if (has_epi) {
                 epi_store(lane * 2, e_bw, e_rw, e_ga, e_gb);
                 for (int i = lane * 2 + 128; i < ncols; i += 128) {
@@ -1400,6 +1402,7 @@ __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, 
     int c_phase = -1, c_unit = 0, c_unit_end = 0, c_j = 0, c_wpt = 1, c_sidx = 0, c_G = 0, c_soff = 0, c_Kv = 0, ucount = 0;
     int c_consumed = 0;   // units the control wave has taken, as last read
     constexpr int c_fmt = FMT;
+    PhaseRegs R;
     // advance to this workgroup's next linear unit, taking part in attention phases on the way
     auto c_seek = [&]() -> bool {
         for (;;) {
@@ -1422,12 +1425,8 @@ __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, 
             c_Kv = (uni(D->K) + kpw - 1) / kpw;
             c_sidx = 0;   // int4: entry of the unit's first tile and group in the staged scales ...
             c_soff = uni(D->lds_bytes) >> 2;   // ... which sit behind the activations
-            PhaseRegs R;
             regs_from_table<FMT == kChainW32>(R, D);
-            if (!wait_go(&sh.go, &sh.abort, c_phase, budget)) return false;
-            if (FMT == kChainW32) stage_block_f32(R, const_cast<unsigned*>(xs), sh.ssq);
-            else stage_block(R, const_cast<unsigned*>(xs), sh.ssq);
-            return true;
+            return true;   // (the caller waits for the phase to open and stages its input)
         }
     };
 
@@ -1445,8 +1444,53 @@ __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, 
     // phases (rare code: seek, attention, staging) around units around j-steps (the loop that has to be tight)
     bool alive = true;
     while (alive && c_seek()) {
+      // Until the phase opens the wave has nothing to do, its ring is full, and whatever of it has landed cannot be used
+      // yet: the memory system would idle through the barrier.  So the oldest steps that have landed move from the ring
+      // into registers (`park`), and the slots they leave are asked to fetch further ahead: up to PARK more j-steps of
+      // weights are on their way while the grid synchronises.  Parked steps are the phase's first ones and are read
+      // back first; the registers are free again before the next phase is looked for.
+      u32x4 park[PARK][TP];
+      int n_parked = 0, park_rd = 0;
+      {
+        const int want = min(PARK, min(c_wpt * (c_unit_end - c_unit), inflight));
+#pragma unroll
+        for (int i = 0; i < PARK; ++i) {
+            if (i < want && uni(lds_ld(&sh.go)) < c_phase) {
+                const GPTRS_LDS u32x4* wp = mine + slot * (SLOT_BYTES / 16);
+                const int oldest = (int)(pend & 3u), younger = loads - oldest;
+                if (oldest) wait_vm_count(younger);
+                pend >>= 2;
+                loads = younger;
+                asm volatile("" ::: "memory");
+#pragma unroll
+                for (int p = 0; p < TP; ++p) park[i][p] = wp[p * NS];
+                --inflight;
+                if (++slot == RING_D) slot = 0;
+                __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): the words are in registers before their slot is asked to take new ones
+                asm volatile("" ::: "memory");
+                if (r_more) request();
+                n_parked = i + 1;
+            }
+        }
+      }
+      if (!wait_go(&sh.go, &sh.abort, c_phase, budget)) break;
+      if (FMT == kChainW32) stage_block_f32(R, const_cast<unsigned*>(xs), sh.ssq);
+      else stage_block<FMT>(R, const_cast<unsigned*>(xs), sh.ssq);
+      bool from_park = false;
       for (; c_unit < c_unit_end; ++c_unit) {
         for (c_j = 0; c_j < c_wpt; ++c_j) {
+        u32x4 cur[TP];
+        from_park = park_rd < n_parked;
+        if (from_park) {
+            switch (park_rd) {
+#define GPTRS_PARK(k) case k: _Pragma("unroll") for (int p = 0; p < TP; ++p) cur[p] = park[k][p]; break;
+                GPTRS_PARK(0) GPTRS_PARK(1)
+                default: _Pragma("unroll") for (int p = 0; p < TP; ++p) cur[p] = park[PARK - 1][p]; break;
+#undef GPTRS_PARK
+            }
+            static_assert(PARK == 3, "cases above");
+            ++park_rd;
+        } else {
         const GPTRS_LDS u32x4* wp = mine + slot * (SLOT_BYTES / 16);
         // the loads of this j-step are the oldest in flight: they have landed once no more than the younger ones remain
         {
@@ -1459,17 +1503,17 @@ __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, 
             loads = younger;
         }
         asm volatile("" ::: "memory");
-        u32x4 cur[TP];
 #pragma unroll
         for (int p = 0; p < TP; ++p) cur[p] = wp[p * NS];
+        --inflight;
+        if (++slot == RING_D) slot = 0;
+        }
         if ((c_j + 1) * NS > c_Kv) {   // the stream's last step: lanes whose words are padding count as zeros
             if (c_j * NS + t >= c_Kv) {
 #pragma unroll
                 for (int p = 0; p < TP; ++p) { cur[p].x = 0u; cur[p].y = 0u; cur[p].z = 0u; cur[p].w = 0u; }
             }
         }
-        --inflight;
-        if (++slot == RING_D) slot = 0;
         // element reads go through scalars: __builtin_bit_cast applied directly to `vec.y` of an
         // ext-vector reads element 0 with this compiler
         if (c_fmt == kChainW16) {
@@ -1539,7 +1583,7 @@ __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, 
                 }
             }
         }
-        if (c_j + 1 < c_wpt && r_more) request();   // (the unit's last step: after the hand-over below)
+        if (!from_park && c_j + 1 < c_wpt && r_more) request();   // (the unit's last step: after the hand-over below; a parked step's slot was refilled when it was parked)
         }   // j-steps
         {
             const int hslot = ucount % NSLOT;
@@ -1558,12 +1602,17 @@ __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, 
                 }
                 if (!alive) break;
             }
-            if ((lane & 15) < 3) sh.red[hslot][wave][3 * (lane >> 4) + (lane & 15)] = v;
+            {
+                // (index recomputed here: as a loop invariant it was kept in a register that the allocator spilled, and its
+                // reload waits for every load in flight)
+                const int t2 = local_tid(), l2 = t2 & 63;
+                if ((l2 & 15) < 3) sh.red[hslot][t2 >> 6][3 * (l2 >> 4) + (l2 & 15)] = v;
+            }
             GPTRS_LDS_RELEASE();
             if (lane == 0) __hip_atomic_fetch_add(&sh.red_cnt[hslot], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             ++ucount;
             c_sidx += TP * c_G;
-            if (r_more) request();
+            if (!from_park && r_more) request();
         }
       }   // units
     }
