@@ -511,7 +511,7 @@ __device__ __forceinline__ void lane_pair(float v, int off, float& a, float& b) 
 // previous phase); only the query row and this step's K/V row are read after it.
 __device__ bool attn_partial(GPTRS_LDS int* go, GPTRS_LDS int* abort, const ChainPhase& P, GPTRS_LDS float* lds, int unit, int phase,
                              unsigned long long budget) {
-    constexpr int PP = 4;   // positions per lane group requested ahead of the barrier
+    constexpr int PP = 5;   // positions per lane group requested ahead of the barrier (32 chunks x 8 lane groups x 5 = 1280 positions)
     const int t = local_tid(), lane = t & 63, wave = uni(t >> 6);
     const bool control = wave == NWS;
     const int dh = P.head_dim, n_q = P.n_q, n_kv = P.n_kv, nch = P.nch, half = P.rot_half;
