@@ -1457,10 +1457,12 @@ __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, 
         for (int i = 0; i < PARK; ++i) {
             if (i < want && uni(lds_ld(&sh.go)) < c_phase) {
                 const GPTRS_LDS u32x4* wp = mine + slot * (SLOT_BYTES / 16);
-                const int oldest = (int)(pend & 3u), younger = loads - oldest;
-                if (oldest) wait_vm_count(younger);
-                pend >>= 2;
-                loads = younger;
+                // The wave has time, so it waits for everything it has in flight rather than for this step alone: the request
+                // it makes below then meets an empty queue and returns at once, and the wave is back at the test of `go`
+                // instead of held in the memory pipeline behind its own older requests when the phase opens.
+                if (loads) wait_vm_imm<0>();
+                pend = 0u;
+                loads = 0;
                 asm volatile("" ::: "memory");
 #pragma unroll
                 for (int p = 0; p < TP; ++p) park[i][p] = wp[p * NS];
