@@ -41,14 +41,15 @@ MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 # rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a copy kernel of known size (commands and raw figures: `profile`).  The
 # figure belongs to ONE version of the kernel: `source_sha256` is the hash of gpt.rs_amd/csrc/kernels_chain.hip it was
 # measured on, and `roofline.traffic` is null whenever the file in the tree hashes differently.
-CHAIN_TRAFFIC = {"bytes": 7.0184e9 + 0.0279e9, "source_sha256": "253fbf93e863204bcf87bf713c9dbdc4213318f03409c700052e1ba5df94fbc0",
+CHAIN_TRAFFIC = {"bytes": 7.0148e9 + 0.0273e9, "w8_bytes": 3.5934e9 + 0.0274e9,
+                 "source_sha256": "ead994fd89037efc14656300c0cddec3b3acd277d523820eebc53d44415b3e0b",
                  "profile": "profiles/chain_kernel_ministral3b_bf16_b1_decode.md"}
 
 
-def chain_traffic_bytes():
+def chain_traffic_bytes(key: str = "bytes"):
     try:
         with open(os.path.join(ROOT, "gpt.rs_amd", "csrc", "kernels_chain.hip"), "rb") as f:
-            return CHAIN_TRAFFIC["bytes"] if hashlib.sha256(f.read()).hexdigest() == CHAIN_TRAFFIC["source_sha256"] else None
+            return CHAIN_TRAFFIC[key] if hashlib.sha256(f.read()).hexdigest() == CHAIN_TRAFFIC["source_sha256"] else None
     except OSError:
         return None
 
@@ -435,7 +436,8 @@ def quant_record(be, cfg, quant: str, prompt, capacity: int, steps: int = 64, wa
         nbytes = sum(algorithmic_bytes_per_step(cfg, 2, prof_start + i, quant, True) for i in range(prof_steps))
         achieved = nbytes / (t_ns * 1e-9) / 1e9
         roof = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                "traffic": None, "kernel": "chain_kernel over %s code words, %d phases per launch" % (quant, phases // max(chains, 1)),
+                "traffic": chain_traffic_bytes("w8_bytes") if quant == "w8" and cfg.num_layers == 26 and len(prompt) == 1024 else None,
+                "kernel": "chain_kernel over %s code words, %d phases per launch" % (quant, phases // max(chains, 1)),
                 "launches": calls, "avg_launch_us": round(t_ns / calls / 1e3, 2), "bytes_per_launch": round(nbytes / calls)}
     return {"metric": "decode tokens/s, Ministral-3B-shape %s weight-only linears (lm_head included), batch 1" % quant,
             "value": round(1.0 / t_step, 2), "unit": "tokens/s", "steps": steps, "warmup": warmup, "ms_per_step": round(t_step * 1e3, 4),
