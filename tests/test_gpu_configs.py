@@ -334,3 +334,44 @@ def test_config4_quantised_layer_full_width(hip, scheme):
     # and the codes are the oracle's: spot check one matrix against the closed form from the dequantised values
     q = np.frombuffer(hip.to_literal(mh.param_handle("blocks.0.attention.w_out.q")), np.int8 if scheme == "w8" else np.uint8)
     assert q.size == (4096 * 3072 if scheme == "w8" else 2048 * 3072)
+
+
+@pytest.mark.parametrize("scheme", ["w8", "w4g128"])
+def test_config4_quantised_batch_of_8_full_width(hip, scheme):
+    """configs[4] at batch 8 through the model: one full-width layer with int8 / int4-g128 linears, 8 sequences of 64
+    tokens through `forward_batch` (prefill: 512 stacked rows on the matrix-core GEMM over the codes; decode: 8 rows on
+    the batched-decode kernel over the codes, one attention launch for the 8 caches).  Every row against the same
+    sequence run alone (64-row prefill, decode through the persistent launch), and rows 0 and 7 against the oracle
+    running the same quantised program op by op with the device's codes."""
+    cfg = models.MinistralConfig(num_layers=1, **FULL)
+    B, T = 8, 64
+    prompts = np.random.default_rng(16).integers(0, cfg.vocab_size, (B, T)).tolist()
+    mh = models.Ministral.random(cfg, hip, seed=5, dtype="Bf16", residual_dtype="F32", quant=scheme)
+    caches = [[None] for _ in range(B)]
+    pre = hip.to_numpy(mh.forward_batch(prompts, 0, caches, 128, last_logits_only=True)).astype(np.float32)
+    toks = [int(np.argmax(pre[b])) for b in range(B)]
+    before = hip.counter("chain_launches")
+    dec = hip.to_numpy(mh.forward_batch([[t] for t in toks], T, caches, 128)).astype(np.float32)
+    assert hip.counter("chain_launches") == before, "a batch decodes on the batched kernels"
+    for b in range(B):
+        c1 = [None]
+        p1 = hip.to_numpy(mh.forward_with_decode_cache(prompts[b], 0, c1, 128, last_logits_only=True))[-1].astype(np.float32)
+        d1 = hip.to_numpy(mh.forward_with_decode_cache([toks[b]], T, c1, 128))[-1].astype(np.float32)
+        ep, ed = np.abs(pre[b] - p1), np.abs(dec[b] - d1)
+        print(f"{scheme} row {b}: batch vs alone, prefill max {ep.max():.4f} mean {ep.mean():.5f}; decode max {ed.max():.4f} mean {ed.mean():.5f}")
+        # the same codes and the same rounding points, other kernels (summation order, a stray rounding tie)
+        assert ep.max() < 0.06 and ep.mean() < 5e-3 and ed.max() < 0.06 and ed.mean() < 5e-3
+    ob = OracleBackend()
+    mo = models.Ministral(cfg, ob, "Bf16", "F32")
+    from parity import TensorSpec
+    for name in mh.param_names:
+        spec = mh.param_specs[name]
+        mo.set_param_bytes(name, TensorSpec(spec.dtype, spec.dims), hip.to_literal(mh.param_handle(name)))
+    with blas_dots():
+        for b in (0, B - 1):
+            co = [None]
+            ref = ob.to_numpy(mo.forward_with_decode_cache(prompts[b], 0, co, 128, last_logits_only=True))[-1]
+            dref = ob.to_numpy(mo.forward_with_decode_cache([toks[b]], T, co, 128))[-1]
+            ep, ed = _report(f"{scheme} row {b} prefill vs oracle", pre[b], ref), _report(f"{scheme} row {b} decode vs oracle", dec[b], dref)
+            # the oracle rounds every op output to bf16, the fused kernels fewer (the bound of the batch-1 test above)
+            assert ep.max() < 0.12 and ep.mean() < 2e-2 and ed.max() < 0.12 and ed.mean() < 2e-2
