@@ -262,6 +262,11 @@ void Backend::evict_packed_sources(const Plan& plan, gptrs_hip_tensor* const* in
         if (!plan.input_weight_only[i] || !inputs[i]) continue;
         const BufferP& b = inputs[i]->buf;
         if (!b || b->evicted || !b->ptr || b->chain_key[2] != 2) continue;
+        // the same tensor passed a second time in a position that reads it: it would be rebuilt on every call
+        bool read_elsewhere = false;
+        for (size_t j = 0; j < n_in && !read_elsewhere; ++j)
+            read_elsewhere = j != i && inputs[j] && inputs[j]->buf == b && !(j < plan.input_weight_only.size() && plan.input_weight_only[j]);
+        if (read_elsewhere) continue;
         auto it = tiled_cache_.find(b->chain_key);
         if (it == tiled_cache_.end()) { b->chain_key = {{0, 0, 0}}; continue; }
         if (it->second.src.lock() != b && it->second.src2.lock() != b) continue;

@@ -99,3 +99,37 @@ def test_a_replaced_weight_is_read_from_its_own_copies(hip):
         hip.set_option("evict_packed_weights", 1)
     assert toks_a == toks_b and all(np.array_equal(a, b) for a, b in zip(logits_a, logits_b))
     assert back_a == back_b
+
+
+def test_a_weight_that_the_same_program_also_reads_stays(hip):
+    """One tensor passed twice, once as the weight of a decode-shaped linear and once in a position that reads its
+    storage (an elementwise add): it is not evicted (it would be rebuilt on every call), and both uses see its values."""
+    from parity import FunctionBuilder, Program, to_bytes
+    k, n = 1024, 1024
+    rng = np.random.default_rng(3)
+    w = (rng.standard_normal((k, n)) * 0.05).astype(np.float32)
+    x = rng.standard_normal((1, k)).astype(np.float32)
+    fb = FunctionBuilder("main")
+    a, b, c = fb.param("Bf16", [1, k]), fb.param("Bf16", [k, n]), fb.param("Bf16", [k, n])
+    fb.set_results([a.matmul(b), c + c])
+    prog = Program(fb)
+    hw = hip.materialize(prog.param_specs[1], to_bytes(w, "Bf16"))
+    hx = hip.materialize(prog.param_specs[0], to_bytes(x, "Bf16"))
+    e0, r0 = hip.counter("weights_evicted"), hip.counter("weights_restored")
+    for _ in range(3):
+        y, d = hip.run_program(prog, [hx, hw, hw])
+    assert hip.counter("weights_evicted") == e0 and hip.counter("weights_restored") == r0
+    wb = hip.to_numpy(hw).astype(np.float32)
+    assert np.array_equal(hip.to_numpy(d).astype(np.float32), 2.0 * wb), "doubling a bf16 value is exact"
+    ref = hip.to_numpy(hx).astype(np.float32) @ wb
+    assert np.allclose(hip.to_numpy(y).astype(np.float32), ref, rtol=2 ** -6, atol=2 ** -6 * float(np.abs(ref).max()))
+    # alone, the same weight does leave once the decode copy exists
+    fb2 = FunctionBuilder("main")
+    a2, b2 = fb2.param("Bf16", [1, k]), fb2.param("Bf16", [k, n])
+    fb2.set_results([a2.matmul(b2)])
+    p2 = Program(fb2)
+    y2 = hip.run_program(p2, [hx, hw])[0]
+    assert hip.counter("weights_evicted") == e0 + 1, "the lone linear runs on the persistent launch, whose copy stands in for the matrix"
+    assert np.array_equal(hip.to_numpy(y2), hip.to_numpy(y))
+    assert bytes(hip.to_literal(hw)) == to_bytes(w, "Bf16"), "read back from the packed copy"
+    assert hip.counter("weights_restored") == r0 + 1
