@@ -65,6 +65,7 @@ constexpr int NC = kChainCounters;
 constexpr int EPI_MAX = 640;     // bias/residual values staged per workgroup and phase: N <= 160 * grid columns
 constexpr int MAXI = 8;          // 8-byte items per thread in the norm staging: K <= 4*MAXI*NT
 constexpr int SLOT_BYTES = TP * NS * 16;     // one j-step of a workgroup: a word per compute lane and tile
+constexpr int PARK_W4 = 1, PARK_W8 = 2;   // ... in the int4 and int8 kernels, whose step arithmetic and staging hold more registers (measured: one step more spills)
 constexpr int PARK = 3;             // j-steps a compute wave can hold in registers while it waits for a phase to open
 constexpr int RING_MIN = 4, RING_MAX = 5;    // j-steps a wave's ring holds (its requests run that far ahead of its reads): 5 where the staged activations leave room
 constexpr int LDS_BYTES = 160 * 1024;        // per workgroup on gfx950
@@ -1449,12 +1450,13 @@ __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, 
       // into registers (`park`), and the slots they leave are asked to fetch further ahead: up to PARK more j-steps of
       // weights are on their way while the grid synchronises.  Parked steps are the phase's first ones and are read
       // back first; the registers are free again before the next phase is looked for.
-      u32x4 park[PARK][TP];
+      constexpr int PARKN = FMT == kChainW4 ? PARK_W4 : (FMT == kChainW8 ? PARK_W8 : PARK);   // (the int4 kernel stages its group scales through registers as well)
+      u32x4 park[PARKN][TP];
       int n_parked = 0, park_rd = 0;
       {
-        const int want = min(PARK, min(c_wpt * (c_unit_end - c_unit), inflight));
+        const int want = min(PARKN, min(c_wpt * (c_unit_end - c_unit), inflight));
 #pragma unroll
-        for (int i = 0; i < PARK; ++i) {
+        for (int i = 0; i < PARKN; ++i) {
             if (i < want && uni(lds_ld(&sh.go)) < c_phase) {
                 const GPTRS_LDS u32x4* wp = mine + slot * (SLOT_BYTES / 16);
                 // The wave has time, so it waits for everything it has in flight rather than for this step alone: the request
@@ -1485,12 +1487,12 @@ __device__ void compute_waves(Shared& sh, const unsigned* xs, PhaseTable table, 
         from_park = park_rd < n_parked;
         if (from_park) {
             switch (park_rd) {
-#define GPTRS_PARK(k) case k: _Pragma("unroll") for (int p = 0; p < TP; ++p) cur[p] = park[k][p]; break;
+#define GPTRS_PARK(k) case k: _Pragma("unroll") for (int p = 0; p < TP; ++p) cur[p] = park[k < PARKN ? k : 0][p]; break;
                 GPTRS_PARK(0) GPTRS_PARK(1)
-                default: _Pragma("unroll") for (int p = 0; p < TP; ++p) cur[p] = park[PARK - 1][p]; break;
+                default: _Pragma("unroll") for (int p = 0; p < TP; ++p) cur[p] = park[PARKN - 1][p]; break;
 #undef GPTRS_PARK
             }
-            static_assert(PARK == 3, "cases above");
+            static_assert(PARK >= 1 && PARK <= 3 && PARK_W4 >= 1 && PARK_W4 <= 3 && PARK_W8 >= 1 && PARK_W8 <= 3, "cases above");
             ++park_rd;
         } else {
         const GPTRS_LDS u32x4* wp = mine + slot * (SLOT_BYTES / 16);
