@@ -236,7 +236,7 @@ class Backend {
     bool opt_gemm_lds_direct = true;
     // f32 chains run only when a linear phase streams at least this much on average (option "chain_f32_min_kb",
     // GPTRS_HIP_CHAIN_F32_MIN_KB): below it a phase's fixed cost is what a stand-alone kernel costs
-    int64_t chain_f32_min_bytes = 8ll << 20;
+    int64_t chain_f32_min_bytes = 4ll << 20;
     int chain_stall_phase = -1;   // tests of the give-up path: the next chain launch expects an arrival too many at this phase
     bool chain_stall_fired = false;   // such a launch has been queued and its time-out not yet reported
     int64_t n_chain_launches = 0, n_chain_phases = 0;

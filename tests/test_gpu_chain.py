@@ -254,7 +254,7 @@ def run_both_f32(hip, build, specs, arrays, atol=5e-4, rtol=1e-4, phases=1):
         assert hip.counter("chain_launches") > before, "the program did not take the chain path"
         assert hip.counter("chain_phases") - ph0 >= phases
     finally:
-        hip.set_option("chain_f32_min_kb", 8192)
+        hip.set_option("chain_f32_min_kb", 4096)
     want = oracle_run(p, arrays)
     hip.set_option("chain", 0)
     try:
@@ -311,7 +311,7 @@ def test_f32_block_tail_chain(hip, d):
 
 
 def test_f32_phases_that_stream_little_keep_their_kernels(hip):
-    """The default policy: f32 linears join a persistent launch from 8 MiB of weights each on average."""
+    """The default policy: f32 linears join a persistent launch from 4 MiB of weights each on average."""
     x = rnd(80, (1, 768))
     small, big = rnd(81, (768, 768), 0.05), rnd(82, (768, 4096), 0.05)
     p_small = prog(lambda fb, a, b: a.matmul(b), [("F32", [1, 768]), ("F32", [768, 768])])
@@ -350,7 +350,7 @@ def test_f32_decode_attention_in_chain(hip, hq, hkv, dh, cap):
             before = hip.counter("chain_phases")
             got = hip_run(hip, p, arrays)
         finally:
-            hip.set_option("chain_f32_min_kb", 8192)
+            hip.set_option("chain_f32_min_kb", 4096)
         # a cache of at most 128 positions is one chunk per kv head: the attention is one phase
         assert hip.counter("chain_phases") - before == (3 if cap <= 128 else 4), "projection, attention and out-projection must share one launch"
         want = oracle_run(p, arrays)

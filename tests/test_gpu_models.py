@@ -239,7 +239,7 @@ def test_gpt_f32_decode_on_the_chain(hip, prompt_len):
         t_chain, l_chain = run_generate(hip, models.Gpt, MID_GPT, 9, 10, "F32", std=0.08, prompt=prompt)
         phases, last = hip.counter("chain_phases") - ph0, hip.counter("last_program_launches")
     finally:
-        hip.set_option("chain_f32_min_kb", 8192)
+        hip.set_option("chain_f32_min_kb", 4096)
         hip.set_option("graphs", 1)
     # per layer qkv, attention (1 phase, or 2 beyond 128 positions), out-projection, fc, projection; then the lm_head
     per_step = 2 * (5 if prompt_len + 10 <= 128 else 6) + 1
