@@ -41,8 +41,8 @@ MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 # rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a copy kernel of known size (commands and raw figures: `profile`).  The
 # figure belongs to ONE version of the kernel: `source_sha256` is the hash of gpt.rs_amd/csrc/kernels_chain.hip it was
 # measured on, and `roofline.traffic` is null whenever the file in the tree hashes differently.
-CHAIN_TRAFFIC = {"bytes": 7.0147e9 + 0.0273e9, "w8_bytes": 3.5951e9 + 0.0274e9,
-                 "source_sha256": "93e5b2b854c49e2a2e64dd0ef986ae99f011c36847b9d1ecd28ed616bdd8e034",
+CHAIN_TRAFFIC = {"bytes": 7.0149e9 + 0.0273e9, "w8_bytes": 3.5937e9 + 0.0274e9,
+                 "source_sha256": "ed3ebc9b622d507ae693373ec872176c091fc4e53d7ff9f3f93152d1901b2a42",
                  "profile": "profiles/chain_kernel_ministral3b_bf16_b1_decode.md"}
 
 

@@ -215,7 +215,7 @@ struct ChainPhase {
     const void* beta;                          // LayerNorm offsets (kChainLayerNorm)
 };
 int chain_grid();  // workgroups per launch (one per CU), 0 when no device is current
-bool chain_supported(int dtype, int64_t m, int64_t k, int64_t n, bool dual, bool norm, int wfmt = kChainW16, bool x_f32 = false);
+bool chain_supported(int dtype, int64_t m, int64_t k, int64_t n, bool dual, bool norm, int wfmt = kChainW16, bool x_f32 = false, bool plain = false);
 size_t chain_weight_bytes(int64_t k, int64_t n, bool dual, int wfmt = kChainW16);
 // w2 != nullptr: SwiGLU pair, columns of w (gate) and w2 (up) interleaved.  wfmt 0: w is bf16 [k,n];
 // 1: si8 [k,n]; 2: packed int4, ui8 [k/2,n]; 3: f32 [k,n] (no pair)

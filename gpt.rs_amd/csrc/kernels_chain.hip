@@ -1237,7 +1237,14 @@ __device__ void control_wave(Shared& sh, unsigned* xs, const ChainPhase* phases,
                         float o[4];
 #pragma unroll
                         for (int c = 0; c < 4; ++c) o[c] = finish(s[c], flags, bi[c], re[c]);
-                        if (out_f32) {
+                        if (tile * 4 + 4 > N) {   // the last tile of a width that is not a multiple of 4: its real columns one by one
+#pragma unroll
+                            for (int c = 0; c < 4; ++c) {
+                                if (tile * 4 + c >= N) continue;
+                                if (out_f32) cstore4(out + 4 * (size_t)(tile * 4 + c), __float_as_uint(o[c]));
+                                else __hip_atomic_store(as_global((unsigned short*)out + (size_t)(tile * 4 + c)), (unsigned short)pack_hw(o[c], 0.f), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            }
+                        } else if (out_f32) {
                             cstore8(out + 4 * (size_t)(tile * 4), (unsigned long long)__float_as_uint(o[0]) | ((unsigned long long)__float_as_uint(o[1]) << 32));
                             cstore8(out + 4 * (size_t)(tile * 4) + 8, (unsigned long long)__float_as_uint(o[2]) | ((unsigned long long)__float_as_uint(o[3]) << 32));
                         } else {
@@ -1738,16 +1745,19 @@ static inline int chain_kpw(int wfmt) { return wfmt == kChainW32 ? 1 : (wfmt == 
 static inline int chain_xbytes(int wfmt) { return wfmt == kChainW32 ? 4 : chain_kpw(wfmt) * 2; }
 static inline int64_t chain_kw(int64_t k, int wfmt) { return cdiv64(cdiv64(k, chain_kpw(wfmt)), NS) * NS; }
 
-bool chain_supported(int dtype, int64_t m, int64_t k, int64_t n, bool dual, bool norm, int wfmt, bool x_f32) {
+bool chain_supported(int dtype, int64_t m, int64_t k, int64_t n, bool dual, bool norm, int wfmt, bool x_f32, bool plain) {
     if (m != 1 || k < 4 || n < 4) return false;
+    // a width that is not a multiple of 4 (GPT-2's head: 50257): the last tile's missing columns are zero in the copy and are not
+    // stored; only for an unquantised layer without bias and residual (staged values and scales come in pairs)
+    const bool ragged_ok = plain && !dual && (wfmt == kChainW16 || wfmt == kChainW32);
     if (wfmt < kChainW16 || wfmt > kChainW32) return false;
     if (wfmt == kChainW32) {   // f32 weights, activations and output; no SwiGLU pair
-        if (dtype != 0 || dual || k % 4 != 0 || n % 4 != 0 || k > 4 * (MAXI / 2) * NT) return false;
+        if (dtype != 0 || dual || k % 4 != 0 || (n % 4 != 0 && !ragged_ok) || k > 4 * (MAXI / 2) * NT) return false;
         return chain_kw(k, wfmt) * chain_xbytes(wfmt) / 4 <= kChainMaxXsWords;
     }
     if (dtype != 2) return false;
     if (x_f32 && (!norm || k > 4 * (MAXI / 2) * NT)) return false;
-    if (k % 4 != 0 || n % (dual ? 2 : 4) != 0) return false;
+    if (k % 4 != 0 || (n % (dual ? 2 : 4) != 0 && !ragged_ok)) return false;
     if (wfmt == kChainW4 && k % 128 != 0) return false;
     if (norm && k > 4 * MAXI * NT) return false;
     if (chain_kw(k, wfmt) * chain_xbytes(wfmt) / 4 > kChainMaxXsWords) return false;

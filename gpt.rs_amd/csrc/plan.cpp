@@ -795,7 +795,7 @@ void Builder::build() {
         const int wfmt = chain_format(in, ldt);
         if (in.norm_ln && wfmt != k::kChainW32) return 0;   // LayerNorm is staged for f32 phases only
         if (wfmt == k::kChainW32 && (in.norm && !in.norm_ln)) return 0;   // ... and RMSNorm for the others
-        if (!k::chain_supported((int)ldt, x.dims[0], x.dims[1], w.dims[1], dual, in.norm, wfmt, in.x_f32)) return 0;
+        if (!k::chain_supported((int)ldt, x.dims[0], x.dims[1], w.dims[1], dual, in.norm, wfmt, in.x_f32, !in.has_bias && !in.has_residual)) return 0;
         k::ChainPhase p{};
         return k::chain_fill_phase(p, x.dims[1], w.dims[1], dual, wfmt) ? 1 : 0;
     };

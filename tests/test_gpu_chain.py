@@ -71,7 +71,7 @@ def run_both(hip, build, specs, arrays, atol, atol_self, rtol=HALF_ULP):
         assert_close(g, q, atol=atol_self, rtol=ULP, what=f"result {i} vs per-linear kernels")
 
 
-@pytest.mark.parametrize("k,n", [(3072, 6144), (4096, 3072), (9216, 3072), (3072, 1000), (512, 40), (64, 12)])
+@pytest.mark.parametrize("k,n", [(3072, 6144), (4096, 3072), (9216, 3072), (3072, 1000), (512, 40), (64, 12), (3072, 1001), (512, 41), (64, 13), (128, 7)])
 def test_single_linear(hip, k, n):
     x, w = rnd(1, (1, k)), rnd(2, (k, n), 2.0 / np.sqrt(k))
     # inputs are exact in bf16: the result is the f32 dot rounded once
@@ -267,7 +267,7 @@ def run_both_f32(hip, build, specs, arrays, atol=5e-4, rtol=1e-4, phases=1):
         assert_close(g, q, atol=atol, rtol=rtol, what=f"result {i} vs per-linear kernels")
 
 
-@pytest.mark.parametrize("k,n", [(768, 2304), (768, 3072), (3072, 768), (768, 768), (200, 52), (4608, 64), (64, 12)])
+@pytest.mark.parametrize("k,n", [(768, 2304), (768, 3072), (3072, 768), (768, 768), (200, 52), (4608, 64), (64, 12), (768, 50257), (200, 53), (64, 14), (64, 5)])
 def test_f32_single_linear(hip, k, n):
     x, w = rnd(31, (1, k)), rnd(32, (k, n), 2.0 / np.sqrt(k))
     run_both_f32(hip, lambda fb, a, b: a.matmul(b), [[1, k], [k, n]], [x, w])
