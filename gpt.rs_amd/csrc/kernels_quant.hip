@@ -32,6 +32,34 @@ __global__ void scales_kernel(const T* __restrict__ w, T* __restrict__ scales, i
     if (s == 0.f) s = 1.0f;
     stw(scales, idx, s);
 }
+// The same for ONE group (the whole column, int8): a thread per column is a few dozen waves walking K one row at a time, so
+// a workgroup of 16 waves takes 64 columns, wave y the rows y, y + 16, ..., and the 16 maxima of a column meet in LDS
+// (a maximum does not depend on the order it is taken in).
+template <typename T>
+__global__ __launch_bounds__(1024) void column_scales_kernel(const T* __restrict__ w, T* __restrict__ scales, int64_t K, int64_t N, float qmax) {
+    __shared__ float part[16][64];
+    const int c = threadIdx.x & 63, y = threadIdx.x >> 6;
+    const int64_t n = (int64_t)blockIdx.x * 64 + c;
+    float amax = 0.f;
+    if (n < N) {
+        int64_t kk = y;
+        for (; kk + 48 < K; kk += 64) {   // four rows in flight
+            const float a = fabsf(ldw(w, kk * N + n)), b = fabsf(ldw(w, (kk + 16) * N + n));
+            const float d = fabsf(ldw(w, (kk + 32) * N + n)), e = fabsf(ldw(w, (kk + 48) * N + n));
+            amax = fmaxf(fmaxf(amax, fmaxf(a, b)), fmaxf(d, e));
+        }
+        for (; kk < K; kk += 16) amax = fmaxf(amax, fabsf(ldw(w, kk * N + n)));
+    }
+    part[y][c] = amax;
+    __syncthreads();
+    if (y == 0 && n < N) {
+#pragma unroll
+        for (int i = 1; i < 16; ++i) amax = fmaxf(amax, part[i][c]);
+        float s = rbf16(amax / qmax);
+        if (s == 0.f) s = 1.0f;
+        stw(scales, n, s);
+    }
+}
 template <typename T>
 __global__ void quant_w8_kernel(const T* __restrict__ w, const T* __restrict__ scales, int8_t* __restrict__ q, int64_t K, int64_t N) {
     const int64_t total = K * N;
@@ -83,8 +111,9 @@ inline unsigned grid_for(int64_t total) {
 
 void quant_w8_scales(hipStream_t s, int dtype, const void* w, void* scales, int64_t k, int64_t n) {
     if (k <= 0 || n <= 0) return;
-    GPTRS_BY_DTYPE((scales_kernel<float><<<grid_for(n), 256, 0, s>>>((const float*)w, (float*)scales, k, n, k, 127.0f)),
-                   (scales_kernel<bf16_t><<<grid_for(n), 256, 0, s>>>((const bf16_t*)w, (bf16_t*)scales, k, n, k, 127.0f)));
+    const unsigned blocks = (unsigned)((n + 63) / 64);
+    GPTRS_BY_DTYPE((column_scales_kernel<float><<<blocks, 1024, 0, s>>>((const float*)w, (float*)scales, k, n, 127.0f)),
+                   (column_scales_kernel<bf16_t><<<blocks, 1024, 0, s>>>((const bf16_t*)w, (bf16_t*)scales, k, n, 127.0f)));
 }
 void quant_w8(hipStream_t s, int dtype, const void* w, const void* scales, int8_t* q, int64_t k, int64_t n) {
     if (k <= 0 || n <= 0) return;
